@@ -1,0 +1,194 @@
+/*
+ * mi355dnn: C ABI of the MI355X (gfx950) dense-contraction kernels.
+ *
+ * This is the drop-in boundary under the reference's kernel entry points
+ *   matmul!/batchedmatmul!   DNNKernels/src/kernels/extern/matmul.jl:78-79,383
+ *   sdpa / sdpa!             DNNKernels/src/kernels/extern/attention.jl:712,773-834
+ *   convolution!             DNNKernels/src/kernels/extern/conv.jl:100-101
+ *   layernorm!               DNNKernels/src/kernels/layernorm.jl:125
+ * which the op handlers call (DNNKernels/src/ops.jl:575-647,1114-1222,1347-1399).
+ *
+ * Conventions
+ *   - Every data pointer is a DEVICE pointer (hipMalloc); `stream` is a
+ *     hipStream_t passed as void* (NULL = the default stream).  Calls enqueue
+ *     work and return; they never synchronise and never allocate.
+ *   - Arrays are row-major C arrays.  The reference's column-major Julia array
+ *     (a,b,c,d) is the same bytes as the row-major [d][c][b][a]
+ *     (DNNKernels/src/safetensors.jl:7-12), so nothing is copied at the boundary.
+ *   - Leading dimensions and strides are in ELEMENTS.
+ *   - Return value: MI_OK, or a decline code.  A decline is the C form of the
+ *     reference's `Decline(reason)` (DNNKernels/src/kernelplans.jl:21-35): no
+ *     work was enqueued and the caller takes its own fallback.  Nothing throws.
+ *   - Scratch comes from the caller (`ws`, `ws_bytes`): the reference hands
+ *     kernels per-op scratch from its bump workspace, valid until the next op
+ *     (DNNKernels/src/workspace.jl:63-106); the *_workspace functions say how
+ *     much a call needs.  ws must be 256-byte aligned.
+ */
+#ifndef MI355DNN_H
+#define MI355DNN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355DNN_VERSION 1
+
+enum mi_status {
+    MI_OK = 0,
+    MI_DECLINE_OPERANDS = 1,    /* null / misaligned / unsupported layout        (Decline(:operands)) */
+    MI_DECLINE_EXTENT = 2,      /* an extent the kernels do not cover            (Decline(:extent))   */
+    MI_DECLINE_WORKSPACE = 3,   /* ws too small or misaligned                                          */
+    MI_DECLINE_BIAS = 4,        /* a bias/mask shape the call cannot apply       (Decline(:bias))     */
+    MI_DECLINE_UNSUPPORTED = 5, /* e.g. grouped convolution                                            */
+    MI_ERROR_LAUNCH = 6,        /* HIP reported an error at launch                                     */
+    MI_ERROR_DEVICE = 7         /* no gfx950 device / library not initialised                          */
+};
+
+enum mi_epilogue { MI_EPI_NONE = 0, MI_EPI_GELU_ERF = 1, MI_EPI_GELU_TANH = 2, MI_EPI_RELU = 3 };
+enum mi_dtype { MI_F16 = 0, MI_F32 = 1 };
+enum mi_wlayout { MI_W_KF = 0, MI_W_FK = 1 };
+enum mi_bias_mode { MI_BIAS_NONE = 0, MI_BIAS_COL = 1, MI_BIAS_ROW = 2 };
+
+/* Which kernel a GEMM call takes; returned by mi_gemm_f16_plan so a host-side
+ * planner (the reference's `mmplan`, matmul.jl:87-95) can be tested without a launch. */
+enum mi_gemm_path { MI_GEMM_DECLINE = 0, MI_GEMM_MFMA = 1, MI_GEMM_SKINNY = 2, MI_GEMM_SCALAR = 3 };
+enum mi_sdpa_path { MI_SDPA_DECLINE = 0, MI_SDPA_FLASH = 1, MI_SDPA_ROWS = 2 };
+enum mi_conv_path { MI_CONV_DECLINE = 0, MI_CONV_GEMM_1X1 = 1, MI_CONV_IM2COL_GEMM = 2, MI_CONV_DIRECT = 3 };
+
+/* Library / device. */
+int mi_version(void);
+/* Selects nothing and allocates nothing: checks that the current HIP device is
+ * gfx950 and raises the kernels' dynamic-LDS limits.  Idempotent.  Replaces the
+ * reference's `caps(backend)` device query (DNNKernels/src/context.jl:55,68). */
+int mi_init(void);
+/* Device facts a planner needs (the fields of Lava.DeviceCaps the reference
+ * reads, context.jl:68): out[0]=mfma available, [1]=tile (16), [2]=wavefront (64),
+ * [3]=LDS bytes per workgroup, [4]=max workgroup size, [5]=compute units. */
+int mi_device_caps(int64_t out[6]);
+
+/* ---------------------------------------------------------------- GEMM
+ * Y[T x F] = epi(round(X[T x K] . W + bias)) (+ residual)
+ *   X   fp16 [T][K], ldX.
+ *   W   fp16, MI_W_KF: [K][F] (the reference's hoisted weight,
+ *       DNNKernels/src/hoistcasts.jl:47-112) or MI_W_FK: [F][K]; ldW.
+ *   bias fp16 or NULL; MI_BIAS_COL: bias[F] (addmm), MI_BIAS_ROW: bias[T]
+ *       (the reference GEMM's per-row bias of the column-major C, matmul.jl:188-217).
+ *   fp32 accumulation seeded with the bias (matmul.jl:21,230-233), one rounding
+ *   to out_dtype, the activation applied to the ROUNDED value (matmul.jl:210-214).
+ *   residual (fp16, same layout as Y, or NULL; fp16 output only) is added after the
+ *   activation with one more rounding: the graph's own add.Tensor (ops.jl:186-197).
+ * Replaces matmul!(ctx, out, A, B, bias; epi) -- matmul.jl:78-79,99-100,133-137,235-273. */
+int mi_gemm_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,
+                int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                int w_layout, int bias_mode, int epi, int out_dtype,
+                void *ws, size_t ws_bytes, void *stream);
+
+/* The same over `nbatch` planes: element strides sY, sX, sW between planes
+ * (0 = operand shared).  Replaces batchedmatmul!(ctx, out, A, B) -- matmul.jl:364-392
+ * and the nbatch form of the GEMMs in sdpa_coopmat! -- attention.jl:697-699. */
+int mi_gemm_f16_batched(void *Y, const void *X, const void *W, const void *bias, const void *residual,
+                        int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                        int w_layout, int bias_mode, int epi, int out_dtype,
+                        int64_t nbatch, int64_t sY, int64_t sX, int64_t sW,
+                        void *ws, size_t ws_bytes, void *stream);
+
+/* Decode-sized T (<= 16): the bandwidth-bound form, split over K across
+ * workgroups with fp32 partial planes in ws and a reducing epilogue.
+ * The reference's counterpart is the fp32-only Lava.gemv! path
+ * (matmul.jl:108-137) and mm_epilogue_kernel! (matmul.jl:192-217). */
+int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,
+                int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                int w_layout, int bias_mode, int epi, int out_dtype,
+                void *ws, size_t ws_bytes, void *stream);
+
+size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int64_t nbatch);
+/* Returns an mi_gemm_path; never launches.  Replaces mmplan / mm_coopmat_plan /
+ * mm_gemv_plan -- matmul.jl:87-95,121-131,172-179. */
+int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,
+                     int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                     int w_layout, int out_dtype, int64_t nbatch, int64_t sY, int64_t sX, int64_t sW);
+
+/* ---------------------------------------------------------------- attention
+ * out(E,Lq,H,B) = softmax_over_keys(scale * q.k + bias) . v
+ *   q (E,Lq,H,B), k (E,Lk,H,B), v (E,Lk,H,B): fp16, each given as a base pointer
+ *   plus four element strides in (E, L, H, B) order -- the reference passes
+ *   root pointer + offsets + strides the same way (flash.jl:1353-1365,1448-1474).
+ *   out is dense (E,Lq,H,B) = row-major [B][H][Lq][E], fp16 or fp32 (the graph's
+ *   declared type, ops.jl:1365-1391).
+ *   bias: optional additive mask laid out (Lk,Lq,H,B) with element strides
+ *   bias_strides[4]; a stride of 0 broadcasts that axis (attention.jl:55-59,
+ *   launch.jl:72-75); bias_dtype MI_F16 / MI_F32.
+ *   kv_len: optional device int32[B]; keys >= kv_len[b] get weight exactly 0
+ *   (what the decoder's 0 / finfo.min mask does, tools/export_whisper_decoder.py:158-165).
+ *   A row with every key excluded yields zeros, not NaN (attention.jl:82-87).
+ * Replaces sdpa(ctx, q, k, v, bias, scale; out) -- attention.jl:712-834 -- and the
+ * fused kernels behind it: attn_flash_cm! + attn_flash_cm_merge! (flash.jl:459-1036,
+ * 1398-1421), attn_softmax_rows! / sdpa_coopmat! (attention.jl:514-705). */
+int mi_sdpa_f16(void *out, int out_dtype,
+                const void *q, const int64_t q_strides[4],
+                const void *k, const int64_t k_strides[4],
+                const void *v, const int64_t v_strides[4],
+                const void *bias, int bias_dtype, const int64_t bias_strides[4],
+                const int32_t *kv_len,
+                int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale,
+                void *ws, size_t ws_bytes, void *stream);
+size_t mi_sdpa_f16_workspace(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, int has_bias);
+/* Returns an mi_sdpa_path; replaces sdpaplan / flashcm_plan -- attention.jl:735-759,
+ * flash.jl:1322-1374.  nsplit_out (optional) receives the key-split count
+ * (splitcount, flash.jl:1288-1303). */
+int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4],
+                     const void *k, const int64_t k_strides[4],
+                     const void *v, const int64_t v_strides[4],
+                     int has_bias, int has_kv_len,
+                     int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale,
+                     int *nsplit_out);
+
+/* ---------------------------------------------------------------- convolution
+ * Reference layout: x (W,H,Cin,N) = row-major [N][Cin][H][W]; w (KW,KH,Cin,Cout) =
+ * [Cout][Cin][KH][KW]; out (OW,OH,Cout,N); bias[Cout] or NULL; stride / padding /
+ * dilation as (x, y) pairs; act MI_EPI_NONE or MI_EPI_RELU; groups must be 1
+ * (anything else declines, as the reference routes grouped convolutions to its
+ * direct kernel).  fp32 accumulation seeded with the bias, one rounding, relu
+ * on the rounded value.
+ * Replaces convolution!(ctx, out, x, w, bias, stride, padding, dilation, groups; act)
+ * -- conv.jl:100-145 -- and convolution_coopmat! / im2col_kernel! /
+ * conv_epilogue_kernel! -- conv_coopmat.jl:246-392. */
+int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
+                  int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                  int64_t KW, int64_t KH, int64_t Cout,
+                  int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                  int64_t dil_x, int64_t dil_y, int64_t groups, int act,
+                  void *ws, size_t ws_bytes, void *stream);
+size_t mi_conv2d_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                               int64_t KW, int64_t KH, int64_t Cout,
+                               int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                               int64_t dil_x, int64_t dil_y);
+/* Returns an mi_conv_path; replaces conv_coopmat_plan / onebyone -- conv_coopmat.jl:83-155,
+ * conv.jl:63-66. */
+int mi_conv2d_f16_plan(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                       int64_t KW, int64_t KH, int64_t Cout,
+                       int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                       int64_t dil_x, int64_t dil_y, int64_t groups);
+/* ATen's output extent -- convsize, conv.jl:309. */
+int64_t mi_convsize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d);
+
+/* ---------------------------------------------------------------- layer norm + glue
+ * `groups` rows of C contiguous fp16 elements; mean in fp32, variance about that
+ * mean in fp32, out = (x-mean)*rstd*gamma + beta rounded to fp16; mean/rstd
+ * (fp32[groups], either may be NULL) returned as native_layer_norm does.
+ * Replaces layernorm!(ctx, out, mean, rstd, a, gamma, beta, C, eps) -- layernorm.jl:44-135. */
+int mi_layernorm_f16(void *out, float *mean, float *rstd, const void *a,
+                     const void *gamma, const void *beta,
+                     int64_t C, int64_t groups, float eps, void *stream);
+
+/* out = fp16(a + b), n elements: the residual add.Tensor in the operand type
+ * (ops.jl:186-197), for callers that do not fold it into the GEMM store. */
+int mi_add_f16(void *out, const void *a, const void *b, int64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355DNN_H */

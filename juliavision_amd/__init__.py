@@ -1,0 +1,13 @@
+"""MI355X-native (gfx950) dense-contraction kernels behind DNNKernels' kernel entry points.
+
+``juliavision_amd.kernels`` mirrors the reference's ``matmul!`` / ``batchedmatmul!`` /
+``sdpa`` / ``convolution!`` / ``layernorm!`` over the C ABI of ``libmi355dnn.so``
+(declared in ``include/mi355dnn.h``).  Importing this package loads nothing; the
+shared object is opened on first use and its absence is an error, never a fallback.
+"""
+from . import _lib  # noqa: F401
+from .kernels import (Ctx, Decline, DeclineError, DeviceCaps, MI355X, Workspace, add_, batchedmatmul_, caps, conv_plan,
+                      convolution_, convsize, layernorm_, matmul_, mmplan, sdpa, sdpaplan)
+
+__all__ = ["Ctx", "Decline", "DeclineError", "DeviceCaps", "MI355X", "Workspace", "add_", "batchedmatmul_", "caps",
+           "conv_plan", "convolution_", "convsize", "layernorm_", "matmul_", "mmplan", "sdpa", "sdpaplan"]

@@ -1,0 +1,56 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/mi355dnn.h"
+
+typedef _Float16 half_t;
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define MI_DEVICE static __device__ __forceinline__
+
+MI_DEVICE u32x4 ldg16(const half_t *p) { return *reinterpret_cast<const u32x4 *>(p); }
+MI_DEVICE u32x2 ldg8(const half_t *p) { return *reinterpret_cast<const u32x2 *>(p); }
+
+// lo16(x) | lo16(y) << 16   and   hi16(x) | hi16(y) << 16
+MI_DEVICE uint32_t pack_lo(uint32_t x, uint32_t y) { return __builtin_amdgcn_perm(y, x, 0x05040100u); }
+MI_DEVICE uint32_t pack_hi(uint32_t x, uint32_t y) { return __builtin_amdgcn_perm(y, x, 0x07060302u); }
+
+MI_DEVICE half8v as_half8(u32x4 v) { return __builtin_bit_cast(half8v, v); }
+
+// Abramowitz & Stegun 7.1.26 in fp32: the same expression as the reference's
+// `erf` (DNNKernels/src/ops.jl:161-169), so a folded gelu is the graph's gelu.
+MI_DEVICE float erf_as(float x) {
+    float a = fabsf(x);
+    float t = 1.0f / (1.0f + 0.3275911f * a);
+    float y = 1.0f - (((((1.061405429f * t - 1.453152027f) * t) + 1.421413741f) * t - 0.284496736f) * t + 0.254829592f) * t * __expf(-a * a);
+    return x < 0.0f ? -y : y;
+}
+// ops.jl:1665-1669 (geluexact), 1677-1682 (gelutanh), 1683 (relu_epi)
+MI_DEVICE float apply_epi(float v, int epi) {
+    switch (epi) {
+    case MI_EPI_GELU_ERF: return 0.5f * v * (1.0f + erf_as(v * 0.70710678118654752440f));
+    case MI_EPI_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    case MI_EPI_RELU: return fmaxf(v, 0.0f);
+    default: return v;
+    }
+}
+
+static inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline size_t round_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
+
+// True once mi_init has run successfully on this process (defined in gemm.hip).
+bool mi_ready();
+int mi_num_cus();
+int mi_sdpa_init();
+// Y[M x N] = A[M x K] . B (+bias) with B either [K][NB-padded N] (b_kn) or [N][K]; defined in gemm.hip.
+int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
+                     long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
+                     long nbatch, long sY, long sA, long sB, hipStream_t st);

@@ -1,0 +1,188 @@
+// Convolution as GEMM for gfx950, in the reference's layout:
+//   x (W,H,Cin,N) = [N][Cin][H][W],  w (KW,KH,Cin,Cout) = [Cout][Cin][KH][KW],
+//   out (OW,OH,Cout,N) = [N][Cout][OH][OW].
+// Per image:  out[Cout][PQ] = w[Cout][CRS] . col[CRS][PQ]   (PQ = OH*OW pixels)
+// so the weight is the K-contiguous operand as it lies, the pixel axis is the
+// contiguous axis of both col and out, and the bias is per output ROW.
+//   1x1 / stride 1 / no padding : col is x itself, no copy (conv.jl:63-66,117-131)
+//   otherwise                   : im2col into scratch, then the same GEMM
+//                                 (conv_coopmat.jl:246-392)
+//   groups != 1                 : the direct kernel (conv.jl:26-51,298-302)
+#include "common.hpp"
+
+namespace {
+
+struct ConvArgs {
+    const half_t *x, *w, *bias;
+    void *out;
+    int Wi, Hi, Cin, N, KW, KH, Cout, OW, OH;
+    int sx, sy, px, py, dx, dy, groups, relu;
+};
+
+// col[c][m], m fastest: c = (ci, kh, kw) with kw fastest, m = (oh, ow) with ow
+// fastest (the order of im2col_kernel!, conv_coopmat.jl:259-286).  Rows c >= CRS
+// and columns m >= PQ are zero, as are taps that fall in the padding.  32-bit
+// index arithmetic throughout.
+__global__ void im2col_kernel(half_t *col, ConvArgs a, int PQP, int CRSP) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int total = PQP * CRSP;
+    if (idx >= total) return;
+    const int n = blockIdx.y;
+    const int m = idx % PQP, c = idx / PQP;
+    const int PQ = a.OW * a.OH, CRS = a.Cin * a.KH * a.KW;
+    half_t val = (half_t)0.0f;
+    if (m < PQ && c < CRS) {
+        const int ow = m % a.OW, oh = m / a.OW;
+        const int kw = c % a.KW, t = c / a.KW, kh = t % a.KH, ci = t / a.KH;
+        const int ix = ow * a.sx - a.px + kw * a.dx, iy = oh * a.sy - a.py + kh * a.dy;
+        if (ix >= 0 && ix < a.Wi && iy >= 0 && iy < a.Hi)
+            val = a.x[(((long)n * a.Cin + ci) * a.Hi + iy) * a.Wi + ix];
+    }
+    col[(long)n * total + idx] = val;
+}
+
+// wp[co][CRSP] = w[co][CRS] zero-padded
+__global__ void padweight_kernel(half_t *wp, const half_t *w, int Cout, int CRS, int CRSP) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= Cout * CRSP) return;
+    const int c = idx % CRSP, co = idx / CRSP;
+    wp[idx] = c < CRS ? w[(long)co * CRS + c] : (half_t)0.0f;
+}
+
+// One thread per output; fp32 accumulator seeded with the bias; the loop order
+// of the reference's conv2d (conv.jl:26-51).
+__global__ void conv_direct_kernel(ConvArgs a) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)a.N * a.Cout * a.OH * a.OW;
+    if (idx >= total) return;
+    const int ox = (int)(idx % a.OW);
+    long t = idx / a.OW;
+    const int oy = (int)(t % a.OH); t /= a.OH;
+    const int co = (int)(t % a.Cout);
+    const int n = (int)(t / a.Cout);
+    const int cing = a.Cin / a.groups, coutg = a.Cout / a.groups;
+    const int g = co / coutg;
+    float acc = a.bias ? (float)a.bias[co] : 0.0f;
+    for (int ci = 0; ci < cing; ci++) {
+        const int xc = g * cing + ci;
+        for (int ky = 0; ky < a.KH; ky++) {
+            const int iy = oy * a.sy - a.py + ky * a.dy;
+            if (iy < 0 || iy >= a.Hi) continue;
+            for (int kx = 0; kx < a.KW; kx++) {
+                const int ix = ox * a.sx - a.px + kx * a.dx;
+                if (ix < 0 || ix >= a.Wi) continue;
+                acc = fmaf((float)a.x[(((long)n * a.Cin + xc) * a.Hi + iy) * a.Wi + ix],
+                           (float)a.w[(((long)co * cing + ci) * a.KH + ky) * a.KW + kx], acc);
+            }
+        }
+    }
+    half_t r = (half_t)acc;
+    if (a.relu && (float)r < 0.0f) r = (half_t)0.0f;
+    reinterpret_cast<half_t *>(a.out)[idx] = r;
+}
+
+bool onebyone(const ConvArgs &a) {   // conv.jl:63-66
+    return a.groups == 1 && a.KW == 1 && a.KH == 1 && a.sx == 1 && a.sy == 1 && a.px == 0 && a.py == 0 && a.dx == 1 && a.dy == 1;
+}
+
+int fill(ConvArgs &a, void *out, const void *x, const void *w, const void *bias,
+         int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, int64_t KW, int64_t KH, int64_t Cout,
+         int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy, int64_t groups, int act) {
+    if (Wi < 1 || Hi < 1 || Cin < 1 || N < 0 || KW < 1 || KH < 1 || Cout < 1) return MI_DECLINE_EXTENT;
+    if (sx < 1 || sy < 1 || dx < 1 || dy < 1 || px < 0 || py < 0 || groups < 1) return MI_DECLINE_EXTENT;
+    if (Cin % groups || Cout % groups) return MI_DECLINE_EXTENT;
+    if (act != MI_EPI_NONE && act != MI_EPI_RELU) return MI_DECLINE_UNSUPPORTED;
+    int64_t OW = mi_convsize(Wi, KW, sx, px, dx), OH = mi_convsize(Hi, KH, sy, py, dy);
+    if (OW < 1 || OH < 1) return MI_DECLINE_EXTENT;
+    if (Wi * Hi * Cin > INT32_MAX || OW * OH * Cout > INT32_MAX || Cin * KW * KH > INT32_MAX / 8 || N > 65535) return MI_DECLINE_EXTENT;
+    a.x = (const half_t *)x; a.w = (const half_t *)w; a.bias = (const half_t *)bias; a.out = out;
+    a.Wi = (int)Wi; a.Hi = (int)Hi; a.Cin = (int)Cin; a.N = (int)N; a.KW = (int)KW; a.KH = (int)KH; a.Cout = (int)Cout;
+    a.OW = (int)OW; a.OH = (int)OH;
+    a.sx = (int)sx; a.sy = (int)sy; a.px = (int)px; a.py = (int)py; a.dx = (int)dx; a.dy = (int)dy;
+    a.groups = (int)groups; a.relu = act == MI_EPI_RELU;
+    return MI_OK;
+}
+
+int conv_path(const ConvArgs &a) {
+    if (a.groups != 1) return MI_CONV_DIRECT;
+    if (onebyone(a)) return MI_CONV_GEMM_1X1;
+    return MI_CONV_IM2COL_GEMM;
+}
+
+void im2col_extents(const ConvArgs &a, int64_t &PQP, int64_t &CRSP) {
+    PQP = round_up((size_t)a.OW * a.OH, 8);
+    CRSP = round_up((size_t)a.Cin * a.KH * a.KW, 8);
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t mi_convsize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d) { return (n + 2 * p - d * (k - 1) - 1) / s + 1; }
+
+int mi_conv2d_f16_plan(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, int64_t KW, int64_t KH, int64_t Cout,
+                       int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy, int64_t groups) {
+    ConvArgs a;
+    if (fill(a, nullptr, nullptr, nullptr, nullptr, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, groups, MI_EPI_NONE) != MI_OK)
+        return MI_CONV_DECLINE;
+    return conv_path(a);
+}
+
+size_t mi_conv2d_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, int64_t KW, int64_t KH, int64_t Cout,
+                               int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy) {
+    ConvArgs a;
+    if (fill(a, nullptr, nullptr, nullptr, nullptr, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, 1, MI_EPI_NONE) != MI_OK) return 0;
+    if (conv_path(a) != MI_CONV_IM2COL_GEMM) return 0;
+    int64_t PQP, CRSP;
+    im2col_extents(a, PQP, CRSP);
+    size_t col = round_up((size_t)N * PQP * CRSP * 2, 256);
+    size_t wp = CRSP != (int64_t)Cin * KH * KW ? round_up((size_t)Cout * CRSP * 2, 256) : 0;
+    return col + wp;
+}
+
+int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
+                  int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, int64_t KW, int64_t KH, int64_t Cout,
+                  int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy, int64_t groups, int act,
+                  void *ws, size_t ws_bytes, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !x || !w) return MI_DECLINE_OPERANDS;
+    ConvArgs a;
+    int rc = fill(a, out, x, w, bias, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, groups, act);
+    if (rc != MI_OK) return rc;
+    if (N == 0) return MI_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int path = conv_path(a);
+    const int PQ = a.OW * a.OH;
+    const int epi = a.relu ? MI_EPI_RELU : MI_EPI_NONE;
+    if (path == MI_CONV_DIRECT) {
+        long total = (long)a.N * a.Cout * PQ;
+        hipLaunchKernelGGL(conv_direct_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a);
+        return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+    }
+    if (path == MI_CONV_GEMM_1X1) {
+        // out[n][Cout][PQ] = w[Cout][Cin] . x[n][Cin][PQ]; the [K][N] operand needs
+        // PQ % 8 == 0 for 16-byte loads, otherwise the scalar GEMM takes it.
+        return mi_internal_gemm(out, w, x, bias, a.Cout, PQ, PQ, a.Cin, PQ, a.Cin, PQ, 1, MI_BIAS_ROW, epi, 0,
+                                a.N, (long)a.Cout * PQ, 0, (long)a.Cin * PQ, st);
+    }
+    int64_t PQP, CRSP;
+    im2col_extents(a, PQP, CRSP);
+    const int CRS = a.Cin * a.KH * a.KW;
+    size_t col_bytes = round_up((size_t)N * PQP * CRSP * 2, 256);
+    size_t wp_bytes = CRSP != CRS ? round_up((size_t)Cout * CRSP * 2, 256) : 0;
+    if (!ws || ws_bytes < col_bytes + wp_bytes || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
+    if (PQP * CRSP > INT32_MAX) return MI_DECLINE_EXTENT;
+    half_t *col = reinterpret_cast<half_t *>(ws);
+    const half_t *wuse = a.w;
+    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)ceil_div(PQP * CRSP, 256), (unsigned)a.N), dim3(256), 0, st, col, a, (int)PQP, (int)CRSP);
+    if (wp_bytes) {
+        half_t *wp = reinterpret_cast<half_t *>(reinterpret_cast<char *>(ws) + col_bytes);
+        hipLaunchKernelGGL(padweight_kernel, dim3((unsigned)ceil_div((int64_t)Cout * CRSP, 256)), dim3(256), 0, st, wp, a.w, a.Cout, CRS, (int)CRSP);
+        wuse = wp;
+    }
+    if (hipGetLastError() != hipSuccess) return MI_ERROR_LAUNCH;
+    return mi_internal_gemm(out, wuse, col, bias, a.Cout, PQ, (int)PQP, (int)CRSP, PQ, CRSP, PQP, 1, MI_BIAS_ROW, epi, 0,
+                            a.N, (long)a.Cout * PQ, 0, PQP * CRSP, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,656 @@
+// fp16 GEMM for gfx950: MFMA 32x32x16 f16 with fp32 accumulation, LDS
+// double-buffered operand tiles, 128-bit global loads, fused bias / activation /
+// residual store; a split-K bandwidth kernel for decode-sized T; a scalar
+// kernel for operands the tiled kernels cannot address.
+//
+// Internal problem statement (row-major):  Y[M x N] = A[M x K] . B  (+ bias)
+//   A is K-contiguous.  B is either N-contiguous [K][N] (B_KN) or K-contiguous
+//   [N][K].  For a linear layer M = tokens, N = features, A = X, B = W.
+#include "common.hpp"
+#include <type_traits>
+
+namespace {
+
+struct GemmArgs {
+    void *Y;
+    const half_t *A, *B, *bias, *residual;
+    int M, N, K;
+    int NB;                 // columns addressable in B (>= N; a multiple of 8 for the [K][N] layout)
+    long ldY, ldA, ldB;
+    long sY, sA, sB;        // batch strides (elements)
+    int bias_mode, epi, out_f32;
+    int tiles_m, tiles_n, group_m;
+    int vec_store;          // Y (and residual) rows allow 16-byte accesses
+};
+
+// ------------------------------------------------------------------------------------------
+// Staging of a K-contiguous operand tile ROWS x BK: each thread moves 16-byte
+// chunks global -> registers -> LDS rows of BK+8 halves (the 16-byte pad makes
+// the 32 rows an MFMA operand read touches fall in distinct bank groups).
+template <int ROWS, int BK, int NT>
+struct KcStage {
+    static constexpr int CPR = BK / 8;
+    static constexpr int CHUNKS = ROWS * CPR;
+    static constexpr int PER = (CHUNKS + NT - 1) / NT;
+    static constexpr int LD = BK + 8;
+    u32x4 r[PER];
+
+    __device__ __forceinline__ void load(const half_t *base, long ld, int row0, int nrows, int k0, int K, int tid) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            int c = tid + i * NT;
+            int row = c / CPR, kc = c % CPR;
+            int gr = min(row0 + row, nrows - 1);
+            int gk = k0 + kc * 8;
+            u32x4 z = {0u, 0u, 0u, 0u};
+            if (CHUNKS % NT == 0 || c < CHUNKS) r[i] = gk < K ? ldg16(base + (long)gr * ld + gk) : z;
+        }
+    }
+    __device__ __forceinline__ void store(half_t *lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            int c = tid + i * NT;
+            int row = c / CPR, kc = c % CPR;
+            if (CHUNKS % NT == 0 || c < CHUNKS) *reinterpret_cast<u32x4 *>(lds + row * LD + kc * 8) = r[i];
+        }
+    }
+};
+
+// Staging of an N-contiguous operand tile [BK][COLS] into the same K-contiguous
+// LDS rows: a thread loads an 8(k) x 8(n) block with eight 16-byte row loads,
+// transposes it in registers (v_perm_b32) and writes eight 16-byte LDS rows.
+template <int COLS, int BK, int NT>
+struct KnStage {
+    static constexpr int KB = BK / 8;
+    static constexpr int BLOCKS = KB * (COLS / 8);
+    static constexpr int PER = (BLOCKS + NT - 1) / NT;
+    static constexpr int LD = BK + 8;
+    u32x4 r[PER][8];
+
+    __device__ __forceinline__ void load(const half_t *base, long ld, int col0, int ncols, int k0, int K, int tid) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            int blk = tid + i * NT;
+            int kb = blk % KB, nb = blk / KB;
+            int gn = min(col0 + nb * 8, ncols - 8);
+            if (BLOCKS % NT == 0 || blk < BLOCKS) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    int gk = k0 + kb * 8 + j;
+                    u32x4 z = {0u, 0u, 0u, 0u};
+                    r[i][j] = gk < K ? ldg16(base + (long)gk * ld + gn) : z;
+                }
+            }
+        }
+    }
+    __device__ __forceinline__ void store(half_t *lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            int blk = tid + i * NT;
+            int kb = blk % KB, nb = blk / KB;
+            if (BLOCKS % NT == 0 || blk < BLOCKS) {
+#pragma unroll
+                for (int w = 0; w < 4; w++) {   // dword w of each row holds columns 2w, 2w+1
+                    u32x4 lo, hi;
+                    lo.x = pack_lo(r[i][0][w], r[i][1][w]); hi.x = pack_hi(r[i][0][w], r[i][1][w]);
+                    lo.y = pack_lo(r[i][2][w], r[i][3][w]); hi.y = pack_hi(r[i][2][w], r[i][3][w]);
+                    lo.z = pack_lo(r[i][4][w], r[i][5][w]); hi.z = pack_hi(r[i][4][w], r[i][5][w]);
+                    lo.w = pack_lo(r[i][6][w], r[i][7][w]); hi.w = pack_hi(r[i][6][w], r[i][7][w]);
+                    *reinterpret_cast<u32x4 *>(lds + (nb * 8 + 2 * w) * LD + kb * 8) = lo;
+                    *reinterpret_cast<u32x4 *>(lds + (nb * 8 + 2 * w + 1) * LD + kb * 8) = hi;
+                }
+            }
+        }
+    }
+};
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+// Workgroup id -> output tile.  The hardware deals consecutive workgroups
+// round-robin over the 8 XCDs, each with its own L2; this hands every XCD one
+// contiguous run of the tile order, and the tile order walks GROUP_M row tiles
+// per column tile so a run reuses a small set of A and B panels.
+__device__ __forceinline__ void tile_of(int pid, int nwg, int tiles_m, int tiles_n, int group_m, int &tm, int &tn) {
+    int xcd = pid & 7, idx = pid >> 3;
+    int full = nwg >> 3, rem = nwg & 7;
+    int logical = xcd * full + min(xcd, rem) + idx;
+    int width = group_m * tiles_n;
+    int g = logical / width, in = logical - g * width;
+    int first = g * group_m;
+    int gsz = min(tiles_m - first, group_m);
+    tm = first + in % gsz;
+    tn = in / gsz;
+}
+
+// ------------------------------------------------------------------------------------------
+// The tiled MFMA kernel.  BM x BN output tile per workgroup, WAVES_M x WAVES_N
+// waves, each owning a (BM/WAVES_M) x (BN/WAVES_N) sub-tile as 32x32 MFMA
+// tiles.  The MFMA is issued "transposed" (rows = n, columns = m) so that a
+// lane's four consecutive accumulator registers are four consecutive n of one
+// output row: an 8-byte fp16 store.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool B_KN>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma_kernel(GemmArgs p) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int LD = BK + 8;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    extern __shared__ __align__(16) char smem[];
+    half_t *As = reinterpret_cast<half_t *>(smem);   // [2][BM][LD]
+    half_t *Bs = As + 2 * BM * LD;                   // [2][BN][LD]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    int tm_, tn_;
+    tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
+    const int m0 = tm_ * BM, n0 = tn_ * BN;
+    const long bz = blockIdx.y;
+    const half_t *A = p.A + bz * p.sA;
+    const half_t *B = p.B + bz * p.sB;
+
+    KcStage<BM, BK, NT> sa;
+    KcStage<BN, BK, NT> sbk;
+    KnStage<BN, BK, NT> sbn;
+
+    float16v acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    const int nk = (p.K + BK - 1) / BK;
+    sa.load(A, p.ldA, m0, p.M, 0, p.K, tid);
+    if (B_KN) sbn.load(B, p.ldB, n0, p.NB, 0, p.K, tid); else sbk.load(B, p.ldB, n0, p.N, 0, p.K, tid);
+    sa.store(As, tid);
+    if (B_KN) sbn.store(Bs, tid); else sbk.store(Bs, tid);
+    __syncthreads();
+
+    const int frow = lane & 31, fk = (lane >> 5) * 8;
+    for (int kt = 0; kt < nk; kt++) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < nk;
+        if (more) {
+            sa.load(A, p.ldA, m0, p.M, (kt + 1) * BK, p.K, tid);
+            if (B_KN) sbn.load(B, p.ldB, n0, p.NB, (kt + 1) * BK, p.K, tid); else sbk.load(B, p.ldB, n0, p.N, (kt + 1) * BK, p.K, tid);
+        }
+        const half_t *as = As + cur * BM * LD + (wm * WTM + frow) * LD + fk;
+        const half_t *bs = Bs + cur * BN * LD + (wn * WTN + frow) * LD + fk;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) {
+            half8v fa[TM], fb[TN];
+#pragma unroll
+            for (int j = 0; j < TM; j++) fa[j] = *reinterpret_cast<const half8v *>(as + j * 32 * LD + ks * 16);
+#pragma unroll
+            for (int i = 0; i < TN; i++) fb[i] = *reinterpret_cast<const half8v *>(bs + i * 32 * LD + ks * 16);
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int j = 0; j < TM; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[i], fa[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            sa.store(As + (cur ^ 1) * BM * LD, tid);
+            if (B_KN) sbn.store(Bs + (cur ^ 1) * BN * LD, tid); else sbk.store(Bs + (cur ^ 1) * BN * LD, tid);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue.  acc[i][j][r]: n = n0 + wn*WTN + 32 i + 8 (r/4) + 4 (lane/32) + r%4,
+    //                          m = m0 + wm*WTM + 32 j + lane%32.
+    // Each wave stages one 32 x WTN sub-tile at a time in its own LDS region
+    // (bias joined in fp32, one rounding), then reads it back row-wise so that the
+    // activation, the residual add and the global stores run on 16-byte vectors
+    // that are contiguous along the output row.
+    constexpr int SLD_H = WTN + 8;                 // halves per staged row (fp16 output)
+    constexpr int SLD_F = WTN + 4;                 // floats per staged row (fp32 output)
+    constexpr int STAGE_BYTES = 32 * SLD_F * 4;
+    static_assert(STAGE_BYTES * WAVES_M * WAVES_N <= 2 * (BM + BN) * LD * 2, "epilogue staging exceeds the operand LDS");
+    char *stage = smem + wave * STAGE_BYTES;
+    const int hl = lane >> 5;
+    static_for<TM>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+        const int mrow = m0 + wm * WTM + 32 * j;
+        const float brow = (p.bias_mode == MI_BIAS_ROW && mrow + frow < p.M) ? (float)p.bias[mrow + frow] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int nl = 32 * i + 8 * g + 4 * hl;
+                const int n = n0 + wn * WTN + nl;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + brow;
+                if (p.bias_mode == MI_BIAS_COL) {
+                    if (n + 3 < p.N) {
+                        half4v bv = *reinterpret_cast<const half4v *>(p.bias + n);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] += (float)bv[e];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) if (n + e < p.N) v[e] += (float)p.bias[n + e];
+                    }
+                }
+                if (p.out_f32) {
+                    float4v o = {v[0], v[1], v[2], v[3]};
+                    *reinterpret_cast<float4v *>(reinterpret_cast<float *>(stage) + frow * SLD_F + nl) = o;
+                } else {
+                    half4v o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(stage) + frow * SLD_H + nl) = o;
+                }
+            }
+        }
+        __syncthreads();
+        if (p.out_f32) {
+            constexpr int CPR = WTN / 4;
+            for (int c = lane; c < 32 * CPR; c += 64) {
+                const int row = c / CPR, ch = c % CPR;
+                const int m = mrow + row, n = n0 + wn * WTN + ch * 4;
+                if (m < p.M && n < p.N) {
+                    float4v x = *reinterpret_cast<const float4v *>(reinterpret_cast<const float *>(stage) + row * SLD_F + ch * 4);
+                    float *yp = reinterpret_cast<float *>(p.Y) + bz * p.sY + (long)m * p.ldY + n;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[e] = apply_epi(x[e], p.epi);
+                    if (p.vec_store && n + 3 < p.N) *reinterpret_cast<float4v *>(yp) = x;
+                    else for (int e = 0; e < 4; e++) if (n + e < p.N) yp[e] = x[e];
+                }
+            }
+        } else {
+            constexpr int CPR = WTN / 8;
+            for (int c = lane; c < 32 * CPR; c += 64) {
+                const int row = c / CPR, ch = c % CPR;
+                const int m = mrow + row, n = n0 + wn * WTN + ch * 8;
+                if (m < p.M && n < p.N) {
+                    half8v x = *reinterpret_cast<const half8v *>(reinterpret_cast<const half_t *>(stage) + row * SLD_H + ch * 8);
+                    const long off = bz * p.sY + (long)m * p.ldY + n;
+                    half_t *yp = reinterpret_cast<half_t *>(p.Y) + off;
+                    if (p.epi != MI_EPI_NONE) {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) x[e] = (half_t)apply_epi((float)x[e], p.epi);
+                    }
+                    if (p.vec_store && n + 7 < p.N) {
+                        if (p.residual) {
+                            half8v rv = as_half8(ldg16(p.residual + off));
+#pragma unroll
+                            for (int e = 0; e < 8; e++) x[e] = (half_t)((float)x[e] + (float)rv[e]);
+                        }
+                        *reinterpret_cast<half8v *>(yp) = x;
+                    } else {
+                        for (int e = 0; e < 8; e++) {
+                            if (n + e < p.N) {
+                                half_t o = x[e];
+                                if (p.residual) o = (half_t)((float)o + (float)p.residual[off + e]);
+                                yp[e] = o;
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    });
+}
+
+// ------------------------------------------------------------------------------------------
+// Scalar kernel: one thread per output, fp32 accumulation seeded with the bias,
+// any strides.  The arithmetic of the reference's mm2 (matmul.jl:17-27).
+__global__ void gemm_scalar_kernel(GemmArgs p, int b_kn) {
+    long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long total = (long)p.M * p.N;
+    if (idx >= total) return;
+    int n = (int)(idx % p.N), m = (int)(idx / p.N);
+    long bz = blockIdx.y;
+    const half_t *A = p.A + bz * p.sA + (long)m * p.ldA;
+    const half_t *B = p.B + bz * p.sB;
+    float acc = p.bias_mode == MI_BIAS_COL ? (float)p.bias[n] : p.bias_mode == MI_BIAS_ROW ? (float)p.bias[m] : 0.0f;
+    if (b_kn) for (int k = 0; k < p.K; k++) acc = fmaf((float)A[k], (float)B[(long)k * p.ldB + n], acc);
+    else      for (int k = 0; k < p.K; k++) acc = fmaf((float)A[k], (float)B[(long)n * p.ldB + k], acc);
+    long off = bz * p.sY + (long)m * p.ldY + n;
+    if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(acc, p.epi);
+    else {
+        half_t o = (half_t)apply_epi((float)(half_t)acc, p.epi);
+        if (p.residual) o = (half_t)((float)o + (float)p.residual[off]);
+        reinterpret_cast<half_t *>(p.Y)[off] = o;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Decode-sized M (<= 16): bandwidth-bound.  Every weight byte is read once with
+// 16-byte loads; K is split over workgroups so that the whole chip pulls on HBM;
+// each split writes an fp32 partial plane, and a small epilogue sums the planes
+// (the reference's split-K planes + mm_epilogue_kernel!, matmul.jl:192-217).
+//
+// KN layout: a thread owns 8 consecutive n; 32 threads span 256 n; the 8 thread
+// rows of a workgroup take interleaved k.  Row partials are reduced through LDS.
+template <int MT>
+__global__ __launch_bounds__(256) void skinny_kn_kernel(GemmArgs p, float *part, int kper) {
+    __shared__ float red[8][256 + 4];
+    __shared__ half_t xs[MT][512];   // the k-slice of A for this workgroup (kper <= 512)
+    const int tid = threadIdx.x, col = tid & 31, row = tid >> 5;
+    const int n = blockIdx.x * 256 + col * 8;
+    const int split = blockIdx.y;
+    const int k0 = split * kper, k1 = min(p.K, k0 + kper);
+    for (int i = tid; i < MT * kper; i += 256) {
+        int m = i / kper, k = i % kper;
+        xs[m][k] = (m < p.M && k0 + k < p.K) ? p.A[(long)m * p.ldA + k0 + k] : (half_t)0.0f;
+    }
+    __syncthreads();
+    float acc[MT][8];
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[m][e] = 0.0f;
+    if (n < p.N) {
+        const half_t *bp = p.B + n;
+        for (int k = k0 + row; k < k1; k += 8) {
+            half8v w = as_half8(ldg16(bp + (long)k * p.ldB));
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                float x = (float)xs[m][k - k0];
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[m][e] = fmaf(x, (float)w[e], acc[m][e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) red[row][col * 8 + e] = acc[m][e];
+        __syncthreads();
+        int nn = blockIdx.x * 256 + tid;
+        if (m < p.M && nn < p.N) {
+            float s = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 8; r++) s += red[r][tid];
+            part[((long)split * p.M + m) * p.N + nn] = s;
+        }
+        __syncthreads();
+    }
+}
+
+// FK layout ([N][K], K-contiguous): one wave per output column n, lanes stride
+// K in 16-byte chunks, wave reduction.  No split needed: N waves fill the chip.
+template <int MT>
+__global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p, float *part) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = blockIdx.x * 4 + wave;
+    if (n >= p.N) return;
+    const half_t *bp = p.B + (long)n * p.ldB;
+    float acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; m++) acc[m] = 0.0f;
+    for (int k = lane * 8; k < p.K; k += 512) {
+        half8v w = as_half8(ldg16(bp + k));
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            if (m < p.M) {
+                half8v x = as_half8(ldg16(p.A + (long)m * p.ldA + k));
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[m] = fmaf((float)x[e], (float)w[e], acc[m]);
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+        float s = acc[m];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        if (lane == 0 && m < p.M) part[(long)m * p.N + n] = s;
+    }
+}
+
+// out[m][n] = epi(round(sum_s part[s][m][n] + bias)) (+ residual)
+__global__ void skinny_epilogue_kernel(GemmArgs p, const float *part, int nsplit) {
+    long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long total = (long)p.M * p.N;
+    if (idx >= total) return;
+    int n = (int)(idx % p.N), m = (int)(idx / p.N);
+    float v = p.bias_mode == MI_BIAS_COL ? (float)p.bias[n] : p.bias_mode == MI_BIAS_ROW ? (float)p.bias[m] : 0.0f;
+    for (int s = 0; s < nsplit; s++) v += part[(long)s * total + idx];
+    long off = (long)m * p.ldY + n;
+    if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(v, p.epi);
+    else {
+        half_t o = (half_t)apply_epi((float)(half_t)v, p.epi);
+        if (p.residual) o = (half_t)((float)o + (float)p.residual[off]);
+        reinterpret_cast<half_t *>(p.Y)[off] = o;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+bool g_ready = false;
+int g_cus = 256;
+
+template <typename KernelT>
+int raise_lds(KernelT kern, int bytes) {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? 0 : 1;
+}
+
+template <int BM, int BN, int BK>
+constexpr int gemm_lds_bytes() { return 2 * (BM + BN) * (BK + 8) * 2; }
+
+#define GEMM_BIG 128, 256, 64, 2, 2
+#define GEMM_MID 128, 128, 64, 2, 2
+#define GEMM_SMALL 64, 64, 64, 2, 2
+
+int skinny_splits(int64_t K, int64_t F) {
+    // Enough workgroups to put ~2 on every CU, k-slices a multiple of 8 and <= 512.
+    int64_t colblocks = ceil_div(F, 256);
+    int64_t want = ceil_div(2 * (int64_t)g_cus, colblocks);
+    int64_t kper = round_up((size_t)ceil_div(K, want), 8);
+    if (kper < 32) kper = 32;
+    if (kper > 512) kper = 512;
+    return (int)ceil_div(K, kper);
+}
+
+bool mfma_addressable(const GemmArgs &a, bool b_kn) {
+    if (a.K % 8 || a.ldA % 8 || a.ldB % 8 || a.sA % 8 || a.sB % 8) return false;
+    if (!aligned_to(a.A, 16) || !aligned_to(a.B, 16)) return false;
+    if (b_kn && (a.NB % 8 || a.NB < 8 || a.NB < a.N)) return false;
+    if (a.bias && a.bias_mode == MI_BIAS_COL && !aligned_to(a.bias, 8)) return false;
+    return a.M >= 1 && a.N >= 1 && a.K >= 8;
+}
+
+template <int BM, int BN, int BK, int WM, int WN>
+int launch_mfma(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
+    a.tiles_m = (int)ceil_div(a.M, BM);
+    a.tiles_n = (int)ceil_div(a.N, BN);
+    a.group_m = a.tiles_m < 6 ? a.tiles_m : 6;
+    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
+                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
+    constexpr int lds = gemm_lds_bytes<BM, BN, BK>();
+    if (b_kn) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, BK, WM, WN, true>), grid, dim3(WM * WN * 64), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, BK, WM, WN, false>), grid, dim3(WM * WN * 64), lds, st, a);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int gemm_path(const GemmArgs &a, bool b_kn, int64_t nbatch) {
+    if (a.M < 1 || a.N < 1 || a.K < 1) return MI_GEMM_DECLINE;
+    bool addr = mfma_addressable(a, b_kn);
+    if (a.M <= 8 && nbatch == 1 && addr) return MI_GEMM_SKINNY;
+    if (addr) return MI_GEMM_MFMA;
+    return MI_GEMM_SCALAR;
+}
+
+int run_skinny(GemmArgs a, bool b_kn, void *ws, size_t ws_bytes, hipStream_t st) {
+    int nsplit = b_kn ? skinny_splits(a.K, a.N) : 1;
+    size_t need = (size_t)nsplit * a.M * a.N * sizeof(float);
+    if (!ws || ws_bytes < need || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
+    float *part = reinterpret_cast<float *>(ws);
+    if (b_kn) {
+        int kper = (int)round_up((size_t)ceil_div(a.K, nsplit), 8);
+        dim3 grid((unsigned)ceil_div(a.N, 256), (unsigned)nsplit);
+        if (a.M <= 1)      hipLaunchKernelGGL(skinny_kn_kernel<1>, grid, dim3(256), 0, st, a, part, kper);
+        else if (a.M <= 4) hipLaunchKernelGGL(skinny_kn_kernel<4>, grid, dim3(256), 0, st, a, part, kper);
+        else if (a.M <= 8) hipLaunchKernelGGL(skinny_kn_kernel<8>, grid, dim3(256), 0, st, a, part, kper);
+        else return MI_DECLINE_EXTENT;
+    } else {
+        dim3 grid((unsigned)ceil_div(a.N, 4));
+        if (a.M <= 1)      hipLaunchKernelGGL(skinny_fk_kernel<1>, grid, dim3(256), 0, st, a, part);
+        else if (a.M <= 4) hipLaunchKernelGGL(skinny_fk_kernel<4>, grid, dim3(256), 0, st, a, part);
+        else if (a.M <= 8) hipLaunchKernelGGL(skinny_fk_kernel<8>, grid, dim3(256), 0, st, a, part);
+        else return MI_DECLINE_EXTENT;
+    }
+    long total = (long)a.M * a.N;
+    hipLaunchKernelGGL(skinny_epilogue_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a, part, nsplit);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bias, const void *residual,
+              int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+              int w_layout, int bias_mode, int epi, int out_dtype, int64_t sY, int64_t sX, int64_t sW) {
+    if (!Y || !X || !W) return MI_DECLINE_OPERANDS;
+    if (T < 0 || K < 0 || F < 0 || T > INT32_MAX || K > INT32_MAX || F > INT32_MAX) return MI_DECLINE_EXTENT;
+    if (w_layout != MI_W_KF && w_layout != MI_W_FK) return MI_DECLINE_OPERANDS;
+    if (out_dtype != MI_F16 && out_dtype != MI_F32) return MI_DECLINE_OPERANDS;
+    if (epi < MI_EPI_NONE || epi > MI_EPI_RELU) return MI_DECLINE_UNSUPPORTED;
+    if (bias_mode < MI_BIAS_NONE || bias_mode > MI_BIAS_ROW) return MI_DECLINE_BIAS;
+    if (bias_mode != MI_BIAS_NONE && !bias) return MI_DECLINE_BIAS;
+    if (residual && out_dtype != MI_F16) return MI_DECLINE_UNSUPPORTED;
+    if (ldX < K || ldY < F || ldW < (w_layout == MI_W_KF ? F : K)) return MI_DECLINE_EXTENT;
+    a.Y = Y; a.A = (const half_t *)X; a.B = (const half_t *)W;
+    a.bias = bias_mode == MI_BIAS_NONE ? nullptr : (const half_t *)bias;
+    a.residual = (const half_t *)residual;
+    a.M = (int)T; a.N = (int)F; a.K = (int)K; a.NB = (int)F;
+    a.ldY = ldY; a.ldA = ldX; a.ldB = ldW; a.sY = sY; a.sA = sX; a.sB = sW;
+    a.bias_mode = bias_mode; a.epi = epi; a.out_f32 = out_dtype == MI_F32;
+    a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
+    return MI_OK;
+}
+
+int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, hipStream_t st, int force_path) {
+    if (!g_ready) return MI_ERROR_DEVICE;
+    if (a.M == 0 || a.N == 0 || nbatch == 0) return MI_OK;
+    int path = force_path ? force_path : gemm_path(a, b_kn, nbatch);
+    if (path == MI_GEMM_DECLINE) return MI_DECLINE_EXTENT;
+    if (path == MI_GEMM_SKINNY) return run_skinny(a, b_kn, ws, ws_bytes, st);
+    if (path == MI_GEMM_MFMA) {
+        if (!mfma_addressable(a, b_kn)) return MI_DECLINE_OPERANDS;
+        // Tile choice: the big tile when it still gives every CU a workgroup,
+        // else smaller tiles so small problems spread over the chip.
+        int64_t big = ceil_div(a.M, 128) * ceil_div(a.N, 256) * nbatch;
+        int64_t mid = ceil_div(a.M, 128) * ceil_div(a.N, 128) * nbatch;
+        if (big >= (g_cus * 3) / 4) return launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
+        if (mid >= (g_cus * 3) / 4) return launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
+        return launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
+    }
+    long total = (long)a.M * a.N;
+    hipLaunchKernelGGL(gemm_scalar_kernel, dim3((unsigned)ceil_div(total, 256), (unsigned)nbatch), dim3(256), 0, st, a, b_kn ? 1 : 0);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+}  // namespace
+
+bool mi_ready() { return g_ready; }
+int mi_num_cus() { return g_cus; }
+
+// Internal entry used by the convolution path (conv.hip): Y[M x N] = A . B with
+// every GemmArgs field meaningful.
+int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
+                     long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
+                     long nbatch, long sY, long sA, long sB, hipStream_t st) {
+    GemmArgs a;
+    a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
+    a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB;
+    a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
+    a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
+    int path = mfma_addressable(a, b_kn != 0) ? MI_GEMM_MFMA : MI_GEMM_SCALAR;
+    return run_gemm(a, b_kn != 0, nbatch, nullptr, 0, st, path);
+}
+
+extern "C" {
+
+int mi_version(void) { return MI355DNN_VERSION; }
+
+int mi_init(void) {
+    if (g_ready) return MI_OK;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MI_ERROR_DEVICE;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return MI_ERROR_DEVICE;
+    if (__builtin_strncmp(prop.gcnArchName, "gfx950", 6) != 0) return MI_ERROR_DEVICE;
+    g_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    int bad = 0;
+    bad |= raise_lds(gemm_mfma_kernel<GEMM_BIG, true>, gemm_lds_bytes<128, 256, 64>());
+    bad |= raise_lds(gemm_mfma_kernel<GEMM_BIG, false>, gemm_lds_bytes<128, 256, 64>());
+    bad |= raise_lds(gemm_mfma_kernel<GEMM_MID, true>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_mfma_kernel<GEMM_MID, false>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_mfma_kernel<GEMM_SMALL, true>, gemm_lds_bytes<64, 64, 64>());
+    bad |= raise_lds(gemm_mfma_kernel<GEMM_SMALL, false>, gemm_lds_bytes<64, 64, 64>());
+    bad |= mi_sdpa_init();
+    if (bad) return MI_ERROR_DEVICE;
+    g_ready = true;
+    return MI_OK;
+}
+
+int mi_device_caps(int64_t out[6]) {
+    if (!out) return MI_DECLINE_OPERANDS;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return MI_ERROR_DEVICE;
+    out[0] = __builtin_strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    out[1] = 16;
+    out[2] = prop.warpSize;
+    out[3] = (int64_t)prop.maxSharedMemoryPerMultiProcessor;
+    out[4] = prop.maxThreadsPerBlock;
+    out[5] = prop.multiProcessorCount;
+    return MI_OK;
+}
+
+size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int64_t nbatch) {
+    if (T < 1 || T > 8 || nbatch > 1) return 0;
+    int nsplit = w_layout == MI_W_KF ? skinny_splits(K, F) : 1;
+    return round_up((size_t)nsplit * T * F * sizeof(float), 256);
+}
+
+int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,
+                     int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                     int w_layout, int out_dtype, int64_t nbatch, int64_t sY, int64_t sX, int64_t sW) {
+    GemmArgs a;
+    int rc = fill_args(a, const_cast<void *>(Y), X, W, nullptr, nullptr, T, K, F, ldY, ldX, ldW, w_layout, MI_BIAS_NONE,
+                       MI_EPI_NONE, out_dtype, sY, sX, sW);
+    if (rc != MI_OK) return MI_GEMM_DECLINE;
+    return gemm_path(a, w_layout == MI_W_KF, nbatch < 1 ? 1 : nbatch);
+}
+
+int mi_gemm_f16_batched(void *Y, const void *X, const void *W, const void *bias, const void *residual,
+                        int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                        int w_layout, int bias_mode, int epi, int out_dtype,
+                        int64_t nbatch, int64_t sY, int64_t sX, int64_t sW,
+                        void *ws, size_t ws_bytes, void *stream) {
+    GemmArgs a;
+    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype, sY, sX, sW);
+    if (rc != MI_OK) return rc;
+    if (nbatch < 0 || nbatch > 65535) return MI_DECLINE_EXTENT;
+    if (K == 0) return MI_DECLINE_EXTENT;
+    return run_gemm(a, w_layout == MI_W_KF, nbatch, ws, ws_bytes, (hipStream_t)stream, 0);
+}
+
+int mi_gemm_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,
+                int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                int w_layout, int bias_mode, int epi, int out_dtype,
+                void *ws, size_t ws_bytes, void *stream) {
+    return mi_gemm_f16_batched(Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype,
+                               1, 0, 0, 0, ws, ws_bytes, stream);
+}
+
+int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,
+                int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                int w_layout, int bias_mode, int epi, int out_dtype,
+                void *ws, size_t ws_bytes, void *stream) {
+    GemmArgs a;
+    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype, 0, 0, 0);
+    if (rc != MI_OK) return rc;
+    if (!g_ready) return MI_ERROR_DEVICE;
+    if (T < 1 || T > 8) return MI_DECLINE_EXTENT;
+    if (!mfma_addressable(a, w_layout == MI_W_KF)) return MI_DECLINE_OPERANDS;
+    return run_skinny(a, w_layout == MI_W_KF, ws, ws_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,147 @@
+// Layer norm and the residual add: the HBM-bound glue between the contractions
+// of an encoder block.  One wavefront per normalisation group, the row held in
+// registers between the three passes (mean, centred variance, normalise) so it
+// is read from memory once; fp32 statistics (layernorm.jl:53-113).
+#include "common.hpp"
+
+namespace {
+
+// A row of C <= 64 * 8 * NCH halves lives in NCH 16-byte chunks per lane.
+template <int NCH>
+__global__ __launch_bounds__(256) void layernorm_vec_kernel(half_t *out, float *mean, float *rstd, const half_t *a,
+                                                            const half_t *gamma, const half_t *beta, int C, long groups, float eps) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long g = (long)blockIdx.x * 4 + wave;
+    if (g >= groups) return;
+    const half_t *row = a + g * C;
+    float x[NCH][8];
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        if (e0 < C) {
+            half8v t = as_half8(ldg16(row + e0));
+#pragma unroll
+            for (int j = 0; j < 8; j++) { x[i][j] = (float)t[j]; s += x[i][j]; }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) x[i][j] = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    const float mu = s / (float)C;
+    float s2 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        if (e0 < C) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) { const float d = x[i][j] - mu; s2 = fmaf(d, d, s2); }
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+    const float r = 1.0f / sqrtf(s2 / (float)C + eps);
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        if (e0 < C) {
+            half8v gv, bv, o;
+            if (gamma) gv = as_half8(ldg16(gamma + e0));
+            if (beta) bv = as_half8(ldg16(beta + e0));
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                float y = (x[i][j] - mu) * r;
+                if (gamma) y *= (float)gv[j];
+                if (beta) y += (float)bv[j];
+                o[j] = (half_t)y;
+            }
+            *reinterpret_cast<half8v *>(out + g * C + e0) = o;
+        }
+    }
+    if (lane == 0) {
+        if (mean) mean[g] = mu;
+        if (rstd) rstd[g] = r;
+    }
+}
+
+// Any C, any alignment: the same three passes reading memory each time.
+__global__ __launch_bounds__(256) void layernorm_any_kernel(half_t *out, float *mean, float *rstd, const half_t *a,
+                                                            const half_t *gamma, const half_t *beta, int C, long groups, float eps) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long g = (long)blockIdx.x * 4 + wave;
+    if (g >= groups) return;
+    const half_t *row = a + g * C;
+    float s = 0.0f;
+    for (int i = lane; i < C; i += 64) s += (float)row[i];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    const float mu = s / (float)C;
+    float s2 = 0.0f;
+    for (int i = lane; i < C; i += 64) { const float d = (float)row[i] - mu; s2 = fmaf(d, d, s2); }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+    const float r = 1.0f / sqrtf(s2 / (float)C + eps);
+    for (int i = lane; i < C; i += 64) {
+        float y = ((float)row[i] - mu) * r;
+        if (gamma) y *= (float)gamma[i];
+        if (beta) y += (float)beta[i];
+        out[g * C + i] = (half_t)y;
+    }
+    if (lane == 0) {
+        if (mean) mean[g] = mu;
+        if (rstd) rstd[g] = r;
+    }
+}
+
+__global__ void add_vec_kernel(half_t *o, const half_t *a, const half_t *b, long n8) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    half8v x = as_half8(ldg16(a + i * 8)), y = as_half8(ldg16(b + i * 8)), r;
+#pragma unroll
+    for (int j = 0; j < 8; j++) r[j] = (half_t)((float)x[j] + (float)y[j]);
+    *reinterpret_cast<half8v *>(o + i * 8) = r;
+}
+__global__ void add_any_kernel(half_t *o, const half_t *a, const half_t *b, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) o[i] = (half_t)((float)a[i] + (float)b[i]);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_layernorm_f16(void *out, float *mean, float *rstd, const void *a, const void *gamma, const void *beta,
+                     int64_t C, int64_t groups, float eps, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !a) return MI_DECLINE_OPERANDS;
+    if (C < 1 || C > INT32_MAX || groups < 0) return MI_DECLINE_EXTENT;
+    if (groups == 0) return MI_OK;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid((unsigned)ceil_div(groups, 4)), block(256);
+    half_t *o = (half_t *)out;
+    const half_t *x = (const half_t *)a, *g = (const half_t *)gamma, *b = (const half_t *)beta;
+    const bool vec = C % 8 == 0 && aligned_to(a, 16) && aligned_to(out, 16) && (!g || aligned_to(g, 16)) && (!b || aligned_to(b, 16));
+    if (vec && C <= 512)       hipLaunchKernelGGL(layernorm_vec_kernel<1>, grid, block, 0, st, o, mean, rstd, x, g, b, (int)C, (long)groups, eps);
+    else if (vec && C <= 1024) hipLaunchKernelGGL(layernorm_vec_kernel<2>, grid, block, 0, st, o, mean, rstd, x, g, b, (int)C, (long)groups, eps);
+    else if (vec && C <= 2048) hipLaunchKernelGGL(layernorm_vec_kernel<4>, grid, block, 0, st, o, mean, rstd, x, g, b, (int)C, (long)groups, eps);
+    else if (vec && C <= 4096) hipLaunchKernelGGL(layernorm_vec_kernel<8>, grid, block, 0, st, o, mean, rstd, x, g, b, (int)C, (long)groups, eps);
+    else                       hipLaunchKernelGGL(layernorm_any_kernel, grid, block, 0, st, o, mean, rstd, x, g, b, (int)C, (long)groups, eps);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_add_f16(void *out, const void *a, const void *b, int64_t n, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !a || !b) return MI_DECLINE_OPERANDS;
+    if (n < 0) return MI_DECLINE_EXTENT;
+    if (n == 0) return MI_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (n % 8 == 0 && aligned_to(out, 16) && aligned_to(a, 16) && aligned_to(b, 16))
+        hipLaunchKernelGGL(add_vec_kernel, dim3((unsigned)ceil_div(n / 8, 256)), dim3(256), 0, st, (half_t *)out, (const half_t *)a, (const half_t *)b, (long)(n / 8));
+    else
+        hipLaunchKernelGGL(add_any_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, (half_t *)out, (const half_t *)a, (const half_t *)b, (long)n);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+}  // extern "C"

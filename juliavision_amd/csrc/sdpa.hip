@@ -1,0 +1,559 @@
+// Scaled-dot-product attention for gfx950.
+//
+//  flash_fwd_kernel   fused attention on MFMA 32x32x16 f16: S^T = K.Q^T and
+//                     O^T = V^T.P^T, so that the score tile leaves the first
+//                     product in exactly the register layout the second product
+//                     consumes -- scores and probabilities never touch LDS or
+//                     HBM.  Online softmax in fp32, one query per lane pair.
+//  sdpa_rows_kernel   one workgroup per (query row, key split): the
+//                     bandwidth-bound form for decode-sized Lq, and the
+//                     always-available path for additive masks, odd head
+//                     sizes and strided operands; split partials are merged by
+//                     sdpa_merge_kernel.
+//
+// Operands are (E, L, H, B) with element strides (the reference's layout,
+// DNNKernels/src/kernels/extern/attention.jl:1-22); out is dense (E, Lq, H, B).
+#include "common.hpp"
+#include <type_traits>
+
+namespace {
+
+struct SdpaArgs {
+    void *out;
+    const half_t *q, *k, *v;
+    long qs[4], ks[4], vs[4];      // (E, L, H, B) element strides
+    const void *bias;
+    long bs[4];                    // (Lk, Lq, H, B) element strides, 0 = broadcast
+    const int *kv_len;
+    float *part_o, *part_ml;       // split partials: [split][row][E], [split][row][2]
+    int E, Lq, Lk, H, B;
+    int out_f32, bias_f32, nsplit;
+    float scale;
+};
+
+constexpr float LOG2E = 1.4426950408889634f;
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Fused kernel.  Workgroup = 4 waves = 128 queries (32 per wave); keys walked in
+// blocks of BC = 64 through double-buffered LDS tiles:
+//   Ks [BC][EP+8]   keys x head-dim, head-dim contiguous  (A operand of S^T = K.Q^T)
+//   Vt [EP][BC+4]   head-dim x keys, keys contiguous      (A operand of O^T = V^T.P^T)
+// V arrives head-dim contiguous, so it is transposed on the way into LDS: a
+// thread takes the same 8 head-dim values of two adjacent keys and writes eight
+// packed key pairs.
+//
+// MFMA 32x32 accumulator layout: lane l, register r holds row 8(r/4)+4(l/32)+r%4,
+// column l%32.  With rows = keys and columns = queries, a lane owns one query
+// and 16 keys per 32-key tile: row maxima and sums need one exchange with lane
+// l^32.  Registers 8b..8b+7 of a tile are, in order, the keys
+// {16b+4h+0..3, 16b+8+4h+0..3} (h = l/32): that is the k-order in which P^T is fed
+// to the second product, and V^T is read from LDS in the same order.
+template <int EP>
+__global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
+    constexpr int BC = 64, BR = 128, NT = 256;
+    constexpr int KLD = EP + 8, VLD = BC + 4;
+    constexpr int KS = EP / 16;       // k16 steps over the head dim
+    constexpr int ET = EP / 32;       // 32-wide head-dim tiles of O
+    constexpr int KCH = EP / 8;       // 16-byte chunks per key row
+    constexpr int K_PER = BC * KCH / NT;
+    constexpr int V_PER = (BC / 2) * KCH / NT;
+    extern __shared__ __align__(16) char smem[];
+    half_t (*Ks)[BC * KLD] = reinterpret_cast<half_t (*)[BC * KLD]>(smem);
+    half_t (*Vt)[EP * VLD] = reinterpret_cast<half_t (*)[EP * VLD]>(smem + 2 * BC * KLD * 2);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hl = lane >> 5, l32 = lane & 31;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int q0 = blockIdx.x * BR + wave * 32;
+    const half_t *qb = p.q + h * p.qs[2] + b * p.qs[3];
+    const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
+    const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
+    int Lk = p.Lk;
+    if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
+    const float c = p.scale * LOG2E;
+
+    // Q^T fragments: column = query l32, k = head-dim 16 ks + 8 hl .. +7
+    half8v qf[KS];
+    {
+        const int qr = min(q0 + l32, p.Lq - 1);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int e = 16 * ks + 8 * hl;
+            u32x4 z = {0u, 0u, 0u, 0u};
+            qf[ks] = as_half8(e < p.E ? ldg16(qb + (long)qr * p.qs[1] + e) : z);
+        }
+    }
+
+    u32x4 kr[K_PER], vr[V_PER][2];
+    auto load_kv = [&](int key0) {
+#pragma unroll
+        for (int i = 0; i < K_PER; i++) {
+            const int cidx = tid + i * NT;
+            const int row = cidx / KCH, ch = cidx % KCH;
+            const int key = min(key0 + row, p.Lk - 1);
+            u32x4 z = {0u, 0u, 0u, 0u};
+            kr[i] = ch * 8 < p.E ? ldg16(kb + (long)key * p.ks[1] + ch * 8) : z;
+        }
+#pragma unroll
+        for (int i = 0; i < V_PER; i++) {
+            const int u = tid + i * NT;
+            const int ch = u % KCH, kp = u / KCH;
+            const int key = key0 + 2 * kp;
+            u32x4 z = {0u, 0u, 0u, 0u};
+            const bool eok = ch * 8 < p.E;
+            vr[i][0] = eok ? ldg16(vb + (long)min(key, p.Lk - 1) * p.vs[1] + ch * 8) : z;
+            vr[i][1] = eok ? ldg16(vb + (long)min(key + 1, p.Lk - 1) * p.vs[1] + ch * 8) : z;
+        }
+    };
+    auto store_kv = [&](int buf, int key0) {
+#pragma unroll
+        for (int i = 0; i < K_PER; i++) {
+            const int cidx = tid + i * NT;
+            const int row = cidx / KCH, ch = cidx % KCH;
+            *reinterpret_cast<u32x4 *>(&Ks[buf][row * KLD + ch * 8]) = kr[i];
+        }
+#pragma unroll
+        for (int i = 0; i < V_PER; i++) {
+            const int u = tid + i * NT;
+            const int ch = u % KCH, kp = u / KCH;
+            // Keys past the end must contribute exactly 0 * v, and v there is a
+            // clamped re-read (finite), so only P needs masking; nothing to zero.
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                *reinterpret_cast<uint32_t *>(&Vt[buf][(ch * 8 + 2 * w) * VLD + 2 * kp]) = pack_lo(vr[i][0][w], vr[i][1][w]);
+                *reinterpret_cast<uint32_t *>(&Vt[buf][(ch * 8 + 2 * w + 1) * VLD + 2 * kp]) = pack_hi(vr[i][0][w], vr[i][1][w]);
+            }
+        }
+        (void)key0;
+    };
+
+    float16v o_acc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o_acc[t][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    const int nblk = (Lk + BC - 1) / BC;
+    if (nblk > 0) {
+        load_kv(0);
+        store_kv(0, 0);
+    }
+    __syncthreads();
+
+    for (int kbk = 0; kbk < nblk; kbk++) {
+        const int cur = kbk & 1, key0 = kbk * BC;
+        const bool more = kbk + 1 < nblk;
+        if (more) load_kv(key0 + BC);
+
+        // S^T tiles: rows = keys, columns = queries
+        float16v s[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[kt][r] = 0.0f;
+            const half_t *kp_ = &Ks[cur][(32 * kt + l32) * KLD + 8 * hl];
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                half8v kf = *reinterpret_cast<const half8v *>(kp_ + 16 * ks);
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kt], 0, 0, 0);
+            }
+        }
+        if (key0 + BC > Lk) {       // the ragged last block: excluded keys get -inf
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = key0 + 32 * kt + 8 * (r >> 2) + 4 * hl + (r & 3);
+                    if (key >= Lk) s[kt][r] = -INFINITY;
+                }
+        }
+        // online softmax (flash.jl:25-38 recurrence), in base 2 with the scale folded
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+        const float mc = m_use * c;
+        float rs = 0.0f;
+        half8v pf[2][2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float pv = __builtin_amdgcn_exp2f(fmaf(s[kt][r], c, -mc));
+                rs += pv;
+                pf[kt][r >> 3][r & 7] = (half_t)pv;
+            }
+        rs += __shfl_xor(rs, 32, 64);
+        l_run = l_run * alpha + rs;
+        m_run = m_new;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int t = 0; t < ET; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o_acc[t][r] *= alpha;
+        }
+        // O^T += V^T . P^T
+#pragma unroll
+        for (int t = 0; t < ET; t++) {
+            const half_t *vp = &Vt[cur][(32 * t + l32) * VLD + 4 * hl];
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int bb = 0; bb < 2; bb++) {
+                    half4v lo = *reinterpret_cast<const half4v *>(vp + 32 * kt + 16 * bb);
+                    half4v hi = *reinterpret_cast<const half4v *>(vp + 32 * kt + 16 * bb + 8);
+                    half8v vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    o_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kt][bb], o_acc[t], 0, 0, 0);
+                }
+        }
+        if (more) store_kv(cur ^ 1, key0 + BC);
+        __syncthreads();
+    }
+
+    // out[b][h][q][e]; lane owns query q0 + l32 and, per tile t and group g, the
+    // four head-dim values e = 32 t + 8 g + 4 hl + 0..3
+    const int qi = q0 + l32;
+    if (qi < p.Lq) {
+        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+        const long base = (((long)b * p.H + h) * p.Lq + qi) * p.E;
+#pragma unroll
+        for (int t = 0; t < ET; t++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int e = 32 * t + 8 * g + 4 * hl;
+                if (e < p.E) {      // E is a multiple of 8, so e..e+3 are all valid
+                    if (p.out_f32) {
+                        float4v o = {o_acc[t][4 * g] * inv, o_acc[t][4 * g + 1] * inv, o_acc[t][4 * g + 2] * inv, o_acc[t][4 * g + 3] * inv};
+                        *reinterpret_cast<float4v *>(reinterpret_cast<float *>(p.out) + base + e) = o;
+                    } else {
+                        half4v o = {(half_t)(o_acc[t][4 * g] * inv), (half_t)(o_acc[t][4 * g + 1] * inv),
+                                    (half_t)(o_acc[t][4 * g + 2] * inv), (half_t)(o_acc[t][4 * g + 3] * inv)};
+                        *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(p.out) + base + e) = o;
+                    }
+                }
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// One workgroup (4 waves) per (query row, key split).  A wave walks keys 8 at a
+// time: 8 lanes share a key, each owning 8-element head-dim chunks c, c+8, ...
+// (NCH chunks, E <= 64 NCH).  Every 8-lane group keeps its own running
+// (m, l, acc); groups, waves and splits are merged with the rescaling identity
+// m = max m_s, l = sum e^{m_s-m} l_s, O = sum e^{m_s-m} O_s  (flash.jl:1385-1391).
+template <int NCH, bool VEC>
+__global__ __launch_bounds__(256) void sdpa_rows_kernel(SdpaArgs p) {
+    __shared__ float red_ml[4][2];
+    __shared__ float red_o[4][64 * NCH];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = lane >> 3, cl = lane & 7;
+    const int split = blockIdx.x % p.nsplit;
+    const int row = blockIdx.x / p.nsplit;      // lq + Lq * h
+    const int lq = row % p.Lq, h = row / p.Lq, b = blockIdx.z;
+    int Lk = p.Lk;
+    if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
+    // split ranges in units of 32 keys (one pass of the workgroup)
+    const int units = (Lk + 31) / 32;
+    const int per = (units + p.nsplit - 1) / p.nsplit;
+    const int kbeg = min(Lk, split * per * 32), kend = min(Lk, (split + 1) * per * 32);
+
+    const half_t *qp = p.q + (long)lq * p.qs[1] + h * p.qs[2] + b * p.qs[3];
+    const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
+    const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
+
+    float qv[NCH][8];
+#pragma unroll
+    for (int ci = 0; ci < NCH; ci++) {
+        const int e0 = (cl + 8 * ci) * 8;
+        if (VEC) {
+            u32x4 z = {0u, 0u, 0u, 0u};
+            half8v t = as_half8(e0 < p.E ? ldg16(qp + e0) : z);
+#pragma unroll
+            for (int j = 0; j < 8; j++) qv[ci][j] = (float)t[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) qv[ci][j] = e0 + j < p.E ? (float)qp[(long)(e0 + j) * p.qs[0]] : 0.0f;
+        }
+    }
+
+    float m = -INFINITY, l = 0.0f;
+    float acc[NCH][8];
+#pragma unroll
+    for (int ci = 0; ci < NCH; ci++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[ci][j] = 0.0f;
+
+    for (int base = kbeg + wave * 8; base < kend; base += 32) {
+        // Every lane of the wave runs the same number of iterations (the shuffles
+        // below need all 64 lanes); a key past the end is computed on a clamped
+        // row and then given weight zero.
+        const int key = base + grp;
+        const bool live = key < kend;
+        const int kk = live ? key : kend - 1;
+        const half_t *kp = kb + (long)kk * p.ks[1];
+        float d = 0.0f;
+#pragma unroll
+        for (int ci = 0; ci < NCH; ci++) {
+            const int e0 = (cl + 8 * ci) * 8;
+            if (VEC) {
+                u32x4 z = {0u, 0u, 0u, 0u};
+                half8v t = as_half8(e0 < p.E ? ldg16(kp + e0) : z);
+#pragma unroll
+                for (int j = 0; j < 8; j++) d = fmaf(qv[ci][j], (float)t[j], d);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (e0 + j < p.E) d = fmaf(qv[ci][j], (float)kp[(long)(e0 + j) * p.ks[0]], d);
+            }
+        }
+        d += __shfl_xor(d, 1, 64);
+        d += __shfl_xor(d, 2, 64);
+        d += __shfl_xor(d, 4, 64);
+        float sc = d * p.scale;
+        if (p.bias && live) {
+            const long bo = (long)kk * p.bs[0] + (long)lq * p.bs[1] + (long)h * p.bs[2] + (long)b * p.bs[3];
+            sc += p.bias_f32 ? reinterpret_cast<const float *>(p.bias)[bo] : (float)reinterpret_cast<const half_t *>(p.bias)[bo];
+        }
+        if (!live) sc = -INFINITY;
+        const float mn = fmaxf(m, sc);
+        const float mu = mn == -INFINITY ? 0.0f : mn;
+        const float al = __expf(m - mu);
+        const float pw = __expf(sc - mu);
+        l = l * al + pw;
+        m = mn;
+        const half_t *vp = vb + (long)kk * p.vs[1];
+#pragma unroll
+        for (int ci = 0; ci < NCH; ci++) {
+            const int e0 = (cl + 8 * ci) * 8;
+            if (VEC) {
+                u32x4 z = {0u, 0u, 0u, 0u};
+                half8v t = as_half8(e0 < p.E ? ldg16(vp + e0) : z);
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc[ci][j] = fmaf(pw, (float)t[j], acc[ci][j] * al);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    float vv = e0 + j < p.E ? (float)vp[(long)(e0 + j) * p.vs[0]] : 0.0f;
+                    acc[ci][j] = fmaf(pw, vv, acc[ci][j] * al);
+                }
+            }
+        }
+    }
+
+    // merge the 8 groups of the wave
+#pragma unroll
+    for (int o = 8; o < 64; o <<= 1) {
+        const float mo = __shfl_xor(m, o, 64), lo = __shfl_xor(l, o, 64);
+        const float mn = fmaxf(m, mo);
+        const float mu = mn == -INFINITY ? 0.0f : mn;
+        const float a0 = __expf(m - mu), a1 = __expf(mo - mu);
+        l = l * a0 + lo * a1;
+#pragma unroll
+        for (int ci = 0; ci < NCH; ci++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[ci][j] = acc[ci][j] * a0 + __shfl_xor(acc[ci][j], o, 64) * a1;
+        m = mn;
+    }
+    // merge the 4 waves through LDS
+    if (lane < 8) {
+#pragma unroll
+        for (int ci = 0; ci < NCH; ci++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) red_o[wave][(cl + 8 * ci) * 8 + j] = acc[ci][j];
+        if (lane == 0) { red_ml[wave][0] = m; red_ml[wave][1] = l; }
+    }
+    __syncthreads();
+    if (tid < 64 * NCH && tid < p.E) {
+        float mm = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; w++) mm = fmaxf(mm, red_ml[w][0]);
+        const float mu = mm == -INFINITY ? 0.0f : mm;
+        float L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float a = __expf(red_ml[w][0] - mu);
+            L += a * red_ml[w][1];
+            O += a * red_o[w][tid];
+        }
+        const long orow = ((long)b * p.H + h) * p.Lq + lq;
+        if (p.nsplit == 1) {
+            const float r = L > 0.0f ? O / L : 0.0f;
+            if (p.out_f32) reinterpret_cast<float *>(p.out)[orow * p.E + tid] = r;
+            else reinterpret_cast<half_t *>(p.out)[orow * p.E + tid] = (half_t)r;
+        } else {
+            const long rows = (long)p.B * p.H * p.Lq;
+            p.part_o[((long)split * rows + orow) * p.E + tid] = O;
+            if (tid == 0) {
+                p.part_ml[((long)split * rows + orow) * 2] = mm;
+                p.part_ml[((long)split * rows + orow) * 2 + 1] = L;
+            }
+        }
+    }
+}
+
+// One thread per (row, e): merges the key splits (attn_flash_cm_merge!, flash.jl:1398-1421).
+__global__ void sdpa_merge_kernel(SdpaArgs p) {
+    const long rows = (long)p.B * p.H * p.Lq;
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * p.E) return;
+    const long row = idx / p.E;
+    const int e = (int)(idx % p.E);
+    float mm = -INFINITY;
+    for (int s = 0; s < p.nsplit; s++) mm = fmaxf(mm, p.part_ml[((long)s * rows + row) * 2]);
+    const float mu = mm == -INFINITY ? 0.0f : mm;
+    float L = 0.0f, O = 0.0f;
+    for (int s = 0; s < p.nsplit; s++) {
+        const float a = __expf(p.part_ml[((long)s * rows + row) * 2] - mu);
+        L += a * p.part_ml[((long)s * rows + row) * 2 + 1];
+        O += a * p.part_o[((long)s * rows + row) * p.E + e];
+    }
+    const float r = L > 0.0f ? O / L : 0.0f;
+    if (p.out_f32) reinterpret_cast<float *>(p.out)[idx] = r;
+    else reinterpret_cast<half_t *>(p.out)[idx] = (half_t)r;
+}
+
+// ------------------------------------------------------------------------------------------
+constexpr int flash_lds_bytes(int EP) { return 2 * 64 * (EP + 8) * 2 + 2 * EP * (64 + 4) * 2; }
+
+bool vec_addressable(const half_t *ptr, const long st[4], int E) {
+    return st[0] == 1 && E % 8 == 0 && st[1] % 8 == 0 && st[2] % 8 == 0 && st[3] % 8 == 0 && aligned_to(ptr, 16);
+}
+
+int rows_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    // Aim at two workgroups per compute unit (the reference's splitcount rule,
+    // flash.jl:1288-1303); a split is at least 64 keys.
+    int64_t rows = Lq * H * B;
+    if (rows <= 0) return 1;
+    int64_t want = ceil_div(2 * (int64_t)mi_num_cus(), rows);
+    int64_t maxs = ceil_div(Lk, 64);
+    if (want > maxs) want = maxs;
+    if (want < 1) want = 1;
+    if (want > 64) want = 64;
+    return (int)want;
+}
+
+int sdpa_path(const SdpaArgs &a) {
+    if (a.E < 1 || a.E > 256 || a.Lq < 0 || a.Lk < 0 || a.H < 1 || a.B < 1) return MI_SDPA_DECLINE;
+    if (a.H > 65535 || a.B > 65535 || (int64_t)a.Lq * a.H * 64 > INT32_MAX) return MI_SDPA_DECLINE;
+    bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
+    bool out_ok = aligned_to(a.out, 16) || a.out == nullptr;
+    if (vec && out_ok && !a.bias && a.scale > 0.0f && a.E <= 128 && a.Lq >= 64 && a.Lk >= 1) return MI_SDPA_FLASH;
+    return MI_SDPA_ROWS;
+}
+
+int fill(SdpaArgs &a, void *out, int out_dtype, const void *q, const int64_t *qs, const void *k, const int64_t *ks,
+         const void *v, const int64_t *vs, const void *bias, int bias_dtype, const int64_t *bs, const int32_t *kv_len,
+         int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale) {
+    if (!q || !k || !v || !qs || !ks || !vs) return MI_DECLINE_OPERANDS;
+    if (bias && !bs) return MI_DECLINE_BIAS;
+    if (out_dtype != MI_F16 && out_dtype != MI_F32) return MI_DECLINE_OPERANDS;
+    if (E > INT32_MAX || Lq > INT32_MAX || Lk > INT32_MAX || H > INT32_MAX || B > INT32_MAX) return MI_DECLINE_EXTENT;
+    a.out = out; a.q = (const half_t *)q; a.k = (const half_t *)k; a.v = (const half_t *)v;
+    for (int i = 0; i < 4; i++) { a.qs[i] = qs[i]; a.ks[i] = ks[i]; a.vs[i] = vs[i]; a.bs[i] = bias ? bs[i] : 0; }
+    a.bias = bias; a.bias_f32 = bias_dtype == MI_F32; a.kv_len = kv_len;
+    a.part_o = a.part_ml = nullptr;
+    a.E = (int)E; a.Lq = (int)Lq; a.Lk = (int)Lk; a.H = (int)H; a.B = (int)B;
+    a.out_f32 = out_dtype == MI_F32; a.nsplit = 1; a.scale = scale;
+    return MI_OK;
+}
+
+template <int NCH>
+void launch_rows(const SdpaArgs &a, bool vec, dim3 grid, hipStream_t st) {
+    if (vec) hipLaunchKernelGGL((sdpa_rows_kernel<NCH, true>), grid, dim3(256), 0, st, a);
+    else     hipLaunchKernelGGL((sdpa_rows_kernel<NCH, false>), grid, dim3(256), 0, st, a);
+}
+
+}  // namespace
+
+// Called once from mi_init: the 128-wide head-dim variant needs more than the
+// default 64 KiB of dynamic LDS.
+int mi_sdpa_init() {
+    int bad = 0;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
+    return bad;
+}
+
+extern "C" {
+
+size_t mi_sdpa_f16_workspace(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, int has_bias) {
+    (void)has_bias;
+    int ns = rows_splits(Lq, Lk, H, B);
+    if (ns <= 1 || Lq >= 64) return 0;
+    size_t rows = (size_t)Lq * H * B;
+    return round_up((size_t)ns * rows * E * sizeof(float), 256) + round_up((size_t)ns * rows * 2 * sizeof(float), 256);
+}
+
+int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                     const void *v, const int64_t v_strides[4], int has_bias, int has_kv_len,
+                     int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale, int *nsplit_out) {
+    (void)has_kv_len;
+    SdpaArgs a;
+    static const int64_t zero4[4] = {0, 0, 0, 0};
+    int rc = fill(a, nullptr, MI_F16, q, q_strides, k, k_strides, v, v_strides, has_bias ? (const void *)q : nullptr, MI_F16,
+                  zero4, nullptr, E, Lq, Lk, H, B, scale);
+    if (rc != MI_OK) return MI_SDPA_DECLINE;
+    int path = sdpa_path(a);
+    if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? rows_splits(Lq, Lk, H, B) : 1;
+    return path;
+}
+
+int mi_sdpa_f16(void *out, int out_dtype,
+                const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                const void *v, const int64_t v_strides[4],
+                const void *bias, int bias_dtype, const int64_t bias_strides[4], const int32_t *kv_len,
+                int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale,
+                void *ws, size_t ws_bytes, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out) return MI_DECLINE_OPERANDS;
+    SdpaArgs a;
+    int rc = fill(a, out, out_dtype, q, q_strides, k, k_strides, v, v_strides, bias, bias_dtype, bias_strides, kv_len, E, Lq, Lk, H, B, scale);
+    if (rc != MI_OK) return rc;
+    if (Lq == 0 || H == 0 || B == 0 || E == 0) return MI_OK;
+    hipStream_t st = (hipStream_t)stream;
+    int path = sdpa_path(a);
+    if (path == MI_SDPA_DECLINE) return MI_DECLINE_EXTENT;
+    if (path == MI_SDPA_FLASH) {
+        dim3 grid((unsigned)ceil_div(Lq, 128), (unsigned)H, (unsigned)B);
+        if (E <= 64) hipLaunchKernelGGL(flash_fwd_kernel<64>, grid, dim3(256), flash_lds_bytes(64), st, a);
+        else         hipLaunchKernelGGL(flash_fwd_kernel<128>, grid, dim3(256), flash_lds_bytes(128), st, a);
+        return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+    }
+    // rows path
+    bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
+    a.nsplit = Lq < 64 ? rows_splits(Lq, Lk, H, B) : 1;
+    if (a.nsplit > 1) {
+        size_t rows = (size_t)Lq * H * B;
+        size_t o_bytes = round_up((size_t)a.nsplit * rows * E * sizeof(float), 256);
+        size_t need = o_bytes + round_up((size_t)a.nsplit * rows * 2 * sizeof(float), 256);
+        if (!ws || ws_bytes < need || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
+        a.part_o = reinterpret_cast<float *>(ws);
+        a.part_ml = reinterpret_cast<float *>(reinterpret_cast<char *>(ws) + o_bytes);
+    }
+    dim3 grid((unsigned)(a.nsplit * Lq * H), 1, (unsigned)B);
+    int nch = (int)ceil_div(E, 64);
+    if (nch == 1) launch_rows<1>(a, vec, grid, st);
+    else if (nch == 2) launch_rows<2>(a, vec, grid, st);
+    else launch_rows<4>(a, vec, grid, st);
+    if (a.nsplit > 1) {
+        long total = (long)Lq * H * B * E;
+        hipLaunchKernelGGL(sdpa_merge_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a);
+    }
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+}  // extern "C"

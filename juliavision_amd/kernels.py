@@ -1,0 +1,416 @@
+"""Host-side mirror of the reference's kernel entry points, over the C ABI.
+
+The reference's op handlers (DNNKernels/src/ops.jl:575-647,1114-1222,1347-1399) call
+``matmul!``, ``batchedmatmul!``, ``sdpa``, ``convolution!`` and ``layernorm!`` with a
+per-run ``Ctx``; a new implementation plugs in as a *plan type* plus one method
+per entry point (DNNKernels/src/kernels/extern/matmul.jl:97-100,
+attention.jl:767-776, kernelplans.jl:1-35).  This module is that seam in
+Python: the same entry points (``!`` spelled ``_``), the same argument meaning,
+``Decline(reason)`` from every planner instead of an exception, and one
+``_run`` method per plan -- each of which is a single call into
+``libmi355dnn.so``.  A Julia shim binds the identical symbols with ``ccall``.
+
+Array convention: a Julia column-major array ``(a, b, c, d)`` is the torch
+tensor of shape ``(d, c, b, a)`` with the same bytes (safetensors.jl:7-12).
+So ``matmul_``'s ``A`` (Julia ``(M, K)``, the hoisted weight) is a torch
+``(K, M)`` tensor, ``B`` (Julia ``(K, N)``, the activations) is torch
+``(N, K)``, ``out`` is torch ``(N, M)``; attention operands (Julia ``(E, L, H, B)``)
+are torch ``(B, H, L, E)`` views with arbitrary strides; convolution operands
+are torch NCHW / OIHW.
+
+PyTorch is used only to own device memory and the stream.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from dataclasses import dataclass
+from typing import NamedTuple, Optional
+
+import torch
+
+from . import _lib as L
+
+
+# ----------------------------------------------------------------------------- Decline / caps / ctx
+
+@dataclass(frozen=True)
+class Decline:
+    """Why a path was not taken (kernelplans.jl:21-35).  Truthiness is False."""
+    reason: str
+
+    def __bool__(self):
+        return False
+
+
+class DeclineError(RuntimeError):
+    """A launch the library refused after a plan had been made."""
+
+    def __init__(self, what: str, status: int):
+        super().__init__(f"{what}: mi355dnn status {status} ({L.STATUS_NAMES.get(status, '?')})")
+        self.status = status
+        self.reason = L.STATUS_NAMES.get(status, "?")
+
+
+class DeviceCaps(NamedTuple):
+    """The device facts planners read -- the named fields of Lava.DeviceCaps
+    (context.jl:68, test_flash.jl:373).  A value, so a test can plan for
+    hardware it does not have."""
+    coopmat: bool
+    tile: int
+    subgroup: int
+    sharedbudget: int
+    workgrouplimit: int
+    cores: int
+
+
+MI355X = DeviceCaps(True, 16, 64, 160 * 1024, 1024, 256)
+
+
+def caps() -> DeviceCaps:
+    """Query the current device (context.jl:55)."""
+    lib = L.init()
+    out = (C.c_int64 * 6)()
+    rc = lib.mi_device_caps(out)
+    if rc != L.OK:
+        raise DeclineError("mi_device_caps", rc)
+    return DeviceCaps(bool(out[0]), int(out[1]), int(out[2]), int(out[3]), int(out[4]), int(out[5]))
+
+
+class Workspace:
+    """Per-op bump scratch (workspace.jl:19-106): ``reset()`` before every op,
+    ``scratch(nbytes)`` hands out 256-byte aligned device memory valid until the
+    next reset.  Grows by reallocation between ops, never inside one."""
+
+    ALIGN = 256
+
+    def __init__(self, device="cuda", nbytes: int = 0):
+        self.device = torch.device(device)
+        self.buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=self.device)
+        self.off = 0
+        self._pending = []
+
+    def reset(self):
+        self.off = 0
+        self._pending.clear()
+
+    def scratch(self, nbytes: int) -> int:
+        if nbytes <= 0:
+            return 0
+        base = self.buf.data_ptr()
+        start = (-(base + self.off)) % self.ALIGN + self.off
+        if start + nbytes > self.buf.numel():
+            # Stream order keeps the old buffer alive for kernels already enqueued.
+            self._pending.append(self.buf)
+            self.buf = torch.empty(max(2 * self.buf.numel(), nbytes + self.ALIGN), dtype=torch.uint8, device=self.device)
+            self.off = 0
+            base = self.buf.data_ptr()
+            start = (-base) % self.ALIGN
+        self.off = start + nbytes
+        return base + start
+
+
+class Ctx:
+    """Per-run context (context.jl:240-331): device caps, workspace, policy flags.
+    ``clampattn`` is accepted for signature parity; the fused kernel here masks
+    ragged tails itself, so the flag changes nothing."""
+
+    def __init__(self, device="cuda", *, ws: Optional[Workspace] = None, dev: Optional[DeviceCaps] = None, clampattn: bool = False):
+        L.init()
+        self.device = torch.device(device)
+        self.dev = dev if dev is not None else caps()
+        self.ws = ws if ws is not None else Workspace(self.device)
+        self.clampattn = clampattn
+
+    @property
+    def stream(self) -> int:
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _is_f16_cuda(*ts) -> bool:
+    return all(isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float16 for t in ts)
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return L.F16
+    if t.dtype == torch.float32:
+        return L.F32
+    raise TypeError(f"unsupported output dtype {t.dtype}")
+
+
+# ----------------------------------------------------------------------------- GEMM
+
+@dataclass(frozen=True)
+class MMMfmaPlan:
+    """Tiled MFMA kernel (the counterpart of MMCoopMatPlan, kernelplans.jl:370-374)."""
+    w_layout: int
+
+
+@dataclass(frozen=True)
+class MMSkinnyPlan:
+    """Split-K bandwidth kernel for T <= 8 (the counterpart of MMGemvPlan, kernelplans.jl:382-385)."""
+    w_layout: int
+
+
+@dataclass(frozen=True)
+class MMScalarPlan:
+    """One thread per output (the reference's Decline path, matmul.jl:140-148)."""
+    w_layout: int
+
+
+def _mat2(t: torch.Tensor):
+    """(layout, ld) of a 2-D operand: 0 = last axis contiguous, 1 = first axis contiguous."""
+    if t.dim() != 2:
+        return None
+    if t.stride(1) == 1 or t.shape[1] == 1:
+        return 0, (t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1))
+    if t.stride(0) == 1:
+        return 1, (t.stride(1) if t.shape[1] > 1 else max(t.shape[0], 1))
+    return None
+
+
+def mmplan(dev: DeviceCaps, out, A, B, bias=None):
+    """Which GEMM path this call takes (mmplan, matmul.jl:87-95).  ``A``: torch (K, F)
+    weight, ``B``: torch (T, K) activations, ``out``: torch (T, F)."""
+    if not _is_f16_cuda(A, B) or not isinstance(out, torch.Tensor) or out.dtype not in (torch.float16, torch.float32):
+        return Decline("operands")
+    la, lb, lo = _mat2(A), _mat2(B), _mat2(out)
+    if la is None or lb is None or lo is None or lb[0] != 0 or lo[0] != 0:
+        return Decline("operands")
+    K, F = A.shape
+    T = B.shape[0]
+    if B.shape[1] != K or tuple(out.shape) != (T, F):
+        return Decline("extent")
+    if bias is not None and not (bias.dim() == 1 and bias.numel() in (F, T)):
+        return Decline("bias")
+    if not dev.coopmat:
+        return Decline("nocoopmat")
+    w_layout = L.W_KF if la[0] == 0 else L.W_FK
+    lib = L.load()
+    path = lib.mi_gemm_f16_plan(out.data_ptr(), B.data_ptr(), A.data_ptr(), T, K, F, lo[1], lb[1], la[1],
+                                w_layout, _dtype_code(out), 1, 0, 0, 0)
+    return {1: MMMfmaPlan, 2: MMSkinnyPlan, 3: MMScalarPlan}.get(path, lambda _: Decline("extent"))(w_layout)
+
+
+def matmul_(ctx: Ctx, out, A, B, bias=None, *, epi="none", residual=None, bias_mode=None):
+    """``out[T,F] = epi(round(B[T,K] . A[K,F] + bias)) (+ residual)`` -- matmul!, matmul.jl:78-79.
+
+    ``epi`` is ``"none" | "gelu" | "gelu_tanh" | "relu"`` (actfn, ops.jl:1684-1685)."""
+    plan = mmplan(ctx.dev, out, A, B, bias)
+    if isinstance(plan, Decline):
+        raise DeclineError(f"matmul_ declined ({plan.reason})", L.DECLINE_OPERANDS)
+    return _matmul_run(ctx, plan, out, A, B, bias, epi, residual, bias_mode)
+
+
+def _matmul_run(ctx, plan, out, A, B, bias, epi, residual, bias_mode):
+    lib = L.init()
+    K, F = A.shape
+    T = B.shape[0]
+    la, lb, lo = _mat2(A), _mat2(B), _mat2(out)
+    if bias is None:
+        bm = L.BIAS_NONE
+    elif bias_mode is not None:
+        bm = {"col": L.BIAS_COL, "row": L.BIAS_ROW}[bias_mode]
+    else:
+        bm = L.BIAS_COL if bias.numel() == F else L.BIAS_ROW
+    if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
+        raise DeclineError("matmul_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
+    need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1)
+    ws = ctx.ws.scratch(need)
+    rc = lib.mi_gemm_f16(out.data_ptr(), B.data_ptr(), A.data_ptr(), _ptr(bias), _ptr(residual),
+                         T, K, F, lo[1], lb[1], la[1], plan.w_layout, bm, L.EPI[epi], _dtype_code(out),
+                         ws, need, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_gemm_f16", rc)
+    return out
+
+
+def batchedmatmul_(ctx: Ctx, out, A, B):
+    """``out[b] = B[b] . A[b]`` over the leading torch axis -- batchedmatmul!, matmul.jl:383.
+    ``A``: torch (Bt, K, F), ``B``: torch (Bt, T, K), ``out``: (Bt, T, F); a leading
+    extent of 1 on ``A`` or ``B`` shares that operand."""
+    lib = L.init()
+    if not _is_f16_cuda(A, B) or A.dim() != 3 or B.dim() != 3 or out.dim() != 3:
+        raise DeclineError("batchedmatmul_: operands", L.DECLINE_OPERANDS)
+    nb = out.shape[0]
+    K, F = A.shape[1:]
+    T = B.shape[1]
+    if A.stride(2) != 1 or B.stride(2) != 1 or out.stride(2) != 1:
+        raise DeclineError("batchedmatmul_: planes must be row-major", L.DECLINE_OPERANDS)
+    sA = 0 if A.shape[0] == 1 else A.stride(0)
+    sB = 0 if B.shape[0] == 1 else B.stride(0)
+    rc = lib.mi_gemm_f16_batched(out.data_ptr(), B.data_ptr(), A.data_ptr(), None, None, T, K, F,
+                                 out.stride(1), B.stride(1), A.stride(1), L.W_KF, L.BIAS_NONE, L.EPI["none"],
+                                 _dtype_code(out), nb, out.stride(0), sB, sA, None, 0, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_gemm_f16_batched", rc)
+    return out
+
+
+# ----------------------------------------------------------------------------- attention
+
+@dataclass(frozen=True)
+class FlashPlan:
+    """Fused MFMA kernel (the counterpart of FlashCMPlan, kernelplans.jl:54-324)."""
+    nsplit: int = 1
+
+
+@dataclass(frozen=True)
+class RowsSDPAPlan:
+    """One workgroup per query row and key split: decode-sized Lq, additive masks,
+    strided or odd-sized heads (takes the place of the three-pass path, attention.jl:790-834)."""
+    nsplit: int = 1
+
+
+def _strides_elbh(t: torch.Tensor):
+    return L.strides4(t.stride(3), t.stride(2), t.stride(1), t.stride(0))
+
+
+def _bias_strides(bias, Lk, Lq, H, B):
+    full = (B, H, Lq, Lk)
+    st = []
+    for ax in (3, 2, 1, 0):
+        if bias.shape[ax] not in (1, full[ax]):
+            return None
+        st.append(0 if bias.shape[ax] == 1 else bias.stride(ax))
+    return L.strides4(*st)
+
+
+def sdpaplan(ctx: Ctx, q, k, v, bias=None, scale=None, kv_len=None):
+    """Which attention implementation a call gets (sdpaplan, attention.jl:735-759)."""
+    if not _is_f16_cuda(q, k, v) or q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        return Decline("operands")
+    Bq, H, Lq, E = q.shape
+    Lk = k.shape[2]
+    if tuple(k.shape) != (Bq, H, Lk, E) or tuple(v.shape) != (Bq, H, Lk, E):
+        return Decline("extent")
+    if bias is not None:
+        if bias.dim() != 4 or bias.dtype not in (torch.float16, torch.float32) or _bias_strides(bias, Lk, Lq, H, Bq) is None:
+            return Decline("bias")
+    if not ctx.dev.coopmat:
+        return Decline("nocoopmat")
+    scale = (1.0 / math.sqrt(E)) if scale is None else float(scale)
+    ns = C.c_int(1)
+    path = L.load().mi_sdpa_f16_plan(q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k), v.data_ptr(), _strides_elbh(v),
+                                     int(bias is not None), int(kv_len is not None), E, Lq, Lk, H, Bq, scale, C.byref(ns))
+    if path == 1:
+        return FlashPlan(ns.value)
+    if path == 2:
+        return RowsSDPAPlan(ns.value)
+    return Decline("extent")
+
+
+def sdpa(ctx: Ctx, q, k, v, bias=None, scale=None, *, out=None, kv_len=None):
+    """``softmax(scale q.k + bias) v`` -- sdpa, attention.jl:712.  ``out`` (torch (B,H,Lq,E),
+    fp16 or fp32, contiguous) is the planner's slot; allocated as fp32 when absent
+    (sdpaout, attention.jl:762-765).  ``kv_len``: optional int32 (B,) tensor of valid keys."""
+    plan = sdpaplan(ctx, q, k, v, bias, scale, kv_len)
+    if isinstance(plan, Decline):
+        raise DeclineError(f"sdpa declined ({plan.reason})", L.DECLINE_OPERANDS)
+    lib = L.init()
+    Bq, H, Lq, E = q.shape
+    Lk = k.shape[2]
+    scale = (1.0 / math.sqrt(E)) if scale is None else float(scale)
+    if out is None:
+        out = torch.empty((Bq, H, Lq, E), dtype=torch.float32, device=q.device)
+    if not out.is_contiguous() or tuple(out.shape) != (Bq, H, Lq, E):
+        raise DeclineError("sdpa: out must be dense (B,H,Lq,E)", L.DECLINE_OPERANDS)
+    bst = _bias_strides(bias, Lk, Lq, H, Bq) if bias is not None else None
+    if kv_len is not None and (kv_len.dtype != torch.int32 or not kv_len.is_cuda or kv_len.numel() != Bq):
+        raise DeclineError("sdpa: kv_len must be a cuda int32 (B,) tensor", L.DECLINE_OPERANDS)
+    need = lib.mi_sdpa_f16_workspace(E, Lq, Lk, H, Bq, int(bias is not None))
+    ws = ctx.ws.scratch(need)
+    rc = lib.mi_sdpa_f16(out.data_ptr(), _dtype_code(out), q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k),
+                         v.data_ptr(), _strides_elbh(v), _ptr(bias), (L.F32 if bias is not None and bias.dtype == torch.float32 else L.F16),
+                         bst, _ptr(kv_len), E, Lq, Lk, H, Bq, scale, ws, need, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_sdpa_f16", rc)
+    return out
+
+
+# ----------------------------------------------------------------------------- convolution
+
+@dataclass(frozen=True)
+class ConvGemmPlan:
+    """1x1 or im2col + MFMA GEMM (the counterpart of ConvCoopMatPlan, kernelplans.jl:405-410)."""
+    path: str
+    workspace: int
+
+
+def convsize(n, k, s, p, d) -> int:
+    """ATen's output extent (convsize, conv.jl:309)."""
+    return (n + 2 * p - d * (k - 1) - 1) // s + 1
+
+
+def conv_plan(dev: DeviceCaps, out, x, w, stride=(1, 1), padding=(0, 0), dilation=(1, 1), groups=1):
+    """conv_coopmat_plan, conv_coopmat.jl:83-155.  stride/padding/dilation are (x, y) pairs."""
+    if not _is_f16_cuda(x, w) or x.dim() != 4 or w.dim() != 4 or not x.is_contiguous() or not w.is_contiguous():
+        return Decline("operands")
+    if not dev.coopmat:
+        return Decline("nocoopmat")
+    N, Cin, Hi, Wi = x.shape
+    Cout, cing, KH, KW = w.shape
+    if cing * groups != Cin:
+        return Decline("extent")
+    lib = L.load()
+    args = (Wi, Hi, Cin, N, KW, KH, Cout, stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1])
+    path = lib.mi_conv2d_f16_plan(*args, groups)
+    if path == 0:
+        return Decline("extent")
+    return ConvGemmPlan(L.CONV_PATHS[path], int(lib.mi_conv2d_f16_workspace(*args)))
+
+
+def convolution_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, groups, *, act="none"):
+    """convolution!(ctx, out, x, w, bias, stride, padding, dilation, groups; act) -- conv.jl:100-145.
+    ``x`` torch (N,Cin,H,W), ``w`` torch (Cout,Cin/groups,KH,KW), ``out`` torch (N,Cout,OH,OW), all
+    contiguous fp16; ``stride``/``padding``/``dilation`` are ``(x, y)`` pairs, the reverse of ATen's
+    ``(h, w)``; ``act`` is ``"none"`` or ``"relu"``."""
+    plan = conv_plan(ctx.dev, out, x, w, stride, padding, dilation, groups)
+    if isinstance(plan, Decline):
+        raise DeclineError(f"convolution_ declined ({plan.reason})", L.DECLINE_OPERANDS)
+    lib = L.init()
+    N, Cin, Hi, Wi = x.shape
+    Cout, _, KH, KW = w.shape
+    OW = convsize(Wi, KW, stride[0], padding[0], dilation[0])
+    OH = convsize(Hi, KH, stride[1], padding[1], dilation[1])
+    if tuple(out.shape) != (N, Cout, OH, OW) or not out.is_contiguous() or out.dtype != torch.float16:
+        raise DeclineError("convolution_: out must be dense fp16 (N,Cout,OH,OW)", L.DECLINE_OPERANDS)
+    ws = ctx.ws.scratch(plan.workspace)
+    rc = lib.mi_conv2d_f16(out.data_ptr(), x.data_ptr(), w.data_ptr(), _ptr(bias), Wi, Hi, Cin, N, KW, KH, Cout,
+                           stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1], groups,
+                           L.EPI[act], ws, plan.workspace, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_conv2d_f16", rc)
+    return out
+
+
+# ----------------------------------------------------------------------------- layer norm, add
+
+def layernorm_(ctx: Ctx, out, mean, rstd, a, gamma, beta, C_: int, eps: float):
+    """layernorm!(ctx, out, mean, rstd, a, gamma, beta, C, eps) -- layernorm.jl:125.
+    ``a`` contiguous fp16 with the normalised axis last; ``mean``/``rstd`` fp32 (groups,) or None."""
+    lib = L.init()
+    if not _is_f16_cuda(a, out) or not a.is_contiguous() or not out.is_contiguous():
+        raise DeclineError("layernorm_: operands", L.DECLINE_OPERANDS)
+    groups = a.numel() // C_
+    rc = lib.mi_layernorm_f16(out.data_ptr(), _ptr(mean), _ptr(rstd), a.data_ptr(), _ptr(gamma), _ptr(beta),
+                              C_, groups, float(eps), ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_layernorm_f16", rc)
+    return out
+
+
+def add_(ctx: Ctx, out, a, b):
+    """out = fp16(a + b), the residual add.Tensor (ops.jl:186-197)."""
+    lib = L.init()
+    if not _is_f16_cuda(a, b, out) or not (a.is_contiguous() and b.is_contiguous() and out.is_contiguous()):
+        raise DeclineError("add_: operands", L.DECLINE_OPERANDS)
+    rc = lib.mi_add_f16(out.data_ptr(), a.data_ptr(), b.data_ptr(), a.numel(), ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_add_f16", rc)
+    return out

@@ -1,0 +1,105 @@
+"""Convolution-as-GEMM, layer norm and residual add on the GPU through the C ABI,
+against the oracle's direct convolution (conv.jl:26-51), two-pass layer norm
+(layernorm.jl:53-113) and fp16 add.  Conv shapes include the reference's own test
+list (test_convtranspose_gemm.jl:188-191, scaled where large) and BASELINE configs 3/4."""
+import numpy as np
+import pytest
+
+import oracle
+from util import assert_parity, poison, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def _conv(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d=1, groups=1, bias=True, relu=False, expect=None, seed=1):
+    import torch
+    import juliavision_amd as jv
+    x = oracle.randn_f16((N, Cin, H, W), seed)
+    w = oracle.randn_f16((Cout, Cin // groups, KH, KW), seed + 1, 0, 0.05)
+    b = oracle.randn_f16((Cout,), seed + 2, 0, 0.5) if bias else None
+    want = oracle.conv2d_f16(x, w, b, (s, s), (p, p), (d, d), groups, relu)
+    out = poison(torch.empty(want.shape, dtype=torch.float16, device="cuda"))
+    dx, dw = to_dev(x), to_dev(w)
+    plan = jv.conv_plan(ctx.dev, out, dx, dw, (s, s), (p, p), (d, d), groups)
+    if expect:
+        assert plan.path == expect, plan
+    ctx.ws.reset()
+    jv.convolution_(ctx, out, dx, dw, None if b is None else to_dev(b), (s, s), (p, p), (d, d), groups, act="relu" if relu else "none")
+    torch.cuda.synchronize()
+    assert_parity(to_host(out), want, what=f"conv {N},{Cin},{H},{W}->{Cout} k{KH} s{s} p{p} g{groups}")
+
+
+@pytest.mark.parametrize("N,Cin,H,W,Cout,K,s,p", [
+    (1, 3, 64, 64, 144, 7, 4, 3),      # stem shape of test_convtranspose_gemm.jl:188 at 64x64
+    (1, 5, 64, 64, 32, 3, 1, 1),
+    (1, 7, 48, 48, 48, 5, 2, 2),
+    (2, 32, 32, 32, 64, 3, 1, 1),
+    (1, 3, 70, 70, 384, 14, 14, 0),    # patch embed 14x14 / stride 14 (config 3) on a 5x5 patch grid
+    (1, 256, 16, 16, 256, 3, 1, 1),    # config 4's 3x3 256->256 on a small map
+])
+def test_conv_im2col(ctx, N, Cin, H, W, Cout, K, s, p):
+    _conv(ctx, N, Cin, H, W, Cout, K, K, s, p, expect="im2col_gemm")
+
+
+def test_conv_1x1_and_relu_and_nobias(ctx):
+    _conv(ctx, 2, 144, 16, 16, 256, 1, 1, 1, 0, expect="gemm_1x1")
+    _conv(ctx, 1, 24, 5, 7, 40, 1, 1, 1, 0, expect="gemm_1x1")          # PQ = 35: scalar GEMM inside
+    _conv(ctx, 1, 16, 12, 12, 32, 3, 3, 1, 1, relu=True, bias=False)
+    _conv(ctx, 1, 8, 20, 20, 16, 3, 3, 2, 2, d=2)
+
+
+def test_conv_grouped_direct(ctx):
+    _conv(ctx, 1, 8, 10, 10, 16, 3, 3, 1, 1, groups=4, expect="direct", relu=True)
+
+
+def test_conv_config3_patch_embed_full(ctx):
+    _conv(ctx, 1, 3, 518, 518, 384, 14, 14, 14, 0, expect="im2col_gemm", seed=5)
+
+
+def test_conv_config4_band(ctx):
+    """3x3 256->256 on 64x64 (M=4096, K=2304, N=256): full size on the GPU, the oracle checks 16 output channels."""
+    import torch
+    import juliavision_amd as jv
+    x = oracle.randn_f16((1, 256, 64, 64), 7)
+    w = oracle.randn_f16((256, 256, 3, 3), 8, 0, 0.02)
+    b = oracle.randn_f16((256,), 9, 0, 0.02)
+    out = poison(torch.empty((1, 256, 64, 64), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.convolution_(ctx, out, to_dev(x), to_dev(w), to_dev(b), (1, 1), (1, 1), (1, 1), 1)
+    torch.cuda.synchronize()
+    got = to_host(out)
+    assert np.all(np.isfinite(got))
+    ch = np.r_[0:8, 248:256]
+    want = oracle.conv2d_f16(x, w[ch], b[ch], (1, 1), (1, 1))
+    assert_parity(got[:, ch], want, what="config4 conv band")
+
+
+@pytest.mark.parametrize("groups,C", [(1500, 1280), (1370, 384), (7, 144), (5, 37), (3, 4096), (2, 5000)])
+@pytest.mark.parametrize("affine", [True, False])
+def test_layernorm(ctx, groups, C, affine):
+    import torch
+    import juliavision_amd as jv
+    a = oracle.randn_f16((groups, C), 3, 0.3, 2.0)
+    g = oracle.randn_f16((C,), 4, 1.0, 0.1) if affine else None
+    b = oracle.randn_f16((C,), 5, 0.0, 0.1) if affine else None
+    want, mu, rs = oracle.layernorm_f16(a, g, b, 1e-5)
+    out = poison(torch.empty((groups, C), dtype=torch.float16, device="cuda"))
+    mean = torch.empty(groups, dtype=torch.float32, device="cuda")
+    rstd = torch.empty(groups, dtype=torch.float32, device="cuda")
+    jv.layernorm_(ctx, out, mean, rstd, to_dev(a), None if g is None else to_dev(g), None if b is None else to_dev(b), C, 1e-5)
+    torch.cuda.synchronize()
+    assert_parity(to_host(out), want, what=f"layernorm {groups}x{C}")
+    np.testing.assert_allclose(to_host(mean), mu, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(to_host(rstd), rs, rtol=1e-4, atol=1e-6)
+
+
+def test_add_bit_exact(ctx):
+    import torch
+    import juliavision_amd as jv
+    for n in (1500 * 1280, 1001):
+        a = oracle.randn_f16((n,), 1)
+        b = oracle.randn_f16((n,), 2)
+        out = torch.empty(n, dtype=torch.float16, device="cuda")
+        jv.add_(ctx, out, to_dev(a), to_dev(b))
+        torch.cuda.synchronize()
+        assert np.array_equal(to_host(out).view(np.uint16), oracle.add_f16(a, b).view(np.uint16))

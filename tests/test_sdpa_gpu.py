@@ -1,0 +1,148 @@
+"""Attention parity on the GPU through the C ABI.
+
+Oracles: the three-pass KA-CPU form (attention.jl:46-112) and the composed
+Float32 softmax(QK^T)V (test_flash.jl:13-24) for the fused kernel, which the
+reference marks cpu=false.  Gate: max rel <= 1e-2, cosine >= 0.9999; the
+reference's own fp16 tolerance is 5e-3 of max (test_flash.jl:142)."""
+import numpy as np
+import pytest
+
+import oracle
+from util import assert_parity, poison, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def _qkv(B, H, Lq, Lk, E, seed, std=1.0):
+    q = oracle.randn_f16((B, H, Lq, E), seed, 0, std)
+    k = oracle.randn_f16((B, H, Lk, E), seed + 1, 0, std)
+    v = oracle.randn_f16((B, H, Lk, E), seed + 2, 0, std)
+    return q, k, v
+
+
+def _check(ctx, q, k, v, *, bias=None, scale=None, kv_len=None, out_dtype="f16", expect=None, what=""):
+    import torch
+    import juliavision_amd as jv
+    dq, dk, dv = (a if isinstance(a, torch.Tensor) else to_dev(a) for a in (q, k, v))
+    hq, hk, hv = (to_host(a) if isinstance(a, torch.Tensor) else a for a in (q, k, v))
+    db = None if bias is None else to_dev(bias)
+    dl = None if kv_len is None else torch.tensor(kv_len, dtype=torch.int32, device="cuda")
+    plan = jv.sdpaplan(ctx, dq, dk, dv, db, scale, dl)
+    if expect is not None:
+        assert type(plan).__name__ == expect, f"{what}: plan {plan}"
+    B, H, Lq, E = hq.shape
+    out = poison(torch.empty((B, H, Lq, E), dtype=torch.float16 if out_dtype == "f16" else torch.float32, device="cuda"))
+    ctx.ws.reset()
+    jv.sdpa(ctx, dq, dk, dv, db, scale, out=out, kv_len=dl)
+    torch.cuda.synchronize()
+    got = to_host(out)
+    ref32 = oracle.sdpa_ref_f32(hq, hk, hv, bias, scale, kv_len=kv_len)
+    assert_parity(got, ref32, what=what + " vs composed f32")
+    tp = oracle.sdpa_threepass_f16(hq, hk, hv, bias, scale, kv_len=kv_len, out_f32=(out_dtype != "f16"))
+    assert_parity(got, tp, what=what + " vs three-pass")
+    return got
+
+
+@pytest.mark.parametrize("B,H,Lq,Lk,E", [
+    (1, 2, 128, 128, 64), (1, 2, 256, 256, 64), (2, 3, 200, 137, 64), (1, 1, 64, 17, 64),
+    (1, 2, 130, 23, 32), (1, 2, 128, 128, 72), (1, 1, 128, 64, 16), (1, 2, 192, 320, 128), (1, 1, 1500, 1500, 64),
+])
+def test_flash_shapes(ctx, B, H, Lq, Lk, E):
+    q, k, v = _qkv(B, H, Lq, Lk, E, 31)
+    _check(ctx, q, k, v, expect="FlashPlan", what=f"flash {B},{H},{Lq},{Lk},{E}")
+
+
+def test_flash_small_inputs_and_f32_out(ctx):
+    # the reference's own test inputs: randn * 0.2 (test_flash.jl:41-43)
+    q, k, v = _qkv(2, 2, 128, 128, 72, 41, std=0.2)
+    _check(ctx, q, k, v, out_dtype="f32", expect="FlashPlan", what="flash 0.2 f32")
+
+
+def test_reference_closed_form_inputs(ctx):
+    # 0.4*sin / cos / sin over ranges 9, 7, 5 (test_coopmat_attention.jl:54-55), (E,L,H,B) = (64,256,2,1)
+    E, L, H, B = 64, 256, 2, 1
+    n = E * L * H * B
+    q = (0.4 * np.sin(np.linspace(0, 9, n))).astype(np.float16).reshape(B, H, L, E)
+    k = (0.4 * np.cos(np.linspace(0, 7, n))).astype(np.float16).reshape(B, H, L, E)
+    v = (0.4 * np.sin(np.linspace(0, 5, n))).astype(np.float16).reshape(B, H, L, E)
+    _check(ctx, q, k, v, expect="FlashPlan", what="closed-form inputs")
+
+
+def test_strided_heads_from_packed_qkv(ctx):
+    """q/k/v as strided views of one packed [T][3][H][E] projection -- how the graph hands them over."""
+    import torch
+    T, H, E = 300, 4, 64
+    packed = to_dev(oracle.randn_f16((1, T, 3, H, E), 51))
+    q = packed[:, :, 0].permute(0, 2, 1, 3)
+    k = packed[:, :, 1].permute(0, 2, 1, 3)
+    v = packed[:, :, 2].permute(0, 2, 1, 3)
+    assert not q.is_contiguous()
+    _check(ctx, q, k, v, expect="FlashPlan", what="strided qkv")
+
+
+def test_rows_path_small_lq_and_ragged(ctx):
+    # ragged shapes of test_flash.jl:189-190 as (E,Lq,Lk,H,B): (16,23,4096,8,1), (32,23,23,8,1), (16,23,17,4,1)
+    for (E, Lq, Lk, H, B) in [(16, 23, 4096, 8, 1), (32, 23, 23, 8, 1), (16, 23, 17, 4, 1), (64, 1, 448, 20, 4), (72, 5, 100, 2, 1), (20, 3, 50, 2, 2)]:
+        q, k, v = _qkv(B, H, Lq, Lk, E, 61)
+        _check(ctx, q, k, v, expect="RowsSDPAPlan", what=f"rows {E},{Lq},{Lk},{H},{B}")
+
+
+def test_additive_mask_and_kv_len_agree(ctx):
+    """The decoder's additive 0 / finfo.min mask (B,H,1,Lk) and kv_len give the same result."""
+    B, H, Lk, E = 4, 20, 448, 64
+    q, k, v = _qkv(B, H, 1, Lk, E, 71)
+    for pos in (3, 447):
+        mask = np.where(np.arange(Lk) <= pos, 0.0, np.finfo(np.float16).min).astype(np.float16).reshape(1, 1, 1, Lk)
+        mask = np.broadcast_to(mask, (B, 1, 1, Lk)).copy()
+        a = _check(ctx, q, k, v, bias=mask, scale=1.0, expect="RowsSDPAPlan", what=f"mask pos {pos}")
+        b = _check(ctx, q, k, v, kv_len=[pos + 1] * B, scale=1.0, expect="RowsSDPAPlan", what=f"kv_len pos {pos}")
+        np.testing.assert_allclose(a.astype(np.float32), b.astype(np.float32), rtol=2e-3, atol=2e-3)
+
+
+def test_full_bias_f32(ctx):
+    B, H, Lq, Lk, E = 1, 2, 70, 90, 64
+    q, k, v = _qkv(B, H, Lq, Lk, E, 81)
+    bias = oracle.randn_f32((B, H, Lq, Lk), 84)
+    _check(ctx, q, k, v, bias=bias, expect="RowsSDPAPlan", what="full f32 bias")
+
+
+def test_all_masked_rows_give_zeros(ctx):
+    import torch
+    B, H, Lq, Lk, E = 2, 2, 128, 64, 64
+    q, k, v = _qkv(B, H, Lq, Lk, E, 91)
+    got = _check(ctx, q, k, v, kv_len=[0, 40], expect="FlashPlan", what="kv_len 0 flash")
+    assert np.all(got[0] == 0)
+    q1 = q[:, :, :1]
+    got = _check(ctx, q1, k, v, kv_len=[0, 40], expect="RowsSDPAPlan", what="kv_len 0 rows")
+    assert np.all(got[0] == 0)
+    mask = np.full((B, 1, 1, Lk), -np.inf, dtype=np.float32)
+    got = _check(ctx, q1, k, v, bias=mask, what="-inf mask")
+    assert np.all(got == 0)
+
+
+def test_rows_sum_to_one(ctx):
+    """softmax weights sum to 1: with v == 1 the output is exactly 1 up to fp16 rounding."""
+    import torch
+    B, H, Lq, Lk, E = 1, 2, 200, 333, 64
+    q, k, _ = _qkv(B, H, Lq, Lk, E, 95)
+    v = np.ones((B, H, Lk, E), dtype=np.float16)
+    got = _check(ctx, q, k, v, what="v=1")
+    assert np.max(np.abs(got.astype(np.float32) - 1.0)) < 2e-3
+
+
+def test_config4_attention_band(ctx):
+    """BASELINE config 4 attention at full size (L=4096, 16 heads x 64); the oracle checks a band of
+    query rows of two heads (the full three-pass form takes minutes on the CPU)."""
+    import torch
+    import juliavision_amd as jv
+    B, H, L, E = 1, 16, 4096, 64
+    q, k, v = _qkv(B, H, L, L, E, 101)
+    out = poison(torch.empty((B, H, L, E), dtype=torch.float16, device="cuda"))
+    jv.sdpa(ctx, to_dev(q), to_dev(k), to_dev(v), None, None, out=out)
+    torch.cuda.synchronize()
+    got = to_host(out)
+    assert np.all(np.isfinite(got))
+    for h in (0, 15):
+        rows = np.r_[0:16, 2040:2056, 4080:4096]
+        want = oracle.sdpa_ref_f32(q[:, h:h + 1, rows], k[:, h:h + 1], v[:, h:h + 1])
+        assert_parity(got[:, h:h + 1, rows], want, what=f"config4 head {h}")
