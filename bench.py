@@ -1,0 +1,364 @@
+#!/usr/bin/env python3
+"""Benchmark of the dense-contraction hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--detail/--no-detail] [--no-cpu]
+
+A *step* is one Whisper-large-v3-turbo-shaped encoder block (BASELINE config 2): batch 1, 1500
+tokens, d_model 1280, 20 heads x 64, FFN 5120 with exact GELU, pre-LayerNorm, fp16 with fp32
+accumulation, on synthetic seeded inputs already resident in HBM:
+
+    LN -> q,k,v = h.Wq/Wk/Wv + b -> SDPA -> (.Wo + b) + x -> LN -> gelu(.W1 + b) -> (.W2 + b) + res
+
+nine kernel launches through the C ABI of libmi355dnn.so.  ``value`` is the block's algorithmic
+TFLOP/s (70.50 GFLOP per block: 58.98 GEMM + 11.52 attention); ``ms_per_step`` is ms per encoder
+block.  ``roofline`` describes the dominant kernel -- the fp16 MFMA GEMM -- at its largest launch
+in the block, the fc1 linear 1500x1280 -> 5120 + bias + GELU (BASELINE config 1's shape), timed
+live with HIP events around that launch in every timed step.  ``cpu_baseline`` is the CPU oracle
+(a C port of the reference's KernelAbstractions-CPU forms) timed on this host on a stated sample.
+``detail`` carries the other configs' kernels (config 1 GEMM in both weight layouts, config 4
+attention and conv, config 3 shapes, config 5 decode linears and attention in GB/s), each timed
+with HIP events over back-to-back launches on rotating buffer sets.
+
+One JSON line is printed on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_F16_TFLOPS = 2500.0       # MI355X dense fp16 MFMA, vendor figure
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, vendor figure
+
+# HBM bytes per launch of the dominant kernel (fc1 GEMM), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of `python bench.py --no-cpu --no-detail`, scaled by the same counters on a plain copy kernel of
+# known size; see profiles/.  None until measured.
+FC1_TRAFFIC_BYTES = None
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--detail", dest="detail", action="store_true", default=True)
+    ap.add_argument("--no-detail", dest="detail", action="store_false")
+    ap.add_argument("--no-cpu", dest="cpu", action="store_false", default=True)
+    return ap.parse_args()
+
+
+# ----------------------------------------------------------------------------- helpers
+
+class Call:
+    """A C-ABI call with its arguments converted once, so that issuing it costs one foreign call."""
+
+    def __init__(self, fn, *args):
+        self.fn = fn
+        assert len(args) == len(fn.argtypes), (fn.__name__, len(args), len(fn.argtypes))
+        self.args = tuple(a if (a is None or isinstance(a, (C._SimpleCData, C.Array))) else t(a)
+                          for t, a in zip(fn.argtypes, args))
+
+    def __call__(self):
+        rc = self.fn(*self.args)
+        if rc != 0:
+            raise RuntimeError(f"{self.fn.__name__} returned status {rc}")
+
+
+def dev(a):
+    import numpy as np
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def event_time(fn, reps, samples=15):
+    """Median seconds per call of fn() over `samples` groups of `reps` back-to-back launches."""
+    import torch
+    fn(); fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(samples):
+        s = torch.cuda.Event(enable_timing=True)
+        e = torch.cuda.Event(enable_timing=True)
+        s.record()
+        for i in range(reps):
+            fn()
+        e.record()
+        e.synchronize()
+        ts.append(s.elapsed_time(e) * 1e-3 / reps)
+    ts.sort()
+    return ts[len(ts) // 2], ts[0], ts[-1]
+
+
+# ----------------------------------------------------------------------------- the encoder block
+
+class EncoderBlock:
+    T, D, H, E, FF = 1500, 1280, 20, 64, 5120
+    FLOP_GEMM = 4 * (2 * 1500 * 1280 * 1280) + 2 * (2 * 1500 * 1280 * 5120)
+    FLOP_ATTN = 4 * 1500 * 1500 * 64 * 20
+    FLOP = FLOP_GEMM + FLOP_ATTN
+    FC1_FLOP = 2 * 1500 * 1280 * 5120
+
+    def __init__(self, lib, stream, seed=1000):
+        import numpy as np
+        import torch
+        import oracle
+        L = self.L = __import__("juliavision_amd")._lib
+        T, D, H, E, FF = self.T, self.D, self.H, self.E, self.FF
+        f16 = torch.float16
+        self.host = {}
+        h = self.host
+        h["x"] = oracle.randn_f16((T, D), seed)
+        for i, n in enumerate(("wq", "wk", "wv", "wo")):
+            h[n] = oracle.randn_f16((D, D), seed + 1 + i, 0, 0.02)
+        h["w1"] = oracle.randn_f16((D, FF), seed + 5, 0, 0.02)
+        h["w2"] = oracle.randn_f16((FF, D), seed + 6, 0, 0.02)
+        for i, (n, m) in enumerate((("bq", D), ("bk", D), ("bv", D), ("bo", D), ("b1", FF), ("b2", D))):
+            h[n] = oracle.randn_f16((m,), seed + 10 + i, 0, 0.02)
+        for i, n in enumerate(("g1", "g2")):
+            h[n] = oracle.randn_f16((D,), seed + 20 + i, 1.0, 0.02)
+        for i, n in enumerate(("be1", "be2")):
+            h[n] = oracle.randn_f16((D,), seed + 22 + i, 0.0, 0.02)
+        d = self.d = {k: dev(v) for k, v in h.items()}
+        for n in ("h1", "q", "k", "v", "a", "o", "h2", "y"):
+            d[n] = torch.empty((T, D), dtype=f16, device="cuda")
+        d["f"] = torch.empty((T, FF), dtype=f16, device="cuda")
+        p = lambda n: d[n].data_ptr()
+
+        def gemm(y, x, w, b, K, F, epi, res=None):
+            return Call(lib.mi_gemm_f16, p(y), p(x), p(w), p(b), (p(res) if res else None), T, K, F, F, K, F,
+                        L.W_KF, L.BIAS_COL, L.EPI[epi], L.F16, None, 0, stream)
+
+        tok = L.strides4(1, D, E, T * D)      # (E, L, H, B) strides of a token-major [T][H][E] buffer
+        scale = 1.0 / np.sqrt(E)
+        self.fc1 = gemm("f", "h2", "w1", "b1", D, FF, "gelu")
+        self.calls_before_fc1 = [
+            Call(lib.mi_layernorm_f16, p("h1"), None, None, p("x"), p("g1"), p("be1"), D, T, 1e-5, stream),
+            gemm("q", "h1", "wq", "bq", D, D, "none"),
+            gemm("k", "h1", "wk", "bk", D, D, "none"),
+            gemm("v", "h1", "wv", "bv", D, D, "none"),
+            Call(lib.mi_sdpa_f16, p("a"), L.F16, tok, p("q"), tok, p("k"), tok, p("v"), tok, None, 0, None, None,
+                 E, T, T, H, 1, scale, None, 0, stream),
+            gemm("o", "a", "wo", "bo", D, D, "none", res="x"),
+            Call(lib.mi_layernorm_f16, p("h2"), None, None, p("o"), p("g2"), p("be2"), D, T, 1e-5, stream),
+        ]
+        self.calls_after_fc1 = [gemm("y", "f", "w2", "b2", FF, D, "none", res="o")]
+
+    def step(self, ev=None):
+        for c in self.calls_before_fc1:
+            c()
+        if ev is not None:
+            ev[0].record()
+        self.fc1()
+        if ev is not None:
+            ev[1].record()
+        for c in self.calls_after_fc1:
+            c()
+
+    # ---- the same block on the CPU oracle, on a sample of the work, scaled to one block
+    def cpu_baseline(self):
+        import numpy as np
+        import oracle
+        h = self.host
+        T, D, H, E = self.T, self.D, self.H, self.E
+        # One whole block: every token row through the six linears and both layer norms, all 20 heads of
+        # the three-pass attention at full length (a few seconds on 16 threads), repeated `reps` times.
+        reps = 3
+        rows, heads = T, H
+        qa = oracle.randn_f16((1, heads, T, E), 5)
+        ka = oracle.randn_f16((1, heads, T, E), 6)
+        va = oracle.randn_f16((1, heads, T, E), 7)
+        t_lin = t_att = 0.0
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            x = h["x"][:rows]
+            h1, _, _ = oracle.layernorm_f16(x, h["g1"], h["be1"], 1e-5)
+            q = oracle.gemm_f16(h1, h["wq"], h["bq"])
+            oracle.gemm_f16(h1, h["wk"], h["bk"])
+            oracle.gemm_f16(h1, h["wv"], h["bv"])
+            o = oracle.gemm_f16(q, h["wo"], h["bo"], residual=x)
+            h2, _, _ = oracle.layernorm_f16(o, h["g2"], h["be2"], 1e-5)
+            f = oracle.gemm_f16(h2, h["w1"], h["b1"], epi="gelu")
+            oracle.gemm_f16(f, h["w2"], h["b2"], residual=o)
+            t1 = time.perf_counter()
+            oracle.sdpa_threepass_f16(qa, ka, va)
+            t2 = time.perf_counter()
+            t_lin += (t1 - t0) / reps
+            t_att += (t2 - t1) / reps
+        sec = t_lin + t_att
+        return {
+            "value": round(self.FLOP / sec / 1e12, 6), "unit": "TFLOP/s", "cores": oracle.threads(), "kind": "port",
+            "sample": f"the whole block, {reps} times: all {T} token rows through the six linears + both layer norms "
+                      f"({t_lin:.2f} s) and all {H} heads of the three-pass attention ({t_att:.2f} s) per block",
+            "ms_per_step": round(sec * 1e3, 1),
+        }
+
+
+# ----------------------------------------------------------------------------- other configs (detail)
+
+def detail_benchmarks(lib, L, stream):
+    import numpy as np
+    import torch
+    out = {}
+    f16 = torch.float16
+    NB = 3   # rotating buffer sets
+
+    def gemm_case(name, T, K, F, layout, epi="none", sets=NB, reps=20):
+        Xs = [torch.randn((T, K), dtype=f16, device="cuda") / K ** 0.5 for _ in range(sets)]
+        Ws = [torch.randn((K, F) if layout == L.W_KF else (F, K), dtype=f16, device="cuda") * 0.02 for _ in range(sets)]
+        b = torch.randn((F,), dtype=f16, device="cuda") * 0.02
+        Ys = [torch.empty((T, F), dtype=f16, device="cuda") for _ in range(min(sets, 3))]
+        need = lib.mi_gemm_f16_workspace(T, K, F, layout, 1)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        calls = [Call(lib.mi_gemm_f16, Ys[i % len(Ys)].data_ptr(), Xs[i].data_ptr(), Ws[i].data_ptr(), b.data_ptr(), None, T, K, F, F, K,
+                      (F if layout == L.W_KF else K), layout, L.BIAS_COL, L.EPI[epi], L.F16, ws.data_ptr(), need, stream) for i in range(sets)]
+        state = {"i": 0}
+
+        def fn():
+            calls[state["i"] % sets]()
+            state["i"] += 1
+        med, lo, hi = event_time(fn, reps)
+        flop = 2.0 * T * K * F
+        wbytes = 2.0 * K * F
+        out[name] = {"us": round(med * 1e6, 2), "us_min": round(lo * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 1),
+                     "frac_mfma_peak": round(flop / med / 1e12 / PEAK_F16_TFLOPS, 4),
+                     "weight_GB/s": round(wbytes / med / 1e9, 1)}
+        return out[name]
+
+    def attn_case(name, B, H, Lq, Lk, E, kv_len=None, sets=NB, reps=10):
+        qs = [torch.randn((B, H, Lq, E), dtype=f16, device="cuda") for _ in range(sets)]
+        ks = [torch.randn((B, H, Lk, E), dtype=f16, device="cuda") for _ in range(sets)]
+        vs = [torch.randn((B, H, Lk, E), dtype=f16, device="cuda") for _ in range(sets)]
+        o = torch.empty((B, H, Lq, E), dtype=f16, device="cuda")
+        kl = None if kv_len is None else torch.full((B,), kv_len, dtype=torch.int32, device="cuda")
+        need = lib.mi_sdpa_f16_workspace(E, Lq, Lk, H, B, 0)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        dq, dk = L.strides4(1, E, E * Lq, E * Lq * H), L.strides4(1, E, E * Lk, E * Lk * H)
+        calls = [Call(lib.mi_sdpa_f16, o.data_ptr(), L.F16, None, qs[i].data_ptr(), dq, ks[i].data_ptr(), dk, vs[i].data_ptr(), dk,
+                      None, 0, None, (kl.data_ptr() if kl is not None else None), E, Lq, Lk, H, B, 1.0 / np.sqrt(E),
+                      ws.data_ptr(), need, stream) for i in range(sets)]
+        state = {"i": 0}
+
+        def fn():
+            calls[state["i"] % sets]()
+            state["i"] += 1
+        med, lo, hi = event_time(fn, reps)
+        keys = Lk if kv_len is None else kv_len
+        flop = 4.0 * Lq * keys * E * H * B
+        kvbytes = 2.0 * 2 * keys * E * H * B
+        out[name] = {"us": round(med * 1e6, 2), "us_min": round(lo * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 2),
+                     "frac_mfma_peak": round(flop / med / 1e12 / PEAK_F16_TFLOPS, 4), "kv_GB/s": round(kvbytes / med / 1e9, 1)}
+
+    # config 1: the linear, both weight layouts
+    gemm_case("c1_linear_1500x1280x5120_W[K][F]_bias", 1500, 1280, 5120, L.W_KF)
+    gemm_case("c1_linear_1500x1280x5120_W[F][K]_bias", 1500, 1280, 5120, L.W_FK)
+    gemm_case("c2_proj_1500x1280x1280", 1500, 1280, 1280, L.W_KF)
+    gemm_case("c2_fc2_1500x5120x1280", 1500, 5120, 1280, L.W_KF)
+    # config 3: ViT-S/14 shapes
+    gemm_case("c3_qkv_1370x384x1152", 1370, 384, 1152, L.W_KF)
+    gemm_case("c3_fc1_1370x384x1536", 1370, 384, 1536, L.W_KF, epi="gelu")
+    gemm_case("c3_fc2_1370x1536x384", 1370, 1536, 384, L.W_KF)
+    attn_case("c3_attn_L1370_6x64", 1, 6, 1370, 1370, 64)
+    attn_case("c2_attn_L1500_20x64", 1, 20, 1500, 1500, 64)
+    # config 4: global attention at 4096 and the 3x3 conv
+    attn_case("c4_attn_L4096_16x64", 1, 16, 4096, 4096, 64)
+    x = torch.randn((1, 256, 64, 64), dtype=f16, device="cuda")
+    w = torch.randn((256, 256, 3, 3), dtype=f16, device="cuda") * 0.02
+    b = torch.randn((256,), dtype=f16, device="cuda") * 0.02
+    o = torch.empty((1, 256, 64, 64), dtype=f16, device="cuda")
+    need = lib.mi_conv2d_f16_workspace(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+    conv = Call(lib.mi_conv2d_f16, o.data_ptr(), x.data_ptr(), w.data_ptr(), b.data_ptr(), 64, 64, 256, 1, 3, 3, 256,
+                1, 1, 1, 1, 1, 1, 1, L.EPI["none"], ws.data_ptr(), need, stream)
+    med, lo, hi = event_time(conv, 10)
+    flop = 2.0 * 4096 * 2304 * 256
+    out["c4_conv3x3_256to256_64x64"] = {"us": round(med * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 2),
+                                        "frac_mfma_peak": round(flop / med / 1e12 / PEAK_F16_TFLOPS, 4)}
+    # config 5: decode-sized linears (HBM-bound on the weights; enough rotating weight sets to exceed the
+    # 256 MB last-level cache) and single-query attention over the caches
+    for bsz in (1, 4, 8):
+        for (K, F) in ((1280, 1280), (1280, 5120)):
+            sets = int(np.ceil(320e6 / (2.0 * K * F)))
+            for lay, tag in ((L.W_KF, "W[K][F]"), (L.W_FK, "W[F][K]")):
+                r = gemm_case(f"c5_linear_b{bsz}_{K}to{F}_{tag}", bsz, K, F, lay, sets=sets, reps=sets)
+                r["frac_hbm_peak"] = round(r["weight_GB/s"] / PEAK_HBM_GBS, 4)
+                del r["TFLOP/s"], r["frac_mfma_peak"]
+        for (nm, Lk, kvl) in (("self_pos447", 448, 448), ("self_pos3", 448, 4), ("cross", 1500, None)):
+            sets = int(np.ceil(320e6 / (4.0 * Lk * 64 * 20 * bsz)))
+            attn_case(f"c5_attn_b{bsz}_{nm}", bsz, 20, 1, Lk, 64, kv_len=kvl, sets=sets, reps=sets)
+            r = out[f"c5_attn_b{bsz}_{nm}"]
+            r["frac_hbm_peak"] = round(r["kv_GB/s"] / PEAK_HBM_GBS, 4)
+            del r["TFLOP/s"], r["frac_mfma_peak"]
+    return out
+
+
+# ----------------------------------------------------------------------------- main
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported (no collective, "
+              "sharding or rank code exists in this path).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import juliavision_amd as jv
+    L = jv._lib
+    lib = L.init()
+    stream = torch.cuda.current_stream().cuda_stream
+    blk = EncoderBlock(lib, stream)
+
+    for _ in range(args.warmup):
+        blk.step()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        blk.step(evs[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    sec = (t1 - t0) / args.steps
+    fc1_ms = sorted(s.elapsed_time(e) for s, e in evs)
+    fc1_avg = sum(fc1_ms) / len(fc1_ms) * 1e-3
+    y = blk.d["y"].float()
+    if not bool(torch.isfinite(y).all()) or float(y.abs().max()) < 1e-3:
+        raise RuntimeError("encoder block produced non-finite or empty output")
+
+    achieved = blk.FC1_FLOP / fc1_avg / 1e12
+    res = {
+        "metric": "fp16 GEMM/attention TFLOP/s + % of MFMA peak; ms per encoder block",
+        "value": round(blk.FLOP / sec / 1e12, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: Whisper-large-v3-turbo-shaped encoder block, batch 1, 1500 tokens, "
+                               "d_model 1280, 20x64 heads, FFN 5120 GELU(erf), pre-LN, fp16 in / fp32 accumulate; "
+                               "70.50 GFLOP per block (58.98 GEMM + 11.52 attention); 9 launches via the C ABI",
+                   "tokens": 1500, "d_model": 1280, "heads": 20, "head_dim": 64, "ffn": 5120,
+                   "weight_layout": "[K][F] (the reference's hoisted layout)"},
+        "frac_mfma_peak": round(blk.FLOP / sec / 1e12 / PEAK_F16_TFLOPS, 4),
+        "roofline": {"kernel": "gemm_mfma_kernel<128,256,64> fc1: Y[1500x5120] = gelu(X[1500x1280].W[1280x5120] + b)",
+                     "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": FC1_TRAFFIC_BYTES,
+                     "flop_per_launch": blk.FC1_FLOP, "avg_launch_us": round(fc1_avg * 1e6, 2),
+                     "median_launch_us": round(fc1_ms[len(fc1_ms) // 2] * 1e3, 2)},
+    }
+    if args.detail:
+        res["detail"] = detail_benchmarks(lib, L, stream)
+    if args.cpu:
+        res["cpu_baseline"] = blk.cpu_baseline()
+    else:
+        res["cpu_baseline"] = None
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

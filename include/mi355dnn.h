@@ -116,8 +116,11 @@ int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,
  *   q (E,Lq,H,B), k (E,Lk,H,B), v (E,Lk,H,B): fp16, each given as a base pointer
  *   plus four element strides in (E, L, H, B) order -- the reference passes
  *   root pointer + offsets + strides the same way (flash.jl:1353-1365,1448-1474).
- *   out is dense (E,Lq,H,B) = row-major [B][H][Lq][E], fp16 or fp32 (the graph's
- *   declared type, ops.jl:1365-1391).
+ *   out is (E,Lq,H,B), fp16 or fp32 (the graph's declared type, ops.jl:1365-1391);
+ *   out_strides NULL means dense = row-major [B][H][Lq][E], which is what the
+ *   reference allocates (attention.jl:762-765).  Element strides in (E,L,H,B)
+ *   order let the caller have the result written token-major ([B][Lq][H][E]),
+ *   i.e. already in the layout the graph's following permute + reshape produces.
  *   bias: optional additive mask laid out (Lk,Lq,H,B) with element strides
  *   bias_strides[4]; a stride of 0 broadcasts that axis (attention.jl:55-59,
  *   launch.jl:72-75); bias_dtype MI_F16 / MI_F32.
@@ -127,7 +130,7 @@ int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,
  * Replaces sdpa(ctx, q, k, v, bias, scale; out) -- attention.jl:712-834 -- and the
  * fused kernels behind it: attn_flash_cm! + attn_flash_cm_merge! (flash.jl:459-1036,
  * 1398-1421), attn_softmax_rows! / sdpa_coopmat! (attention.jl:514-705). */
-int mi_sdpa_f16(void *out, int out_dtype,
+int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
                 const void *q, const int64_t q_strides[4],
                 const void *k, const int64_t k_strides[4],
                 const void *v, const int64_t v_strides[4],

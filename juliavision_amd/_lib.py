@@ -36,7 +36,7 @@ SIGNATURES = {
     "mi_gemv_f16": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
     "mi_gemm_f16_workspace": (_sz, [_i64, _i64, _i64, _int, _i64]),
     "mi_gemm_f16_plan": (_int, [_vp] * 3 + [_i64] * 6 + [_int] * 2 + [_i64] * 4),
-    "mi_sdpa_f16": (_int, [_vp, _int, _vp, _i64p, _vp, _i64p, _vp, _i64p, _vp, _int, _i64p, _vp] + [_i64] * 5 + [_f32, _vp, _sz, _vp]),
+    "mi_sdpa_f16": (_int, [_vp, _int, _i64p, _vp, _i64p, _vp, _i64p, _vp, _i64p, _vp, _int, _i64p, _vp] + [_i64] * 5 + [_f32, _vp, _sz, _vp]),
     "mi_sdpa_f16_workspace": (_sz, [_i64] * 5 + [_int]),
     "mi_sdpa_f16_plan": (_int, [_vp, _i64p, _vp, _i64p, _vp, _i64p, _int, _int] + [_i64] * 5 + [_f32, C.POINTER(C.c_int)]),
     "mi_conv2d_f16": (_int, [_vp] * 4 + [_i64] * 14 + [_int, _vp, _sz, _vp]),

@@ -21,7 +21,7 @@ namespace {
 struct SdpaArgs {
     void *out;
     const half_t *q, *k, *v;
-    long qs[4], ks[4], vs[4];      // (E, L, H, B) element strides
+    long qs[4], ks[4], vs[4], os[4];   // (E, L, H, B) element strides
     const void *bias;
     long bs[4];                    // (Lk, Lq, H, B) element strides, 0 = broadcast
     const int *kv_len;
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
     const int qi = q0 + l32;
     if (qi < p.Lq) {
         const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-        const long base = (((long)b * p.H + h) * p.Lq + qi) * p.E;
+        const long base = (long)b * p.os[3] + (long)h * p.os[2] + (long)qi * p.os[1];
 #pragma unroll
         for (int t = 0; t < ET; t++)
 #pragma unroll
@@ -392,8 +392,9 @@ __global__ __launch_bounds__(256) void sdpa_rows_kernel(SdpaArgs p) {
         const long orow = ((long)b * p.H + h) * p.Lq + lq;
         if (p.nsplit == 1) {
             const float r = L > 0.0f ? O / L : 0.0f;
-            if (p.out_f32) reinterpret_cast<float *>(p.out)[orow * p.E + tid] = r;
-            else reinterpret_cast<half_t *>(p.out)[orow * p.E + tid] = (half_t)r;
+            const long oo = (long)b * p.os[3] + (long)h * p.os[2] + (long)lq * p.os[1] + (long)tid * p.os[0];
+            if (p.out_f32) reinterpret_cast<float *>(p.out)[oo] = r;
+            else reinterpret_cast<half_t *>(p.out)[oo] = (half_t)r;
         } else {
             const long rows = (long)p.B * p.H * p.Lq;
             p.part_o[((long)split * rows + orow) * p.E + tid] = O;
@@ -422,8 +423,10 @@ __global__ void sdpa_merge_kernel(SdpaArgs p) {
         O += a * p.part_o[((long)s * rows + row) * p.E + e];
     }
     const float r = L > 0.0f ? O / L : 0.0f;
-    if (p.out_f32) reinterpret_cast<float *>(p.out)[idx] = r;
-    else reinterpret_cast<half_t *>(p.out)[idx] = (half_t)r;
+    const long lq = row % p.Lq, hb = row / p.Lq, h = hb % p.H, b = hb / p.H;
+    const long oo = b * p.os[3] + h * p.os[2] + lq * p.os[1] + (long)e * p.os[0];
+    if (p.out_f32) reinterpret_cast<float *>(p.out)[oo] = r;
+    else reinterpret_cast<half_t *>(p.out)[oo] = (half_t)r;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -450,12 +453,12 @@ int sdpa_path(const SdpaArgs &a) {
     if (a.E < 1 || a.E > 256 || a.Lq < 0 || a.Lk < 0 || a.H < 1 || a.B < 1) return MI_SDPA_DECLINE;
     if (a.H > 65535 || a.B > 65535 || (int64_t)a.Lq * a.H * 64 > INT32_MAX) return MI_SDPA_DECLINE;
     bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
-    bool out_ok = aligned_to(a.out, 16) || a.out == nullptr;
+    bool out_ok = (aligned_to(a.out, 16) || a.out == nullptr) && a.os[0] == 1 && a.os[1] % 8 == 0 && a.os[2] % 8 == 0 && a.os[3] % 8 == 0;
     if (vec && out_ok && !a.bias && a.scale > 0.0f && a.E <= 128 && a.Lq >= 64 && a.Lk >= 1) return MI_SDPA_FLASH;
     return MI_SDPA_ROWS;
 }
 
-int fill(SdpaArgs &a, void *out, int out_dtype, const void *q, const int64_t *qs, const void *k, const int64_t *ks,
+int fill(SdpaArgs &a, void *out, int out_dtype, const int64_t *os, const void *q, const int64_t *qs, const void *k, const int64_t *ks,
          const void *v, const int64_t *vs, const void *bias, int bias_dtype, const int64_t *bs, const int32_t *kv_len,
          int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale) {
     if (!q || !k || !v || !qs || !ks || !vs) return MI_DECLINE_OPERANDS;
@@ -464,6 +467,8 @@ int fill(SdpaArgs &a, void *out, int out_dtype, const void *q, const int64_t *qs
     if (E > INT32_MAX || Lq > INT32_MAX || Lk > INT32_MAX || H > INT32_MAX || B > INT32_MAX) return MI_DECLINE_EXTENT;
     a.out = out; a.q = (const half_t *)q; a.k = (const half_t *)k; a.v = (const half_t *)v;
     for (int i = 0; i < 4; i++) { a.qs[i] = qs[i]; a.ks[i] = ks[i]; a.vs[i] = vs[i]; a.bs[i] = bias ? bs[i] : 0; }
+    if (os) { for (int i = 0; i < 4; i++) a.os[i] = os[i]; }
+    else { a.os[0] = 1; a.os[1] = E; a.os[2] = E * Lq; a.os[3] = E * Lq * H; }
     a.bias = bias; a.bias_f32 = bias_dtype == MI_F32; a.kv_len = kv_len;
     a.part_o = a.part_ml = nullptr;
     a.E = (int)E; a.Lq = (int)Lq; a.Lk = (int)Lk; a.H = (int)H; a.B = (int)B;
@@ -504,7 +509,7 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
     (void)has_kv_len;
     SdpaArgs a;
     static const int64_t zero4[4] = {0, 0, 0, 0};
-    int rc = fill(a, nullptr, MI_F16, q, q_strides, k, k_strides, v, v_strides, has_bias ? (const void *)q : nullptr, MI_F16,
+    int rc = fill(a, nullptr, MI_F16, nullptr, q, q_strides, k, k_strides, v, v_strides, has_bias ? (const void *)q : nullptr, MI_F16,
                   zero4, nullptr, E, Lq, Lk, H, B, scale);
     if (rc != MI_OK) return MI_SDPA_DECLINE;
     int path = sdpa_path(a);
@@ -512,7 +517,7 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
     return path;
 }
 
-int mi_sdpa_f16(void *out, int out_dtype,
+int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
                 const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
                 const void *v, const int64_t v_strides[4],
                 const void *bias, int bias_dtype, const int64_t bias_strides[4], const int32_t *kv_len,
@@ -521,7 +526,7 @@ int mi_sdpa_f16(void *out, int out_dtype,
     if (!mi_ready()) return MI_ERROR_DEVICE;
     if (!out) return MI_DECLINE_OPERANDS;
     SdpaArgs a;
-    int rc = fill(a, out, out_dtype, q, q_strides, k, k_strides, v, v_strides, bias, bias_dtype, bias_strides, kv_len, E, Lq, Lk, H, B, scale);
+    int rc = fill(a, out, out_dtype, out_strides, q, q_strides, k, k_strides, v, v_strides, bias, bias_dtype, bias_strides, kv_len, E, Lq, Lk, H, B, scale);
     if (rc != MI_OK) return rc;
     if (Lq == 0 || H == 0 || B == 0 || E == 0) return MI_OK;
     hipStream_t st = (hipStream_t)stream;

@@ -307,7 +307,7 @@ def sdpaplan(ctx: Ctx, q, k, v, bias=None, scale=None, kv_len=None):
 
 def sdpa(ctx: Ctx, q, k, v, bias=None, scale=None, *, out=None, kv_len=None):
     """``softmax(scale q.k + bias) v`` -- sdpa, attention.jl:712.  ``out`` (torch (B,H,Lq,E),
-    fp16 or fp32, contiguous) is the planner's slot; allocated as fp32 when absent
+    fp16 or fp32; dense, or a strided view such as a token-major buffer permuted) is the planner's slot; allocated as fp32 when absent
     (sdpaout, attention.jl:762-765).  ``kv_len``: optional int32 (B,) tensor of valid keys."""
     plan = sdpaplan(ctx, q, k, v, bias, scale, kv_len)
     if isinstance(plan, Decline):
@@ -318,14 +318,14 @@ def sdpa(ctx: Ctx, q, k, v, bias=None, scale=None, *, out=None, kv_len=None):
     scale = (1.0 / math.sqrt(E)) if scale is None else float(scale)
     if out is None:
         out = torch.empty((Bq, H, Lq, E), dtype=torch.float32, device=q.device)
-    if not out.is_contiguous() or tuple(out.shape) != (Bq, H, Lq, E):
-        raise DeclineError("sdpa: out must be dense (B,H,Lq,E)", L.DECLINE_OPERANDS)
+    if tuple(out.shape) != (Bq, H, Lq, E):
+        raise DeclineError("sdpa: out must have shape (B,H,Lq,E)", L.DECLINE_OPERANDS)
     bst = _bias_strides(bias, Lk, Lq, H, Bq) if bias is not None else None
     if kv_len is not None and (kv_len.dtype != torch.int32 or not kv_len.is_cuda or kv_len.numel() != Bq):
         raise DeclineError("sdpa: kv_len must be a cuda int32 (B,) tensor", L.DECLINE_OPERANDS)
     need = lib.mi_sdpa_f16_workspace(E, Lq, Lk, H, Bq, int(bias is not None))
     ws = ctx.ws.scratch(need)
-    rc = lib.mi_sdpa_f16(out.data_ptr(), _dtype_code(out), q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k),
+    rc = lib.mi_sdpa_f16(out.data_ptr(), _dtype_code(out), (None if out.is_contiguous() else _strides_elbh(out)), q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k),
                          v.data_ptr(), _strides_elbh(v), _ptr(bias), (L.F32 if bias is not None and bias.dtype == torch.float32 else L.F16),
                          bst, _ptr(kv_len), E, Lq, Lk, H, Bq, scale, ws, need, ctx.stream)
     if rc != L.OK:

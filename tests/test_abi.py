@@ -1,0 +1,133 @@
+"""The C-ABI library loads and exports every symbol ``include/mi355dnn.h`` declares, and its
+planners (which launch nothing) answer without a GPU: every refusal is a named decline that can
+be asserted by constructing the call, the reference's own way of testing plans
+(DNNKernels/test/test_flash.jl:358-365, test_coopmat_attention.jl:92-134)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from juliavision_amd import _lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mi355dnn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = _declared()
+    assert len(names) >= 17
+    lib = L.load()
+    for n in names:
+        assert hasattr(lib, n), n
+        assert n in L.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(L.SIGNATURES) == set(names)
+    assert lib.mi_version() == 1
+
+
+def test_compute_calls_refuse_without_a_device():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    lib = L.load()
+    assert lib.mi_layernorm_f16(0x1000, None, None, 0x2000, None, None, 8, 1, 1e-5, None) == L.ERROR_DEVICE
+    assert lib.mi_add_f16(0x1000, 0x1000, 0x1000, 8, None) == L.ERROR_DEVICE
+    with pytest.raises(RuntimeError):
+        L.init()
+
+
+def _gemm_plan(T, K, F, *, ldY=None, ldX=None, ldW=None, layout=L.W_KF, y=0x10000, x=0x20000, w=0x30000, dt=L.F16, nb=1):
+    ldY = F if ldY is None else ldY
+    ldX = K if ldX is None else ldX
+    ldW = (F if layout == L.W_KF else K) if ldW is None else ldW
+    return L.GEMM_PATHS[L.load().mi_gemm_f16_plan(y, x, w, T, K, F, ldY, ldX, ldW, layout, dt, nb, T * ldY, T * ldX, 0)]
+
+
+def test_gemm_planner():
+    assert _gemm_plan(1500, 1280, 5120) == "mfma"
+    assert _gemm_plan(1500, 1280, 5120, layout=L.W_FK) == "mfma"
+    assert _gemm_plan(1370, 384, 1152) == "mfma"
+    for T in (1, 4, 8):
+        assert _gemm_plan(T, 1280, 1280) == "skinny"
+        assert _gemm_plan(T, 1280, 5120, layout=L.W_FK) == "skinny"
+    assert _gemm_plan(9, 1280, 1280) == "mfma"
+    assert _gemm_plan(8, 1280, 1280, nb=2) == "mfma"
+    # extents or pointers the 16-byte loads cannot address fall to the scalar kernel, as a ragged
+    # extent falls off the reference's fast kernel (tools/census_gemm_declines.jl:8-14)
+    assert _gemm_plan(1288, 1284, 1288) == "scalar"
+    assert _gemm_plan(64, 64, 60) == "scalar"                    # [K][F] rows of 60 halves
+    assert _gemm_plan(64, 64, 60, layout=L.W_FK) == "mfma"       # [F][K] rows are K-contiguous
+    assert _gemm_plan(64, 64, 64, x=0x20002) == "scalar"
+    assert _gemm_plan(64, 64, 64, ldX=60) == "decline"
+    assert _gemm_plan(0, 64, 64) == "decline"
+    assert _gemm_plan(64, 64, 64, dt=7) == "decline"
+
+
+def test_gemm_workspace():
+    lib = L.load()
+    assert lib.mi_gemm_f16_workspace(1500, 1280, 5120, L.W_KF, 1) == 0
+    n = lib.mi_gemm_f16_workspace(4, 1280, 1280, L.W_KF, 1)
+    assert n > 0 and n % 256 == 0 and n % (4 * 1280 * 4) == 0
+    assert lib.mi_gemm_f16_workspace(4, 1280, 1280, L.W_FK, 1) == 4 * 1280 * 4
+
+
+def _sdpa_plan(E, Lq, Lk, H, B, *, bias=0, scale=0.125, qs=None, ptr=0x10000):
+    dense = lambda L_: L.strides4(1, E, E * L_, E * L_ * H)
+    ns = C.c_int(0)
+    path = L.load().mi_sdpa_f16_plan(ptr, qs or dense(Lq), 0x20000, dense(Lk), 0x30000, dense(Lk), bias, 0, E, Lq, Lk, H, B, scale, C.byref(ns))
+    return L.SDPA_PATHS[path], ns.value
+
+
+def test_sdpa_planner():
+    assert _sdpa_plan(64, 4096, 4096, 16, 1) == ("flash", 1)
+    assert _sdpa_plan(64, 1500, 1500, 20, 1)[0] == "flash"
+    assert _sdpa_plan(72, 256, 256, 8, 16)[0] == "flash"
+    assert _sdpa_plan(64, 1500, 1500, 20, 1, bias=1)[0] == "rows"          # Decline(:bias) of the fused plan, flash.jl:1327
+    assert _sdpa_plan(64, 1, 448, 20, 1)[0] == "rows"
+    assert _sdpa_plan(20, 128, 128, 2, 1)[0] == "rows"                     # E not a multiple of 8
+    assert _sdpa_plan(64, 128, 128, 2, 1, qs=L.strides4(2, 128, 128 * 128, 0))[0] == "rows"   # head dim not contiguous
+    assert _sdpa_plan(64, 128, 128, 2, 1, ptr=0x10002)[0] == "rows"
+    assert _sdpa_plan(64, 128, 128, 2, 1, scale=-1.0)[0] == "rows"
+    assert _sdpa_plan(512, 128, 128, 2, 1)[0] == "decline"
+    # key splits for decode-sized Lq aim at two workgroups per CU (flash.jl:1288-1303): 20 rows -> many splits,
+    # 160 rows -> fewer, never more than one split per 64 keys
+    p1, n1 = _sdpa_plan(64, 1, 1500, 20, 1)
+    p8, n8 = _sdpa_plan(64, 1, 1500, 20, 8)
+    assert p1 == p8 == "rows" and n1 == 24 and 1 <= n8 < n1
+    assert _sdpa_plan(64, 1, 448, 20, 1)[1] == 7
+    assert _sdpa_plan(64, 23, 17, 4, 1)[1] == 1
+
+
+def test_conv_planner_and_extents():
+    lib = L.load()
+    plan = lambda *a: L.CONV_PATHS[lib.mi_conv2d_f16_plan(*a)]
+    assert plan(518, 518, 3, 1, 14, 14, 384, 14, 14, 0, 0, 1, 1, 1) == "im2col_gemm"
+    assert plan(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 1) == "im2col_gemm"
+    assert plan(256, 256, 144, 1, 1, 1, 256, 1, 1, 0, 0, 1, 1, 1) == "gemm_1x1"     # onebyone, conv.jl:63-66
+    assert plan(256, 256, 144, 1, 1, 1, 256, 2, 2, 0, 0, 1, 1, 1) == "im2col_gemm"
+    assert plan(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 4) == "direct"
+    assert plan(64, 64, 255, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 4) == "decline"
+    assert plan(2, 2, 3, 1, 5, 5, 8, 1, 1, 0, 0, 1, 1, 1) == "decline"              # empty output
+    assert lib.mi_convsize(518, 14, 14, 0, 1) == 37 and lib.mi_convsize(256, 7, 4, 3, 1) == 64
+    # im2col scratch: col[CRS->8][PQ->8] fp16 (+ padded weights when CRS % 8 != 0)
+    ws = lib.mi_conv2d_f16_workspace(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
+    assert ws == 2304 * 4096 * 2
+    ws3 = lib.mi_conv2d_f16_workspace(518, 518, 3, 1, 14, 14, 384, 14, 14, 0, 0, 1, 1)
+    assert ws3 == -(-(592 * 1376 * 2) // 256) * 256 + 384 * 592 * 2
+    assert lib.mi_conv2d_f16_workspace(256, 256, 144, 1, 1, 1, 256, 1, 1, 0, 0, 1, 1) == 0
+
+
+def test_host_planners_decline_by_name_on_cpu_tensors():
+    import torch
+    import juliavision_amd as jv
+    a = torch.zeros((8, 8), dtype=torch.float16)
+    assert jv.mmplan(jv.MI355X, a, a, a) == jv.Decline("operands")
+    assert not jv.mmplan(jv.MI355X, a, a, a)
+    x = torch.zeros((1, 8, 8, 8), dtype=torch.float16)
+    assert jv.conv_plan(jv.MI355X, x, x, x) == jv.Decline("operands")
+    assert jv.convsize(518, 14, 14, 0, 1) == 37

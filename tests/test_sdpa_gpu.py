@@ -146,3 +146,20 @@ def test_config4_attention_band(ctx):
         rows = np.r_[0:16, 2040:2056, 4080:4096]
         want = oracle.sdpa_ref_f32(q[:, h:h + 1, rows], k[:, h:h + 1], v[:, h:h + 1])
         assert_parity(got[:, h:h + 1, rows], want, what=f"config4 head {h}")
+
+
+def test_token_major_output(ctx):
+    """out given as a strided view: the result lands token-major ([B][L][H][E]), the layout the graph's
+    permute + reshape after attention produces, with no copy."""
+    import torch
+    import juliavision_amd as jv
+    B, H, L, E = 1, 4, 300, 64
+    q, k, v = _qkv(B, H, L, L, E, 111)
+    for lq in (L, 3):
+        buf = poison(torch.empty((B, lq, H, E), dtype=torch.float16, device="cuda"))
+        out = buf.permute(0, 2, 1, 3)
+        ctx.ws.reset()
+        jv.sdpa(ctx, to_dev(q[:, :, :lq]), to_dev(k), to_dev(v), None, None, out=out)
+        torch.cuda.synchronize()
+        want = oracle.sdpa_ref_f32(q[:, :, :lq], k, v)
+        assert_parity(to_host(buf).transpose(0, 2, 1, 3), want, what=f"token-major out Lq={lq}")
