@@ -9,7 +9,7 @@ accumulation, on synthetic seeded inputs already resident in HBM:
 
     LN -> q,k,v = h.Wq/Wk/Wv + b -> SDPA -> (.Wo + b) + x -> LN -> gelu(.W1 + b) -> (.W2 + b) + res
 
-nine kernel launches through the C ABI of libmi355dnn.so.  ``value`` is the block's algorithmic
+seven kernel launches through the C ABI (the q, k, v projections are one batched launch) of libmi355dnn.so.  ``value`` is the block's algorithmic
 TFLOP/s (70.50 GFLOP per block: 58.98 GEMM + 11.52 attention); ``ms_per_step`` is ms per encoder
 block.  ``roofline`` describes the dominant kernel -- the fp16 MFMA GEMM -- at its largest launch
 in the block, the fc1 linear 1500x1280 -> 5120 + bias + GELU (BASELINE config 1's shape), timed
@@ -115,19 +115,21 @@ class EncoderBlock:
         self.host = {}
         h = self.host
         h["x"] = oracle.randn_f16((T, D), seed)
-        for i, n in enumerate(("wq", "wk", "wv", "wo")):
-            h[n] = oracle.randn_f16((D, D), seed + 1 + i, 0, 0.02)
+        h["wqkv"] = oracle.randn_f16((3, D, D), seed + 1, 0, 0.02)      # Wq, Wk, Wv, each [K][F]
+        h["wo"] = oracle.randn_f16((D, D), seed + 4, 0, 0.02)
         h["w1"] = oracle.randn_f16((D, FF), seed + 5, 0, 0.02)
         h["w2"] = oracle.randn_f16((FF, D), seed + 6, 0, 0.02)
-        for i, (n, m) in enumerate((("bq", D), ("bk", D), ("bv", D), ("bo", D), ("b1", FF), ("b2", D))):
-            h[n] = oracle.randn_f16((m,), seed + 10 + i, 0, 0.02)
+        h["bqkv"] = oracle.randn_f16((3, D), seed + 10, 0, 0.02)
+        for i, (n, m) in enumerate((("bo", D), ("b1", FF), ("b2", D))):
+            h[n] = oracle.randn_f16((m,), seed + 13 + i, 0, 0.02)
         for i, n in enumerate(("g1", "g2")):
             h[n] = oracle.randn_f16((D,), seed + 20 + i, 1.0, 0.02)
         for i, n in enumerate(("be1", "be2")):
             h[n] = oracle.randn_f16((D,), seed + 22 + i, 0.0, 0.02)
         d = self.d = {k: dev(v) for k, v in h.items()}
-        for n in ("h1", "q", "k", "v", "a", "o", "h2", "y"):
+        for n in ("h1", "a", "o", "h2", "y"):
             d[n] = torch.empty((T, D), dtype=f16, device="cuda")
+        d["qkv"] = torch.empty((3, T, D), dtype=f16, device="cuda")
         d["f"] = torch.empty((T, FF), dtype=f16, device="cuda")
         p = lambda n: d[n].data_ptr()
 
@@ -140,11 +142,11 @@ class EncoderBlock:
         self.fc1 = gemm("f", "h2", "w1", "b1", D, FF, "gelu")
         self.calls_before_fc1 = [
             Call(lib.mi_layernorm_f16, p("h1"), None, None, p("x"), p("g1"), p("be1"), D, T, 1e-5, stream),
-            gemm("q", "h1", "wq", "bq", D, D, "none"),
-            gemm("k", "h1", "wk", "bk", D, D, "none"),
-            gemm("v", "h1", "wv", "bv", D, D, "none"),
-            Call(lib.mi_sdpa_f16, p("a"), L.F16, tok, p("q"), tok, p("k"), tok, p("v"), tok, None, 0, None, None,
-                 E, T, T, H, 1, scale, None, 0, stream),
+            # the three projections read the same h1: one batched launch (plane strides: Y T*D, X 0, W D*D, bias D)
+            Call(lib.mi_gemm_f16_batched, p("qkv"), p("h1"), p("wqkv"), p("bqkv"), None, T, D, D, D, D, D,
+                 L.W_KF, L.BIAS_COL, L.EPI["none"], L.F16, 3, T * D, 0, D * D, D, None, 0, stream),
+            Call(lib.mi_sdpa_f16, p("a"), L.F16, tok, p("qkv"), tok, p("qkv") + 2 * T * D, tok, p("qkv") + 4 * T * D, tok,
+                 None, 0, None, None, E, T, T, H, 1, scale, None, 0, stream),
             gemm("o", "a", "wo", "bo", D, D, "none", res="x"),
             Call(lib.mi_layernorm_f16, p("h2"), None, None, p("o"), p("g2"), p("be2"), D, T, 1e-5, stream),
         ]
@@ -179,9 +181,9 @@ class EncoderBlock:
             t0 = time.perf_counter()
             x = h["x"][:rows]
             h1, _, _ = oracle.layernorm_f16(x, h["g1"], h["be1"], 1e-5)
-            q = oracle.gemm_f16(h1, h["wq"], h["bq"])
-            oracle.gemm_f16(h1, h["wk"], h["bk"])
-            oracle.gemm_f16(h1, h["wv"], h["bv"])
+            q = oracle.gemm_f16(h1, h["wqkv"][0], h["bqkv"][0])
+            oracle.gemm_f16(h1, h["wqkv"][1], h["bqkv"][1])
+            oracle.gemm_f16(h1, h["wqkv"][2], h["bqkv"][2])
             o = oracle.gemm_f16(q, h["wo"], h["bo"], residual=x)
             h2, _, _ = oracle.layernorm_f16(o, h["g2"], h["be2"], 1e-5)
             f = oracle.gemm_f16(h2, h["w1"], h["b1"], epi="gelu")
@@ -341,7 +343,7 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "BASELINE config 2: Whisper-large-v3-turbo-shaped encoder block, batch 1, 1500 tokens, "
                                "d_model 1280, 20x64 heads, FFN 5120 GELU(erf), pre-LN, fp16 in / fp32 accumulate; "
-                               "70.50 GFLOP per block (58.98 GEMM + 11.52 attention); 9 launches via the C ABI",
+                               "70.50 GFLOP per block (58.98 GEMM + 11.52 attention); 7 launches via the C ABI",
                    "tokens": 1500, "d_model": 1280, "heads": 20, "head_dim": 64, "ffn": 5120,
                    "weight_layout": "[K][F] (the reference's hoisted layout)"},
         "frac_mfma_peak": round(blk.FLOP / sec / 1e12 / PEAK_F16_TFLOPS, 4),

@@ -86,13 +86,15 @@ int mi_gemm_f16(void *Y, const void *X, const void *W, const void *bias, const v
                 int w_layout, int bias_mode, int epi, int out_dtype,
                 void *ws, size_t ws_bytes, void *stream);
 
-/* The same over `nbatch` planes: element strides sY, sX, sW between planes
+/* The same over `nbatch` planes: element strides sY, sX, sW, sBias between planes
  * (0 = operand shared).  Replaces batchedmatmul!(ctx, out, A, B) -- matmul.jl:364-392
- * and the nbatch form of the GEMMs in sdpa_coopmat! -- attention.jl:697-699. */
+ * and the nbatch form of the GEMMs in sdpa_coopmat! -- attention.jl:697-699.  With
+ * sX = 0 it also runs several addmm ops that read the same activations (the q, k, v
+ * projections of one attention, ops.jl:1347-1356 three times) as one launch. */
 int mi_gemm_f16_batched(void *Y, const void *X, const void *W, const void *bias, const void *residual,
                         int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
                         int w_layout, int bias_mode, int epi, int out_dtype,
-                        int64_t nbatch, int64_t sY, int64_t sX, int64_t sW,
+                        int64_t nbatch, int64_t sY, int64_t sX, int64_t sW, int64_t sBias,
                         void *ws, size_t ws_bytes, void *stream);
 
 /* Decode-sized T (<= 16): the bandwidth-bound form, split over K across

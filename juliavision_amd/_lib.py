@@ -32,7 +32,7 @@ SIGNATURES = {
     "mi_init": (_int, []),
     "mi_device_caps": (_int, [_i64p]),
     "mi_gemm_f16": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
-    "mi_gemm_f16_batched": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_i64] * 4 + [_vp, _sz, _vp]),
+    "mi_gemm_f16_batched": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_i64] * 5 + [_vp, _sz, _vp]),
     "mi_gemv_f16": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
     "mi_gemm_f16_workspace": (_sz, [_i64, _i64, _i64, _int, _i64]),
     "mi_gemm_f16_plan": (_int, [_vp] * 3 + [_i64] * 6 + [_int] * 2 + [_i64] * 4),

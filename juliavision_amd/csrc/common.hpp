@@ -12,6 +12,8 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
 
 #define MI_DEVICE static __device__ __forceinline__
 
@@ -28,7 +30,7 @@ MI_DEVICE half8v as_half8(u32x4 v) { return __builtin_bit_cast(half8v, v); }
 // `erf` (DNNKernels/src/ops.jl:161-169), so a folded gelu is the graph's gelu.
 MI_DEVICE float erf_as(float x) {
     float a = fabsf(x);
-    float t = 1.0f / (1.0f + 0.3275911f * a);
+    float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * a);
     float y = 1.0f - (((((1.061405429f * t - 1.453152027f) * t) + 1.421413741f) * t - 0.284496736f) * t + 0.254829592f) * t * __expf(-a * a);
     return x < 0.0f ? -y : y;
 }

@@ -17,7 +17,7 @@ struct GemmArgs {
     int M, N, K;
     int NB;                 // columns addressable in B (>= N; a multiple of 8 for the [K][N] layout)
     long ldY, ldA, ldB;
-    long sY, sA, sB;        // batch strides (elements)
+    long sY, sA, sB, sBias; // batch strides (elements)
     int bias_mode, epi, out_f32;
     int tiles_m, tiles_n, group_m;
     int vec_store;          // Y (and residual) rows allow 16-byte accesses
@@ -129,6 +129,108 @@ __device__ __forceinline__ void tile_of(int pid, int nwg, int tiles_m, int tiles
 }
 
 // ------------------------------------------------------------------------------------------
+// Accumulator tile -> memory, shared by the tiled kernels.
+// acc[i][j][r]: n = n0 + wn*WTN + 32 i + 8 (r/4) + 4 (lane/32) + r%4,  m = m0 + wm*WTM + 32 j + lane%32.
+// Each wave stages one 32 x WTN sub-tile at a time in its own LDS region (bias
+// joined in fp32, one rounding), then reads it back row-wise so that the
+// activation, the residual add and the global stores run on 16-byte vectors
+// that are contiguous along the output row.  The caller has synchronised the
+// workgroup after its last read of the operand tiles.
+template <int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
+__device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN][TM], char *smem, int m0, int n0, int wm, int wn,
+                                           int wave, int lane, long bz) {
+    const int frow = lane & 31;
+    const half_t *bias = p.bias ? p.bias + bz * p.sBias : nullptr;
+    constexpr int SLD_H = WTN + 8;                 // halves per staged row (fp16 output)
+    constexpr int SLD_F = WTN + 4;                 // floats per staged row (fp32 output)
+    constexpr int STAGE_BYTES = 32 * SLD_F * 4;
+    static_assert(STAGE_BYTES * NWAVES <= LDS_BYTES, "epilogue staging exceeds the operand LDS");
+    char *stage = smem + wave * STAGE_BYTES;
+    const int hl = lane >> 5;
+    static_for<TM>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+        const int mrow = m0 + wm * WTM + 32 * j;
+        const float brow = (p.bias_mode == MI_BIAS_ROW && mrow + frow < p.M) ? (float)bias[mrow + frow] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int nl = 32 * i + 8 * g + 4 * hl;
+                const int n = n0 + wn * WTN + nl;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + brow;
+                if (p.bias_mode == MI_BIAS_COL) {
+                    if (n + 3 < p.N) {
+                        half4v bv = *reinterpret_cast<const half4v *>(bias + n);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] += (float)bv[e];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) if (n + e < p.N) v[e] += (float)bias[n + e];
+                    }
+                }
+                if (p.out_f32) {
+                    float4v o = {v[0], v[1], v[2], v[3]};
+                    *reinterpret_cast<float4v *>(reinterpret_cast<float *>(stage) + frow * SLD_F + nl) = o;
+                } else {
+                    half4v o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(stage) + frow * SLD_H + nl) = o;
+                }
+            }
+        }
+        __syncthreads();
+        if (p.out_f32) {
+            constexpr int CPR = WTN / 4;
+            for (int c = lane; c < 32 * CPR; c += 64) {
+                const int row = c / CPR, ch = c % CPR;
+                const int m = mrow + row, n = n0 + wn * WTN + ch * 4;
+                if (m < p.M && n < p.N) {
+                    float4v x = *reinterpret_cast<const float4v *>(reinterpret_cast<const float *>(stage) + row * SLD_F + ch * 4);
+                    float *yp = reinterpret_cast<float *>(p.Y) + bz * p.sY + (long)m * p.ldY + n;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[e] = apply_epi(x[e], p.epi);
+                    if (p.vec_store && n + 3 < p.N) *reinterpret_cast<float4v *>(yp) = x;
+                    else for (int e = 0; e < 4; e++) if (n + e < p.N) yp[e] = x[e];
+                }
+            }
+        } else {
+            constexpr int CPR = WTN / 8;
+            for (int c = lane; c < 32 * CPR; c += 64) {
+                const int row = c / CPR, ch = c % CPR;
+                const int m = mrow + row, n = n0 + wn * WTN + ch * 8;
+                if (m < p.M && n < p.N) {
+                    half8v x = *reinterpret_cast<const half8v *>(reinterpret_cast<const half_t *>(stage) + row * SLD_H + ch * 8);
+                    const long off = bz * p.sY + (long)m * p.ldY + n;
+                    half_t *yp = reinterpret_cast<half_t *>(p.Y) + off;
+                    if (p.epi != MI_EPI_NONE) {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) x[e] = (half_t)apply_epi((float)x[e], p.epi);
+                    }
+                    if (p.vec_store && n + 7 < p.N) {
+                        if (p.residual) {
+                            half8v rv = as_half8(ldg16(p.residual + off));
+#pragma unroll
+                            for (int e = 0; e < 8; e++) x[e] = (half_t)((float)x[e] + (float)rv[e]);
+                        }
+                        *reinterpret_cast<half8v *>(yp) = x;
+                    } else {
+                        for (int e = 0; e < 8; e++) {
+                            if (n + e < p.N) {
+                                half_t o = x[e];
+                                if (p.residual) o = (half_t)((float)o + (float)p.residual[off + e]);
+                                yp[e] = o;
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    });
+}
+
+// ------------------------------------------------------------------------------------------
 // The tiled MFMA kernel.  BM x BN output tile per workgroup, WAVES_M x WAVES_N
 // waves, each owning a (BM/WAVES_M) x (BN/WAVES_N) sub-tile as 32x32 MFMA
 // tiles.  The MFMA is issued "transposed" (rows = n, columns = m) so that a
@@ -202,99 +304,167 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma_kernel(GemmAr
         __syncthreads();
     }
 
-    // Epilogue.  acc[i][j][r]: n = n0 + wn*WTN + 32 i + 8 (r/4) + 4 (lane/32) + r%4,
-    //                          m = m0 + wm*WTM + 32 j + lane%32.
-    // Each wave stages one 32 x WTN sub-tile at a time in its own LDS region
-    // (bias joined in fp32, one rounding), then reads it back row-wise so that the
-    // activation, the residual add and the global stores run on 16-byte vectors
-    // that are contiguous along the output row.
-    constexpr int SLD_H = WTN + 8;                 // halves per staged row (fp16 output)
-    constexpr int SLD_F = WTN + 4;                 // floats per staged row (fp32 output)
-    constexpr int STAGE_BYTES = 32 * SLD_F * 4;
-    static_assert(STAGE_BYTES * WAVES_M * WAVES_N <= 2 * (BM + BN) * LD * 2, "epilogue staging exceeds the operand LDS");
-    char *stage = smem + wave * STAGE_BYTES;
-    const int hl = lane >> 5;
-    static_for<TM>([&](auto J) {
-        constexpr int j = decltype(J)::value;
-        const int mrow = m0 + wm * WTM + 32 * j;
-        const float brow = (p.bias_mode == MI_BIAS_ROW && mrow + frow < p.M) ? (float)p.bias[mrow + frow] : 0.0f;
+    store_tile<TM, TN, WTM, WTN, WAVES_M * WAVES_N, 2 * (BM + BN) * LD * 2>(p, acc, smem, m0, n0, wm, wn, wave, lane, bz);
+}
+
+// ------------------------------------------------------------------------------------------
+// The software-pipelined kernel for K % 64 == 0 (every linear of the encoder
+// configurations).  Same tiles and LDS layout as gemm_mfma_kernel, but the K loop
+// is written out as a four-phase pipeline per 64-deep tile:
+//   phase 0: read fragments of k-step 1 | MFMAs of k-step 0   (+ issue the global loads of tile kt+2)
+//   phase 1: read fragments of k-step 2 | MFMAs of k-step 1 | write the A part of tile kt+1 to the other LDS buffer
+//   phase 2: read fragments of k-step 3 | MFMAs of k-step 2 | write the B part of tile kt+1
+//   barrier
+//   phase 3: read fragments of k-step 0 of tile kt+1 | MFMAs of k-step 3
+// Global loads run two tiles ahead through two register sets, so a load has a
+// whole tile of MFMAs to land before its LDS write; the only barrier of a tile sits
+// where its successor's first fragment read can be hidden behind the last k-step.
+// Two waves per SIMD (8 waves on a 128 x 256 tile) cover each other's waits.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool B_KN>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(GemmArgs p) {
+    constexpr int BK = 64, LD = BK + 8, NT = WAVES_M * WAVES_N * 64;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
+    constexpr int PA = BM * 8 / NT, PB = BN * 8 / NT;     // 16-byte chunks per thread per tile
+    // The [K][N] operand keeps its layout in LDS: BK rows of BN halves, padded by
+    // 32 halves so that the four rows a transposing read touches fall in distinct
+    // bank groups.  Its MFMA fragments come from ds_read_b64_tr_b16 (see fread).
+    constexpr int BLD = BN + 32, CPRB = BN / 8;
+    static_assert(PA >= 1 && PB >= 1, "tile too small for this workgroup");
+    constexpr int BSZ = B_KN ? BK * BLD : BN * LD;      // halves per B buffer
+    extern __shared__ __align__(16) char smem[];
+    half_t *As = reinterpret_cast<half_t *>(smem);   // [2][BM][LD]
+    half_t *Bs = As + 2 * BM * LD;                   // [2][BN][LD] or [2][BK][BLD]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    int tm_, tn_;
+    tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
+    const int m0 = tm_ * BM, n0 = tn_ * BN;
+    const long bz = blockIdx.y;
+    const half_t *A = p.A + bz * p.sA;
+    const half_t *B = p.B + bz * p.sB;
+
+    // Per-thread global sources; rows and columns past the edge re-read the last
+    // valid one (their results are never stored).
+    const half_t *ap[PA], *bp[PB];
 #pragma unroll
-        for (int i = 0; i < TN; i++) {
+    for (int i = 0; i < PA; i++) { const int c = tid + i * NT; ap[i] = A + (long)min(m0 + (c >> 3), p.M - 1) * p.ldA + (c & 7) * 8; }
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int nl = 32 * i + 8 * g + 4 * hl;
-                const int n = n0 + wn * WTN + nl;
-                float v[4];
+    for (int i = 0; i < PB; i++) {
+        const int c = tid + i * NT;
+        if (!B_KN) bp[i] = B + (long)min(n0 + (c >> 3), p.N - 1) * p.ldB + (c & 7) * 8;
+        else       bp[i] = B + (long)(c / CPRB) * p.ldB + min(n0 + (c % CPRB) * 8, p.NB - 8);
+    }
+    u32x4 ga[2][PA], gb[2][PB];
+    auto gload = [&](int set, int kt) {
+        const long ko = (long)kt * BK;
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + brow;
-                if (p.bias_mode == MI_BIAS_COL) {
-                    if (n + 3 < p.N) {
-                        half4v bv = *reinterpret_cast<const half4v *>(p.bias + n);
+        for (int i = 0; i < PA; i++) ga[set][i] = ldg16(ap[i] + ko);
 #pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] += (float)bv[e];
-                    } else {
+        for (int i = 0; i < PB; i++) gb[set][i] = ldg16(bp[i] + (B_KN ? ko * p.ldB : ko));
+    };
+    auto lwrite_a = [&](int set, int buf) {
 #pragma unroll
-                        for (int e = 0; e < 4; e++) if (n + e < p.N) v[e] += (float)p.bias[n + e];
-                    }
-                }
-                if (p.out_f32) {
-                    float4v o = {v[0], v[1], v[2], v[3]};
-                    *reinterpret_cast<float4v *>(reinterpret_cast<float *>(stage) + frow * SLD_F + nl) = o;
-                } else {
-                    half4v o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                    *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(stage) + frow * SLD_H + nl) = o;
-                }
-            }
+        for (int i = 0; i < PA; i++) { const int c = tid + i * NT; *reinterpret_cast<u32x4 *>(As + buf * BM * LD + (c >> 3) * LD + (c & 7) * 8) = ga[set][i]; }
+    };
+    auto lwrite_b = [&](int set, int buf) {
+#pragma unroll
+        for (int i = 0; i < PB; i++) {
+            const int c = tid + i * NT;
+            half_t *dst = !B_KN ? Bs + buf * BSZ + (c >> 3) * LD + (c & 7) * 8 : Bs + buf * BSZ + (c / CPRB) * BLD + (c % CPRB) * 8;
+            *reinterpret_cast<u32x4 *>(dst) = gb[set][i];
         }
-        __syncthreads();
-        if (p.out_f32) {
-            constexpr int CPR = WTN / 4;
-            for (int c = lane; c < 32 * CPR; c += 64) {
-                const int row = c / CPR, ch = c % CPR;
-                const int m = mrow + row, n = n0 + wn * WTN + ch * 4;
-                if (m < p.M && n < p.N) {
-                    float4v x = *reinterpret_cast<const float4v *>(reinterpret_cast<const float *>(stage) + row * SLD_F + ch * 4);
-                    float *yp = reinterpret_cast<float *>(p.Y) + bz * p.sY + (long)m * p.ldY + n;
+    };
+
+    float16v acc[TN][TM];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) x[e] = apply_epi(x[e], p.epi);
-                    if (p.vec_store && n + 3 < p.N) *reinterpret_cast<float4v *>(yp) = x;
-                    else for (int e = 0; e < 4; e++) if (n + e < p.N) yp[e] = x[e];
-                }
-            }
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    const int frow = lane & 31, fk = (lane >> 5) * 8;
+    const int aoff = (wm * WTM + frow) * LD + fk, boff = (wn * WTN + frow) * LD + fk;
+    // [K][N] fragments: within each block of 16 lanes, lane i of ds_read_b64_tr_b16
+    // receives, for j = 0..3, element i%4 of the 8 bytes addressed by lane 4j + i/4.
+    // Pointing lane s at row (k0 + s/4), columns (n0 + 4 (s%4) .. +3) therefore hands
+    // lane i the four consecutive k of column n0 + i: the MFMA operand layout.
+    const int tboff = (fk + ((lane & 15) >> 2)) * BLD + wn * WTN + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    half8v fa[2][TM], fb[2][TN];
+    auto fread = [&](int fs, int buf, int ks) {
+        const half_t *as = As + buf * BM * LD + aoff + ks * 16;
+#pragma unroll
+        for (int j = 0; j < TM; j++) fa[fs][j] = *reinterpret_cast<const half8v *>(as + j * 32 * LD);
+        if (!B_KN) {
+            const half_t *bs = Bs + buf * BSZ + boff + ks * 16;
+#pragma unroll
+            for (int i = 0; i < TN; i++) fb[fs][i] = *reinterpret_cast<const half8v *>(bs + i * 32 * LD);
         } else {
-            constexpr int CPR = WTN / 8;
-            for (int c = lane; c < 32 * CPR; c += 64) {
-                const int row = c / CPR, ch = c % CPR;
-                const int m = mrow + row, n = n0 + wn * WTN + ch * 8;
-                if (m < p.M && n < p.N) {
-                    half8v x = *reinterpret_cast<const half8v *>(reinterpret_cast<const half_t *>(stage) + row * SLD_H + ch * 8);
-                    const long off = bz * p.sY + (long)m * p.ldY + n;
-                    half_t *yp = reinterpret_cast<half_t *>(p.Y) + off;
-                    if (p.epi != MI_EPI_NONE) {
+            const half_t *bs = Bs + buf * BSZ + tboff + ks * 16 * BLD;
 #pragma unroll
-                        for (int e = 0; e < 8; e++) x[e] = (half_t)apply_epi((float)x[e], p.epi);
-                    }
-                    if (p.vec_store && n + 7 < p.N) {
-                        if (p.residual) {
-                            half8v rv = as_half8(ldg16(p.residual + off));
-#pragma unroll
-                            for (int e = 0; e < 8; e++) x[e] = (half_t)((float)x[e] + (float)rv[e]);
-                        }
-                        *reinterpret_cast<half8v *>(yp) = x;
-                    } else {
-                        for (int e = 0; e < 8; e++) {
-                            if (n + e < p.N) {
-                                half_t o = x[e];
-                                if (p.residual) o = (half_t)((float)o + (float)p.residual[off + e]);
-                                yp[e] = o;
-                            }
-                        }
-                    }
-                }
+            for (int i = 0; i < TN; i++) {
+                short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(bs + i * 32));
+                short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(bs + i * 32 + 4 * BLD));
+                short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                fb[fs][i] = __builtin_bit_cast(half8v, both);
             }
         }
+    };
+    auto mma = [&](int fs) {
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int j = 0; j < TM; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[fs][i], fa[fs][j], acc[i][j], 0, 0, 0);
+    };
+
+    const int nk = p.K / BK;   // the launcher guarantees K % 64 == 0 and nk >= 2
+    gload(0, 0);
+    gload(1, 1);
+    lwrite_a(0, 0);
+    lwrite_b(0, 0);
+    __syncthreads();
+    fread(0, 0, 0);
+
+    // MODE 0: steady state; 1: second-to-last tile (nothing left to fetch); 2: last tile.
+    // Tile kt is computed from LDS buffer `cur`; register set `gw` holds tile kt+1, set `gl` receives tile kt+2.
+    auto body = [&](auto MODE_, int kt, int cur, int gw, int gl) {
+        constexpr int MODE = decltype(MODE_)::value;
+        if constexpr (MODE == 0) gload(gl, kt + 2);
+        fread(1, cur, 1);
+        mma(0);
+        __builtin_amdgcn_sched_barrier(0);
+        fread(0, cur, 2);
+        mma(1);
+        if constexpr (MODE < 2) lwrite_a(gw, cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        fread(1, cur, 3);
+        mma(0);
+        if constexpr (MODE < 2) lwrite_b(gw, cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
-    });
+        if constexpr (MODE < 2) fread(0, cur ^ 1, 0);
+        mma(1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using M0 = std::integral_constant<int, 0>;
+    using M1 = std::integral_constant<int, 1>;
+    using M2 = std::integral_constant<int, 2>;
+    const int npairs = (nk - 2) >> 1;       // steady-state tiles come in (buffer 0, buffer 1) pairs
+    int kt = 0;
+    for (int pr = 0; pr < npairs; pr++, kt += 2) {
+        body(M0{}, kt, 0, 1, 0);
+        body(M0{}, kt + 1, 1, 0, 1);
+    }
+    if (nk & 1) {
+        body(M0{}, kt, 0, 1, 0);
+        body(M1{}, kt + 1, 1, 0, 1);
+        body(M2{}, kt + 2, 0, 1, 0);
+    } else {
+        body(M1{}, kt, 0, 1, 0);
+        body(M2{}, kt + 1, 1, 0, 1);
+    }
+    __syncthreads();
+    store_tile<TM, TN, WTM, WTN, WAVES_M * WAVES_N, 2 * (BM * LD + BSZ) * 2>(p, acc, smem, m0, n0, wm, wn, wave, lane, bz);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -308,7 +478,8 @@ __global__ void gemm_scalar_kernel(GemmArgs p, int b_kn) {
     long bz = blockIdx.y;
     const half_t *A = p.A + bz * p.sA + (long)m * p.ldA;
     const half_t *B = p.B + bz * p.sB;
-    float acc = p.bias_mode == MI_BIAS_COL ? (float)p.bias[n] : p.bias_mode == MI_BIAS_ROW ? (float)p.bias[m] : 0.0f;
+    const half_t *bias = p.bias ? p.bias + bz * p.sBias : nullptr;
+    float acc = p.bias_mode == MI_BIAS_COL ? (float)bias[n] : p.bias_mode == MI_BIAS_ROW ? (float)bias[m] : 0.0f;
     if (b_kn) for (int k = 0; k < p.K; k++) acc = fmaf((float)A[k], (float)B[(long)k * p.ldB + n], acc);
     else      for (int k = 0; k < p.K; k++) acc = fmaf((float)A[k], (float)B[(long)n * p.ldB + k], acc);
     long off = bz * p.sY + (long)m * p.ldY + n;
@@ -432,7 +603,10 @@ int raise_lds(KernelT kern, int bytes) {
 }
 
 template <int BM, int BN, int BK>
-constexpr int gemm_lds_bytes() { return 2 * (BM + BN) * (BK + 8) * 2; }
+constexpr int gemm_lds_bytes() {
+    constexpr int kc = BN * (BK + 8), kn = BK * (BN + 32);       // B buffer in either layout
+    return 2 * (BM * (BK + 8) + (kc > kn ? kc : kn)) * 2;
+}
 
 #define GEMM_BIG 128, 256, 64, 2, 2
 #define GEMM_MID 128, 128, 64, 2, 2
@@ -454,6 +628,20 @@ bool mfma_addressable(const GemmArgs &a, bool b_kn) {
     if (b_kn && (a.NB % 8 || a.NB < 8 || a.NB < a.N)) return false;
     if (a.bias && a.bias_mode == MI_BIAS_COL && !aligned_to(a.bias, 8)) return false;
     return a.M >= 1 && a.N >= 1 && a.K >= 8;
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_pipe(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
+    a.tiles_m = (int)ceil_div(a.M, BM);
+    a.tiles_n = (int)ceil_div(a.N, BN);
+    a.group_m = a.tiles_m < 6 ? a.tiles_m : 6;
+    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
+                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
+    constexpr int lds = gemm_lds_bytes<BM, BN, 64>();
+    if (b_kn) hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, true>), grid, dim3(WM * WN * 64), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, false>), grid, dim3(WM * WN * 64), lds, st, a);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
 template <int BM, int BN, int BK, int WM, int WN>
@@ -504,7 +692,7 @@ int run_skinny(GemmArgs a, bool b_kn, void *ws, size_t ws_bytes, hipStream_t st)
 
 int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bias, const void *residual,
               int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
-              int w_layout, int bias_mode, int epi, int out_dtype, int64_t sY, int64_t sX, int64_t sW) {
+              int w_layout, int bias_mode, int epi, int out_dtype, int64_t sY, int64_t sX, int64_t sW, int64_t sBias = 0) {
     if (!Y || !X || !W) return MI_DECLINE_OPERANDS;
     if (T < 0 || K < 0 || F < 0 || T > INT32_MAX || K > INT32_MAX || F > INT32_MAX) return MI_DECLINE_EXTENT;
     if (w_layout != MI_W_KF && w_layout != MI_W_FK) return MI_DECLINE_OPERANDS;
@@ -518,7 +706,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.bias = bias_mode == MI_BIAS_NONE ? nullptr : (const half_t *)bias;
     a.residual = (const half_t *)residual;
     a.M = (int)T; a.N = (int)F; a.K = (int)K; a.NB = (int)F;
-    a.ldY = ldY; a.ldA = ldX; a.ldB = ldW; a.sY = sY; a.sA = sX; a.sB = sW;
+    a.ldY = ldY; a.ldA = ldX; a.ldB = ldW; a.sY = sY; a.sA = sX; a.sB = sW; a.sBias = sBias;
     a.bias_mode = bias_mode; a.epi = epi; a.out_f32 = out_dtype == MI_F32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
     return MI_OK;
@@ -536,8 +724,9 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         // else smaller tiles so small problems spread over the chip.
         int64_t big = ceil_div(a.M, 128) * ceil_div(a.N, 256) * nbatch;
         int64_t mid = ceil_div(a.M, 128) * ceil_div(a.N, 128) * nbatch;
-        if (big >= (g_cus * 3) / 4) return launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
-        if (mid >= (g_cus * 3) / 4) return launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
+        const bool pipe = a.K % 64 == 0 && a.K >= 128;
+        if (big >= (g_cus * 3) / 4) return pipe ? launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
+        if (mid >= (g_cus * 3) / 8) return pipe ? launch_pipe<128, 128, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
         return launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
     }
     long total = (long)a.M * a.N;
@@ -557,7 +746,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
                      long nbatch, long sY, long sA, long sB, hipStream_t st) {
     GemmArgs a;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
-    a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB;
+    a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
     int path = mfma_addressable(a, b_kn != 0) ? MI_GEMM_MFMA : MI_GEMM_SCALAR;
@@ -583,6 +772,10 @@ int mi_init(void) {
     bad |= raise_lds(gemm_mfma_kernel<GEMM_MID, false>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_mfma_kernel<GEMM_SMALL, true>, gemm_lds_bytes<64, 64, 64>());
     bad |= raise_lds(gemm_mfma_kernel<GEMM_SMALL, false>, gemm_lds_bytes<64, 64, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, true>, gemm_lds_bytes<128, 256, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, false>, gemm_lds_bytes<128, 256, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, true>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, false>, gemm_lds_bytes<128, 128, 64>());
     bad |= mi_sdpa_init();
     if (bad) return MI_ERROR_DEVICE;
     g_ready = true;
@@ -622,10 +815,10 @@ int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,
 int mi_gemm_f16_batched(void *Y, const void *X, const void *W, const void *bias, const void *residual,
                         int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
                         int w_layout, int bias_mode, int epi, int out_dtype,
-                        int64_t nbatch, int64_t sY, int64_t sX, int64_t sW,
+                        int64_t nbatch, int64_t sY, int64_t sX, int64_t sW, int64_t sBias,
                         void *ws, size_t ws_bytes, void *stream) {
     GemmArgs a;
-    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype, sY, sX, sW);
+    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype, sY, sX, sW, sBias);
     if (rc != MI_OK) return rc;
     if (nbatch < 0 || nbatch > 65535) return MI_DECLINE_EXTENT;
     if (K == 0) return MI_DECLINE_EXTENT;
@@ -637,7 +830,7 @@ int mi_gemm_f16(void *Y, const void *X, const void *W, const void *bias, const v
                 int w_layout, int bias_mode, int epi, int out_dtype,
                 void *ws, size_t ws_bytes, void *stream) {
     return mi_gemm_f16_batched(Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype,
-                               1, 0, 0, 0, ws, ws_bytes, stream);
+                               1, 0, 0, 0, 0, ws, ws_bytes, stream);
 }
 
 int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,

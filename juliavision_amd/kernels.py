@@ -246,7 +246,7 @@ def batchedmatmul_(ctx: Ctx, out, A, B):
     sB = 0 if B.shape[0] == 1 else B.stride(0)
     rc = lib.mi_gemm_f16_batched(out.data_ptr(), B.data_ptr(), A.data_ptr(), None, None, T, K, F,
                                  out.stride(1), B.stride(1), A.stride(1), L.W_KF, L.BIAS_NONE, L.EPI["none"],
-                                 _dtype_code(out), nb, out.stride(0), sB, sA, None, 0, ctx.stream)
+                                 _dtype_code(out), nb, out.stride(0), sB, sA, 0, None, 0, ctx.stream)
     if rc != L.OK:
         raise DeclineError("mi_gemm_f16_batched", rc)
     return out

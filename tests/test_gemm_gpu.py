@@ -100,3 +100,24 @@ def test_batched(ctx):
         jv.batchedmatmul_(ctx, out, to_dev(W), to_dev(X))
         torch.cuda.synchronize()
         assert_parity(to_host(out), want, what=f"bmm {nb} {T} {K} {F}")
+
+
+def test_batched_shared_activations_with_per_plane_bias(ctx):
+    """q, k, v projections as one launch through the C ABI: X shared (plane stride 0), W, bias and Y per plane."""
+    import torch
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    T, K, F = 300, 256, 384
+    X = oracle.randn_f16((T, K), 31, 0, 1.0 / np.sqrt(K))
+    W = oracle.randn_f16((3, K, F), 32)
+    b = oracle.randn_f16((3, F), 33, 0, 0.5)
+    dX, dW, db = to_dev(X), to_dev(W), to_dev(b)
+    out = poison(torch.empty((3, T, F), dtype=torch.float16, device="cuda"))
+    rc = lib.mi_gemm_f16_batched(out.data_ptr(), dX.data_ptr(), dW.data_ptr(), db.data_ptr(), None, T, K, F, F, K, F,
+                                 L.W_KF, L.BIAS_COL, L.EPI["none"], L.F16, 3, T * F, 0, K * F, F, None, 0,
+                                 torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = to_host(out)
+    for i in range(3):
+        assert_parity(got[i], oracle.gemm_f16(X, W[i], b[i]), what=f"qkv plane {i}")
