@@ -16,7 +16,9 @@ LIB = os.path.join(HERE, "libmi355dnn.so")
 SOURCES = ["gemm.hip", "sdpa.hip", "conv.hip", "layernorm.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+# -fno-honor-nans: no kernel relies on NaN propagation (infinities stay honoured: they are the masks);
+#   without it every fmaxf operand is first canonicalised with an extra v_max_f32.
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-honor-nans",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 

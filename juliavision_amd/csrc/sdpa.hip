@@ -43,12 +43,11 @@ __device__ __forceinline__ void static_for(F &&f) {
 
 // ------------------------------------------------------------------------------------------
 // Fused kernel.  Workgroup = 4 waves = 128 queries (32 per wave); keys walked in
-// blocks of BC = 64 through double-buffered LDS tiles:
-//   Ks [BC][EP+8]   keys x head-dim, head-dim contiguous  (A operand of S^T = K.Q^T)
-//   Vt [EP][BC+4]   head-dim x keys, keys contiguous      (A operand of O^T = V^T.P^T)
-// V arrives head-dim contiguous, so it is transposed on the way into LDS: a
-// thread takes the same 8 head-dim values of two adjacent keys and writes eight
-// packed key pairs.
+// blocks of BC = 64 through double-buffered LDS tiles, both as they lie in memory:
+//   Ks [BC][EP+8]    keys x head-dim   (A operand of S^T = K.Q^T, plain 16-byte reads)
+//   Vs [BC][EP+32]   keys x head-dim   (A operand of O^T = V^T.P^T through
+//                    ds_read_b64_tr_b16, which transposes 4 keys x 16 head-dim
+//                    values per 16 lanes on the way out of LDS)
 //
 // MFMA 32x32 accumulator layout: lane l, register r holds row 8(r/4)+4(l/32)+r%4,
 // column l%32.  With rows = keys and columns = queries, a lane owns one query
@@ -56,18 +55,34 @@ __device__ __forceinline__ void static_for(F &&f) {
 // l^32.  Registers 8b..8b+7 of a tile are, in order, the keys
 // {16b+4h+0..3, 16b+8+4h+0..3} (h = l/32): that is the k-order in which P^T is fed
 // to the second product, and V^T is read from LDS in the same order.
+//
+// Softmax bookkeeping is arranged to cost as few vector instructions as possible,
+// because at head size 64 the exponentials, not the MFMAs, are the long pole:
+//   * Q is pre-multiplied by scale*log2(e) (in fp32, rounded to fp16 once), so the
+//     first product is already in the base-2 exponent domain;
+//   * the reference point M of the running softmax is subtracted by the MFMA itself:
+//     the accumulator of the first product starts from a register tuple holding -M,
+//     so the product delivers t = s - M and p = exp2(t) needs no further arithmetic;
+//   * M is a *stale* maximum: it only moves when a row's block maximum exceeds it by
+//     more than 2^8 (or on the first block).  p then lies in (0, 256], exact in
+//     fp16/fp32, and O and l are rescaled only on those rare moves.  The result is
+//     the same softmax -- every term carries the same factor 2^-M -- with the
+//     rescaling of flash.jl:25-38 applied lazily (the reference's `lazyrescale`,
+//     flash.jl:1041-1096, skips it when no maximum grew; this skips it until one
+//     grew by a factor of 256);
+//   * row sums accumulate the fp16 probabilities pairwise with v_dot2_f32_f16.
 template <int EP>
 __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
     constexpr int BC = 64, BR = 128, NT = 256;
-    constexpr int KLD = EP + 8, VLD = BC + 4;
+    constexpr int KLD = EP + 8, VLD = EP + 32;
     constexpr int KS = EP / 16;       // k16 steps over the head dim
     constexpr int ET = EP / 32;       // 32-wide head-dim tiles of O
     constexpr int KCH = EP / 8;       // 16-byte chunks per key row
-    constexpr int K_PER = BC * KCH / NT;
-    constexpr int V_PER = (BC / 2) * KCH / NT;
+    constexpr int PER = BC * KCH / NT;
+    constexpr float TH = 8.0f;
     extern __shared__ __align__(16) char smem[];
     half_t (*Ks)[BC * KLD] = reinterpret_cast<half_t (*)[BC * KLD]>(smem);
-    half_t (*Vt)[EP * VLD] = reinterpret_cast<half_t (*)[EP * VLD]>(smem + 2 * BC * KLD * 2);
+    half_t (*Vs)[BC * VLD] = reinterpret_cast<half_t (*)[BC * VLD]>(smem + 2 * BC * KLD * 2);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hl = lane >> 5, l32 = lane & 31;
@@ -80,7 +95,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
     if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
     const float c = p.scale * LOG2E;
 
-    // Q^T fragments: column = query l32, k = head-dim 16 ks + 8 hl .. +7
+    // Q^T fragments: column = query l32, k = head-dim 16 ks + 8 hl .. +7, times scale*log2(e)
     half8v qf[KS];
     {
         const int qr = min(q0 + l32, p.Lq - 1);
@@ -88,51 +103,54 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
         for (int ks = 0; ks < KS; ks++) {
             const int e = 16 * ks + 8 * hl;
             u32x4 z = {0u, 0u, 0u, 0u};
-            qf[ks] = as_half8(e < p.E ? ldg16(qb + (long)qr * p.qs[1] + e) : z);
+            half8v t = as_half8(e < p.E ? ldg16(qb + (long)qr * p.qs[1] + e) : z);
+#pragma unroll
+            for (int j = 0; j < 8; j++) qf[ks][j] = (half_t)((float)t[j] * c);
         }
     }
 
-    u32x4 kr[K_PER], vr[V_PER][2];
+    // Per-thread sources of its PER 16-byte chunks of a key block; a block whose
+    // 64 keys all exist is fetched with one 64-bit add per chunk, the ragged last
+    // one re-reads the last valid key for the rows past the end.
+    u32x4 kr[PER], vr[PER];
+    const half_t *kp0[PER], *vp0[PER];
+    bool eok[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int cidx = tid + i * NT;
+        const int row = cidx / KCH, ch = cidx % KCH;
+        eok[i] = ch * 8 < p.E;
+        kp0[i] = kb + (long)row * p.ks[1] + (eok[i] ? ch * 8 : 0);
+        vp0[i] = vb + (long)row * p.vs[1] + (eok[i] ? ch * 8 : 0);
+    }
     auto load_kv = [&](int key0) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        if (key0 + BC <= p.Lk && p.E == EP) {     // the common case: no predicate, no clamp
+            const long ko = (long)key0 * p.ks[1], vo = (long)key0 * p.vs[1];
 #pragma unroll
-        for (int i = 0; i < K_PER; i++) {
-            const int cidx = tid + i * NT;
-            const int row = cidx / KCH, ch = cidx % KCH;
-            const int key = min(key0 + row, p.Lk - 1);
-            u32x4 z = {0u, 0u, 0u, 0u};
-            kr[i] = ch * 8 < p.E ? ldg16(kb + (long)key * p.ks[1] + ch * 8) : z;
-        }
+            for (int i = 0; i < PER; i++) {
+                kr[i] = ldg16(kp0[i] + ko);
+                vr[i] = ldg16(vp0[i] + vo);
+            }
+        } else {
 #pragma unroll
-        for (int i = 0; i < V_PER; i++) {
-            const int u = tid + i * NT;
-            const int ch = u % KCH, kp = u / KCH;
-            const int key = key0 + 2 * kp;
-            u32x4 z = {0u, 0u, 0u, 0u};
-            const bool eok = ch * 8 < p.E;
-            vr[i][0] = eok ? ldg16(vb + (long)min(key, p.Lk - 1) * p.vs[1] + ch * 8) : z;
-            vr[i][1] = eok ? ldg16(vb + (long)min(key + 1, p.Lk - 1) * p.vs[1] + ch * 8) : z;
+            for (int i = 0; i < PER; i++) {
+                const int cidx = tid + i * NT;
+                const int row = cidx / KCH, ch = cidx % KCH;
+                const int key = min(key0 + row, p.Lk - 1);
+                kr[i] = eok[i] ? ldg16(kb + (long)key * p.ks[1] + ch * 8) : z;
+                vr[i] = eok[i] ? ldg16(vb + (long)key * p.vs[1] + ch * 8) : z;
+            }
         }
     };
-    auto store_kv = [&](int buf, int key0) {
+    auto store_kv = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < K_PER; i++) {
+        for (int i = 0; i < PER; i++) {
             const int cidx = tid + i * NT;
             const int row = cidx / KCH, ch = cidx % KCH;
             *reinterpret_cast<u32x4 *>(&Ks[buf][row * KLD + ch * 8]) = kr[i];
+            *reinterpret_cast<u32x4 *>(&Vs[buf][row * VLD + ch * 8]) = vr[i];
         }
-#pragma unroll
-        for (int i = 0; i < V_PER; i++) {
-            const int u = tid + i * NT;
-            const int ch = u % KCH, kp = u / KCH;
-            // Keys past the end must contribute exactly 0 * v, and v there is a
-            // clamped re-read (finite), so only P needs masking; nothing to zero.
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                *reinterpret_cast<uint32_t *>(&Vt[buf][(ch * 8 + 2 * w) * VLD + 2 * kp]) = pack_lo(vr[i][0][w], vr[i][1][w]);
-                *reinterpret_cast<uint32_t *>(&Vt[buf][(ch * 8 + 2 * w + 1) * VLD + 2 * kp]) = pack_hi(vr[i][0][w], vr[i][1][w]);
-            }
-        }
-        (void)key0;
     };
 
     float16v o_acc[ET];
@@ -140,34 +158,40 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
     for (int t = 0; t < ET; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o_acc[t][r] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
+    float16v negm;                      // every register holds -M for this lane's query
+#pragma unroll
+    for (int r = 0; r < 16; r++) negm[r] = 0.0f;
+    float m_ref = 0.0f, l_run = 0.0f;
+    bool first = true;
 
     const int nblk = (Lk + BC - 1) / BC;
     if (nblk > 0) {
         load_kv(0);
-        store_kv(0, 0);
+        store_kv(0);
     }
     __syncthreads();
 
-    for (int kbk = 0; kbk < nblk; kbk++) {
+    // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
+    const int vtoff = (4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const half2v ones = {(half_t)1.0f, (half_t)1.0f};
+
+    auto block = [&](auto MASK_, int kbk) {
+        constexpr bool MASK = decltype(MASK_)::value;
         const int cur = kbk & 1, key0 = kbk * BC;
         const bool more = kbk + 1 < nblk;
         if (more) load_kv(key0 + BC);
 
-        // S^T tiles: rows = keys, columns = queries
+        // t = s*scale*log2(e) - M, straight out of the MFMA chain
         float16v s[2];
 #pragma unroll
         for (int kt = 0; kt < 2; kt++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) s[kt][r] = 0.0f;
             const half_t *kp_ = &Ks[cur][(32 * kt + l32) * KLD + 8 * hl];
+            s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], negm, 0, 0, 0);
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                half8v kf = *reinterpret_cast<const half8v *>(kp_ + 16 * ks);
-                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s[kt], 0, 0, 0);
-            }
+            for (int ks = 1; ks < KS; ks++)
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_ + 16 * ks), qf[ks], s[kt], 0, 0, 0);
         }
-        if (key0 + BC > Lk) {       // the ragged last block: excluded keys get -inf
+        if constexpr (MASK) {           // the ragged last block: excluded keys get -inf
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -176,55 +200,66 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
                     if (key >= Lk) s[kt][r] = -INFINITY;
                 }
         }
-        // online softmax (flash.jl:25-38 recurrence), in base 2 with the scale folded
-        float mx = -INFINITY;
+        float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
+        for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, s[0][r]), s[1][r]);
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-        const float mc = m_use * c;
-        float rs = 0.0f;
-        half8v pf[2][2];
+        // Move the reference point only when a row outgrew it by 2^TH (or on the first block).
+        const bool grow = (mx > TH || first) && mx != -INFINITY;
+        if (__any(grow)) {
+            const float d = grow ? mx : 0.0f;
+            const float alpha = __builtin_amdgcn_exp2f(-d);
+            m_ref += d;
+            l_run *= alpha;
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+            for (int r = 0; r < 16; r++) negm[r] = -m_ref;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float pv = __builtin_amdgcn_exp2f(fmaf(s[kt][r], c, -mc));
-                rs += pv;
-                pf[kt][r >> 3][r & 7] = (half_t)pv;
-            }
-        rs += __shfl_xor(rs, 32, 64);
-        l_run = l_run * alpha + rs;
-        m_run = m_new;
-        if (__any(alpha != 1.0f)) {
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[kt][r] -= d;
 #pragma unroll
             for (int t = 0; t < ET; t++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) o_acc[t][r] *= alpha;
         }
+        first = false;
+        half8v pf[2][2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(s[kt][r]), p1 = __builtin_amdgcn_exp2f(s[kt][r + 1]);
+                const half2v pk = {(half_t)p0, (half_t)p1};
+                pf[kt][r >> 3][r & 7] = pk[0];
+                pf[kt][r >> 3][(r & 7) + 1] = pk[1];
+                l_run = __builtin_amdgcn_fdot2(pk, ones, l_run, false);
+            }
         // O^T += V^T . P^T
 #pragma unroll
         for (int t = 0; t < ET; t++) {
-            const half_t *vp = &Vt[cur][(32 * t + l32) * VLD + 4 * hl];
+            const half_t *vp = &Vs[cur][vtoff + 32 * t];
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
                 for (int bb = 0; bb < 2; bb++) {
-                    half4v lo = *reinterpret_cast<const half4v *>(vp + 32 * kt + 16 * bb);
-                    half4v hi = *reinterpret_cast<const half4v *>(vp + 32 * kt + 16 * bb + 8);
-                    half8v vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    o_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kt][bb], o_acc[t], 0, 0, 0);
+                    const half_t *vq = vp + (32 * kt + 16 * bb) * VLD;
+                    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(vq));
+                    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(vq + 8 * VLD));
+                    short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    o_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, both), pf[kt][bb], o_acc[t], 0, 0, 0);
                 }
         }
-        if (more) store_kv(cur ^ 1, key0 + BC);
+        if (more) store_kv(cur ^ 1);
         __syncthreads();
-    }
+    };
+    const int nfull = Lk / BC;           // blocks with every key valid
+    for (int kbk = 0; kbk < nfull; kbk++) block(std::false_type{}, kbk);
+    if (nfull < nblk) block(std::true_type{}, nfull);
 
-    // out[b][h][q][e]; lane owns query q0 + l32 and, per tile t and group g, the
+    // Both lanes of a query hold half of its row sum.
+    l_run += __shfl_xor(l_run, 32, 64);
+
+    // out(e, q, h, b); lane owns query q0 + l32 and, per tile t and group g, the
     // four head-dim values e = 32 t + 8 g + 4 hl + 0..3
     const int qi = q0 + l32;
     if (qi < p.Lq) {
@@ -430,7 +465,7 @@ __global__ void sdpa_merge_kernel(SdpaArgs p) {
 }
 
 // ------------------------------------------------------------------------------------------
-constexpr int flash_lds_bytes(int EP) { return 2 * 64 * (EP + 8) * 2 + 2 * EP * (64 + 4) * 2; }
+constexpr int flash_lds_bytes(int EP) { return 2 * 64 * (EP + 8) * 2 + 2 * 64 * (EP + 32) * 2; }
 
 bool vec_addressable(const half_t *ptr, const long st[4], int E) {
     return st[0] == 1 && E % 8 == 0 && st[1] % 8 == 0 && st[2] % 8 == 0 && st[3] % 8 == 0 && aligned_to(ptr, 16);
