@@ -43,7 +43,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 
 // ------------------------------------------------------------------------------------------
 // Fused kernel.  Workgroup = 4 waves = 128 queries (32 per wave); keys walked in
-// blocks of BC = 64 through double-buffered LDS tiles, both as they lie in memory:
+// blocks of BC = 64 through three LDS stages, both operands as they lie in memory:
 //   Ks [BC][EP+8]    keys x head-dim   (A operand of S^T = K.Q^T, plain 16-byte reads)
 //   Vs [BC][EP+32]   keys x head-dim   (A operand of O^T = V^T.P^T through
 //                    ds_read_b64_tr_b16, which transposes 4 keys x 16 head-dim
@@ -61,18 +61,20 @@ __device__ __forceinline__ void static_for(F &&f) {
 //   * Q is pre-multiplied by scale*log2(e) (in fp32, rounded to fp16 once), so the
 //     first product is already in the base-2 exponent domain;
 //   * the reference point M of the running softmax is subtracted by the MFMA itself:
-//     the accumulator of the first product starts from a register tuple holding -M,
-//     so the product delivers t = s - M and p = exp2(t) needs no further arithmetic;
-//   * M is a *stale* maximum: it only moves when a row's block maximum exceeds it by
-//     more than 2^8 (or on the first block).  p then lies in (0, 256], exact in
-//     fp16/fp32, and O and l are rescaled only on those rare moves.  The result is
-//     the same softmax -- every term carries the same factor 2^-M -- with the
-//     rescaling of flash.jl:25-38 applied lazily (the reference's `lazyrescale`,
-//     flash.jl:1041-1096, skips it when no maximum grew; this skips it until one
-//     grew by a factor of 256);
+//     the first product carries one extra k-step whose operands contribute
+//     1.0 * (-M[query]) to every score, so it delivers t = s - M and p = exp2(t)
+//     needs no further arithmetic (M is kept fp16-representable so that what is
+//     subtracted is exactly what the bookkeeping assumes);
+//   * M is a *stale* reference, not the running maximum: it moves on the first
+//     block and when a probability leaves fp16 range (t >= 16, seen as an infinite
+//     row sum), and then to the block maximum.  In between no maximum is computed
+//     at all.  The result is the same softmax -- every term of a row carries the
+//     same factor 2^-M -- with the rescaling of flash.jl:25-38 applied lazily (the
+//     reference's `lazyrescale`, flash.jl:1041-1096, skips it when no maximum grew;
+//     this skips it until fp16 would overflow);
 //   * row sums accumulate the fp16 probabilities pairwise with v_dot2_f32_f16.
 template <int EP>
-__global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
+__global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
     constexpr int BC = 64, BR = 128, NT = 256;
     constexpr int KLD = EP + 8, VLD = EP + 32;
     constexpr int KS = EP / 16;       // k16 steps over the head dim
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
     constexpr float TH = 8.0f;
     extern __shared__ __align__(16) char smem[];
     half_t (*Ks)[BC * KLD] = reinterpret_cast<half_t (*)[BC * KLD]>(smem);
-    half_t (*Vs)[BC * VLD] = reinterpret_cast<half_t (*)[BC * VLD]>(smem + 2 * BC * KLD * 2);
+    half_t (*Vs)[BC * VLD] = reinterpret_cast<half_t (*)[BC * VLD]>(smem + 3 * BC * KLD * 2);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hl = lane >> 5, l32 = lane & 31;
@@ -158,72 +160,44 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
     for (int t = 0; t < ET; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o_acc[t][r] = 0.0f;
-    float16v negm;                      // every register holds -M for this lane's query
+    // The reference point M rides along as one more k-step of the first product:
+    // an operand pair that contributes 1.0 * (-M[query]) to every score.
+    half8v kext, qext;
 #pragma unroll
-    for (int r = 0; r < 16; r++) negm[r] = 0.0f;
-    float m_ref = 0.0f, l_run = 0.0f;
+    for (int j = 0; j < 8; j++) { kext[j] = (half_t)0.0f; qext[j] = (half_t)0.0f; }
+    if (hl == 0) kext[0] = (half_t)1.0f;
+    float m_ref = 0.0f, l_run = 0.0f;    // m_ref is always exactly representable in fp16
     bool first = true;
 
+    // Three LDS stages: while block j is in its softmax and second product, the first
+    // product of block j+1 already runs (its MFMAs fill the matrix pipe under the
+    // exponentials), and block j+2 is on its way from memory into the third stage.
     const int nblk = (Lk + BC - 1) / BC;
-    if (nblk > 0) {
-        load_kv(0);
-        store_kv(0);
-    }
+    if (nblk > 0) { load_kv(0); store_kv(0); }
+    if (nblk > 1) { load_kv(BC); store_kv(1); }
     __syncthreads();
 
     // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
     const int vtoff = (4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const int ktoff = l32 * KLD + 8 * hl;
     const half2v ones = {(half_t)1.0f, (half_t)1.0f};
+    const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    auto block = [&](auto MASK_, int kbk) {
-        constexpr bool MASK = decltype(MASK_)::value;
-        const int cur = kbk & 1, key0 = kbk * BC;
-        const bool more = kbk + 1 < nblk;
-        if (more) load_kv(key0 + BC);
-
-        // t = s*scale*log2(e) - M, straight out of the MFMA chain
-        float16v s[2];
+    // t = s*scale*log2(e) - M, straight out of the MFMA chain
+    auto qk = [&](float16v (&s)[2], int st) {
+        const half_t *kbase = &Ks[st][ktoff];
 #pragma unroll
         for (int kt = 0; kt < 2; kt++) {
-            const half_t *kp_ = &Ks[cur][(32 * kt + l32) * KLD + 8 * hl];
-            s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], negm, 0, 0, 0);
+            const half_t *kp_ = kbase + 32 * kt * KLD;
+            s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], zero16, 0, 0, 0);
 #pragma unroll
             for (int ks = 1; ks < KS; ks++)
                 s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_ + 16 * ks), qf[ks], s[kt], 0, 0, 0);
+            s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, s[kt], 0, 0, 0);
         }
-        if constexpr (MASK) {           // the ragged last block: excluded keys get -inf
-#pragma unroll
-            for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int key = key0 + 32 * kt + 8 * (r >> 2) + 4 * hl + (r & 3);
-                    if (key >= Lk) s[kt][r] = -INFINITY;
-                }
-        }
-        float mx = fmaxf(s[0][0], s[1][0]);
-#pragma unroll
-        for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, s[0][r]), s[1][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        // Move the reference point only when a row outgrew it by 2^TH (or on the first block).
-        const bool grow = (mx > TH || first) && mx != -INFINITY;
-        if (__any(grow)) {
-            const float d = grow ? mx : 0.0f;
-            const float alpha = __builtin_amdgcn_exp2f(-d);
-            m_ref += d;
-            l_run *= alpha;
-#pragma unroll
-            for (int r = 0; r < 16; r++) negm[r] = -m_ref;
-#pragma unroll
-            for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) s[kt][r] -= d;
-#pragma unroll
-            for (int t = 0; t < ET; t++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o_acc[t][r] *= alpha;
-        }
-        first = false;
-        half8v pf[2][2];
+    };
+    // p = 2^t as fp16 MFMA operands; the row sum takes the rounded values, pairwise
+    auto probs = [&](const float16v (&s)[2], half8v (&pf)[2][2], float &l) {
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -232,12 +206,78 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
                 const half2v pk = {(half_t)p0, (half_t)p1};
                 pf[kt][r >> 3][r & 7] = pk[0];
                 pf[kt][r >> 3][(r & 7) + 1] = pk[1];
-                l_run = __builtin_amdgcn_fdot2(pk, ones, l_run, false);
+                l = __builtin_amdgcn_fdot2(pk, ones, l, false);
             }
+    };
+
+    float16v sa[2], sb[2];
+    if (nblk > 0) qk(sa, 0);
+
+    // One key block: sc holds its scores (computed one iteration earlier), sn receives the next block's.
+    auto iter = [&](auto MASK_, float16v (&sc)[2], float16v (&sn)[2], int j) {
+        constexpr bool MASK = decltype(MASK_)::value;
+        const int key0 = j * BC;
+        const int st = j % 3, st1 = (j + 1) % 3, st2 = (j + 2) % 3;
+        const bool next2 = j + 2 < nblk;
+        if (next2) load_kv(key0 + 2 * BC);
+        if constexpr (MASK) {           // the ragged last block: excluded keys get -inf
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = key0 + 32 * kt + 8 * (r >> 2) + 4 * hl + (r & 3);
+                    if (key >= Lk) sc[kt][r] = -INFINITY;
+                }
+        }
+        // Fast path: exponentiate against the current reference point while the next block's
+        // first product runs underneath.  (After the last block that product multiplies a stale
+        // stage: wasted, harmless, and it keeps this stretch free of branches so that the two
+        // instruction streams can be interleaved: one MFMA, then a handful of vector instructions.)
+        __builtin_amdgcn_sched_barrier(0);
+        qk(sn, st1);
+        half8v pf[2][2];
+        float l_new = l_run;
+        probs(sc, pf, l_new);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * KS, 0);
+#pragma unroll
+        for (int g = 0; g < 2 * KS + 2; g++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + 2), 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // A probability that left fp16 range (t >= 16) shows up as an infinite row sum.  Then, and on
+        // the first block, settle a new reference point: the block maximum, for the rows that outgrew
+        // the old one by 2^TH; rescale what was accumulated; redo the exponentials.
+        if (__any(first || !(l_new < INFINITY))) {
+            float mx = fmaxf(sc[0][0], sc[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sc[0][r]), sc[1][r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const bool grow = (mx > TH || first) && mx != -INFINITY;
+            const half_t m16 = (half_t)(m_ref + (grow ? mx : 0.0f));
+            const float d = (float)m16 - m_ref;
+            const float alpha = __builtin_amdgcn_exp2f(-d);
+            m_ref += d;
+            l_run *= alpha;
+            if (hl == 0) qext[0] = -m16;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) { sc[kt][r] -= d; sn[kt][r] -= d; }   // sn was formed against the old M
+#pragma unroll
+            for (int t = 0; t < ET; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o_acc[t][r] *= alpha;
+            l_new = l_run;
+            probs(sc, pf, l_new);
+        }
+        l_run = l_new;
+        first = false;
         // O^T += V^T . P^T
+        const half_t *vbase = &Vs[st][vtoff];
 #pragma unroll
         for (int t = 0; t < ET; t++) {
-            const half_t *vp = &Vs[cur][vtoff + 32 * t];
+            const half_t *vp = vbase + 32 * t;
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -249,12 +289,21 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(SdpaArgs p) {
                     o_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, both), pf[kt][bb], o_acc[t], 0, 0, 0);
                 }
         }
-        if (more) store_kv(cur ^ 1);
+        if (next2) store_kv(st2);
         __syncthreads();
     };
     const int nfull = Lk / BC;           // blocks with every key valid
-    for (int kbk = 0; kbk < nfull; kbk++) block(std::false_type{}, kbk);
-    if (nfull < nblk) block(std::true_type{}, nfull);
+    int j = 0;
+    for (; j + 2 <= nfull; j += 2) {
+        iter(std::false_type{}, sa, sb, j);
+        iter(std::false_type{}, sb, sa, j + 1);
+    }
+    if (j < nfull) {
+        iter(std::false_type{}, sa, sb, j);
+        if (j + 1 < nblk) iter(std::true_type{}, sb, sa, j + 1);
+    } else if (j < nblk) {
+        iter(std::true_type{}, sa, sb, j);
+    }
 
     // Both lanes of a query hold half of its row sum.
     l_run += __shfl_xor(l_run, 32, 64);
@@ -465,7 +514,7 @@ __global__ void sdpa_merge_kernel(SdpaArgs p) {
 }
 
 // ------------------------------------------------------------------------------------------
-constexpr int flash_lds_bytes(int EP) { return 2 * 64 * (EP + 8) * 2 + 2 * 64 * (EP + 32) * 2; }
+constexpr int flash_lds_bytes(int EP) { return 3 * 64 * (EP + 8) * 2 + 3 * 64 * (EP + 32) * 2; }
 
 bool vec_addressable(const half_t *ptr, const long st[4], int E) {
     return st[0] == 1 && E % 8 == 0 && st[1] % 8 == 0 && st[2] % 8 == 0 && st[3] % 8 == 0 && aligned_to(ptr, 16);
