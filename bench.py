@@ -133,9 +133,14 @@ class EncoderBlock:
         d["f"] = torch.empty((T, FF), dtype=f16, device="cuda")
         p = lambda n: d[n].data_ptr()
 
+        # per-op scratch, as the reference's bump workspace hands it out (split-K planes of the narrow linears)
+        ws_bytes = max(lib.mi_gemm_f16_workspace(T, K_, F_, L.W_KF, 1) for (K_, F_) in ((D, D), (D, FF), (FF, D)))
+        self.ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device="cuda")
+        wsp = self.ws.data_ptr()
+
         def gemm(y, x, w, b, K, F, epi, res=None):
             return Call(lib.mi_gemm_f16, p(y), p(x), p(w), p(b), (p(res) if res else None), T, K, F, F, K, F,
-                        L.W_KF, L.BIAS_COL, L.EPI[epi], L.F16, None, 0, stream)
+                        L.W_KF, L.BIAS_COL, L.EPI[epi], L.F16, wsp, ws_bytes, stream)
 
         tok = L.strides4(1, D, E, T * D)      # (E, L, H, B) strides of a token-major [T][H][E] buffer
         scale = 1.0 / np.sqrt(E)

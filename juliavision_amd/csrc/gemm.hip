@@ -593,6 +593,42 @@ __global__ void skinny_epilogue_kernel(GemmArgs p, const float *part, int nsplit
     }
 }
 
+// Split-K epilogue: out = epi(round(sum_s part[s] + bias)) (+ residual), four columns per thread.
+// The counterpart of mm_epilogue_kernel! (matmul.jl:192-217): the planes are fp32 M x N.
+__global__ void splitk_epilogue_kernel(GemmArgs p, const float *part, int nsplit) {
+    const long idx = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    const long total = (long)p.M * p.N;
+    if (idx >= total) return;
+    const int n = (int)(idx % p.N), m = (int)(idx / p.N);
+    float4v v = *reinterpret_cast<const float4v *>(part + idx);
+    for (int s = 1; s < nsplit; s++) {
+        float4v w = *reinterpret_cast<const float4v *>(part + (long)s * total + idx);
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] += w[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+        v[e] += p.bias_mode == MI_BIAS_COL ? (float)p.bias[n + e] : p.bias_mode == MI_BIAS_ROW ? (float)p.bias[m] : 0.0f;
+    const long off = (long)m * p.ldY + n;
+    if (p.out_f32) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) reinterpret_cast<float *>(p.Y)[off + e] = apply_epi(v[e], p.epi);
+    } else {
+        half4v o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (half_t)apply_epi((float)(half_t)v[e], p.epi);
+        if (p.residual) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = (half_t)((float)o[e] + (float)p.residual[off + e]);
+        }
+        if (p.vec_store) *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(p.Y) + off) = o;
+        else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) reinterpret_cast<half_t *>(p.Y)[off + e] = o[e];
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 bool g_ready = false;
 int g_cus = 256;
@@ -658,6 +694,21 @@ int launch_mfma(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
+// K-slices for a GEMM whose 128 x 128 output tiles number fewer than the CUs: as many as fit two
+// workgroups per CU, each slice a multiple of 64 and deep enough; N must allow 4-wide rows.
+int splitk_count(int64_t M, int64_t N, int64_t K) {
+    if (M <= 8 || N % 4 || K % 64) return 1;
+    const int64_t tiles = ceil_div(M, 128) * ceil_div(N, 128);
+    if (ceil_div(M, 128) * ceil_div(N, 256) >= (g_cus * 3) / 4 || tiles * 2 > g_cus) return 1;
+    int64_t s = (2 * (int64_t)g_cus) / tiles;
+    if (s > 8) s = 8;
+    // A slice must be deep enough to pay for the second pass over the output: 1024, or 512 when
+    // the tiles would otherwise leave three quarters of the chip idle.
+    const int64_t kmin = tiles * 4 <= g_cus ? 512 : 1024;
+    while (s > 1 && (K % (s * 64) != 0 || K / s < kmin)) s--;
+    return (int)s;
+}
+
 int gemm_path(const GemmArgs &a, bool b_kn, int64_t nbatch) {
     if (a.M < 1 || a.N < 1 || a.K < 1) return MI_GEMM_DECLINE;
     bool addr = mfma_addressable(a, b_kn);
@@ -720,6 +771,24 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
     if (path == MI_GEMM_SKINNY) return run_skinny(a, b_kn, ws, ws_bytes, st);
     if (path == MI_GEMM_MFMA) {
         if (!mfma_addressable(a, b_kn)) return MI_DECLINE_OPERANDS;
+        // Split K over workgroups when the output alone cannot fill the chip: each K-slice is one plane
+        // of a batched launch (plane strides: A advances along k, Y one fp32 M x N plane in ws), and a
+        // second small kernel sums the planes and applies bias, activation and residual.
+        const int split = nbatch == 1 ? splitk_count(a.M, a.N, a.K) : 1;
+        if (split > 1 && ws && aligned_to(ws, 256) && ws_bytes >= (size_t)split * a.M * a.N * sizeof(float)) {
+            GemmArgs s1 = a;
+            s1.Y = ws; s1.out_f32 = 1; s1.bias = nullptr; s1.bias_mode = MI_BIAS_NONE; s1.epi = MI_EPI_NONE; s1.residual = nullptr;
+            s1.ldY = a.N; s1.sY = (long)a.M * a.N;
+            s1.K = a.K / split;
+            s1.sA = s1.K; s1.sB = b_kn ? (long)s1.K * a.ldB : s1.K; s1.sBias = 0;
+            int rc = launch_pipe<128, 128, 2, 2>(s1, b_kn, split, st);
+            if (rc != MI_OK) return rc;
+            GemmArgs s2 = a;
+            s2.vec_store = !a.out_f32 && a.ldY % 4 == 0 && aligned_to(a.Y, 8);
+            const long quads = ((long)a.M * a.N) / 4;
+            hipLaunchKernelGGL(splitk_epilogue_kernel, dim3((unsigned)ceil_div(quads, 256)), dim3(256), 0, st, s2, reinterpret_cast<const float *>(ws), split);
+            return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+        }
         // Tile choice: the big tile when it still gives every CU a workgroup,
         // else smaller tiles so small problems spread over the chip.
         int64_t big = ceil_div(a.M, 128) * ceil_div(a.N, 256) * nbatch;
@@ -797,7 +866,11 @@ int mi_device_caps(int64_t out[6]) {
 }
 
 size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int64_t nbatch) {
-    if (T < 1 || T > 8 || nbatch > 1) return 0;
+    if (T < 1 || nbatch > 1) return 0;
+    if (T > 8) {
+        const int split = splitk_count(T, F, K);
+        return split > 1 ? round_up((size_t)split * T * F * sizeof(float), 256) : 0;
+    }
     int nsplit = w_layout == MI_W_KF ? skinny_splits(K, F) : 1;
     return round_up((size_t)nsplit * T * F * sizeof(float), 256);
 }

@@ -121,3 +121,16 @@ def test_batched_shared_activations_with_per_plane_bias(ctx):
     got = to_host(out)
     for i in range(3):
         assert_parity(got[i], oracle.gemm_f16(X, W[i], b[i]), what=f"qkv plane {i}")
+
+
+@pytest.mark.parametrize("layout", ["kf", "fk"])
+def test_split_k_narrow_outputs(ctx, layout):
+    """Few output tiles and a deep K: the library splits K over workgroups (fp32 planes in the workspace,
+    summed by a second kernel that applies bias, activation and residual)."""
+    from juliavision_amd import _lib as L
+    lib = L.load()
+    assert lib.mi_gemm_f16_workspace(1500, 5120, 1280, L.W_KF, 1) >= 2 * 1500 * 1280 * 4
+    assert lib.mi_gemm_f16_workspace(200, 2048, 256, L.W_KF, 1) > 0
+    _run(ctx, 200, 2048, 256, layout=layout, epi="gelu", residual=True)
+    _run(ctx, 200, 2048, 256, layout=layout, out_f32=True)
+    _run(ctx, 1500, 5120, 1280, layout=layout, residual=True, seed=7)
