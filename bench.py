@@ -39,8 +39,8 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, vendor figure
 
 # HBM bytes per launch of the dominant kernel (fc1 GEMM), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of `python bench.py --no-cpu --no-detail`, scaled by the same counters on a plain copy kernel of
-# known size; see profiles/.  None until measured.
-FC1_TRAFFIC_BYTES = None
+# known size (--calibrate-copy).
+FC1_TRAFFIC_BYTES = 57_309_184       # profiles/fc1_gemm_hbm_traffic.txt: FETCH 20 483 KiB x 2.000 + WRITE 15 000 KiB x 1.000
 
 
 def parse_args():
@@ -51,6 +51,12 @@ def parse_args():
     ap.add_argument("--detail", dest="detail", action="store_true", default=True)
     ap.add_argument("--no-detail", dest="detail", action="store_false")
     ap.add_argument("--no-cpu", dest="cpu", action="store_false", default=True)
+    ap.add_argument("--only", default=None, metavar="SUBSTR",
+                    help="run only the detail cases whose name contains SUBSTR (e.g. c4_attn, c1_linear) and print them; "
+                         "for profiling one kernel with rocprofv3")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy three times, so that a rocprofv3 --pmc run of this "
+                         "command holds a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
     return ap.parse_args()
 
 
@@ -165,6 +171,7 @@ class EncoderBlock:
         self.fc1()
         if ev is not None:
             ev[1].record()
+            ev[2].record()       # nothing between ev[1] and ev[2]: what one event marker itself costs on this stream
         for c in self.calls_after_fc1:
             c()
 
@@ -209,7 +216,7 @@ class EncoderBlock:
 
 # ----------------------------------------------------------------------------- other configs (detail)
 
-def detail_benchmarks(lib, L, stream):
+def detail_benchmarks(lib, L, stream, only=None):
     import numpy as np
     import torch
     out = {}
@@ -217,6 +224,8 @@ def detail_benchmarks(lib, L, stream):
     NB = 3   # rotating buffer sets
 
     def gemm_case(name, T, K, F, layout, epi="none", sets=NB, reps=20):
+        if only is not None and only not in name:
+            return None
         Xs = [torch.randn((T, K), dtype=f16, device="cuda") / K ** 0.5 for _ in range(sets)]
         Ws = [torch.randn((K, F) if layout == L.W_KF else (F, K), dtype=f16, device="cuda") * 0.02 for _ in range(sets)]
         b = torch.randn((F,), dtype=f16, device="cuda") * 0.02
@@ -239,6 +248,8 @@ def detail_benchmarks(lib, L, stream):
         return out[name]
 
     def attn_case(name, B, H, Lq, Lk, E, kv_len=None, sets=NB, reps=10):
+        if only is not None and only not in name:
+            return
         qs = [torch.randn((B, H, Lq, E), dtype=f16, device="cuda") for _ in range(sets)]
         ks = [torch.randn((B, H, Lk, E), dtype=f16, device="cuda") for _ in range(sets)]
         vs = [torch.randn((B, H, Lk, E), dtype=f16, device="cuda") for _ in range(sets)]
@@ -273,35 +284,50 @@ def detail_benchmarks(lib, L, stream):
     gemm_case("c3_fc2_1370x1536x384", 1370, 1536, 384, L.W_KF)
     attn_case("c3_attn_L1370_6x64", 1, 6, 1370, 1370, 64)
     attn_case("c2_attn_L1500_20x64", 1, 20, 1500, 1500, 64)
+    def conv_case():
+        x = torch.randn((1, 256, 64, 64), dtype=f16, device="cuda")
+        w = torch.randn((256, 256, 3, 3), dtype=f16, device="cuda") * 0.02
+        b = torch.randn((256,), dtype=f16, device="cuda") * 0.02
+        o = torch.empty((1, 256, 64, 64), dtype=f16, device="cuda")
+        need = lib.mi_conv2d_f16_workspace(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        conv = Call(lib.mi_conv2d_f16, o.data_ptr(), x.data_ptr(), w.data_ptr(), b.data_ptr(), 64, 64, 256, 1, 3, 3, 256,
+                    1, 1, 1, 1, 1, 1, 1, L.EPI["none"], ws.data_ptr(), need, stream)
+        med, lo, hi = event_time(conv, 10)
+        flop = 2.0 * 4096 * 2304 * 256
+        out["c4_conv3x3_256to256_64x64"] = {"us": round(med * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 2),
+                                            "frac_mfma_peak": round(flop / med / 1e12 / PEAK_F16_TFLOPS, 4)}
+
+    def decode_cases():
+        # config 5: decode-sized linears (HBM-bound on the weights; enough rotating weight sets to exceed the
+        # 256 MB last-level cache) and single-query attention over the caches
+        for bsz in (1, 4, 8):
+            for (K, F) in ((1280, 1280), (1280, 5120)):
+                sets = int(np.ceil(320e6 / (2.0 * K * F)))
+                for lay, tag in ((L.W_KF, "W[K][F]"), (L.W_FK, "W[F][K]")):
+                    name = f"c5_linear_b{bsz}_{K}to{F}_{tag}"
+                    if only is not None and only not in name:
+                        continue
+                    r = gemm_case(name, bsz, K, F, lay, sets=sets, reps=sets)
+                    r["frac_hbm_peak"] = round(r["weight_GB/s"] / PEAK_HBM_GBS, 4)
+                    del r["TFLOP/s"], r["frac_mfma_peak"]
+            for (nm, Lk, kvl) in (("self_pos447", 448, 448), ("self_pos3", 448, 4), ("cross", 1500, None)):
+                name = f"c5_attn_b{bsz}_{nm}"
+                if only is not None and only not in name:
+                    continue
+                sets = int(np.ceil(320e6 / (4.0 * Lk * 64 * 20 * bsz)))
+                attn_case(name, bsz, 20, 1, Lk, 64, kv_len=kvl, sets=sets, reps=sets)
+                r = out[name]
+                r["frac_hbm_peak"] = round(r["kv_GB/s"] / PEAK_HBM_GBS, 4)
+                del r["TFLOP/s"], r["frac_mfma_peak"]
+
     # config 4: global attention at 4096 and the 3x3 conv
     attn_case("c4_attn_L4096_16x64", 1, 16, 4096, 4096, 64)
-    x = torch.randn((1, 256, 64, 64), dtype=f16, device="cuda")
-    w = torch.randn((256, 256, 3, 3), dtype=f16, device="cuda") * 0.02
-    b = torch.randn((256,), dtype=f16, device="cuda") * 0.02
-    o = torch.empty((1, 256, 64, 64), dtype=f16, device="cuda")
-    need = lib.mi_conv2d_f16_workspace(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
-    ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
-    conv = Call(lib.mi_conv2d_f16, o.data_ptr(), x.data_ptr(), w.data_ptr(), b.data_ptr(), 64, 64, 256, 1, 3, 3, 256,
-                1, 1, 1, 1, 1, 1, 1, L.EPI["none"], ws.data_ptr(), need, stream)
-    med, lo, hi = event_time(conv, 10)
-    flop = 2.0 * 4096 * 2304 * 256
-    out["c4_conv3x3_256to256_64x64"] = {"us": round(med * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 2),
-                                        "frac_mfma_peak": round(flop / med / 1e12 / PEAK_F16_TFLOPS, 4)}
-    # config 5: decode-sized linears (HBM-bound on the weights; enough rotating weight sets to exceed the
-    # 256 MB last-level cache) and single-query attention over the caches
-    for bsz in (1, 4, 8):
-        for (K, F) in ((1280, 1280), (1280, 5120)):
-            sets = int(np.ceil(320e6 / (2.0 * K * F)))
-            for lay, tag in ((L.W_KF, "W[K][F]"), (L.W_FK, "W[F][K]")):
-                r = gemm_case(f"c5_linear_b{bsz}_{K}to{F}_{tag}", bsz, K, F, lay, sets=sets, reps=sets)
-                r["frac_hbm_peak"] = round(r["weight_GB/s"] / PEAK_HBM_GBS, 4)
-                del r["TFLOP/s"], r["frac_mfma_peak"]
-        for (nm, Lk, kvl) in (("self_pos447", 448, 448), ("self_pos3", 448, 4), ("cross", 1500, None)):
-            sets = int(np.ceil(320e6 / (4.0 * Lk * 64 * 20 * bsz)))
-            attn_case(f"c5_attn_b{bsz}_{nm}", bsz, 20, 1, Lk, 64, kv_len=kvl, sets=sets, reps=sets)
-            r = out[f"c5_attn_b{bsz}_{nm}"]
-            r["frac_hbm_peak"] = round(r["kv_GB/s"] / PEAK_HBM_GBS, 4)
-            del r["TFLOP/s"], r["frac_mfma_peak"]
+    if only is None or only in "c4_conv3x3_256to256_64x64":
+        conv_case()
+    decode_cases()
+    if only is not None:
+        return {k: v for k, v in out.items() if only in k}
     return out
 
 
@@ -318,12 +344,22 @@ def main():
     L = jv._lib
     lib = L.init()
     stream = torch.cuda.current_stream().cuda_stream
+    if args.only is not None:
+        print(json.dumps({"only": args.only, "detail": detail_benchmarks(lib, L, stream, args.only)}))
+        return
     blk = EncoderBlock(lib, stream)
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         blk.step()
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    evs = [tuple(torch.cuda.Event(enable_timing=True) for _ in range(3)) for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -331,7 +367,11 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     sec = (t1 - t0) / args.steps
-    fc1_ms = sorted(s.elapsed_time(e) for s, e in evs)
+    # An event is a marker packet of its own in the queue: the bracket [ev0, ev1] holds the fc1 kernel plus one
+    # marker; [ev1, ev2] holds one marker and nothing else.  Their difference is the kernel's own duration.
+    bracket_ms = [e0.elapsed_time(e1) for e0, e1, _ in evs]
+    marker_ms = [e1.elapsed_time(e2) for _, e1, e2 in evs]
+    fc1_ms = sorted(b - m for b, m in zip(bracket_ms, marker_ms))
     fc1_avg = sum(fc1_ms) / len(fc1_ms) * 1e-3
     y = blk.d["y"].float()
     if not bool(torch.isfinite(y).all()) or float(y.abs().max()) < 1e-3:
@@ -352,11 +392,13 @@ def main():
                    "tokens": 1500, "d_model": 1280, "heads": 20, "head_dim": 64, "ffn": 5120,
                    "weight_layout": "[K][F] (the reference's hoisted layout)"},
         "frac_mfma_peak": round(blk.FLOP / sec / 1e12 / PEAK_F16_TFLOPS, 4),
-        "roofline": {"kernel": "gemm_mfma_kernel<128,256,64> fc1: Y[1500x5120] = gelu(X[1500x1280].W[1280x5120] + b)",
+        "roofline": {"kernel": "gemm_pipe_kernel<128,256,2,4,KN> fc1: Y[1500x5120] = gelu(X[1500x1280].W[1280x5120] + b)",
                      "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": FC1_TRAFFIC_BYTES,
                      "flop_per_launch": blk.FC1_FLOP, "avg_launch_us": round(fc1_avg * 1e6, 2),
-                     "median_launch_us": round(fc1_ms[len(fc1_ms) // 2] * 1e3, 2)},
+                     "median_launch_us": round(fc1_ms[len(fc1_ms) // 2] * 1e3, 2),
+                     "avg_event_bracket_us": round(sum(bracket_ms) / len(bracket_ms) * 1e3, 2),
+                     "avg_event_marker_us": round(sum(marker_ms) / len(marker_ms) * 1e3, 2)},
     }
     if args.detail:
         res["detail"] = detail_benchmarks(lib, L, stream)
