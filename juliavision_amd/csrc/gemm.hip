@@ -179,7 +179,9 @@ __device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN
                 }
             }
         }
-        __syncthreads();
+        // A wave reads back only what it staged itself, and its LDS operations complete in order:
+        // no workgroup barrier, only a stop for the compiler.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (p.out_f32) {
             constexpr int CPR = WTN / 4;
             for (int c = lane; c < 32 * CPR; c += 64) {
@@ -226,7 +228,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN
                 }
             }
         }
-        __syncthreads();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     });
 }
 
@@ -429,21 +431,36 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
     // Tile kt is computed from LDS buffer `cur`; register set `gw` holds tile kt+1, set `gl` receives tile kt+2.
     auto body = [&](auto MODE_, int kt, int cur, int gw, int gl) {
         constexpr int MODE = decltype(MODE_)::value;
+        constexpr int NM = TM * TN;               // MFMAs per k-step
+        constexpr int NR = TM + (B_KN ? 2 * TN : TN);   // fragment reads per k-step
+        // Each k-step is pinned to: its fragment reads first, then its MFMAs with the step's
+        // memory instructions dealt out between them, so that neither the LDS pipe nor the
+        // vector-memory path sees a burst.
         if constexpr (MODE == 0) gload(gl, kt + 2);
         fread(1, cur, 1);
         mma(0);
+        __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
+#pragma unroll
+        for (int g = 0; g < NM; g++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x020, (PA + PB + NM - 1) / NM, 0); }
         __builtin_amdgcn_sched_barrier(0);
         fread(0, cur, 2);
         mma(1);
         if constexpr (MODE < 2) lwrite_a(gw, cur ^ 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
+#pragma unroll
+        for (int g = 0; g < NM; g++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x200, (PA + NM - 1) / NM, 0); }
         __builtin_amdgcn_sched_barrier(0);
         fread(1, cur, 3);
         mma(0);
         if constexpr (MODE < 2) lwrite_b(gw, cur ^ 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
+#pragma unroll
+        for (int g = 0; g < NM; g++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x200, (PB + NM - 1) / NM, 0); }
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         if constexpr (MODE < 2) fread(0, cur ^ 1, 0);
         mma(1);
+        __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
     using M0 = std::integral_constant<int, 0>;
