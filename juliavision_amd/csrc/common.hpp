@@ -55,4 +55,4 @@ int mi_sdpa_init();
 // Y[M x N] = A[M x K] . B (+bias) with B either [K][NB-padded N] (b_kn) or [N][K]; defined in gemm.hip.
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
-                     long nbatch, long sY, long sA, long sB, hipStream_t st);
+                     long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st);

@@ -21,24 +21,33 @@ struct ConvArgs {
 
 // col[c][m], m fastest: c = (ci, kh, kw) with kw fastest, m = (oh, ow) with ow
 // fastest (the order of im2col_kernel!, conv_coopmat.jl:259-286).  Rows c >= CRS
-// and columns m >= PQ are zero, as are taps that fall in the padding.  32-bit
-// index arithmetic throughout.
+// and columns m >= PQ are zero, as are taps that fall in the padding.  A thread
+// produces eight consecutive pixels of one row c (one 16-byte store), so the
+// index decomposition is paid once per eight elements; 32-bit arithmetic throughout.
 __global__ void im2col_kernel(half_t *col, ConvArgs a, int PQP, int CRSP) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    const int total = PQP * CRSP;
-    if (idx >= total) return;
+    const int groups = PQP >> 3;
+    if (idx >= groups * CRSP) return;
     const int n = blockIdx.y;
-    const int m = idx % PQP, c = idx / PQP;
+    const int m0 = (idx % groups) * 8, c = idx / groups;
     const int PQ = a.OW * a.OH, CRS = a.Cin * a.KH * a.KW;
-    half_t val = (half_t)0.0f;
-    if (m < PQ && c < CRS) {
-        const int ow = m % a.OW, oh = m / a.OW;
+    half8v val;
+#pragma unroll
+    for (int j = 0; j < 8; j++) val[j] = (half_t)0.0f;
+    if (c < CRS) {
         const int kw = c % a.KW, t = c / a.KW, kh = t % a.KH, ci = t / a.KH;
-        const int ix = ow * a.sx - a.px + kw * a.dx, iy = oh * a.sy - a.py + kh * a.dy;
-        if (ix >= 0 && ix < a.Wi && iy >= 0 && iy < a.Hi)
-            val = a.x[(((long)n * a.Cin + ci) * a.Hi + iy) * a.Wi + ix];
+        const half_t *xp = a.x + ((long)n * a.Cin + ci) * a.Hi * a.Wi;
+        int ow = m0 % a.OW, oh = m0 / a.OW;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            if (m0 + j < PQ) {
+                const int ix = ow * a.sx - a.px + kw * a.dx, iy = oh * a.sy - a.py + kh * a.dy;
+                if (ix >= 0 && ix < a.Wi && iy >= 0 && iy < a.Hi) val[j] = xp[iy * a.Wi + ix];
+            }
+            if (++ow == a.OW) { ow = 0; oh++; }
+        }
     }
-    col[(long)n * total + idx] = val;
+    *reinterpret_cast<half8v *>(col + (long)n * PQP * CRSP + (long)c * PQP + m0) = val;
 }
 
 // wp[co][CRSP] = w[co][CRS] zero-padded
@@ -137,7 +146,7 @@ size_t mi_conv2d_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, i
     im2col_extents(a, PQP, CRSP);
     size_t col = round_up((size_t)N * PQP * CRSP * 2, 256);
     size_t wp = CRSP != (int64_t)Cin * KH * KW ? round_up((size_t)Cout * CRSP * 2, 256) : 0;
-    return col + wp;
+    return col + wp + mi_gemm_f16_workspace(Cout, CRSP, (int64_t)a.OW * a.OH, MI_W_KF, N);
 }
 
 int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
@@ -163,18 +172,19 @@ int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
         // out[n][Cout][PQ] = w[Cout][Cin] . x[n][Cin][PQ]; the [K][N] operand needs
         // PQ % 8 == 0 for 16-byte loads, otherwise the scalar GEMM takes it.
         return mi_internal_gemm(out, w, x, bias, a.Cout, PQ, PQ, a.Cin, PQ, a.Cin, PQ, 1, MI_BIAS_ROW, epi, 0,
-                                a.N, (long)a.Cout * PQ, 0, (long)a.Cin * PQ, st);
+                                a.N, (long)a.Cout * PQ, 0, (long)a.Cin * PQ, nullptr, 0, st);
     }
     int64_t PQP, CRSP;
     im2col_extents(a, PQP, CRSP);
     const int CRS = a.Cin * a.KH * a.KW;
     size_t col_bytes = round_up((size_t)N * PQP * CRSP * 2, 256);
     size_t wp_bytes = CRSP != CRS ? round_up((size_t)Cout * CRSP * 2, 256) : 0;
-    if (!ws || ws_bytes < col_bytes + wp_bytes || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
+    const size_t gemm_bytes = mi_gemm_f16_workspace(Cout, CRSP, PQ, MI_W_KF, N);
+    if (!ws || ws_bytes < col_bytes + wp_bytes + gemm_bytes || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
     if (PQP * CRSP > INT32_MAX) return MI_DECLINE_EXTENT;
     half_t *col = reinterpret_cast<half_t *>(ws);
     const half_t *wuse = a.w;
-    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)ceil_div(PQP * CRSP, 256), (unsigned)a.N), dim3(256), 0, st, col, a, (int)PQP, (int)CRSP);
+    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)ceil_div(PQP / 8 * CRSP, 256), (unsigned)a.N), dim3(256), 0, st, col, a, (int)PQP, (int)CRSP);
     if (wp_bytes) {
         half_t *wp = reinterpret_cast<half_t *>(reinterpret_cast<char *>(ws) + col_bytes);
         hipLaunchKernelGGL(padweight_kernel, dim3((unsigned)ceil_div((int64_t)Cout * CRSP, 256)), dim3(256), 0, st, wp, a.w, a.Cout, CRS, (int)CRSP);
@@ -182,7 +192,7 @@ int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
     }
     if (hipGetLastError() != hipSuccess) return MI_ERROR_LAUNCH;
     return mi_internal_gemm(out, wuse, col, bias, a.Cout, PQ, (int)PQP, (int)CRSP, PQ, CRSP, PQP, 1, MI_BIAS_ROW, epi, 0,
-                            a.N, (long)a.Cout * PQ, 0, PQP * CRSP, st);
+                            a.N, (long)a.Cout * PQ, 0, PQP * CRSP, reinterpret_cast<char *>(ws) + col_bytes + wp_bytes, gemm_bytes, st);
 }
 
 }  // extern "C"

@@ -829,14 +829,14 @@ int mi_num_cus() { return g_cus; }
 // every GemmArgs field meaningful.
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
-                     long nbatch, long sY, long sA, long sB, hipStream_t st) {
+                     long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st) {
     GemmArgs a;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
     int path = mfma_addressable(a, b_kn != 0) ? MI_GEMM_MFMA : MI_GEMM_SCALAR;
-    return run_gemm(a, b_kn != 0, nbatch, nullptr, 0, st, path);
+    return run_gemm(a, b_kn != 0, nbatch, ws, ws_bytes, st, path);
 }
 
 extern "C" {
