@@ -73,9 +73,15 @@ __device__ __forceinline__ void static_for(F &&f) {
 //     reference's `lazyrescale`, flash.jl:1041-1096, skips it when no maximum grew;
 //     this skips it until fp16 would overflow);
 //   * row sums accumulate the fp16 probabilities pairwise with v_dot2_f32_f16.
-template <int EP>
-__global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
-    constexpr int BC = 64, BR = 128, NT = 256;
+//
+// PP ("ping-pong"): eight waves per workgroup, 256 queries.  Waves w and w+4 share a SIMD and are kept
+// half a key block apart by two workgroup barriers per block, so that while one of them is in its
+// exponentials (with the next block's first product underneath) the other is in its second product:
+// the matrix pipe and the vector ALU of a SIMD are then busy with different waves instead of both
+// waves wanting the same unit at the same time.  Waves 0-3 do all the global -> LDS staging.
+template <int EP, bool PP>
+__global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
+    constexpr int BC = 64, BR = PP ? 256 : 128, NT = 256;     // NT: threads that stage K and V
     constexpr int KLD = EP + 8, VLD = EP + 32;
     constexpr int KS = EP / 16;       // k16 steps over the head dim
     constexpr int ET = EP / 32;       // 32-wide head-dim tiles of O
@@ -86,7 +92,10 @@ __global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaAr
     half_t (*Ks)[BC * KLD] = reinterpret_cast<half_t (*)[BC * KLD]>(smem);
     half_t (*Vs)[BC * VLD] = reinterpret_cast<half_t (*)[BC * VLD]>(smem + 3 * BC * KLD * 2);
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tid = threadIdx.x & 255;                       // index among the staging threads
+    const int grp = wave >> 2;                               // PP: 0 = waves 0-3, 1 = waves 4-7
+    const bool loader = !PP || grp == 0;
     const int hl = lane >> 5, l32 = lane & 31;
     const int h = blockIdx.y, b = blockIdx.z;
     const int q0 = blockIdx.x * BR + wave * 32;
@@ -96,6 +105,12 @@ __global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaAr
     int Lk = p.Lk;
     if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
     const float c = p.scale * LOG2E;
+    // barrier between the half-block intervals of the ping-pong: LDS traffic of this wave done, nothing else waited for
+    auto pp_barrier = [&]() {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
 
     // Q^T fragments: column = query l32, k = head-dim 16 ks + 8 hl .. +7, times scale*log2(e)
     half8v qf[KS];
@@ -173,8 +188,8 @@ __global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaAr
     // product of block j+1 already runs (its MFMAs fill the matrix pipe under the
     // exponentials), and block j+2 is on its way from memory into the third stage.
     const int nblk = (Lk + BC - 1) / BC;
-    if (nblk > 0) { load_kv(0); store_kv(0); }
-    if (nblk > 1) { load_kv(BC); store_kv(1); }
+    if (nblk > 0 && loader) { load_kv(0); store_kv(0); }
+    if (nblk > 1 && loader) { load_kv(BC); store_kv(1); }
     __syncthreads();
 
     // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
@@ -218,7 +233,7 @@ __global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaAr
         constexpr bool MASK = decltype(MASK_)::value;
         const int key0 = j * BC;
         const int st = j % 3, st1 = (j + 1) % 3, st2 = (j + 2) % 3;
-        const bool next2 = j + 2 < nblk;
+        const bool next2 = j + 2 < nblk && loader;
         if (next2) load_kv(key0 + 2 * BC);
         if constexpr (MASK) {           // the ragged last block: excluded keys get -inf
 #pragma unroll
@@ -273,6 +288,13 @@ __global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaAr
         }
         l_run = l_new;
         first = false;
+        if constexpr (PP) {
+            // Second half of the block.  Block j+2 goes into the stage whose last readers (the other
+            // group's second product of block j-1) finished before the barrier just passed; the barrier
+            // that ends this interval publishes it before anyone's first product of block j+2.
+            pp_barrier();
+            if (next2) store_kv(st2);
+        }
         // O^T += V^T . P^T
         const half_t *vbase = &Vs[st][vtoff];
 #pragma unroll
@@ -289,10 +311,15 @@ __global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaAr
                     o_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, both), pf[kt][bb], o_acc[t], 0, 0, 0);
                 }
         }
-        if (next2) store_kv(st2);
-        __syncthreads();
+        if constexpr (PP) {
+            pp_barrier();
+        } else {
+            if (next2) store_kv(st2);
+            __syncthreads();
+        }
     };
     const int nfull = Lk / BC;           // blocks with every key valid
+    if (PP && grp == 1) pp_barrier();    // waves 4-7 run half a block behind waves 0-3
     int j = 0;
     for (; j + 2 <= nfull; j += 2) {
         iter(std::false_type{}, sa, sb, j);
@@ -305,6 +332,7 @@ __global__ __launch_bounds__(256, EP <= 64 ? 2 : 1) void flash_fwd_kernel(SdpaAr
         iter(std::true_type{}, sa, sb, j);
     }
 
+    if (PP && grp == 0) pp_barrier();    // ... so waves 0-3 meet their last barrier here
     // Both lanes of a query hold half of its row sum.
     l_run += __shfl_xor(l_run, 32, 64);
 
@@ -572,8 +600,9 @@ void launch_rows(const SdpaArgs &a, bool vec, dim3 grid, hipStream_t st) {
 // default 64 KiB of dynamic LDS.
 int mi_sdpa_init() {
     int bad = 0;
-    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
-    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     return bad;
 }
 
@@ -617,9 +646,16 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
     int path = sdpa_path(a);
     if (path == MI_SDPA_DECLINE) return MI_DECLINE_EXTENT;
     if (path == MI_SDPA_FLASH) {
-        dim3 grid((unsigned)ceil_div(Lq, 128), (unsigned)H, (unsigned)B);
-        if (E <= 64) hipLaunchKernelGGL(flash_fwd_kernel<64>, grid, dim3(256), flash_lds_bytes(64), st, a);
-        else         hipLaunchKernelGGL(flash_fwd_kernel<128>, grid, dim3(256), flash_lds_bytes(128), st, a);
+        // The 8-wave ping-pong kernel when 256-query workgroups still cover most of the chip.
+        const bool pp = E <= 64 && ceil_div(Lq, 256) * H * B * 4 >= (int64_t)mi_num_cus() * 3;
+        if (pp) {
+            dim3 grid((unsigned)ceil_div(Lq, 256), (unsigned)H, (unsigned)B);
+            hipLaunchKernelGGL((flash_fwd_kernel<64, true>), grid, dim3(512), flash_lds_bytes(64), st, a);
+        } else {
+            dim3 grid((unsigned)ceil_div(Lq, 128), (unsigned)H, (unsigned)B);
+            if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false>), grid, dim3(256), flash_lds_bytes(64), st, a);
+            else         hipLaunchKernelGGL((flash_fwd_kernel<128, false>), grid, dim3(256), flash_lds_bytes(128), st, a);
+        }
         return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
     }
     // rows path

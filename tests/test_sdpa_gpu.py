@@ -163,3 +163,16 @@ def test_token_major_output(ctx):
         torch.cuda.synchronize()
         want = oracle.sdpa_ref_f32(q[:, :, :lq], k, v)
         assert_parity(to_host(buf).transpose(0, 2, 1, 3), want, what=f"token-major out Lq={lq}")
+
+
+def test_eight_wave_kernel_on_large_grids(ctx):
+    """Grids that fill the chip with 256-query workgroups take the 8-wave variant of the fused kernel:
+    ragged query and key counts, per-batch kv_len (one of them 0), strided heads."""
+    import torch
+    B, H, Lq, Lk, E = 4, 16, 700, 777, 64
+    q, k, v = _qkv(B, H, Lq, Lk, E, 121)
+    _check(ctx, q, k, v, expect="FlashPlan", what="8-wave ragged")
+    got = _check(ctx, q, k, v, kv_len=[777, 0, 65, 300], expect="FlashPlan", what="8-wave kv_len")
+    assert np.all(got[1] == 0)
+    _check(ctx, q, k[:, :, :64], v[:, :, :64], expect="FlashPlan", what="8-wave one block")
+    _check(ctx, q, k[:, :, :129], v[:, :, :129], out_dtype="f32", expect="FlashPlan", what="8-wave three blocks f32")
