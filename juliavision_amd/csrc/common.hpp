@@ -44,6 +44,14 @@ MI_DEVICE float apply_epi(float v, int epi) {
     }
 }
 
+template <int EPI>
+MI_DEVICE float apply_epi_c(float v) {
+    if constexpr (EPI == MI_EPI_GELU_ERF) return 0.5f * v * (1.0f + erf_as(v * 0.70710678118654752440f));
+    else if constexpr (EPI == MI_EPI_GELU_TANH) return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    else if constexpr (EPI == MI_EPI_RELU) return fmaxf(v, 0.0f);
+    else return v;
+}
+
 static inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline size_t round_up(size_t a, size_t b) { return (a + b - 1) / b * b; }

@@ -136,9 +136,31 @@ __device__ __forceinline__ void tile_of(int pid, int nwg, int tiles_m, int tiles
 // activation, the residual add and the global stores run on 16-byte vectors
 // that are contiguous along the output row.  The caller has synchronised the
 // workgroup after its last read of the operand tiles.
-template <int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
-__device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN][TM], char *smem, int m0, int n0, int wm, int wn,
-                                           int wave, int lane, long bz) {
+// The column bias of a wave's sub-tile, in the accumulator's order: cb[i][g] covers
+// n = n0 + wn*WTN + 32 i + 8 g + 4 (lane/32) .. +3.  Fetched by the kernels ahead of their last
+// k-step so that the epilogue does not start with a trip to memory.
+template <int TN, int WTN>
+__device__ __forceinline__ void load_col_bias(const GemmArgs &p, half4v (&cb)[TN][4], int n0, int wn, int lane, long bz) {
+    const half4v z = {(half_t)0.0f, (half_t)0.0f, (half_t)0.0f, (half_t)0.0f};
+    const bool on = p.bias_mode == MI_BIAS_COL;
+    const half_t *bias = on ? p.bias + bz * p.sBias : nullptr;
+    const bool vec = (reinterpret_cast<uintptr_t>(bias) & 7) == 0;
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const int n = n0 + wn * WTN + 32 * i + 8 * g + 4 * (lane >> 5);
+            cb[i][g] = z;
+            if (on) {
+                if (n + 3 < p.N && vec) cb[i][g] = *reinterpret_cast<const half4v *>(bias + n);
+                else for (int e = 0; e < 4; e++) if (n + e < p.N) cb[i][g][e] = bias[n + e];
+            }
+        }
+}
+
+template <int EPI, int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
+__device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], char *smem, int m0, int n0, int wm, int wn,
+                                               int wave, int lane, long bz) {
     const int frow = lane & 31;
     const half_t *bias = p.bias ? p.bias + bz * p.sBias : nullptr;
     constexpr int SLD_H = WTN + 8;                 // halves per staged row (fp16 output)
@@ -159,17 +181,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN
                 const int n = n0 + wn * WTN + nl;
                 float v[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + brow;
-                if (p.bias_mode == MI_BIAS_COL) {
-                    if (n + 3 < p.N) {
-                        half4v bv = *reinterpret_cast<const half4v *>(bias + n);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] += (float)bv[e];
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; e++) if (n + e < p.N) v[e] += (float)bias[n + e];
-                    }
-                }
+                for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + brow + (float)cb[i][g][e];
                 if (p.out_f32) {
                     float4v o = {v[0], v[1], v[2], v[3]};
                     *reinterpret_cast<float4v *>(reinterpret_cast<float *>(stage) + frow * SLD_F + nl) = o;
@@ -191,7 +203,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN
                     float4v x = *reinterpret_cast<const float4v *>(reinterpret_cast<const float *>(stage) + row * SLD_F + ch * 4);
                     float *yp = reinterpret_cast<float *>(p.Y) + bz * p.sY + (long)m * p.ldY + n;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) x[e] = apply_epi(x[e], p.epi);
+                    for (int e = 0; e < 4; e++) x[e] = apply_epi_c<EPI>(x[e]);
                     if (p.vec_store && n + 3 < p.N) *reinterpret_cast<float4v *>(yp) = x;
                     else for (int e = 0; e < 4; e++) if (n + e < p.N) yp[e] = x[e];
                 }
@@ -205,9 +217,9 @@ __device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN
                     half8v x = *reinterpret_cast<const half8v *>(reinterpret_cast<const half_t *>(stage) + row * SLD_H + ch * 8);
                     const long off = bz * p.sY + (long)m * p.ldY + n;
                     half_t *yp = reinterpret_cast<half_t *>(p.Y) + off;
-                    if (p.epi != MI_EPI_NONE) {
+                    if constexpr (EPI != MI_EPI_NONE) {
 #pragma unroll
-                        for (int e = 0; e < 8; e++) x[e] = (half_t)apply_epi((float)x[e], p.epi);
+                        for (int e = 0; e < 8; e++) x[e] = (half_t)apply_epi_c<EPI>((float)x[e]);
                     }
                     if (p.vec_store && n + 7 < p.N) {
                         if (p.residual) {
@@ -230,6 +242,19 @@ __device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     });
+}
+
+// The activation is a compile-time choice inside the store loops: one uniform branch per tile
+// instead of one per element.
+template <int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
+__device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], char *smem, int m0, int n0, int wm, int wn,
+                                           int wave, int lane, long bz) {
+    switch (p.epi) {
+    case MI_EPI_GELU_ERF: store_tile_epi<MI_EPI_GELU_ERF, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz); break;
+    case MI_EPI_GELU_TANH: store_tile_epi<MI_EPI_GELU_TANH, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz); break;
+    case MI_EPI_RELU: store_tile_epi<MI_EPI_RELU, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz); break;
+    default: store_tile_epi<MI_EPI_NONE, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz); break;
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -306,7 +331,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma_kernel(GemmAr
         __syncthreads();
     }
 
-    store_tile<TM, TN, WTM, WTN, WAVES_M * WAVES_N, 2 * (BM + BN) * LD * 2>(p, acc, smem, m0, n0, wm, wn, wave, lane, bz);
+    half4v cb[TN][4];
+    load_col_bias<TN, WTN>(p, cb, n0, wn, lane, bz);
+    store_tile<TM, TN, WTM, WTN, WAVES_M * WAVES_N, 2 * (BM + BN) * LD * 2>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -472,16 +499,19 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
         body(M0{}, kt, 0, 1, 0);
         body(M0{}, kt + 1, 1, 0, 1);
     }
+    half4v cb[TN][4];
     if (nk & 1) {
         body(M0{}, kt, 0, 1, 0);
         body(M1{}, kt + 1, 1, 0, 1);
+        load_col_bias<TN, WTN>(p, cb, n0, wn, lane, bz);
         body(M2{}, kt + 2, 0, 1, 0);
     } else {
         body(M1{}, kt, 0, 1, 0);
+        load_col_bias<TN, WTN>(p, cb, n0, wn, lane, bz);
         body(M2{}, kt + 1, 1, 0, 1);
     }
     __syncthreads();
-    store_tile<TM, TN, WTM, WTN, WAVES_M * WAVES_N, 2 * (BM * LD + BSZ) * 2>(p, acc, smem, m0, n0, wm, wn, wave, lane, bz);
+    store_tile<TM, TN, WTM, WTN, WAVES_M * WAVES_N, 2 * (BM * LD + BSZ) * 2>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz);
 }
 
 // ------------------------------------------------------------------------------------------
