@@ -539,24 +539,44 @@ __global__ void gemm_scalar_kernel(GemmArgs p, int b_kn) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Decode-sized M (<= 16): bandwidth-bound.  Every weight byte is read once with
-// 16-byte loads; K is split over workgroups so that the whole chip pulls on HBM;
-// each split writes an fp32 partial plane, and a small epilogue sums the planes
-// (the reference's split-K planes + mm_epilogue_kernel!, matmul.jl:192-217).
+// Decode-sized M (<= 8): bandwidth- and latency-bound.  Every weight byte is read once with
+// 16-byte loads, a thread's loads are all issued before the first is used, and the activations
+// (a few KB) are staged in LDS.  Products go through v_dot2_f32_f16: fp16 pairs, fp32 sum.
 //
-// KN layout: a thread owns 8 consecutive n; 32 threads span 256 n; the 8 thread
-// rows of a workgroup take interleaved k.  Row partials are reduced through LDS.
+// [K][F] weights: a thread owns 8 consecutive columns, 16 threads span 128 columns, the 16 thread
+// rows of a workgroup take interleaved k-pairs.  K is split over workgroups so that the whole chip
+// pulls on HBM; each split writes an fp32 partial plane and skinny_epilogue_kernel sums the planes
+// (the reference's split-K planes + mm_epilogue_kernel!, matmul.jl:192-217).
+constexpr int SKN_COLS = 128;      // columns per workgroup
+constexpr int SKN_KMAX = 256;      // deepest k-slice: 16 loads of 16 bytes per thread, all in flight at once
+constexpr int SKN_LOADS = SKN_KMAX / 32;
+
 template <int MT>
 __global__ __launch_bounds__(256) void skinny_kn_kernel(GemmArgs p, float *part, int kper) {
-    __shared__ float red[8][256 + 4];
-    __shared__ half_t xs[MT][512];   // the k-slice of A for this workgroup (kper <= 512)
-    const int tid = threadIdx.x, col = tid & 31, row = tid >> 5;
-    const int n = blockIdx.x * 256 + col * 8;
+    __shared__ __align__(16) half_t xs[MT][SKN_KMAX];
+    __shared__ float red[4][MT][SKN_COLS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cx = tid & 15, ky = tid >> 4;            // ky = 0..15: k-pairs 2 ky, 2 ky + 1 (+ 32 i)
+    const int n = blockIdx.x * SKN_COLS + cx * 8;
     const int split = blockIdx.y;
-    const int k0 = split * kper, k1 = min(p.K, k0 + kper);
-    for (int i = tid; i < MT * kper; i += 256) {
-        int m = i / kper, k = i % kper;
-        xs[m][k] = (m < p.M && k0 + k < p.K) ? p.A[(long)m * p.ldA + k0 + k] : (half_t)0.0f;
+    const int k0 = split * kper, klen = min(p.K - k0, kper);     // kper % 32 == 0, K % 8 == 0
+    // weights first: they are what the memory system has to deliver
+    u32x4 w[SKN_LOADS][2];
+    const bool ncol = n < p.N;                          // NB % 8 == 0: a thread's 8 columns are in the row or all past N
+    const half_t *bp = p.B + (long)k0 * p.ldB + n;
+#pragma unroll
+    for (int i = 0; i < SKN_LOADS; i++) {
+        const int k = 32 * i + 2 * ky;
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        if (32 * i < kper) {
+            w[i][0] = (ncol && k < klen) ? ldg16(bp + (long)k * p.ldB) : z;
+            w[i][1] = (ncol && k + 1 < klen) ? ldg16(bp + (long)(k + 1) * p.ldB) : z;
+        }
+    }
+    for (int c = tid; c < MT * (kper >> 3); c += 256) {
+        const int m = c / (kper >> 3), ch = c % (kper >> 3);
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        *reinterpret_cast<u32x4 *>(&xs[m][ch * 8]) = (m < p.M && ch * 8 < klen) ? ldg16(p.A + (long)m * p.ldA + k0 + ch * 8) : z;
     }
     __syncthreads();
     float acc[MT][8];
@@ -564,79 +584,126 @@ __global__ __launch_bounds__(256) void skinny_kn_kernel(GemmArgs p, float *part,
     for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[m][e] = 0.0f;
-    if (n < p.N) {
-        const half_t *bp = p.B + n;
-        for (int k = k0 + row; k < k1; k += 8) {
-            half8v w = as_half8(ldg16(bp + (long)k * p.ldB));
+#pragma unroll
+    for (int i = 0; i < SKN_LOADS; i++) {
+        if (32 * i < kper) {
+            const int k = 32 * i + 2 * ky;
+            // (w[k][n+e], w[k+1][n+e]) pairs
+            uint32_t pr[8];
+#pragma unroll
+            for (int q = 0; q < 4; q++) { pr[2 * q] = pack_lo(w[i][0][q], w[i][1][q]); pr[2 * q + 1] = pack_hi(w[i][0][q], w[i][1][q]); }
 #pragma unroll
             for (int m = 0; m < MT; m++) {
-                float x = (float)xs[m][k - k0];
+                const half2v x = *reinterpret_cast<const half2v *>(&xs[m][k]);
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[m][e] = fmaf(x, (float)w[e], acc[m][e]);
+                for (int e = 0; e < 8; e++) acc[m][e] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, pr[e]), x, acc[m][e], false);
             }
         }
     }
+    // a wave holds 4 thread rows of the same 16 column groups: fold them, then the 4 waves through LDS
 #pragma unroll
-    for (int m = 0; m < MT; m++) {
+    for (int m = 0; m < MT; m++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) red[row][col * 8 + e] = acc[m][e];
-        __syncthreads();
-        int nn = blockIdx.x * 256 + tid;
-        if (m < p.M && nn < p.N) {
-            float s = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 8; r++) s += red[r][tid];
-            part[((long)split * p.M + m) * p.N + nn] = s;
+        for (int e = 0; e < 8; e++) {
+            float v = acc[m][e];
+            v += __shfl_xor(v, 16, 64);
+            v += __shfl_xor(v, 32, 64);
+            if (lane < 16) red[wave][m][cx * 8 + e] = v;
         }
-        __syncthreads();
+    __syncthreads();
+    for (int c = tid; c < MT * SKN_COLS; c += 256) {
+        const int m = c / SKN_COLS, col = c % SKN_COLS;
+        const int nn = blockIdx.x * SKN_COLS + col;
+        if (m < p.M && nn < p.N) part[((long)split * p.M + m) * p.N + nn] = (red[0][m][col] + red[1][m][col]) + (red[2][m][col] + red[3][m][col]);
     }
 }
 
-// FK layout ([N][K], K-contiguous): one wave per output column n, lanes stride
-// K in 16-byte chunks, wave reduction.  No split needed: N waves fill the chip.
-template <int MT>
-__global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p, float *part) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n = blockIdx.x * 4 + wave;
-    if (n >= p.N) return;
-    const half_t *bp = p.B + (long)n * p.ldB;
-    float acc[MT];
-#pragma unroll
-    for (int m = 0; m < MT; m++) acc[m] = 0.0f;
-    for (int k = lane * 8; k < p.K; k += 512) {
-        half8v w = as_half8(ldg16(bp + k));
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            if (m < p.M) {
-                half8v x = as_half8(ldg16(p.A + (long)m * p.ldA + k));
-#pragma unroll
-                for (int e = 0; e < 8; e++) acc[m] = fmaf((float)x[e], (float)w[e], acc[m]);
-            }
-        }
-    }
-#pragma unroll
-    for (int m = 0; m < MT; m++) {
-        float s = acc[m];
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-        if (lane == 0 && m < p.M) part[(long)m * p.N + n] = s;
-    }
-}
-
-// out[m][n] = epi(round(sum_s part[s][m][n] + bias)) (+ residual)
+// out[m][n] = epi(round(sum_s part[s][m][n] + bias)) (+ residual).  A thread's plane loads are
+// issued eight at a time, so the sum costs a few memory round trips, not one per plane.
 __global__ void skinny_epilogue_kernel(GemmArgs p, const float *part, int nsplit) {
     long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     long total = (long)p.M * p.N;
     if (idx >= total) return;
     int n = (int)(idx % p.N), m = (int)(idx / p.N);
     float v = p.bias_mode == MI_BIAS_COL ? (float)p.bias[n] : p.bias_mode == MI_BIAS_ROW ? (float)p.bias[m] : 0.0f;
-    for (int s = 0; s < nsplit; s++) v += part[(long)s * total + idx];
+    int s = 0;
+    for (; s + 8 <= nsplit; s += 8) {
+        float t[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[j] = part[(long)(s + j) * total + idx];
+        v += ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
+    }
+    for (; s < nsplit; s++) v += part[(long)s * total + idx];
     long off = (long)m * p.ldY + n;
     if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(v, p.epi);
     else {
         half_t o = (half_t)apply_epi((float)(half_t)v, p.epi);
         if (p.residual) o = (half_t)((float)o + (float)p.residual[off]);
         reinterpret_cast<half_t *>(p.Y)[off] = o;
+    }
+}
+
+// [F][K] weights (K-contiguous): one wave per output column, lanes stride K in 16-byte chunks,
+// wave reduction, and the epilogue in the same launch: no workspace, no second kernel.  The
+// activations are staged in LDS once per workgroup (dynamic: MT rows of K halves).
+template <int MT>
+__global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p, int rows_per_wave) {
+    extern __shared__ __align__(16) char smem[];
+    half_t *xs = reinterpret_cast<half_t *>(smem);       // [MT][K]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kch = p.K >> 3;
+    for (int c = tid; c < MT * kch; c += 256) {
+        const int m = c / kch, ch = c % kch;
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        *reinterpret_cast<u32x4 *>(xs + (long)m * p.K + ch * 8) = m < p.M ? ldg16(p.A + (long)m * p.ldA + ch * 8) : z;
+    }
+    __syncthreads();
+    for (int r = 0; r < rows_per_wave; r++) {
+        const int n = (blockIdx.x * 4 + wave) * rows_per_wave + r;
+        if (n >= p.N) break;                              // uniform over the wave
+        const half_t *bp = p.B + (long)n * p.ldB;
+        float acc[MT];
+#pragma unroll
+        for (int m = 0; m < MT; m++) acc[m] = 0.0f;
+        for (int kb = lane * 8; kb < p.K; kb += 4 * 512) {
+            u32x4 w[4];
+            const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < 4; i++) w[i] = kb + 512 * i < p.K ? ldg16(bp + kb + 512 * i) : z;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (kb + 512 * i < p.K) {
+#pragma unroll
+                    for (int m = 0; m < MT; m++) {
+                        const u32x4 x = *reinterpret_cast<const u32x4 *>(xs + (long)m * p.K + kb + 512 * i);
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            const uint32_t wq = w[i][q], xq = x[q];     // bit_cast wants an addressable scalar, not a vector element
+                            acc[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, wq), __builtin_bit_cast(half2v, xq), acc[m], false);
+                        }
+                    }
+                }
+            }
+        }
+        float mine = 0.0f;                                // lane m keeps row m's sum
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            float sres = acc[m];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) sres += __shfl_xor(sres, o, 64);
+            if (lane == m) mine = sres;
+        }
+        if (lane < p.M) {
+            const int m = lane;
+            float v = mine + (p.bias_mode == MI_BIAS_COL ? (float)p.bias[n] : p.bias_mode == MI_BIAS_ROW ? (float)p.bias[m] : 0.0f);
+            const long off = (long)m * p.ldY + n;
+            if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(v, p.epi);
+            else {
+                half_t o = (half_t)apply_epi((float)(half_t)v, p.epi);
+                if (p.residual) o = (half_t)((float)o + (float)p.residual[off]);
+                reinterpret_cast<half_t *>(p.Y)[off] = o;
+            }
+        }
     }
 }
 
@@ -695,15 +762,18 @@ constexpr int gemm_lds_bytes() {
 #define GEMM_MID 128, 128, 64, 2, 2
 #define GEMM_SMALL 64, 64, 64, 2, 2
 
-int skinny_splits(int64_t K, int64_t F) {
-    // Enough workgroups to put ~2 on every CU, k-slices a multiple of 8 and <= 512.
-    int64_t colblocks = ceil_div(F, 256);
-    int64_t want = ceil_div(2 * (int64_t)g_cus, colblocks);
-    int64_t kper = round_up((size_t)ceil_div(K, want), 8);
-    if (kper < 32) kper = 32;
-    if (kper > 512) kper = 512;
-    return (int)ceil_div(K, kper);
+// k-slice depth for the [K][F] skinny kernel: enough workgroups to put ~2 on every CU, slices a
+// multiple of 32 within [64, SKN_KMAX].
+int skinny_kper(int64_t K, int64_t F) {
+    const int64_t colblocks = ceil_div(F, SKN_COLS);
+    const int64_t want = ceil_div(2 * (int64_t)g_cus, colblocks);
+    int64_t kper = (int64_t)round_up((size_t)ceil_div(K, want), 32);
+    if (kper < 64) kper = 64;
+    if (kper > SKN_KMAX) kper = SKN_KMAX;
+    return (int)kper;
 }
+int skinny_splits(int64_t K, int64_t F) { return (int)ceil_div(K, skinny_kper(K, F)); }
+constexpr size_t SKINNY_FK_LDS_MAX = 128 * 1024;    // activations of the [F][K] kernel: M rows of K halves
 
 bool mfma_addressable(const GemmArgs &a, bool b_kn) {
     if (a.K % 8 || a.ldA % 8 || a.ldB % 8 || a.sA % 8 || a.sB % 8) return false;
@@ -759,32 +829,38 @@ int splitk_count(int64_t M, int64_t N, int64_t K) {
 int gemm_path(const GemmArgs &a, bool b_kn, int64_t nbatch) {
     if (a.M < 1 || a.N < 1 || a.K < 1) return MI_GEMM_DECLINE;
     bool addr = mfma_addressable(a, b_kn);
-    if (a.M <= 8 && nbatch == 1 && addr) return MI_GEMM_SKINNY;
+    if (a.M <= 8 && nbatch == 1 && addr && (b_kn || (size_t)8 * a.K * sizeof(half_t) <= SKINNY_FK_LDS_MAX)) return MI_GEMM_SKINNY;
     if (addr) return MI_GEMM_MFMA;
     return MI_GEMM_SCALAR;
 }
 
 int run_skinny(GemmArgs a, bool b_kn, void *ws, size_t ws_bytes, hipStream_t st) {
-    int nsplit = b_kn ? skinny_splits(a.K, a.N) : 1;
-    size_t need = (size_t)nsplit * a.M * a.N * sizeof(float);
-    if (!ws || ws_bytes < need || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
-    float *part = reinterpret_cast<float *>(ws);
     if (b_kn) {
-        int kper = (int)round_up((size_t)ceil_div(a.K, nsplit), 8);
-        dim3 grid((unsigned)ceil_div(a.N, 256), (unsigned)nsplit);
+        const int kper = skinny_kper(a.K, a.N), nsplit = (int)ceil_div(a.K, kper);
+        size_t need = (size_t)nsplit * a.M * a.N * sizeof(float);
+        if (!ws || ws_bytes < need || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
+        float *part = reinterpret_cast<float *>(ws);
+        dim3 grid((unsigned)ceil_div(a.N, SKN_COLS), (unsigned)nsplit);
         if (a.M <= 1)      hipLaunchKernelGGL(skinny_kn_kernel<1>, grid, dim3(256), 0, st, a, part, kper);
+        else if (a.M <= 2) hipLaunchKernelGGL(skinny_kn_kernel<2>, grid, dim3(256), 0, st, a, part, kper);
         else if (a.M <= 4) hipLaunchKernelGGL(skinny_kn_kernel<4>, grid, dim3(256), 0, st, a, part, kper);
         else if (a.M <= 8) hipLaunchKernelGGL(skinny_kn_kernel<8>, grid, dim3(256), 0, st, a, part, kper);
         else return MI_DECLINE_EXTENT;
+        long total = (long)a.M * a.N;
+        hipLaunchKernelGGL(skinny_epilogue_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a, part, nsplit);
     } else {
-        dim3 grid((unsigned)ceil_div(a.N, 4));
-        if (a.M <= 1)      hipLaunchKernelGGL(skinny_fk_kernel<1>, grid, dim3(256), 0, st, a, part);
-        else if (a.M <= 4) hipLaunchKernelGGL(skinny_fk_kernel<4>, grid, dim3(256), 0, st, a, part);
-        else if (a.M <= 8) hipLaunchKernelGGL(skinny_fk_kernel<8>, grid, dim3(256), 0, st, a, part);
-        else return MI_DECLINE_EXTENT;
+        const int mt = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8;
+        const size_t lds = (size_t)mt * a.K * sizeof(half_t);
+        if (a.M > 8 || lds > SKINNY_FK_LDS_MAX) return MI_DECLINE_EXTENT;
+        // rows per wave: as many as still leave every CU a workgroup, at most eight (a workgroup stages
+        // all M activation rows once, whatever the number of weight rows it then streams)
+        int rpw = 1;
+        dim3 grid((unsigned)ceil_div(a.N, 4 * rpw));
+        if (mt == 1)      hipLaunchKernelGGL(skinny_fk_kernel<1>, grid, dim3(256), lds, st, a, rpw);
+        else if (mt == 2) hipLaunchKernelGGL(skinny_fk_kernel<2>, grid, dim3(256), lds, st, a, rpw);
+        else if (mt == 4) hipLaunchKernelGGL(skinny_fk_kernel<4>, grid, dim3(256), lds, st, a, rpw);
+        else              hipLaunchKernelGGL(skinny_fk_kernel<8>, grid, dim3(256), lds, st, a, rpw);
     }
-    long total = (long)a.M * a.N;
-    hipLaunchKernelGGL(skinny_epilogue_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a, part, nsplit);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
@@ -892,6 +968,10 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, false>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, true>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, false>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(skinny_fk_kernel<1>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<2>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<4>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<8>, (int)SKINNY_FK_LDS_MAX);
     bad |= mi_sdpa_init();
     if (bad) return MI_ERROR_DEVICE;
     g_ready = true;
@@ -918,8 +998,8 @@ size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int6
         const int split = splitk_count(T, F, K);
         return split > 1 ? round_up((size_t)split * T * F * sizeof(float), 256) : 0;
     }
-    int nsplit = w_layout == MI_W_KF ? skinny_splits(K, F) : 1;
-    return round_up((size_t)nsplit * T * F * sizeof(float), 256);
+    if (w_layout != MI_W_KF) return 0;      // the [F][K] skinny kernel finishes its outputs itself
+    return round_up((size_t)skinny_splits(K, F) * T * F * sizeof(float), 256);
 }
 
 int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,

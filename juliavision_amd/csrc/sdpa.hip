@@ -409,21 +409,38 @@ __global__ __launch_bounds__(256) void sdpa_rows_kernel(SdpaArgs p) {
 #pragma unroll
         for (int j = 0; j < 8; j++) acc[ci][j] = 0.0f;
 
-    for (int base = kbeg + wave * 8; base < kend; base += 32) {
-        // Every lane of the wave runs the same number of iterations (the shuffles
-        // below need all 64 lanes); a key past the end is computed on a clamped
-        // row and then given weight zero.
+    // Every lane of the wave runs the same number of iterations (the shuffles below need all 64
+    // lanes); a key past the end is computed on a clamped row and then given weight zero.  With
+    // 16-byte addressable operands the next iteration's K and V chunks are requested before the
+    // current ones are used, so a wave waits for memory once, not once per 8 keys.
+    u32x4 kc[NCH], vc[NCH];
+    auto fetch = [&](int base, u32x4 (&kx)[NCH], u32x4 (&vx)[NCH]) {
+        const int key = base + grp;
+        const int kk = key < kend ? key : kend - 1;
+        const half_t *kp = kb + (long)kk * p.ks[1], *vp = vb + (long)kk * p.vs[1];
+#pragma unroll
+        for (int ci = 0; ci < NCH; ci++) {
+            const int e0 = (cl + 8 * ci) * 8;
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            kx[ci] = e0 < p.E ? ldg16(kp + e0) : z;
+            vx[ci] = e0 < p.E ? ldg16(vp + e0) : z;
+        }
+    };
+    const int base0 = kbeg + wave * 8;
+    if (VEC && base0 < kend) fetch(base0, kc, vc);
+    for (int base = base0; base < kend; base += 32) {
         const int key = base + grp;
         const bool live = key < kend;
         const int kk = live ? key : kend - 1;
         const half_t *kp = kb + (long)kk * p.ks[1];
+        u32x4 kn[NCH], vn[NCH];
+        if (VEC && base + 32 < kend) fetch(base + 32, kn, vn);
         float d = 0.0f;
 #pragma unroll
         for (int ci = 0; ci < NCH; ci++) {
             const int e0 = (cl + 8 * ci) * 8;
             if (VEC) {
-                u32x4 z = {0u, 0u, 0u, 0u};
-                half8v t = as_half8(e0 < p.E ? ldg16(kp + e0) : z);
+                half8v t = as_half8(kc[ci]);
 #pragma unroll
                 for (int j = 0; j < 8; j++) d = fmaf(qv[ci][j], (float)t[j], d);
             } else {
@@ -452,8 +469,7 @@ __global__ __launch_bounds__(256) void sdpa_rows_kernel(SdpaArgs p) {
         for (int ci = 0; ci < NCH; ci++) {
             const int e0 = (cl + 8 * ci) * 8;
             if (VEC) {
-                u32x4 z = {0u, 0u, 0u, 0u};
-                half8v t = as_half8(e0 < p.E ? ldg16(vp + e0) : z);
+                half8v t = as_half8(vc[ci]);
 #pragma unroll
                 for (int j = 0; j < 8; j++) acc[ci][j] = fmaf(pw, (float)t[j], acc[ci][j] * al);
             } else {
@@ -463,6 +479,10 @@ __global__ __launch_bounds__(256) void sdpa_rows_kernel(SdpaArgs p) {
                     acc[ci][j] = fmaf(pw, vv, acc[ci][j] * al);
                 }
             }
+        }
+        if (VEC) {
+#pragma unroll
+            for (int ci = 0; ci < NCH; ci++) { kc[ci] = kn[ci]; vc[ci] = vn[ci]; }
         }
     }
 
@@ -525,14 +545,32 @@ __global__ void sdpa_merge_kernel(SdpaArgs p) {
     if (idx >= rows * p.E) return;
     const long row = idx / p.E;
     const int e = (int)(idx % p.E);
-    float mm = -INFINITY;
-    for (int s = 0; s < p.nsplit; s++) mm = fmaxf(mm, p.part_ml[((long)s * rows + row) * 2]);
-    const float mu = mm == -INFINITY ? 0.0f : mm;
-    float L = 0.0f, O = 0.0f;
-    for (int s = 0; s < p.nsplit; s++) {
-        const float a = __expf(p.part_ml[((long)s * rows + row) * 2] - mu);
-        L += a * p.part_ml[((long)s * rows + row) * 2 + 1];
-        O += a * p.part_o[((long)s * rows + row) * p.E + e];
+    // Splits are taken eight at a time with every load of a batch issued before the first is used;
+    // the running maximum is carried from batch to batch by the rescaling identity.
+    float mm = -INFINITY, L = 0.0f, O = 0.0f;
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        float ms[8], ls[8], os_[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int s = min(s0 + j, p.nsplit - 1);
+            const float2v ml = *reinterpret_cast<const float2v *>(p.part_ml + ((long)s * rows + row) * 2);
+            ms[j] = s0 + j < p.nsplit ? ml[0] : -INFINITY;
+            ls[j] = ml[1];
+            os_[j] = p.part_o[((long)s * rows + row) * p.E + e];
+        }
+        float mb = mm;
+#pragma unroll
+        for (int j = 0; j < 8; j++) mb = fmaxf(mb, ms[j]);
+        const float mu = mb == -INFINITY ? 0.0f : mb;
+        const float a0 = __expf(mm - mu);
+        L *= a0; O *= a0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float a = __expf(ms[j] - mu);     // a split past the end has m = -inf: weight 0
+            L += a * ls[j];
+            O += a * os_[j];
+        }
+        mm = mb;
     }
     const float r = L > 0.0f ? O / L : 0.0f;
     const long lq = row % p.Lq, hb = row / p.Lq, h = hb % p.H, b = hb / p.H;

@@ -73,7 +73,7 @@ def test_gemm_workspace():
     assert lib.mi_gemm_f16_workspace(1500, 1280, 5120, L.W_KF, 1) == 0
     n = lib.mi_gemm_f16_workspace(4, 1280, 1280, L.W_KF, 1)
     assert n > 0 and n % 256 == 0 and n % (4 * 1280 * 4) == 0
-    assert lib.mi_gemm_f16_workspace(4, 1280, 1280, L.W_FK, 1) == 4 * 1280 * 4
+    assert lib.mi_gemm_f16_workspace(4, 1280, 1280, L.W_FK, 1) == 0      # that kernel finishes its outputs itself
 
 
 def _sdpa_plan(E, Lq, Lk, H, B, *, bias=0, scale=0.125, qs=None, ptr=0x10000):
