@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, vendor figure
 # HBM bytes per launch of the dominant kernel (fc1 GEMM), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of `python bench.py --no-cpu --no-detail`, scaled by the same counters on a plain copy kernel of
 # known size (--calibrate-copy).
-FC1_TRAFFIC_BYTES = 57_309_184       # profiles/fc1_gemm_hbm_traffic.txt: FETCH 20 483 KiB x 2.000 + WRITE 15 000 KiB x 1.000
+FC1_TRAFFIC_BYTES = 57_253_949       # profiles/fc1_gemm_hbm_traffic.txt: FETCH 20 456 KiB x 2.000 + WRITE 15 000 KiB x 1.000
 
 
 def parse_args():
@@ -216,6 +216,53 @@ class EncoderBlock:
 
 # ----------------------------------------------------------------------------- other configs (detail)
 
+def decoder_layer_case(bsz, layout="kf", steps=200):
+    """One Whisper-decoder-shaped layer per token (d 1280, 20x64 heads, FFN 5120, self cache 448 with the
+    position at its end, cross cache 1500), weights in the reference's hoisted [K][F] layout: the eager step
+    (Python host + one launch per kernel) and the same step replayed as a captured graph."""
+    import time
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd.decode import DecodeBuffers, DecoderLayerWeights, KVCache, StepGraph, decoder_layer_step
+    d, H, E, ffn = 1280, 20, 64, 5120
+    ctx = jv.Ctx("cuda")
+    f16 = torch.float16
+    w = (lambda k, f: torch.randn((k, f), dtype=f16, device="cuda") * 0.02) if layout == "kf" else \
+        (lambda k, f: (torch.randn((f, k), dtype=f16, device="cuda") * 0.02).t())
+    v = lambda n, m=0.0: torch.randn((n,), dtype=f16, device="cuda") * 0.02 + m
+    W = DecoderLayerWeights(v(d, 1.0), v(d), w(d, 3 * d), v(3 * d), w(d, d), v(d), v(d, 1.0), v(d), w(d, d), v(d), w(d, d), v(d),
+                            v(d, 1.0), v(d), w(d, ffn), v(ffn), w(ffn, d), v(d))
+    cache = KVCache(1, bsz, H, E)
+    for t in (cache.self_k, cache.self_v, cache.cross_k, cache.cross_v):
+        t.normal_()
+    buf = DecodeBuffers(bsz, d, ffn)
+    x = torch.randn((bsz, d), dtype=f16, device="cuda")
+    y = torch.empty_like(x)
+
+    def step():
+        cache.advance(ctx)
+        decoder_layer_step(ctx, W, cache, 0, x, y, buf)
+
+    def timed(fn):
+        cache.length.fill_(447)                  # every step then attends the full 448-slot cache
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    eager = timed(step)
+    graph = StepGraph(step)
+    replay = timed(graph.replay)
+    weights = 2.0 * (3 * d * d + 3 * d * d + 2 * d * ffn)
+    kv = 2.0 * 2 * bsz * H * E * (448 + 1500)
+    return {"eager_us": round(eager * 1e6, 1), "graph_us": round(replay * 1e6, 1), "launches": 21 if layout == "kf" else 15,
+            "GB/s_graph": round((weights + kv) / replay / 1e9, 1), "frac_hbm_peak_graph": round((weights + kv) / replay / 1e9 / PEAK_HBM_GBS, 4)}
+
+
 def detail_benchmarks(lib, L, stream, only=None):
     import numpy as np
     import torch
@@ -320,6 +367,14 @@ def detail_benchmarks(lib, L, stream, only=None):
                 r = out[name]
                 r["frac_hbm_peak"] = round(r["kv_GB/s"] / PEAK_HBM_GBS, 4)
                 del r["TFLOP/s"], r["frac_mfma_peak"]
+
+    # config 5, whole decoder layer per token: the per-op dispatch the reference is bound by
+    # (~63 us per op, plans/whisper-decoder.md:161-166) against one graph launch of the same work
+    for bsz in (1, 4, 8):
+        for lay, tag in (("kf", "W[K][F]"), ("fk", "W[F][K]")):
+            name = f"c5_decoder_layer_b{bsz}_{tag}"
+            if only is None or only in name:
+                out[name] = decoder_layer_case(bsz, lay)
 
     # config 4: global attention at 4096 and the 3x3 conv
     attn_case("c4_attn_L4096_16x64", 1, 16, 4096, 4096, 64)

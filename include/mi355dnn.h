@@ -193,6 +193,30 @@ int mi_layernorm_f16(void *out, float *mean, float *rstd, const void *a,
  * (ops.jl:186-197), for callers that do not fold it into the GEMM store. */
 int mi_add_f16(void *out, const void *a, const void *b, int64_t n, void *stream);
 
+/* ---- decode-step cache maintenance ------------------------------------------
+ * The reference's decoder step is functional: the exported graph writes the new
+ * token's K/V with index_put, returns the whole cache through cat, and
+ * decodestep! copies ~18 MB back per token (WhisperRunner/src/decode.jl:186-203).
+ * These two calls replace that round trip with an in-place write driven by a
+ * device-resident length per batch row, the same int32 array mi_sdpa_f16 takes
+ * as kv_len -- so a step enqueues identical work whatever the position, and a
+ * captured graph of it can be replayed (the reference's Lava.capture/replay,
+ * plans/whisper-decoder.md:244-259).
+ *
+ * Order within a step: mi_kv_advance(+1) once, then per layer mi_kv_append_f16
+ * (writes slot kv_len[b]-1) and attention with kv_len.
+ *
+ * cache_k/cache_v: (E, Lmax, H, B) with element strides cache_strides, E contiguous.
+ * k_new/v_new: (E, 1, H, B) with element strides new_strides (the L stride is unused).
+ * A row whose kv_len is 0 or exceeds Lmax is left untouched. */
+int mi_kv_append_f16(void *cache_k, void *cache_v, const int64_t cache_strides[4], int64_t Lmax,
+                     const void *k_new, const void *v_new, const int64_t new_strides[4],
+                     const int32_t *kv_len, int64_t E, int64_t H, int64_t B, void *stream);
+
+/* kv_len[b] = clamp(kv_len[b] + delta, 0, cap) for b < B, on the device
+ * (KVCache.position += 1, decode.jl:201, without the host in the loop). */
+int mi_kv_advance(int32_t *kv_len, int64_t B, int32_t delta, int32_t cap, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

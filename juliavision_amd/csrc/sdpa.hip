@@ -72,7 +72,8 @@ __device__ __forceinline__ void static_for(F &&f) {
 //     same factor 2^-M -- with the rescaling of flash.jl:25-38 applied lazily (the
 //     reference's `lazyrescale`, flash.jl:1041-1096, skips it when no maximum grew;
 //     this skips it until fp16 would overflow);
-//   * row sums accumulate the fp16 probabilities pairwise with v_dot2_f32_f16.
+//   * row sums are plain fp32 adds of the probabilities: they overlap with the MFMAs of the
+//     other wave on the SIMD, which v_dot2_f32_f16 was measured not to do.
 //
 // PP ("ping-pong"): eight waves per workgroup, 256 queries.  Waves w and w+4 share a SIMD and are kept
 // half a key block apart by two workgroup barriers per block, so that while one of them is in its
@@ -97,8 +98,21 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     const int grp = wave >> 2;                               // PP: 0 = waves 0-3, 1 = waves 4-7
     const bool loader = !PP || grp == 0;
     const int hl = lane >> 5, l32 = lane & 31;
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int q0 = blockIdx.x * BR + wave * 32;
+    // Workgroups are dealt to the 8 XCDs round-robin in launch order; renumbering them so that each XCD
+    // owns a contiguous run keeps all query blocks of a head on one XCD, whose L2 then holds that head's
+    // K and V once instead of every XCD holding every head's.
+    int qblk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    {
+        const int nqb = gridDim.x, total = nqb * gridDim.y * gridDim.z;
+        if ((total & 7) == 0) {
+            int id = blockIdx.x + nqb * (blockIdx.y + gridDim.y * blockIdx.z);
+            id = (id & 7) * (total >> 3) + (id >> 3);
+            qblk = id % nqb;
+            h = (id / nqb) % gridDim.y;
+            b = id / (nqb * gridDim.y);
+        }
+    }
+    const int q0 = qblk * BR + wave * 32;
     const half_t *qb = p.q + h * p.qs[2] + b * p.qs[3];
     const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
     const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
@@ -195,7 +209,6 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
     const int vtoff = (4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
     const int ktoff = l32 * KLD + 8 * hl;
-    const half2v ones = {(half_t)1.0f, (half_t)1.0f};
     const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // t = s*scale*log2(e) - M, straight out of the MFMA chain
@@ -211,7 +224,8 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
             s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, s[kt], 0, 0, 0);
         }
     };
-    // p = 2^t as fp16 MFMA operands; the row sum takes the rounded values, pairwise
+    // p = 2^t as fp16 MFMA operands; the row sum is kept in fp32 with plain adds (v_dot2_f32_f16 on the
+    // packed pairs costs fewer instructions but does not run under MFMAs: measured 8 % slower)
     auto probs = [&](const float16v (&s)[2], half8v (&pf)[2][2], float &l) {
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
@@ -221,7 +235,7 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
                 const half2v pk = {(half_t)p0, (half_t)p1};
                 pf[kt][r >> 3][r & 7] = pk[0];
                 pf[kt][r >> 3][(r & 7) + 1] = pk[1];
-                l = __builtin_amdgcn_fdot2(pk, ones, l, false);
+                l += p0 + p1;
             }
     };
 
@@ -257,7 +271,7 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
 #pragma unroll
         for (int g = 0; g < 2 * KS + 2; g++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + 2), 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + 2), 0);     // the remaining vector work trails the last MFMA
         }
         __builtin_amdgcn_sched_barrier(0);
         // A probability that left fp16 range (t >= 16) shows up as an infinite row sum.  Then, and on
