@@ -56,7 +56,7 @@ enum mi_bias_mode { MI_BIAS_NONE = 0, MI_BIAS_COL = 1, MI_BIAS_ROW = 2 };
  * planner (the reference's `mmplan`, matmul.jl:87-95) can be tested without a launch. */
 enum mi_gemm_path { MI_GEMM_DECLINE = 0, MI_GEMM_MFMA = 1, MI_GEMM_SKINNY = 2, MI_GEMM_SCALAR = 3 };
 enum mi_sdpa_path { MI_SDPA_DECLINE = 0, MI_SDPA_FLASH = 1, MI_SDPA_ROWS = 2 };
-enum mi_conv_path { MI_CONV_DECLINE = 0, MI_CONV_GEMM_1X1 = 1, MI_CONV_IM2COL_GEMM = 2, MI_CONV_DIRECT = 3 };
+enum mi_conv_path { MI_CONV_DECLINE = 0, MI_CONV_GEMM_1X1 = 1, MI_CONV_IM2COL_GEMM = 2, MI_CONV_DIRECT = 3, MI_CONV_IMPLICIT_GEMM = 4 };
 
 /* Library / device. */
 int mi_version(void);
@@ -160,7 +160,10 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4],
  * on the rounded value.
  * Replaces convolution!(ctx, out, x, w, bias, stride, padding, dilation, groups; act)
  * -- conv.jl:100-145 -- and convolution_coopmat! / im2col_kernel! /
- * conv_epilogue_kernel! -- conv_coopmat.jl:246-392. */
+ * conv_epilogue_kernel! -- conv_coopmat.jl:246-392; the implicit-GEMM path (stride_x 1,
+ * OW % 8 == 0, Cin*KH*KW % 64 == 0) is the MFMA counterpart of conv2d_igemm! --
+ * conv_implicit.jl:53-355: the im2col matrix is never written, the GEMM gathers its
+ * operand from a zero-padded copy of x in the workspace. */
 int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
                   int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
                   int64_t KW, int64_t KH, int64_t Cout,

@@ -21,7 +21,7 @@ W_KF, W_FK = 0, 1
 BIAS_NONE, BIAS_COL, BIAS_ROW = 0, 1, 2
 GEMM_PATHS = {0: "decline", 1: "mfma", 2: "skinny", 3: "scalar"}
 SDPA_PATHS = {0: "decline", 1: "flash", 2: "rows"}
-CONV_PATHS = {0: "decline", 1: "gemm_1x1", 2: "im2col_gemm", 3: "direct"}
+CONV_PATHS = {0: "decline", 1: "gemm_1x1", 2: "im2col_gemm", 3: "direct", 4: "implicit_gemm"}
 
 _i64, _int, _vp, _sz, _f32 = C.c_int64, C.c_int, C.c_void_p, C.c_size_t, C.c_float
 _i64p = C.POINTER(C.c_int64)

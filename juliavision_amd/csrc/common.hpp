@@ -57,6 +57,21 @@ static inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cas
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline size_t round_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
 
+// Implicit-GEMM convolution: how the GEMM finds its [K][N] operand (the im2col matrix) in a
+// zero-padded copy of the input instead of in memory.  The K axis is ordered (kh, kw, ci) with ci
+// fastest (the weights are re-laid to match), so a 64-deep tile is 64 consecutive channels of one
+// tap: row k of the tile and column n = (oh, ow) is xp[img][ci0 + k][oh*sy + kh*dy][ow + kw*dx],
+// and eight consecutive columns of a row are eight consecutive halves of xp (stride 1 along x).
+struct ConvGather {
+    const half_t *xp;      // padded input [img][Cin][Hp][Wp]; nullptr = ordinary GEMM
+    long img;              // elements per image
+    long odd;              // xp[i] for odd i is also stored at xp[odd + i], a 4-byte aligned address: a second copy of
+                           // the padded input, one element to the left, follows the first
+    int HpWp, Wp, OW, sy, dyWp, dx, KW;
+    int cpt;               // 64-channel tiles per tap: Cin / 64
+    int split;             // 1: the launch's planes are K-slices of one image, 0: they are images
+};
+
 // True once mi_init has run successfully on this process (defined in gemm.hip).
 bool mi_ready();
 int mi_num_cus();
@@ -64,4 +79,5 @@ int mi_sdpa_init();
 // Y[M x N] = A[M x K] . B (+bias) with B either [K][NB-padded N] (b_kn) or [N][K]; defined in gemm.hip.
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
-                     long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st);
+                     long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st,
+                     const ConvGather *gather = nullptr);

@@ -50,6 +50,53 @@ __global__ void im2col_kernel(half_t *col, ConvArgs a, int PQP, int CRSP) {
     *reinterpret_cast<half8v *>(col + (long)n * PQP * CRSP + (long)c * PQP + m0) = val;
 }
 
+// xp[n][ci][Hp][Wp]: x with py rows of zeros above and below and px (and the round-up to a multiple
+// of 8) columns left and right; one 16-byte store per thread.  What the implicit-GEMM path reads.
+// The same launch re-lays the weights as w2[co][kh][kw][ci] (blocks past the padding work, image 0
+// only): the K order in which the implicit GEMM walks the taps.
+__global__ void conv_pad_kernel(half_t *xp, half_t *w2, ConvArgs a, int Hp, int Wp, int pad_blocks, long shifted) {
+    if ((int)blockIdx.x >= pad_blocks) {
+        if (blockIdx.y != 0) return;
+        // a thread gathers eight channels of one (co, tap) and stores them with one 16-byte write; with the tap
+        // as the fastest thread index a wave reads a dense stretch of the source
+        const int idx = (blockIdx.x - pad_blocks) * blockDim.x + threadIdx.x;
+        const int taps = a.KH * a.KW, c8s = a.Cin >> 3;
+        if (idx >= a.Cout * c8s * taps) return;
+        const int tap = idx % taps, t = idx / taps, c8 = t % c8s, co = t / c8s;
+        const half_t *src = a.w + ((long)co * a.Cin + c8 * 8) * taps + tap;
+        half8v v;
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = src[j * taps];
+        *reinterpret_cast<half8v *>(w2 + ((long)co * taps + tap) * a.Cin + c8 * 8) = v;
+        return;
+    }
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int cpr = Wp >> 3;
+    if (idx >= cpr * Hp * a.Cin) return;
+    const int n = blockIdx.y;
+    const int c8 = (idx % cpr) * 8, t = idx / cpr, yp = t % Hp, ci = t / Hp;
+    const int iy = yp - a.py;
+    // elements c8 .. c8+8 of the padded row: the first eight go to the copy proper, the last eight to the
+    // copy that sits one element to the left (its chunk at the same position)
+    half_t e[9];
+#pragma unroll
+    for (int j = 0; j < 9; j++) e[j] = (half_t)0.0f;
+    if (iy >= 0 && iy < a.Hi) {
+        const half_t *row = a.x + (((long)n * a.Cin + ci) * a.Hi + iy) * a.Wi;
+#pragma unroll
+        for (int j = 0; j < 9; j++) {
+            const int ix = c8 + j - a.px;
+            if (ix >= 0 && ix < a.Wi) e[j] = row[ix];
+        }
+    }
+    half8v v0, v1;
+#pragma unroll
+    for (int j = 0; j < 8; j++) { v0[j] = e[j]; v1[j] = e[j + 1]; }
+    const long at = (((long)n * a.Cin + ci) * Hp + yp) * Wp + c8;
+    *reinterpret_cast<half8v *>(xp + at) = v0;
+    *reinterpret_cast<half8v *>(xp + shifted + at) = v1;
+}
+
 // wp[co][CRSP] = w[co][CRS] zero-padded
 __global__ void padweight_kernel(half_t *wp, const half_t *w, int Cout, int CRS, int CRSP) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
@@ -112,10 +159,22 @@ int fill(ConvArgs &a, void *out, const void *x, const void *w, const void *bias,
     return MI_OK;
 }
 
+// Implicit GEMM needs eight consecutive output pixels to be eight consecutive input columns (stride 1
+// along x, OW a multiple of 8) and 64-deep K tiles that are 64 channels of one tap (Cin % 64 == 0).
+bool implicit_ok(const ConvArgs &a) {
+    return a.sx == 1 && a.OW % 8 == 0 && a.Cin % 64 == 0 && (long)a.Cin * a.KH * a.KW >= 128;
+}
+
 int conv_path(const ConvArgs &a) {
     if (a.groups != 1) return MI_CONV_DIRECT;
     if (onebyone(a)) return MI_CONV_GEMM_1X1;
+    if (implicit_ok(a)) return MI_CONV_IMPLICIT_GEMM;
     return MI_CONV_IM2COL_GEMM;
+}
+
+void padded_extents(const ConvArgs &a, int &Hp, int &Wp) {
+    Hp = a.Hi + 2 * a.py;
+    Wp = (int)round_up((size_t)(a.Wi + 2 * a.px), 8);
 }
 
 void im2col_extents(const ConvArgs &a, int64_t &PQP, int64_t &CRSP) {
@@ -141,6 +200,12 @@ size_t mi_conv2d_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, i
                                int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy) {
     ConvArgs a;
     if (fill(a, nullptr, nullptr, nullptr, nullptr, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, 1, MI_EPI_NONE) != MI_OK) return 0;
+    if (conv_path(a) == MI_CONV_IMPLICIT_GEMM) {
+        int Hp, Wp;
+        padded_extents(a, Hp, Wp);
+        return 2 * round_up((size_t)N * Cin * Hp * Wp * 2, 256) + round_up((size_t)Cout * Cin * KH * KW * 2, 256) +
+               mi_gemm_f16_workspace(Cout, Cin * KH * KW, (int64_t)a.OW * a.OH, MI_W_KF, N);
+    }
     if (conv_path(a) != MI_CONV_IM2COL_GEMM) return 0;
     int64_t PQP, CRSP;
     im2col_extents(a, PQP, CRSP);
@@ -173,6 +238,27 @@ int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
         // PQ % 8 == 0 for 16-byte loads, otherwise the scalar GEMM takes it.
         return mi_internal_gemm(out, w, x, bias, a.Cout, PQ, PQ, a.Cin, PQ, a.Cin, PQ, 1, MI_BIAS_ROW, epi, 0,
                                 a.N, (long)a.Cout * PQ, 0, (long)a.Cin * PQ, nullptr, 0, st);
+    }
+    if (path == MI_CONV_IMPLICIT_GEMM) {
+        int Hp, Wp;
+        padded_extents(a, Hp, Wp);
+        const int CRS = a.Cin * a.KH * a.KW;
+        const size_t xp1 = round_up((size_t)a.N * a.Cin * Hp * Wp * 2, 256), xp_bytes = 2 * xp1;     // the copy and its shifted twin
+        const size_t w2_bytes = round_up((size_t)a.Cout * CRS * 2, 256);
+        const size_t gemm_bytes = mi_gemm_f16_workspace(a.Cout, CRS, PQ, MI_W_KF, a.N);
+        if (!ws || ws_bytes < xp_bytes + w2_bytes + gemm_bytes || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
+        if ((long)a.Cin * Hp * Wp > INT32_MAX || (long)a.Cout * CRS > INT32_MAX) return MI_DECLINE_EXTENT;
+        half_t *xp = reinterpret_cast<half_t *>(ws);
+        half_t *w2 = reinterpret_cast<half_t *>(reinterpret_cast<char *>(ws) + xp_bytes);
+        const int pad_blocks = (int)ceil_div((int64_t)(Wp / 8) * Hp * a.Cin, 256), w_blocks = (int)ceil_div((int64_t)a.Cout * CRS / 8, 256);
+        hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)(pad_blocks + w_blocks), (unsigned)a.N), dim3(256), 0, st, xp, w2, a, Hp, Wp, pad_blocks, (long)(xp1 / 2));
+        if (hipGetLastError() != hipSuccess) return MI_ERROR_LAUNCH;
+        ConvGather g;
+        g.xp = xp; g.img = (long)a.Cin * Hp * Wp; g.odd = (long)(xp1 / 2) - 1; g.HpWp = Hp * Wp; g.Wp = Wp; g.OW = a.OW; g.sy = a.sy;
+        g.dyWp = a.dy * Wp; g.dx = a.dx; g.KW = a.KW; g.cpt = a.Cin / 64; g.split = 0;
+        // B is never dereferenced in this mode; xp stands in so that the operand checks see an aligned pointer
+        return mi_internal_gemm(out, w2, xp, bias, a.Cout, PQ, PQ, CRS, PQ, CRS, PQ, 1, MI_BIAS_ROW, epi, 0,
+                                a.N, (long)a.Cout * PQ, 0, 0, reinterpret_cast<char *>(ws) + xp_bytes + w2_bytes, gemm_bytes, st, &g);
     }
     int64_t PQP, CRSP;
     im2col_extents(a, PQP, CRSP);

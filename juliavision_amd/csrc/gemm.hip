@@ -21,6 +21,7 @@ struct GemmArgs {
     int bias_mode, epi, out_f32;
     int tiles_m, tiles_n, group_m;
     int vec_store;          // Y (and residual) rows allow 16-byte accesses
+    ConvGather cv;          // cv.xp != nullptr: B is the im2col matrix of a convolution, gathered on the fly
 };
 
 // ------------------------------------------------------------------------------------------
@@ -349,8 +350,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma_kernel(GemmAr
 // whole tile of MFMAs to land before its LDS write; the only barrier of a tile sits
 // where its successor's first fragment read can be hidden behind the last k-step.
 // Two waves per SIMD (8 waves on a 128 x 256 tile) cover each other's waits.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool B_KN>
+// BMODE: 0 = B is [N][K], 1 = B is [K][N], 2 = B is [K][N] gathered from a padded image (implicit-GEMM convolution).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BMODE>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(GemmArgs p) {
+    constexpr bool B_KN = BMODE != 0, CONV = BMODE == 2;
     constexpr int BK = 64, LD = BK + 8, NT = WAVES_M * WAVES_N * 64;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
     constexpr int PA = BM * 8 / NT, PB = BN * 8 / NT;     // 16-byte chunks per thread per tile
@@ -383,13 +386,41 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
         if (!B_KN) bp[i] = B + (long)min(n0 + (c >> 3), p.N - 1) * p.ldB + (c & 7) * 8;
         else       bp[i] = B + (long)(c / CPRB) * p.ldB + min(n0 + (c % CPRB) * 8, p.NB - 8);
     }
+    // Implicit GEMM: every chunk of this thread lies in the same eight columns (NT is a multiple of
+    // CPRB), i.e. at one pixel offset, in channels 16 apart; which tap and which 64 channels a tile
+    // covers is the same for the whole workgroup.
+    const half_t *cpix = nullptr;
+    int ctile0 = 0;
+    if constexpr (CONV) {
+        static_assert(NT % CPRB == 0 && NT / CPRB == 16, "a thread's chunks share their columns, 16 rows apart");
+        const int ncol = min(n0 + (tid % CPRB) * 8, p.NB - 8);
+        const int oh = ncol / p.cv.OW, ow = ncol % p.cv.OW;
+        cpix = p.cv.xp + (p.cv.split ? 0 : bz * p.cv.img) + (long)oh * p.cv.sy * p.cv.Wp + ow + (long)(tid / CPRB) * p.cv.HpWp;
+        ctile0 = p.cv.split ? (int)bz * (p.K / BK) : 0;
+    }
     u32x4 ga[2][PA], gb[2][PB];
     auto gload = [&](int set, int kt) {
         const long ko = (long)kt * BK;
 #pragma unroll
         for (int i = 0; i < PA; i++) ga[set][i] = ldg16(ap[i] + ko);
 #pragma unroll
-        for (int i = 0; i < PB; i++) gb[set][i] = ldg16(bp[i] + (B_KN ? ko * p.ldB : ko));
+        for (int i = 0; i < PB; i++) {
+            if constexpr (CONV) {
+                const int t = ctile0 + kt, tap = t / p.cv.cpt, ci0 = (t - tap * p.cv.cpt) * BK;
+                const int kh = tap / p.cv.KW, kw = tap - kh * p.cv.KW;
+                const int toff = ci0 * p.cv.HpWp + kh * p.cv.dyWp + kw * p.cv.dx;       // same for every lane
+                // The eight halves start kw*dx elements into an aligned row, i.e. at a 2-byte boundary, and
+                // vector loads want 4-byte alignment: odd starts are read from the second copy of the padded
+                // input, which is the first shifted by one element (the choice is the same for every lane).
+                const uint32_t *src = reinterpret_cast<const uint32_t *>(cpix + toff + ((toff & 1) ? p.cv.odd : 0L) + (long)i * 16 * p.cv.HpWp);
+                uint32_t w4[4];
+                __builtin_memcpy(w4, src, 16);
+#pragma unroll
+                for (int q = 0; q < 4; q++) gb[set][i][q] = w4[q];
+            } else {
+                gb[set][i] = ldg16(bp[i] + (B_KN ? ko * p.ldB : ko));
+            }
+        }
     };
     auto lwrite_a = [&](int set, int buf) {
 #pragma unroll
@@ -792,8 +823,9 @@ int launch_pipe(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
                             : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
     constexpr int lds = gemm_lds_bytes<BM, BN, 64>();
-    if (b_kn) hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, true>), grid, dim3(WM * WN * 64), lds, st, a);
-    else      hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, false>), grid, dim3(WM * WN * 64), lds, st, a);
+    if (a.cv.xp)   hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 2>), grid, dim3(WM * WN * 64), lds, st, a);
+    else if (b_kn) hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 1>), grid, dim3(WM * WN * 64), lds, st, a);
+    else           hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 0>), grid, dim3(WM * WN * 64), lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
@@ -883,6 +915,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.ldY = ldY; a.ldA = ldX; a.ldB = ldW; a.sY = sY; a.sA = sX; a.sB = sW; a.sBias = sBias;
     a.bias_mode = bias_mode; a.epi = epi; a.out_f32 = out_dtype == MI_F32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
+    a.cv = ConvGather{};
     return MI_OK;
 }
 
@@ -904,6 +937,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
             s1.ldY = a.N; s1.sY = (long)a.M * a.N;
             s1.K = a.K / split;
             s1.sA = s1.K; s1.sB = b_kn ? (long)s1.K * a.ldB : s1.K; s1.sBias = 0;
+            s1.cv.split = 1;
             int rc = launch_pipe<128, 128, 2, 2>(s1, b_kn, split, st);
             if (rc != MI_OK) return rc;
             GemmArgs s2 = a;
@@ -917,8 +951,9 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         int64_t big = ceil_div(a.M, 128) * ceil_div(a.N, 256) * nbatch;
         int64_t mid = ceil_div(a.M, 128) * ceil_div(a.N, 128) * nbatch;
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
+        if (a.cv.xp && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
         if (big >= (g_cus * 3) / 4) return pipe ? launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
-        if (mid >= (g_cus * 3) / 8) return pipe ? launch_pipe<128, 128, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
+        if (mid >= (g_cus * 3) / 8 || a.cv.xp) return pipe ? launch_pipe<128, 128, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
         return launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
     }
     long total = (long)a.M * a.N;
@@ -935,13 +970,18 @@ int mi_num_cus() { return g_cus; }
 // every GemmArgs field meaningful.
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
-                     long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st) {
+                     long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st,
+                     const ConvGather *gather) {
     GemmArgs a;
+    a.cv = ConvGather{};
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
-    int path = mfma_addressable(a, b_kn != 0) ? MI_GEMM_MFMA : MI_GEMM_SCALAR;
+    if (gather) a.cv = *gather;
+    const bool addr = mfma_addressable(a, b_kn != 0);
+    if (gather && !addr) return MI_DECLINE_OPERANDS;
+    int path = addr ? MI_GEMM_MFMA : MI_GEMM_SCALAR;
     return run_gemm(a, b_kn != 0, nbatch, ws, ws_bytes, st, path);
 }
 
@@ -968,6 +1008,8 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, false>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, true>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, false>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 2>, gemm_lds_bytes<128, 256, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, 2>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(skinny_fk_kernel<1>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<2>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<4>, (int)SKINNY_FK_LDS_MAX);

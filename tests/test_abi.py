@@ -107,16 +107,21 @@ def test_conv_planner_and_extents():
     lib = L.load()
     plan = lambda *a: L.CONV_PATHS[lib.mi_conv2d_f16_plan(*a)]
     assert plan(518, 518, 3, 1, 14, 14, 384, 14, 14, 0, 0, 1, 1, 1) == "im2col_gemm"
-    assert plan(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 1) == "im2col_gemm"
+    assert plan(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 1) == "implicit_gemm"   # stride 1, OW % 8 == 0, Cin % 64 == 0
+    assert plan(64, 64, 32, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 1) == "im2col_gemm"      # 32 channels do not fill a 64-deep tile
+    assert plan(60, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 1) == "im2col_gemm"     # OW = 60
     assert plan(256, 256, 144, 1, 1, 1, 256, 1, 1, 0, 0, 1, 1, 1) == "gemm_1x1"     # onebyone, conv.jl:63-66
     assert plan(256, 256, 144, 1, 1, 1, 256, 2, 2, 0, 0, 1, 1, 1) == "im2col_gemm"
     assert plan(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 4) == "direct"
     assert plan(64, 64, 255, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1, 4) == "decline"
     assert plan(2, 2, 3, 1, 5, 5, 8, 1, 1, 0, 0, 1, 1, 1) == "decline"              # empty output
     assert lib.mi_convsize(518, 14, 14, 0, 1) == 37 and lib.mi_convsize(256, 7, 4, 3, 1) == 64
-    # im2col scratch: col[CRS->8][PQ->8] fp16 (+ padded weights when CRS % 8 != 0)
+    # implicit GEMM scratch: the zero-padded input [Cin][H+2][W+2 -> 72] fp16 twice (the second copy shifted by one
+    # element, for taps that start at an odd column), the weights re-laid tap-major,
+    # four fp32 split-K planes of the 256 x 4096 output
     ws = lib.mi_conv2d_f16_workspace(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
-    assert ws == 2304 * 4096 * 2 + 4 * 256 * 4096 * 4           # col + four fp32 split-K planes of the 256 x 4096 output
+    assert ws == 2 * 256 * 66 * 72 * 2 + 256 * 2304 * 2 + 4 * 256 * 4096 * 4
+    # im2col scratch: col[CRS->8][PQ->8] fp16 (+ padded weights when CRS % 8 != 0)
     ws3 = lib.mi_conv2d_f16_workspace(518, 518, 3, 1, 14, 14, 384, 14, 14, 0, 0, 1, 1)
     assert ws3 == -(-(592 * 1376 * 2) // 256) * 256 + 384 * 592 * 2
     assert lib.mi_conv2d_f16_workspace(256, 256, 144, 1, 1, 1, 256, 1, 1, 0, 0, 1, 1) == 0

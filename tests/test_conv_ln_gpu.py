@@ -12,19 +12,22 @@ pytestmark = pytest.mark.gpu
 
 
 def _conv(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d=1, groups=1, bias=True, relu=False, expect=None, seed=1):
+    """``s``, ``p``, ``d``: one number for both axes or an ``(x, y)`` pair."""
     import torch
     import juliavision_amd as jv
+    pair = lambda v: v if isinstance(v, tuple) else (v, v)
+    s, p, d = pair(s), pair(p), pair(d)
     x = oracle.randn_f16((N, Cin, H, W), seed)
     w = oracle.randn_f16((Cout, Cin // groups, KH, KW), seed + 1, 0, 0.05)
     b = oracle.randn_f16((Cout,), seed + 2, 0, 0.5) if bias else None
-    want = oracle.conv2d_f16(x, w, b, (s, s), (p, p), (d, d), groups, relu)
+    want = oracle.conv2d_f16(x, w, b, s[::-1], p[::-1], d[::-1], groups, relu)      # the oracle takes (y, x) pairs as torch does
     out = poison(torch.empty(want.shape, dtype=torch.float16, device="cuda"))
     dx, dw = to_dev(x), to_dev(w)
-    plan = jv.conv_plan(ctx.dev, out, dx, dw, (s, s), (p, p), (d, d), groups)
+    plan = jv.conv_plan(ctx.dev, out, dx, dw, s, p, d, groups)
     if expect:
         assert plan.path == expect, plan
     ctx.ws.reset()
-    jv.convolution_(ctx, out, dx, dw, None if b is None else to_dev(b), (s, s), (p, p), (d, d), groups, act="relu" if relu else "none")
+    jv.convolution_(ctx, out, dx, dw, None if b is None else to_dev(b), s, p, d, groups, act="relu" if relu else "none")
     torch.cuda.synchronize()
     assert_parity(to_host(out), want, what=f"conv {N},{Cin},{H},{W}->{Cout} k{KH} s{s} p{p} g{groups}")
 
@@ -35,10 +38,22 @@ def _conv(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d=1, groups=1, bias=True, relu=
     (1, 7, 48, 48, 48, 5, 2, 2),
     (2, 32, 32, 32, 64, 3, 1, 1),
     (1, 3, 70, 70, 384, 14, 14, 0),    # patch embed 14x14 / stride 14 (config 3) on a 5x5 patch grid
-    (1, 256, 16, 16, 256, 3, 1, 1),    # config 4's 3x3 256->256 on a small map
 ])
 def test_conv_im2col(ctx, N, Cin, H, W, Cout, K, s, p):
     _conv(ctx, N, Cin, H, W, Cout, K, K, s, p, expect="im2col_gemm")
+
+
+@pytest.mark.parametrize("N,Cin,H,W,Cout,KH,KW,s,p,d,kw", [
+    (1, 256, 16, 16, 256, 3, 3, 1, 1, 1, {}),                      # config 4's 3x3 256->256 on a small map
+    (2, 64, 24, 24, 100, 3, 3, 1, 1, 1, {"relu": True}),           # two images, ragged Cout, relu
+    (1, 64, 40, 40, 64, 7, 7, 1, 3, 1, {"bias": False}),           # taps shifted by -3..3 columns: odd and even starts
+    (1, 128, 20, 24, 96, 5, 5, 1, (4, 2), (2, 1), {}),             # dilation 2 along x only, unequal padding
+    (1, 64, 18, 16, 48, 3, 1, (1, 2), (0, 1), 1, {}),              # 3 rows x 1 column, stride 2 along y, no x padding
+    (1, 192, 12, 32, 32, 1, 3, 1, (1, 0), 1, {}),                  # KH = 1, KW = 3
+    (3, 64, 9, 10, 40, 3, 3, 1, (0, 2), 1, {"relu": True}),        # OW = 8 without x padding, three images
+])
+def test_conv_implicit_gemm(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, kw):
+    _conv(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, expect="implicit_gemm", **kw)
 
 
 def test_conv_1x1_and_relu_and_nobias(ctx):
