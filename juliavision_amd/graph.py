@@ -1,0 +1,441 @@
+"""A minimal loader/executor for exported op graphs, dispatching to the MI355X kernels.
+
+The reference runs ``torch.export`` graphs serialised as JSON -- ``buffers``
+(``weight`` / ``external`` / ``transient`` / ``view`` / ``host``) and ``ops``
+(``aten`` name, ``in``, ``out``, ``attrs`` with positional constants as ``arg<j>``),
+written by ``tools/export_graphs.py:111-230`` and read by ``graph.jl:125-149`` --
+through one handler per ATen op (``runop!``, ``execute.jl:493-539``, ``ops.jl``).
+This module reads the same schema, keeps the handler-per-op shape, and covers
+the ops of the dense-contraction path:
+
+    linear / addmm / mm, scaled_dot_product_attention, layer_norm /
+    native_layer_norm, gelu, relu, add.Tensor, convolution, and the view ops
+    between them.
+
+Two of the reference's rewrites matter for that path and have counterparts here:
+
+* ``foldrelu.jl:60-125`` folds an activation into the producing ``addmm``'s
+  epilogue: ``fold_activations``.
+* ``hoistcasts.jl:47-112`` (``hoistpermutes``) pre-transposes ``addmm`` weights
+  at load time.  Nothing to hoist here: the GEMM reads ``[F][K]`` weights through
+  a transposed view (``MI_W_FK``), so the permute stays a view.
+
+and two more fall out of what the kernels accept: the residual ``add.Tensor``
+after a linear rides in its GEMM store (``fold_residuals``; the reference's own
+next item, plans/perf-plan.md:4074-4095), and attention writes its output
+token-major when the graph transposes it straight back (``fold_sdpa_transpose``).
+
+An op outside the list raises :class:`UnsupportedOp`; there is no eager fallback.
+``convert`` produces the schema from an ``ExportedProgram`` (static shapes only),
+so a graph can be built and run without the reference's tooling.
+"""
+from __future__ import annotations
+
+import json
+import math
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+import torch
+
+from . import kernels as K
+
+VIEW_OPS = {"view.default", "_unsafe_view.default", "reshape.default", "transpose.int", "permute.default", "t.default",
+            "unsqueeze.default", "squeeze.dim", "expand.default", "alias.default", "detach.default", "slice.Tensor",
+            "select.int", "flatten.using_ints", "unflatten.int", "contiguous.default"}
+DROP_OPS = {"_assert_tensor_metadata.default", "_assert_scalar.default", "sym_constrain_range_for_size.default"}
+LINEAR_OPS = {"linear.default", "addmm.default", "mm.default"}
+ACTIVATIONS = {"gelu.default": "gelu", "relu.default": "relu"}
+
+
+class UnsupportedOp(NotImplementedError):
+    """An ATen op with no kernel on this path (the reference would route it to one of its other kernels)."""
+
+
+# ----------------------------------------------------------------------------- schema
+
+def _const(x):
+    if isinstance(x, float) and not math.isfinite(x):
+        return "-inf" if x < 0 else ("inf" if x > 0 else "nan")
+    if isinstance(x, (int, float, bool, str)) or x is None:
+        return x
+    if isinstance(x, (list, tuple)):
+        return [_const(v) for v in x]
+    if isinstance(x, torch.dtype):
+        return str(x).replace("torch.", "")
+    if isinstance(x, torch.device):
+        return None
+    return str(x)
+
+
+def convert(ep, name: str = "graph") -> Dict[str, Any]:
+    """``ExportedProgram`` -> the buffers/ops dictionary (the schema of export_graphs.py:111-230, static
+    shapes).  Parameters and buffers become ``weight`` buffers keyed by their state-dict name, user inputs
+    and outputs ``external``, view ops ``view`` buffers that alias their parent, everything else an op
+    with a ``transient`` result and a ``live`` interval in op indices."""
+    import torch.fx as fx
+    sig = ep.graph_signature
+    key_of = dict(sig.inputs_to_parameters)
+    key_of.update(sig.inputs_to_buffers)
+    key_of.update(getattr(sig, "inputs_to_lifted_tensor_constants", {}))
+    buffers: Dict[str, Dict[str, Any]] = {}
+    ops: List[Dict[str, Any]] = []
+    inputs, outputs = [], []
+    born, last = {}, {}
+
+    def describe(nid, val, kind, **extra):
+        b = {"id": nid, "kind": kind}
+        if isinstance(val, (tuple, list)):
+            b["shapes"] = [list(v.shape) if hasattr(v, "shape") else None for v in val]
+            b["dtypes"] = [str(v.dtype).replace("torch.", "") if hasattr(v, "dtype") else None for v in val]
+        elif val is not None and hasattr(val, "shape"):
+            b["shape"] = [int(d) for d in val.shape]
+            b["dtype"] = str(val.dtype).replace("torch.", "")
+        b.update(extra)
+        buffers[nid] = b
+
+    for n in ep.graph.nodes:
+        if n.op == "placeholder":
+            if n.name in key_of:
+                describe(n.name, n.meta.get("val"), "weight", key=key_of[n.name])
+            else:
+                describe(n.name, n.meta.get("val"), "external")
+                inputs.append(n.name)
+        elif n.op == "call_function":
+            target = str(n.target).replace("aten.", "")
+            if target in DROP_OPS:
+                continue
+            at = len(ops)
+            args, attrs = [], {}
+            for j, a in enumerate(n.args):
+                if isinstance(a, fx.Node):
+                    args.append(a.name)
+                    last[a.name] = at
+                elif isinstance(a, (list, tuple)) and any(isinstance(v, fx.Node) for v in a):
+                    for v in a:
+                        if isinstance(v, fx.Node):
+                            args.append(v.name)
+                            last[v.name] = at
+                    attrs[f"arg{j}"] = [f"${v.name}" if isinstance(v, fx.Node) else _const(v) for v in a]
+                else:
+                    attrs[f"arg{j}"] = _const(a)
+            for k, v in n.kwargs.items():
+                if isinstance(v, fx.Node):
+                    args.append(v.name)
+                    last[v.name] = at
+                else:
+                    attrs[k] = _const(v)
+            val = n.meta.get("val")
+            born[n.name] = at
+            if "getitem" in target or target in VIEW_OPS:
+                describe(n.name, val, "view", of=args[0] if args else None, op=target, attrs=attrs)
+                continue
+            describe(n.name, val, "transient")
+            ops.append({"id": n.name, "aten": target, "in": args, "out": n.name,
+                        "attrs": {k: v for k, v in attrs.items() if v is not None}})
+        elif n.op == "output":
+            flat = n.args[0] if isinstance(n.args[0], (list, tuple)) else [n.args[0]]
+            outputs += [a.name for a in flat if isinstance(a, fx.Node)]
+    for bid, b in buffers.items():
+        if b["kind"] == "transient":
+            if bid in outputs:
+                b["kind"] = "external"
+            else:
+                b["live"] = [born.get(bid, 0), last.get(bid, len(ops))]
+    return {"name": name, "symbols": [], "inputs": inputs, "outputs": outputs, "buffers": list(buffers.values()),
+            "ops": ops, "fusion_groups": [], "barriers": []}
+
+
+@dataclass
+class Graph:
+    """The parsed form (GraphSpec, graph.jl:125-149): buffers by id, ops in order."""
+    name: str
+    inputs: List[str]
+    outputs: List[str]
+    buffers: Dict[str, Dict[str, Any]]
+    ops: List[Dict[str, Any]]
+    notes: List[str] = field(default_factory=list)      # what the rewrites did, for inspection
+
+    @classmethod
+    def load(cls, src) -> "Graph":
+        d = json.load(open(src)) if isinstance(src, str) else src
+        if d.get("symbols"):
+            raise UnsupportedOp(f"graph {d.get('name')}: symbolic extents {d['symbols']} (this executor is static-shape)")
+        return cls(d["name"], list(d["inputs"]), list(d["outputs"]), {b["id"]: dict(b) for b in d["buffers"]},
+                   [dict(o, attrs=dict(o.get("attrs", {}))) for o in d["ops"]])
+
+    # -- queries the rewrites share
+    def root(self, bid: str) -> str:
+        """The buffer a chain of views bottoms out in."""
+        while self.buffers[bid]["kind"] == "view":
+            bid = self.buffers[bid]["of"]
+        return bid
+
+    def readers(self, bid: str) -> List[str]:
+        """Ops and views that take ``bid`` as an input."""
+        r = [o["id"] for o in self.ops if bid in o["in"]]
+        r += [b["id"] for b in self.buffers.values() if b["kind"] == "view" and b.get("of") == bid]
+        return r
+
+    def op(self, oid: str) -> Optional[Dict[str, Any]]:
+        return next((o for o in self.ops if o["id"] == oid), None)
+
+
+# ----------------------------------------------------------------------------- rewrites
+
+def fold_activations(g: Graph) -> Graph:
+    """gelu / relu whose only producer is a linear op read by nothing else becomes that op's epilogue
+    (foldrelu.jl:60-125); the activation's buffer then aliases the linear's output."""
+    for act in [o for o in g.ops if o["aten"] in ACTIVATIONS]:
+        if act["aten"] == "gelu.default" and act["attrs"].get("approximate", "none") != "none":
+            continue                                    # only the erf form is the folded epilogue's arithmetic
+        src = act["in"][0]
+        prod = g.op(src)
+        if prod is None or prod["aten"] not in LINEAR_OPS or g.readers(src) != [act["id"]] or src in g.outputs:
+            continue
+        prod["attrs"]["epilogue"] = ACTIVATIONS[act["aten"]]
+        g.ops.remove(act)
+        g.buffers[act["id"]].update(kind="view", of=src, op="alias.default", attrs={})
+        g.notes.append(f"fold {act['aten']} into {prod['id']}")
+    return g
+
+
+def fold_residuals(g: Graph) -> Graph:
+    """``add.Tensor(x, y)`` where one side is (a view chain of) a linear op's output that nothing else reads:
+    the add moves into that GEMM's store, after the activation, with its own rounding -- bit-identical to
+    the separate op."""
+    for add in [o for o in g.ops if o["aten"] == "add.Tensor"]:
+        if add["attrs"].get("alpha", 1) != 1 or len(add["in"]) != 2:
+            continue
+        for mine, other in (add["in"], add["in"][::-1]):
+            chain = [mine]
+            while g.buffers[chain[-1]]["kind"] == "view":
+                chain.append(g.buffers[chain[-1]]["of"])
+            prod = g.op(chain[-1])
+            single = all(len(g.readers(c)) == 1 for c in chain) and not any(c in g.outputs for c in chain)
+            if prod is None or prod["aten"] not in LINEAR_OPS or not single or "residual" in prod["attrs"]:
+                continue
+            if g.buffers[other].get("shape") != g.buffers[mine].get("shape") or other == mine:
+                continue
+            # the other operand must exist before the GEMM runs
+            if g.op(g.root(other)) is not None and g.ops.index(g.op(g.root(other))) > g.ops.index(prod):
+                continue
+            prod["attrs"]["residual"] = "$" + other
+            prod["in"].append(other)
+            g.ops.remove(add)
+            g.buffers[add["id"]].update(kind="view", of=mine, op="alias.default", attrs={})
+            if add["id"] in g.outputs:                 # the GEMM's result is now what the caller gets
+                g.buffers[chain[-1]]["kind"] = "external"
+            g.notes.append(f"fold add {add['id']} into {prod['id']}")
+            break
+    return g
+
+
+def fold_sdpa_transpose(g: Graph) -> Graph:
+    """Attention whose only reader swaps the head and token axes back (``transpose(1, 2)`` /
+    ``permute(0, 2, 1, 3)``): the kernel writes token-major, the swap becomes the view it already is, and
+    the ``reshape`` that follows is a free view instead of a copy."""
+    for o in g.ops:
+        if o["aten"] != "scaled_dot_product_attention.default":
+            continue
+        rd = g.readers(o["id"])
+        if len(rd) != 1 or g.buffers[rd[0]]["kind"] != "view":
+            continue
+        v = g.buffers[rd[0]]
+        swap = (v["op"] == "transpose.int" and sorted(x % 4 for x in (v["attrs"].get("arg1"), v["attrs"].get("arg2"))) == [1, 2]) or \
+               (v["op"] == "permute.default" and [x % 4 for x in v["attrs"].get("arg1", [])] == [0, 2, 1, 3])
+        if swap:
+            o["attrs"]["token_major"] = True
+            g.notes.append(f"{o['id']} writes token-major")
+    return g
+
+
+def optimize(g: Graph) -> Graph:
+    return fold_sdpa_transpose(fold_residuals(fold_activations(g)))
+
+
+# ----------------------------------------------------------------------------- execution
+
+_DTYPES = {"float16": torch.float16, "float32": torch.float32, "int64": torch.int64, "int32": torch.int32, "bool": torch.bool}
+
+
+class Executor:
+    """Binds a graph to weights and a context and runs it op by op (Model / call, execute.jl:493-539).
+    Transient buffers are allocated once at construction; nothing is allocated per run."""
+
+    def __init__(self, graph: Graph, weights: Dict[str, torch.Tensor], ctx: Optional[K.Ctx] = None, device="cuda"):
+        self.g = graph
+        self.ctx = ctx if ctx is not None else K.Ctx(device)
+        self.device = torch.device(device)
+        self.t: Dict[str, torch.Tensor] = {}
+        for b in graph.buffers.values():
+            if b["kind"] == "weight":
+                w = weights[b["key"]]
+                if list(w.shape) != list(b["shape"]):
+                    raise ValueError(f"weight {b['key']}: shape {tuple(w.shape)} but the graph declares {b['shape']}")
+                self.t[b["id"]] = w.to(self.device, _DTYPES[b["dtype"]]).contiguous()
+        for o in graph.ops:                               # check every op has a handler before anything runs
+            if o["aten"] not in self.HANDLERS:
+                raise UnsupportedOp(f"{graph.name}: no kernel on this path for aten.{o['aten']} (op {o['id']})")
+        for o in graph.ops:
+            b = graph.buffers[o["out"]]
+            if "shape" not in b:
+                continue
+            shape = list(b["shape"])
+            if o["attrs"].get("token_major"):             # (B, H, L, E) stored as (B, L, H, E)
+                self.t[o["out"]] = torch.empty([shape[0], shape[2], shape[1], shape[3]], dtype=_DTYPES[b["dtype"]],
+                                               device=self.device).transpose(1, 2)
+            else:
+                self.t[o["out"]] = torch.empty(shape, dtype=_DTYPES[b["dtype"]], device=self.device)
+
+    # -- operands
+    def get(self, bid: str) -> torch.Tensor:
+        if bid in self.t:
+            return self.t[bid]
+        b = self.g.buffers[bid]
+        if b["kind"] != "view":
+            raise KeyError(f"buffer {bid} ({b['kind']}) has no value yet")
+        return self._view(b)
+
+    def _view(self, b) -> torch.Tensor:
+        src, a, op = self.get(b["of"]), b.get("attrs", {}), b["op"]
+        if "getitem" in op:
+            if a.get("arg1", 0) != 0:
+                raise UnsupportedOp(f"{b['id']}: only the first result of a multi-result op is kept")
+            return src
+        if op in ("view.default", "_unsafe_view.default", "reshape.default"):
+            want = list(a["arg1"])
+            try:
+                return src.view(want)
+            except RuntimeError:
+                raise UnsupportedOp(f"{b['id']}: reshape of {tuple(src.shape)} strides {src.stride()} to {want} needs a copy")
+        if op == "transpose.int":
+            return src.transpose(a["arg1"], a["arg2"])
+        if op == "permute.default":
+            return src.permute(a["arg1"])
+        if op == "t.default":
+            return src.t()
+        if op == "unsqueeze.default":
+            return src.unsqueeze(a["arg1"])
+        if op == "squeeze.dim":
+            return src.squeeze(a["arg1"])
+        if op == "expand.default":
+            return src.expand(a["arg1"])
+        if op in ("alias.default", "detach.default"):
+            return src
+        if op == "contiguous.default":
+            if not src.is_contiguous():
+                raise UnsupportedOp(f"{b['id']}: contiguous() of a strided tensor needs a copy")
+            return src
+        if op == "slice.Tensor":
+            dim, lo, hi, step = a.get("arg1", 0), a.get("arg2"), a.get("arg3"), a.get("arg4", 1)
+            idx = [slice(None)] * src.dim()
+            idx[dim] = slice(lo, None if hi is None or hi >= 2 ** 62 else hi, step)
+            return src[tuple(idx)]
+        if op == "select.int":
+            return src.select(a["arg1"], a["arg2"])
+        if op == "flatten.using_ints":
+            return src.flatten(a.get("arg1", 0), a.get("arg2", -1))
+        if op == "unflatten.int":
+            return src.unflatten(a["arg1"], a["arg2"])
+        raise UnsupportedOp(f"view op {op}")
+
+    @staticmethod
+    def _rows(t: torch.Tensor) -> torch.Tensor:
+        """(..., K) -> (T, K) without a copy."""
+        if t.dim() == 2:
+            return t
+        try:
+            return t.view(-1, t.shape[-1])
+        except RuntimeError:
+            raise UnsupportedOp(f"linear over a tensor of shape {tuple(t.shape)} strides {t.stride()} needs a copy")
+
+    # -- handlers (runop!, ops.jl)
+    def _linear(self, o):
+        at, ins, attrs = o["aten"], o["in"], o["attrs"]
+        res_id = attrs["residual"][1:] if "residual" in attrs else None
+        ins = ins[:-1] if res_id else ins                # fold_residuals appended it last
+        if at == "linear.default":                       # (x, weight[F,K], bias?)
+            x, w = self.get(ins[0]), self.get(ins[1]).t()
+            bias = self.get(ins[2]) if len(ins) > 2 else None
+        elif at == "addmm.default":                      # (bias, x, w[K,F]); ops.jl:1347-1363
+            if attrs.get("beta", 1) != 1 or attrs.get("alpha", 1) != 1:
+                raise UnsupportedOp(f"{o['id']}: addmm with beta/alpha other than 1")
+            bias, x, w = self.get(ins[0]), self.get(ins[1]), self.get(ins[2])
+        else:                                            # mm (x, w[K,F])
+            x, w, bias = self.get(ins[0]), self.get(ins[1]), None
+        out = self.t[o["out"]]
+        res = self._rows(self.get(res_id)) if res_id else None
+        self.ctx.ws.reset()
+        K.matmul_(self.ctx, self._rows(out), w, self._rows(x), bias, epi=attrs.get("epilogue", "none"), residual=res)
+
+    def _sdpa(self, o):
+        a = o["attrs"]
+        if a.get("is_causal") or a.get("dropout_p", 0.0) not in (0, 0.0) or a.get("enable_gqa"):
+            raise UnsupportedOp(f"{o['id']}: causal flag / dropout / gqa are not exported on this path (masks arrive as attn_mask)")
+        q, k, v = (self.get(i) for i in o["in"][:3])
+        bias = self.get(o["in"][3]) if len(o["in"]) > 3 else None
+        self.ctx.ws.reset()
+        K.sdpa(self.ctx, q, k, v, bias, a.get("scale"), out=self.t[o["out"]])
+
+    def _layer_norm(self, o):
+        ins, a = o["in"], o["attrs"]
+        x = self.get(ins[0])
+        shape = a["arg1"]
+        if len(shape) != 1 or shape[0] != x.shape[-1]:
+            raise UnsupportedOp(f"{o['id']}: layer_norm over {shape} (only the last axis)")
+        gamma = self.get(ins[1]) if len(ins) > 1 else None
+        beta = self.get(ins[2]) if len(ins) > 2 else None
+        eps = a.get("arg4", a.get("eps", 1e-5))
+        K.layernorm_(self.ctx, self.t[o["out"]], None, None, x, gamma, beta, x.shape[-1], eps)
+
+    def _native_layer_norm(self, o):
+        ins, a = o["in"], o["attrs"]
+        x = self.get(ins[0])
+        shape = a["arg1"]
+        if len(shape) != 1 or shape[0] != x.shape[-1]:
+            raise UnsupportedOp(f"{o['id']}: layer_norm over {shape} (only the last axis)")
+        b = self.g.buffers[o["out"]]
+        if o["out"] not in self.t:                        # multi-result: only the normalised tensor is materialised
+            self.t[o["out"]] = torch.empty(b["shapes"][0], dtype=_DTYPES[b["dtypes"][0]], device=self.device)
+        K.layernorm_(self.ctx, self.t[o["out"]], None, None, x, self.get(ins[1]) if len(ins) > 1 else None,
+                     self.get(ins[2]) if len(ins) > 2 else None, x.shape[-1], a.get("arg4", 1e-5))
+
+    def _add(self, o):
+        if o["attrs"].get("alpha", 1) != 1 or len(o["in"]) != 2:
+            raise UnsupportedOp(f"{o['id']}: add with a scalar operand or alpha")
+        a, b = self.get(o["in"][0]), self.get(o["in"][1])
+        if a.shape != b.shape:
+            raise UnsupportedOp(f"{o['id']}: broadcasting add {tuple(a.shape)} + {tuple(b.shape)}")
+        K.add_(self.ctx, self.t[o["out"]], a, b)
+
+    def _activation(self, o):
+        raise UnsupportedOp(f"{o['id']}: a stand-alone {o['aten']} (run optimize() so that it folds into its linear)")
+
+    def _convolution(self, o):
+        a, ins = o["attrs"], o["in"]
+        x, w = self.get(ins[0]), self.get(ins[1])
+        bias = self.get(ins[2]) if len(ins) > 2 else None
+        stride, padding, dilation = a["arg3"], a["arg4"], a["arg5"]
+        if a.get("arg6") or any(a.get("arg7", [0, 0])):
+            raise UnsupportedOp(f"{o['id']}: transposed convolution")
+        self.ctx.ws.reset()
+        K.convolution_(self.ctx, self.t[o["out"]], x, w, bias, tuple(stride[::-1]), tuple(padding[::-1]), tuple(dilation[::-1]), a.get("arg8", 1))
+
+    HANDLERS = {"linear.default": _linear, "addmm.default": _linear, "mm.default": _linear,
+                "scaled_dot_product_attention.default": _sdpa, "layer_norm.default": _layer_norm,
+                "native_layer_norm.default": _native_layer_norm, "add.Tensor": _add,
+                "gelu.default": _activation, "relu.default": _activation, "convolution.default": _convolution}
+
+    def __call__(self, *inputs: torch.Tensor):
+        if len(inputs) != len(self.g.inputs):
+            raise ValueError(f"{self.g.name} takes {len(self.g.inputs)} inputs")
+        for bid, x in zip(self.g.inputs, inputs):
+            b = self.g.buffers[bid]
+            if list(x.shape) != list(b["shape"]) or x.dtype != _DTYPES[b["dtype"]] or not x.is_cuda:
+                raise ValueError(f"input {bid}: expected cuda {b['dtype']} {b['shape']}")
+            self.t[bid] = x
+        for o in self.g.ops:
+            self.HANDLERS[o["aten"]](self, o)
+        outs = [self.get(bid) for bid in self.g.outputs]
+        return outs[0] if len(outs) == 1 else outs

@@ -1,0 +1,147 @@
+"""The exported-graph loader/executor: schema conversion and rewrites on the CPU, execution on the GPU against
+the same module evaluated by torch in fp32 (the module's own arithmetic, independent of this library)."""
+import json
+
+import numpy as np
+import pytest
+
+from util import assert_parity
+
+
+def _block(d=128, heads=2, ffn=256, seed=0):
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+
+    class Block(nn.Module):
+        """A pre-LN encoder block written the way the exported models are: separate q/k/v linears (k without bias,
+        as in Whisper), SDPA on (B, H, T, E) views, GELU MLP, two residual adds."""
+
+        def __init__(self):
+            super().__init__()
+            self.h = heads
+            self.ln1, self.ln2 = nn.LayerNorm(d), nn.LayerNorm(d)
+            self.q, self.k, self.v, self.o = nn.Linear(d, d), nn.Linear(d, d, bias=False), nn.Linear(d, d), nn.Linear(d, d)
+            self.fc1, self.fc2 = nn.Linear(d, ffn), nn.Linear(ffn, d)
+
+        def forward(self, x):
+            B, T, D = x.shape
+            y = self.ln1(x)
+            sp = lambda t: t.view(B, T, self.h, D // self.h).transpose(1, 2)
+            a = F.scaled_dot_product_attention(sp(self.q(y)), sp(self.k(y)), sp(self.v(y)))
+            x = x + self.o(a.transpose(1, 2).reshape(B, T, D))
+            return x + self.fc2(F.gelu(self.fc1(self.ln2(x))))
+
+    torch.manual_seed(seed)
+    m = Block().eval()
+    with torch.no_grad():
+        for p in m.parameters():
+            if p.dim() == 1:
+                p.copy_(torch.randn_like(p) * 0.1 + (1.0 if p is m.ln1.weight or p is m.ln2.weight else 0.0))
+    return m.half()
+
+
+def _export(m, T=70, d=128):
+    import torch
+    x = torch.randn(1, T, d).half()
+    return torch.export.export(m, (x,)), x
+
+
+def test_convert_writes_the_reference_schema():
+    from juliavision_amd import graph as G
+    m = _block()
+    ep, _ = _export(m)
+    d = G.convert(ep, "block")
+    json.loads(json.dumps(d))                                         # plain JSON
+    assert set(d) >= {"name", "symbols", "inputs", "outputs", "buffers", "ops", "fusion_groups", "barriers"}
+    kinds = {b["id"]: b["kind"] for b in d["buffers"]}
+    assert d["inputs"] == ["x"] and kinds["x"] == "external" and kinds[d["outputs"][0]] == "external"
+    weights = [b for b in d["buffers"] if b["kind"] == "weight"]
+    assert {b["key"] for b in weights} == set(m.state_dict())
+    assert kinds["view"] == "view" and kinds["transpose"] == "view"
+    aten = [o["aten"] for o in d["ops"]]
+    assert aten.count("linear.default") == 6 and aten.count("scaled_dot_product_attention.default") == 1
+    assert aten.count("layer_norm.default") == 2 and aten.count("gelu.default") == 1 and aten.count("add.Tensor") == 2
+    lin = next(o for o in d["ops"] if o["id"] == "linear")
+    assert lin["in"] == ["layer_norm", "p_q_weight", "p_q_bias"] and lin["out"] == "linear"
+    tr = next(b for b in d["buffers"] if b["id"] == "transpose")
+    assert tr["of"] == "view" and tr["op"] == "transpose.int" and tr["attrs"]["arg1"] == 1 and tr["attrs"]["arg2"] == 2
+    live = next(b for b in d["buffers"] if b["id"] == "layer_norm")["live"]
+    assert live[0] == 0 and live[1] == aten.index("scaled_dot_product_attention.default") - 1   # last read by the v projection
+
+
+def test_rewrites_fold_activation_residuals_and_attention_layout():
+    from juliavision_amd import graph as G
+    ep, _ = _export(_block())
+    g = G.optimize(G.Graph.load(G.convert(ep, "block")))
+    aten = [o["aten"] for o in g.ops]
+    assert "gelu.default" not in aten and "add.Tensor" not in aten
+    fc1 = g.op("linear_4")
+    assert fc1["attrs"]["epilogue"] == "gelu" and g.buffers["gelu"]["kind"] == "view" and g.buffers["gelu"]["of"] == "linear_4"
+    assert g.op("linear_3")["attrs"]["residual"] == "$x" and g.op("linear_5")["attrs"]["residual"] == "$add"
+    assert g.op("scaled_dot_product_attention")["attrs"]["token_major"] is True
+    assert len(g.ops) == 9                                              # 2 LN + 6 linears + attention
+    assert g.root("add_1") == "linear_5" and len(g.notes) == 4
+    # an activation that something else also reads must stay where it is
+    d = G.convert(ep, "block")
+    d["outputs"].append("linear_4")
+    g2 = G.fold_activations(G.Graph.load(d))
+    assert any(o["aten"] == "gelu.default" for o in g2.ops)
+
+
+def test_unsupported_op_is_named():
+    import torch
+    from juliavision_amd import graph as G
+
+    class M(torch.nn.Module):
+        def forward(self, x):
+            return torch.softmax(x, -1)
+
+    ep = torch.export.export(M(), (torch.randn(2, 8).half(),))
+    g = G.Graph.load(G.convert(ep, "m"))
+    assert [o["aten"] for o in g.ops] == ["softmax.int"]
+    assert "softmax.int" not in G.Executor.HANDLERS
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fold", [True, False])
+def test_exported_block_runs_on_the_kernels(ctx, fold):
+    import torch
+    from juliavision_amd import graph as G
+    m = _block(seed=3)
+    ep, x = _export(m)
+    g = G.Graph.load(G.convert(ep, "block"))
+    if fold:
+        g = G.optimize(g)
+    else:
+        g = G.fold_sdpa_transpose(G.fold_activations(g))          # residual adds stay separate ops
+        assert sum(o["aten"] == "add.Tensor" for o in g.ops) == 2
+    run = G.Executor(g, m.state_dict(), ctx)
+    with torch.no_grad():
+        want = m.float()(x.float()).numpy()
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    assert_parity(got.float().cpu().numpy(), want, what=f"exported block fold={fold}")
+    x2 = torch.randn_like(x)                                       # same executor, new input: nothing is cached
+    with torch.no_grad():
+        want2 = m(x2.float()).numpy()
+    assert_parity(run(x2.cuda()).float().cpu().numpy(), want2, what="second call")
+
+
+@pytest.mark.gpu
+def test_executor_refuses_what_it_cannot_run(ctx):
+    import torch
+    from juliavision_amd import graph as G
+
+    class M(torch.nn.Module):
+        def forward(self, x):
+            return torch.softmax(x, -1)
+
+    ep = torch.export.export(M(), (torch.randn(2, 8).half(),))
+    with pytest.raises(G.UnsupportedOp, match="softmax"):
+        G.Executor(G.Graph.load(G.convert(ep, "m")), {}, ctx)
+    ep2, _ = _export(_block())
+    g = G.fold_activations(G.Graph.load(G.convert(ep2, "block")))   # attention output still needs a copy for its reshape
+    run = G.Executor(g, _block().state_dict(), ctx)
+    with pytest.raises(G.UnsupportedOp, match="needs a copy"):
+        run(torch.randn(1, 70, 128).half().cuda())
