@@ -97,8 +97,11 @@ int mi_gemm_f16_batched(void *Y, const void *X, const void *W, const void *bias,
                         int64_t nbatch, int64_t sY, int64_t sX, int64_t sW, int64_t sBias,
                         void *ws, size_t ws_bytes, void *stream);
 
-/* Decode-sized T (<= 16): the bandwidth-bound form, split over K across
- * workgroups with fp32 partial planes in ws and a reducing epilogue.
+/* Decode-sized T (<= 8; more declines with MI_DECLINE_EXTENT): the
+ * bandwidth-bound form.  [K][F] weights: K split across workgroups, fp32
+ * partial planes in ws, a reducing epilogue (ws from mi_gemm_f16_workspace).
+ * [F][K] weights: one launch, no workspace.  mi_gemm_f16 takes the same route
+ * by itself for T <= 8; this entry forces it.
  * The reference's counterpart is the fp32-only Lava.gemv! path
  * (matmul.jl:108-137) and mm_epilogue_kernel! (matmul.jl:192-217). */
 int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,

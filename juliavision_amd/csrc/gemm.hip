@@ -938,7 +938,9 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
             s1.K = a.K / split;
             s1.sA = s1.K; s1.sB = b_kn ? (long)s1.K * a.ldB : s1.K; s1.sBias = 0;
             s1.cv.split = 1;
-            int rc = launch_pipe<128, 128, 2, 2>(s1, b_kn, split, st);
+            // the 128 x 256 tile (two waves per SIMD) when the slices still give most CUs a workgroup
+            const bool big_tiles = ceil_div(a.M, 128) * ceil_div(a.N, 256) * split >= (g_cus * 3) / 4;
+            int rc = big_tiles ? launch_pipe<128, 256, 2, 4>(s1, b_kn, split, st) : launch_pipe<128, 128, 2, 2>(s1, b_kn, split, st);
             if (rc != MI_OK) return rc;
             GemmArgs s2 = a;
             s2.vec_store = !a.out_f32 && a.ldY % 4 == 0 && aligned_to(a.Y, 8);

@@ -50,6 +50,25 @@ def test_gemm_no_bias_row_bias_residual(ctx):
     _run(ctx, 4, 128, 136, residual=True, epi="gelu")
 
 
+@pytest.mark.parametrize("layout", ["kf", "fk"])
+@pytest.mark.parametrize("T,K,F", [
+    (1, 8, 8), (2, 72, 136), (3, 264, 200), (5, 1288, 392), (6, 4104, 128), (7, 640, 1032), (8, 2048, 136),
+])
+def test_decode_sized_rows_ragged_extents(ctx, T, K, F, layout):
+    """T <= 8 takes the bandwidth kernels: K not a multiple of their 32- and 512-deep strides, F not a multiple of
+    their 128-column blocks, every row count their templates round up from."""
+    import juliavision_amd as jv
+    import torch
+    W = torch.zeros((K, F), dtype=torch.float16, device="cuda")
+    W = W if layout == "kf" else torch.zeros((F, K), dtype=torch.float16, device="cuda").t()
+    plan = jv.mmplan(ctx.dev, torch.zeros((T, F), dtype=torch.float16, device="cuda"), W, torch.zeros((T, K), dtype=torch.float16, device="cuda"))
+    assert type(plan).__name__ == "MMSkinnyPlan"
+    _run(ctx, T, K, F, layout=layout, seed=40 + T)
+    _run(ctx, T, K, F, layout=layout, epi="gelu", residual=True, seed=50 + T)
+    _run(ctx, T, K, F, layout=layout, bias=False, out_f32=True, seed=60 + T)
+    _run(ctx, T, K, F, layout=layout, bias_mode="row", epi="relu", seed=70 + T)
+
+
 def test_gemm_unaligned_takes_scalar_path(ctx):
     import juliavision_amd as jv
     import torch
