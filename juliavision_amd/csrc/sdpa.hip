@@ -112,12 +112,25 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
             b = id / (nqb * gridDim.y);
         }
     }
+    // Key splits (small grids only): the x index carries (query block, split); a split walks a run of whole
+    // key blocks and leaves (O, M, l) partials for sdpa_merge_kernel instead of the normalised output.
+    const int split = PP ? 0 : qblk % p.nsplit;
+    if (!PP) qblk /= p.nsplit;
     const int q0 = qblk * BR + wave * 32;
     const half_t *qb = p.q + h * p.qs[2] + b * p.qs[3];
     const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
     const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
     int Lk = p.Lk;
     if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
+    int LkLoad = p.Lk;                 // keys that exist in memory (rows past it are re-reads of the last one)
+    if (!PP && p.nsplit > 1) {
+        const int per = (((p.Lk + BC - 1) / BC + p.nsplit - 1) / p.nsplit) * BC;      // keys per split, whole blocks
+        const int kbeg = split * per;
+        kb += (long)kbeg * p.ks[1];
+        vb += (long)kbeg * p.vs[1];
+        Lk = max(0, min(Lk - kbeg, per));
+        LkLoad = max(1, min(p.Lk - kbeg, per));
+    }
     const float c = p.scale * LOG2E;
     // barrier between the half-block intervals of the ping-pong: LDS traffic of this wave done, nothing else waited for
     auto pp_barrier = [&]() {
@@ -127,16 +140,17 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     };
 
     // Q^T fragments: column = query l32, k = head-dim 16 ks + 8 hl .. +7, times scale*log2(e)
+    // (requested here, scaled after the first two key blocks have been requested as well: the workgroup's
+    // start-up then costs one trip to memory, not three)
     half8v qf[KS];
+    u32x4 qraw[KS];
     {
         const int qr = min(q0 + l32, p.Lq - 1);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             const int e = 16 * ks + 8 * hl;
             u32x4 z = {0u, 0u, 0u, 0u};
-            half8v t = as_half8(e < p.E ? ldg16(qb + (long)qr * p.qs[1] + e) : z);
-#pragma unroll
-            for (int j = 0; j < 8; j++) qf[ks][j] = (half_t)((float)t[j] * c);
+            qraw[ks] = e < p.E ? ldg16(qb + (long)qr * p.qs[1] + e) : z;
         }
     }
 
@@ -154,35 +168,37 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
         kp0[i] = kb + (long)row * p.ks[1] + (eok[i] ? ch * 8 : 0);
         vp0[i] = vb + (long)row * p.vs[1] + (eok[i] ? ch * 8 : 0);
     }
-    auto load_kv = [&](int key0) {
+    auto load_into = [&](u32x4 (&kx)[PER], u32x4 (&vx)[PER], int key0) {
         const u32x4 z = {0u, 0u, 0u, 0u};
-        if (key0 + BC <= p.Lk && p.E == EP) {     // the common case: no predicate, no clamp
+        if (key0 + BC <= LkLoad && p.E == EP) {   // the common case: no predicate, no clamp
             const long ko = (long)key0 * p.ks[1], vo = (long)key0 * p.vs[1];
 #pragma unroll
             for (int i = 0; i < PER; i++) {
-                kr[i] = ldg16(kp0[i] + ko);
-                vr[i] = ldg16(vp0[i] + vo);
+                kx[i] = ldg16(kp0[i] + ko);
+                vx[i] = ldg16(vp0[i] + vo);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < PER; i++) {
                 const int cidx = tid + i * NT;
                 const int row = cidx / KCH, ch = cidx % KCH;
-                const int key = min(key0 + row, p.Lk - 1);
-                kr[i] = eok[i] ? ldg16(kb + (long)key * p.ks[1] + ch * 8) : z;
-                vr[i] = eok[i] ? ldg16(vb + (long)key * p.vs[1] + ch * 8) : z;
+                const int key = min(key0 + row, LkLoad - 1);
+                kx[i] = eok[i] ? ldg16(kb + (long)key * p.ks[1] + ch * 8) : z;
+                vx[i] = eok[i] ? ldg16(vb + (long)key * p.vs[1] + ch * 8) : z;
             }
         }
     };
-    auto store_kv = [&](int buf) {
+    auto store_from = [&](const u32x4 (&kx)[PER], const u32x4 (&vx)[PER], int buf) {
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int cidx = tid + i * NT;
             const int row = cidx / KCH, ch = cidx % KCH;
-            *reinterpret_cast<u32x4 *>(&Ks[buf][row * KLD + ch * 8]) = kr[i];
-            *reinterpret_cast<u32x4 *>(&Vs[buf][row * VLD + ch * 8]) = vr[i];
+            *reinterpret_cast<u32x4 *>(&Ks[buf][row * KLD + ch * 8]) = kx[i];
+            *reinterpret_cast<u32x4 *>(&Vs[buf][row * VLD + ch * 8]) = vx[i];
         }
     };
+    auto load_kv = [&](int key0) { load_into(kr, vr, key0); };
+    auto store_kv = [&](int buf) { store_from(kr, vr, buf); };
 
     float16v o_acc[ET];
 #pragma unroll
@@ -202,8 +218,19 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     // product of block j+1 already runs (its MFMAs fill the matrix pipe under the
     // exponentials), and block j+2 is on its way from memory into the third stage.
     const int nblk = (Lk + BC - 1) / BC;
-    if (nblk > 0 && loader) { load_kv(0); store_kv(0); }
-    if (nblk > 1 && loader) { load_kv(BC); store_kv(1); }
+    {
+        u32x4 kr1[PER], vr1[PER];
+        if (nblk > 0 && loader) load_kv(0);
+        if (nblk > 1 && loader) load_into(kr1, vr1, BC);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const half8v t = as_half8(qraw[ks]);
+#pragma unroll
+            for (int j = 0; j < 8; j++) qf[ks][j] = (half_t)((float)t[j] * c);
+        }
+        if (nblk > 0 && loader) store_kv(0);
+        if (nblk > 1 && loader) store_from(kr1, vr1, 1);
+    }
     __syncthreads();
 
     // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
@@ -350,28 +377,75 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     // Both lanes of a query hold half of its row sum.
     l_run += __shfl_xor(l_run, 32, 64);
 
-    // out(e, q, h, b); lane owns query q0 + l32 and, per tile t and group g, the
-    // four head-dim values e = 32 t + 8 g + 4 hl + 0..3
-    const int qi = q0 + l32;
-    if (qi < p.Lq) {
-        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-        const long base = (long)b * p.os[3] + (long)h * p.os[2] + (long)qi * p.os[1];
+    // out(e, q, h, b); lane owns query q0 + l32 and, per tile t and group g, the four head-dim values
+    // e = 32 t + 8 g + 4 hl + 0..3: stored from the registers, a wave's store instruction would touch 32 rows
+    // with 16 or 32 bytes each.  Instead each wave lays its 32 x E tile out in its own stretch of the (now
+    // idle) operand LDS and reads it back row-wise, so that every store instruction covers whole rows.
+    // A wave reads only what it wrote itself and its LDS operations complete in order: no workgroup barrier.
+    const bool partial = !PP && p.nsplit > 1;
+    const bool as_f32 = partial || p.out_f32;
+    constexpr int SLF = EP + 4, SLH = EP + 8;              // staged row lengths (floats, halves)
+    float *stf = reinterpret_cast<float *>(smem) + wave * 32 * SLF;
+    half_t *sth = reinterpret_cast<half_t *>(smem) + wave * 32 * SLH;
+    const float inv = partial ? 1.0f : (l_run > 0.0f ? 1.0f / l_run : 0.0f);
+    const long rows = (long)p.B * p.H * p.Lq;
+    if (partial && hl == 0 && q0 + l32 < p.Lq) {
+        // the reference point in natural-log units (it was kept in the base-2 domain), -inf for a split without a key
+        const long row = ((long)b * p.H + h) * p.Lq + q0 + l32;
+        float2v ml = {l_run > 0.0f ? m_ref * 0.6931471805599453f : -INFINITY, l_run};
+        *reinterpret_cast<float2v *>(p.part_ml + ((long)split * rows + row) * 2) = ml;
+    }
+    if (PP && as_f32) {
+        // eight waves of fp32 rows do not fit the operand LDS: this combination stores from the registers
+        const int qi = q0 + l32;
+        if (qi < p.Lq) {
+            const long base = (long)b * p.os[3] + (long)h * p.os[2] + (long)qi * p.os[1];
 #pragma unroll
-        for (int t = 0; t < ET; t++)
+            for (int t = 0; t < ET; t++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int e = 32 * t + 8 * g + 4 * hl;
-                if (e < p.E) {      // E is a multiple of 8, so e..e+3 are all valid
-                    if (p.out_f32) {
+                for (int g = 0; g < 4; g++) {
+                    const int e = 32 * t + 8 * g + 4 * hl;
+                    if (e < p.E) {
                         float4v o = {o_acc[t][4 * g] * inv, o_acc[t][4 * g + 1] * inv, o_acc[t][4 * g + 2] * inv, o_acc[t][4 * g + 3] * inv};
                         *reinterpret_cast<float4v *>(reinterpret_cast<float *>(p.out) + base + e) = o;
-                    } else {
-                        half4v o = {(half_t)(o_acc[t][4 * g] * inv), (half_t)(o_acc[t][4 * g + 1] * inv),
-                                    (half_t)(o_acc[t][4 * g + 2] * inv), (half_t)(o_acc[t][4 * g + 3] * inv)};
-                        *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(p.out) + base + e) = o;
                     }
                 }
+        }
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < ET; t++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const int e = 32 * t + 8 * g + 4 * hl;
+            if (as_f32) {
+                float4v o = {o_acc[t][4 * g] * inv, o_acc[t][4 * g + 1] * inv, o_acc[t][4 * g + 2] * inv, o_acc[t][4 * g + 3] * inv};
+                *reinterpret_cast<float4v *>(stf + l32 * SLF + e) = o;
+            } else {
+                half4v o = {(half_t)(o_acc[t][4 * g] * inv), (half_t)(o_acc[t][4 * g + 1] * inv),
+                            (half_t)(o_acc[t][4 * g + 2] * inv), (half_t)(o_acc[t][4 * g + 3] * inv)};
+                *reinterpret_cast<half4v *>(sth + l32 * SLH + e) = o;
             }
+        }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (as_f32) {
+        constexpr int CPR = EP / 4;                        // 16-byte chunks per row
+        float *dst0 = partial ? p.part_o + ((long)split * rows + ((long)b * p.H + h) * p.Lq) * p.E
+                              : reinterpret_cast<float *>(p.out) + (long)b * p.os[3] + (long)h * p.os[2];
+        const long rstride = partial ? p.E : p.os[1];
+        for (int c = lane; c < 32 * CPR; c += 64) {
+            const int row = c / CPR, e = (c % CPR) * 4;
+            if (q0 + row < p.Lq && e < p.E)
+                *reinterpret_cast<float4v *>(dst0 + (long)(q0 + row) * rstride + e) = *reinterpret_cast<const float4v *>(stf + row * SLF + e);
+        }
+    } else {
+        constexpr int CPR = EP / 8;
+        half_t *dst0 = reinterpret_cast<half_t *>(p.out) + (long)b * p.os[3] + (long)h * p.os[2];
+        for (int c = lane; c < 32 * CPR; c += 64) {
+            const int row = c / CPR, e = (c % CPR) * 8;
+            if (q0 + row < p.Lq && e < p.E)
+                *reinterpret_cast<u32x4 *>(dst0 + (long)(q0 + row) * p.os[1] + e) = *reinterpret_cast<const u32x4 *>(sth + row * SLH + e);
+        }
     }
 }
 
@@ -613,6 +687,23 @@ int rows_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     return (int)want;
 }
 
+// Key splits for the fused kernel.  A workgroup spends about 1 us per 64-key block plus 3 us of start-up,
+// and the merge is a second launch of about 6 us, so splitting pays only when the query blocks leave most
+// of the chip idle and every split still walks a dozen blocks (config 3's 66 workgroups x 22 blocks do
+// not: 21.9 us unsplit, 21.1 us at best split three ways).
+int flash_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    const int64_t wgs = ceil_div(Lq, 128) * H * B, cus = mi_num_cus();
+    if (wgs * 2 > cus) return 1;
+    int64_t want = ceil_div(cus * 3 / 2, wgs);
+    const int64_t blocks = ceil_div(Lk, 64);
+    if (want > blocks / 12) want = blocks / 12;
+    if (want > 16) want = 16;
+    if (want < 2) return 1;
+    // no empty split: with `per` blocks each, the last one must still start inside the keys
+    while (want > 1 && ceil_div(blocks, want) * (want - 1) >= blocks) want--;
+    return (int)want;
+}
+
 int sdpa_path(const SdpaArgs &a) {
     if (a.E < 1 || a.E > 256 || a.Lq < 0 || a.Lk < 0 || a.H < 1 || a.B < 1) return MI_SDPA_DECLINE;
     if (a.H > 65535 || a.B > 65535 || (int64_t)a.Lq * a.H * 64 > INT32_MAX) return MI_SDPA_DECLINE;
@@ -661,9 +752,10 @@ int mi_sdpa_init() {
 extern "C" {
 
 size_t mi_sdpa_f16_workspace(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, int has_bias) {
-    (void)has_bias;
-    int ns = rows_splits(Lq, Lk, H, B);
-    if (ns <= 1 || Lq >= 64) return 0;
+    // sized for the path the call will most likely take: the fused kernel's key splits for Lq >= 64 without
+    // an additive mask (unused if the operands turn out not to be 16-byte addressable), the rows kernel's below
+    int ns = Lq >= 64 ? (has_bias ? 1 : flash_splits(Lq, Lk, H, B)) : rows_splits(Lq, Lk, H, B);
+    if (ns <= 1) return 0;
     size_t rows = (size_t)Lq * H * B;
     return round_up((size_t)ns * rows * E * sizeof(float), 256) + round_up((size_t)ns * rows * 2 * sizeof(float), 256);
 }
@@ -678,7 +770,8 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
                   zero4, nullptr, E, Lq, Lk, H, B, scale);
     if (rc != MI_OK) return MI_SDPA_DECLINE;
     int path = sdpa_path(a);
-    if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? rows_splits(Lq, Lk, H, B) : 1;
+    if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? rows_splits(Lq, Lk, H, B)
+                                  : path == MI_SDPA_FLASH ? flash_splits(Lq, Lk, H, B) : 1;
     return path;
 }
 
@@ -704,9 +797,23 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
             dim3 grid((unsigned)ceil_div(Lq, 256), (unsigned)H, (unsigned)B);
             hipLaunchKernelGGL((flash_fwd_kernel<64, true>), grid, dim3(512), flash_lds_bytes(64), st, a);
         } else {
-            dim3 grid((unsigned)ceil_div(Lq, 128), (unsigned)H, (unsigned)B);
+            // few query blocks: split the keys over workgroups too, if the caller brought the workspace for it
+            a.nsplit = flash_splits(Lq, Lk, H, B);
+            const size_t rows = (size_t)Lq * H * B;
+            const size_t o_bytes = round_up((size_t)a.nsplit * rows * E * sizeof(float), 256);
+            if (a.nsplit > 1 && ws && aligned_to(ws, 256) && ws_bytes >= o_bytes + round_up((size_t)a.nsplit * rows * 2 * sizeof(float), 256)) {
+                a.part_o = reinterpret_cast<float *>(ws);
+                a.part_ml = reinterpret_cast<float *>(reinterpret_cast<char *>(ws) + o_bytes);
+            } else {
+                a.nsplit = 1;
+            }
+            dim3 grid((unsigned)(ceil_div(Lq, 128) * a.nsplit), (unsigned)H, (unsigned)B);
             if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false>), grid, dim3(256), flash_lds_bytes(64), st, a);
             else         hipLaunchKernelGGL((flash_fwd_kernel<128, false>), grid, dim3(256), flash_lds_bytes(128), st, a);
+            if (a.nsplit > 1) {
+                const long total = (long)Lq * H * B * E;
+                hipLaunchKernelGGL(sdpa_merge_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a);
+            }
         }
         return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
     }

@@ -176,3 +176,38 @@ def test_eight_wave_kernel_on_large_grids(ctx):
     assert np.all(got[1] == 0)
     _check(ctx, q, k[:, :, :64], v[:, :, :64], expect="FlashPlan", what="8-wave one block")
     _check(ctx, q, k[:, :, :129], v[:, :, :129], out_dtype="f32", expect="FlashPlan", what="8-wave three blocks f32")
+
+
+def test_fused_kernel_splits_keys_on_small_grids(ctx):
+    """Few query blocks and very many keys: the fused kernel also splits the keys over workgroups and a merge joins
+    the partials.  Ragged last split, per-batch kv_len that leaves the later split without a key (one row of the
+    batch with none at all), fp32 and token-major outputs; config 3's shape stays in one pass."""
+    import torch
+    import juliavision_amd as jv
+    q, k, v = _qkv(1, 6, 1370, 1370, 64, 131)
+    plan = jv.sdpaplan(ctx, to_dev(q), to_dev(k), to_dev(v))
+    assert type(plan).__name__ == "FlashPlan" and plan.nsplit == 1, plan
+    _check(ctx, q, k, v, expect="FlashPlan", what="config 3 attention")
+    q, k, v = _qkv(1, 2, 300, 2000, 64, 135)
+    assert jv.sdpaplan(ctx, to_dev(q), to_dev(k), to_dev(v)).nsplit == 2
+    _check(ctx, q, k, v, expect="FlashPlan", what="two key splits, ragged second")
+    q, k, v = _qkv(3, 2, 200, 1700, 64, 141)
+    assert jv.sdpaplan(ctx, to_dev(q), to_dev(k), to_dev(v)).nsplit == 2
+    got = _check(ctx, q, k, v, kv_len=[1700, 0, 70], out_dtype="f32", expect="FlashPlan", what="key splits with kv_len")
+    assert np.all(got[1] == 0)
+    buf = poison(torch.empty((3, 200, 2, 64), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.sdpa(ctx, to_dev(q), to_dev(k), to_dev(v), None, None, out=buf.permute(0, 2, 1, 3))
+    torch.cuda.synchronize()
+    assert_parity(to_host(buf).transpose(0, 2, 1, 3), oracle.sdpa_ref_f32(q, k, v), what="key splits, token-major out")
+    # without a workspace the same call runs unsplit and must agree
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    dq, dk, dv = to_dev(q), to_dev(k), to_dev(v)
+    out = poison(torch.empty((3, 2, 200, 64), dtype=torch.float16, device="cuda"))
+    st = lambda t: L.strides4(t.stride(3), t.stride(2), t.stride(1), t.stride(0))
+    rc = lib.mi_sdpa_f16(out.data_ptr(), L.F16, None, dq.data_ptr(), st(dq), dk.data_ptr(), st(dk), dv.data_ptr(), st(dv),
+                         None, L.F16, None, None, 64, 200, 1700, 2, 3, 0.125, None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert_parity(to_host(out), oracle.sdpa_ref_f32(q, k, v), what="no workspace: one pass")
