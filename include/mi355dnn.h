@@ -109,6 +109,19 @@ int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const v
                 int w_layout, int bias_mode, int epi, int out_dtype,
                 void *ws, size_t ws_bytes, void *stream);
 
+/* Y = epi(layernorm(X) . W + bias) (+ residual) for T <= 8 in one pass over the weights:
+ * the rows of X are normalised over K (fp32 statistics, gamma/beta fp16 or NULL, the
+ * result rounded to fp16) while they are staged, in the arithmetic and summation order
+ * of mi_layernorm_f16, so the result is bit-identical to that call followed by
+ * mi_gemv_f16.  The reference runs the two as separate ops (layernorm!,
+ * layernorm.jl:125, then matmul!, matmul.jl:78-79); folding the norm into the GEMM's
+ * prologue is item 3 of its plans/kernels-to-port.md.  Workspace as for mi_gemv_f16. */
+int mi_ln_gemv_f16(void *Y, const void *X, const void *gamma, const void *beta, float eps,
+                   const void *W, const void *bias, const void *residual,
+                   int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                   int w_layout, int bias_mode, int epi, int out_dtype,
+                   void *ws, size_t ws_bytes, void *stream);
+
 size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int64_t nbatch);
 /* Returns an mi_gemm_path; never launches.  Replaces mmplan / mm_coopmat_plan /
  * mm_gemv_plan -- matmul.jl:87-95,121-131,172-179. */

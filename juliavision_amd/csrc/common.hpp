@@ -53,6 +53,15 @@ MI_DEVICE float apply_epi_c(float v) {
     else return v;
 }
 
+// One layer-normalised element, rounded to fp16: shared by the layer-norm kernels and the GEMV that folds
+// the norm into its prologue, so that the two produce the same bits.
+MI_DEVICE half_t ln_norm1(float x, float mu, float r, bool has_g, float g, bool has_b, float b) {
+    float y = (x - mu) * r;
+    if (has_g) y *= g;
+    if (has_b) y += b;
+    return (half_t)y;
+}
+
 static inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline size_t round_up(size_t a, size_t b) { return (a + b - 1) / b * b; }

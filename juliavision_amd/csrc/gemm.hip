@@ -22,6 +22,11 @@ struct GemmArgs {
     int tiles_m, tiles_n, group_m;
     int vec_store;          // Y (and residual) rows allow 16-byte accesses
     ConvGather cv;          // cv.xp != nullptr: B is the im2col matrix of a convolution, gathered on the fly
+    // Decode-sized kernels only: the rows of A are layer-normalised over K on their way into LDS
+    // (ln_on; gamma, beta may be null), exactly as layernorm_vec_kernel would have written them.
+    const half_t *ln_gamma, *ln_beta;
+    float ln_eps;
+    int ln_on;
 };
 
 // ------------------------------------------------------------------------------------------
@@ -578,6 +583,79 @@ __global__ void gemm_scalar_kernel(GemmArgs p, int b_kn) {
 // rows of a workgroup take interleaved k-pairs.  K is split over workgroups so that the whole chip
 // pulls on HBM; each split writes an fp32 partial plane and skinny_epilogue_kernel sums the planes
 // (the reference's split-K planes + mm_epilogue_kernel!, matmul.jl:192-217).
+// Layer-norm statistics of up to MT rows of A, one wave per row, in the summation order of
+// layernorm_vec_kernel (a lane takes the 16-byte chunks lane, lane + 64, ...; butterfly over the wave):
+// the fused result is bit-identical to running that kernel first.  stats[m] = (mean, rstd).
+template <int MT>
+__device__ __forceinline__ void ln_row_stats(const GemmArgs &p, float (*stats)[2], int tid) {
+    const int lane = tid & 63, wave = tid >> 6;
+    constexpr int NCH = 8;                                   // rows up to 4096 halves stay in registers between the passes
+    for (int m = wave; m < MT && m < p.M; m += 4) {
+        const half_t *row = p.A + (long)m * p.ldA;
+        float s = 0.0f, s2 = 0.0f;
+        if (p.K <= NCH * 512) {
+            u32x4 raw[NCH];
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const int e0 = (lane + 64 * i) * 8;
+                const u32x4 z = {0u, 0u, 0u, 0u};
+                raw[i] = e0 < p.K ? ldg16(row + e0) : z;
+            }
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                if ((lane + 64 * i) * 8 < p.K) {
+                    const half8v t = as_half8(raw[i]);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) s += (float)t[j];
+                }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+            const float mu = s / (float)p.K;
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                if ((lane + 64 * i) * 8 < p.K) {
+                    const half8v t = as_half8(raw[i]);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) { const float d = (float)t[j] - mu; s2 = fmaf(d, d, s2); }
+                }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+            if (lane == 0) { stats[m][0] = mu; stats[m][1] = 1.0f / sqrtf(s2 / (float)p.K + p.ln_eps); }
+        } else {
+            for (int e0 = lane * 8; e0 < p.K; e0 += 512) {
+                const half8v t = as_half8(ldg16(row + e0));
+#pragma unroll
+                for (int j = 0; j < 8; j++) s += (float)t[j];
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+            const float mu = s / (float)p.K;
+            for (int e0 = lane * 8; e0 < p.K; e0 += 512) {
+                const half8v t = as_half8(ldg16(row + e0));
+#pragma unroll
+                for (int j = 0; j < 8; j++) { const float d = (float)t[j] - mu; s2 = fmaf(d, d, s2); }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+            if (lane == 0) { stats[m][0] = mu; stats[m][1] = 1.0f / sqrtf(s2 / (float)p.K + p.ln_eps); }
+        }
+    }
+}
+
+// Eight activations of row statistics (mu, r) at column k0 of A, normalised and rounded as layernorm_vec_kernel does.
+__device__ __forceinline__ u32x4 ln_apply8(const GemmArgs &p, u32x4 raw, float mu, float r, int k0) {
+    const half8v x = as_half8(raw);
+    half8v gv, bv, o;
+    if (p.ln_gamma) gv = as_half8(ldg16(p.ln_gamma + k0));
+    if (p.ln_beta) bv = as_half8(ldg16(p.ln_beta + k0));
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        o[j] = ln_norm1((float)x[j], mu, r, p.ln_gamma != nullptr, p.ln_gamma ? (float)gv[j] : 0.0f, p.ln_beta != nullptr, p.ln_beta ? (float)bv[j] : 0.0f);
+    return __builtin_bit_cast(u32x4, o);
+}
+
 constexpr int SKN_COLS = 128;      // columns per workgroup
 constexpr int SKN_KMAX = 256;      // deepest k-slice: 16 loads of 16 bytes per thread, all in flight at once
 constexpr int SKN_LOADS = SKN_KMAX / 32;
@@ -586,6 +664,7 @@ template <int MT>
 __global__ __launch_bounds__(256) void skinny_kn_kernel(GemmArgs p, float *part, int kper) {
     __shared__ __align__(16) half_t xs[MT][SKN_KMAX];
     __shared__ float red[4][MT][SKN_COLS];
+    __shared__ float lnst[MT][2];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cx = tid & 15, ky = tid >> 4;            // ky = 0..15: k-pairs 2 ky, 2 ky + 1 (+ 32 i)
     const int n = blockIdx.x * SKN_COLS + cx * 8;
@@ -604,10 +683,18 @@ __global__ __launch_bounds__(256) void skinny_kn_kernel(GemmArgs p, float *part,
             w[i][1] = (ncol && k + 1 < klen) ? ldg16(bp + (long)(k + 1) * p.ldB) : z;
         }
     }
+    if (p.ln_on) {                                      // uniform
+        ln_row_stats<MT>(p, lnst, tid);
+        __syncthreads();
+    }
     for (int c = tid; c < MT * (kper >> 3); c += 256) {
         const int m = c / (kper >> 3), ch = c % (kper >> 3);
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        *reinterpret_cast<u32x4 *>(&xs[m][ch * 8]) = (m < p.M && ch * 8 < klen) ? ldg16(p.A + (long)m * p.ldA + k0 + ch * 8) : z;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (m < p.M && ch * 8 < klen) {
+            v = ldg16(p.A + (long)m * p.ldA + k0 + ch * 8);
+            if (p.ln_on) v = ln_apply8(p, v, lnst[m][0], lnst[m][1], k0 + ch * 8);
+        }
+        *reinterpret_cast<u32x4 *>(&xs[m][ch * 8]) = v;
     }
     __syncthreads();
     float acc[MT][8];
@@ -682,11 +769,20 @@ __global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p, int rows_per
     extern __shared__ __align__(16) char smem[];
     half_t *xs = reinterpret_cast<half_t *>(smem);       // [MT][K]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ float lnst[MT][2];
     const int kch = p.K >> 3;
+    if (p.ln_on) {                                      // uniform
+        ln_row_stats<MT>(p, lnst, tid);
+        __syncthreads();
+    }
     for (int c = tid; c < MT * kch; c += 256) {
         const int m = c / kch, ch = c % kch;
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        *reinterpret_cast<u32x4 *>(xs + (long)m * p.K + ch * 8) = m < p.M ? ldg16(p.A + (long)m * p.ldA + ch * 8) : z;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (m < p.M) {
+            v = ldg16(p.A + (long)m * p.ldA + ch * 8);
+            if (p.ln_on) v = ln_apply8(p, v, lnst[m][0], lnst[m][1], ch * 8);
+        }
+        *reinterpret_cast<u32x4 *>(xs + (long)m * p.K + ch * 8) = v;
     }
     __syncthreads();
     for (int r = 0; r < rows_per_wave; r++) {
@@ -916,6 +1012,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.bias_mode = bias_mode; a.epi = epi; a.out_f32 = out_dtype == MI_F32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
     a.cv = ConvGather{};
+    a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     return MI_OK;
 }
 
@@ -976,6 +1073,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
                      const ConvGather *gather) {
     GemmArgs a;
     a.cv = ConvGather{};
+    a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
@@ -1087,6 +1185,23 @@ int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const v
     if (!g_ready) return MI_ERROR_DEVICE;
     if (T < 1 || T > 8) return MI_DECLINE_EXTENT;
     if (!mfma_addressable(a, w_layout == MI_W_KF)) return MI_DECLINE_OPERANDS;
+    return run_skinny(a, w_layout == MI_W_KF, ws, ws_bytes, (hipStream_t)stream);
+}
+
+int mi_ln_gemv_f16(void *Y, const void *X, const void *gamma, const void *beta, float eps,
+                   const void *W, const void *bias, const void *residual,
+                   int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                   int w_layout, int bias_mode, int epi, int out_dtype,
+                   void *ws, size_t ws_bytes, void *stream) {
+    GemmArgs a;
+    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype, 0, 0, 0);
+    if (rc != MI_OK) return rc;
+    if (!g_ready) return MI_ERROR_DEVICE;
+    if (T < 1 || T > 8) return MI_DECLINE_EXTENT;
+    if (!mfma_addressable(a, w_layout == MI_W_KF)) return MI_DECLINE_OPERANDS;
+    if ((gamma && !aligned_to(gamma, 16)) || (beta && !aligned_to(beta, 16))) return MI_DECLINE_OPERANDS;
+    if (w_layout == MI_W_FK && (size_t)8 * K * sizeof(half_t) > SKINNY_FK_LDS_MAX) return MI_DECLINE_EXTENT;
+    a.ln_on = 1; a.ln_gamma = (const half_t *)gamma; a.ln_beta = (const half_t *)beta; a.ln_eps = eps;
     return run_skinny(a, w_layout == MI_W_KF, ws, ws_bytes, (hipStream_t)stream);
 }
 

@@ -51,12 +51,8 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(half_t *out, float *
             if (gamma) gv = as_half8(ldg16(gamma + e0));
             if (beta) bv = as_half8(ldg16(beta + e0));
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                float y = (x[i][j] - mu) * r;
-                if (gamma) y *= (float)gv[j];
-                if (beta) y += (float)bv[j];
-                o[j] = (half_t)y;
-            }
+            for (int j = 0; j < 8; j++)
+                o[j] = ln_norm1(x[i][j], mu, r, gamma != nullptr, gamma ? (float)gv[j] : 0.0f, beta != nullptr, beta ? (float)bv[j] : 0.0f);
             *reinterpret_cast<half8v *>(out + g * C + e0) = o;
         }
     }

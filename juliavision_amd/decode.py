@@ -19,7 +19,7 @@ from typing import Callable, List, Optional
 import torch
 
 from . import _lib as L
-from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, matmul_, sdpa
+from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, sdpa
 
 
 class KVCache:
@@ -98,30 +98,35 @@ def decoder_layer_step(ctx: Ctx, W: DecoderLayerWeights, cache: KVCache, layer: 
                        buf: DecodeBuffers, eps: float = 1e-5):
     """One token through one decoder layer: self-attention over the cache (the new
     row appended in place first), cross-attention over the window's encoder K/V,
-    GELU MLP; residuals ride in the GEMV epilogues.  ``cache.advance`` must have
+    GELU MLP; the three layer norms ride in the prologues of the GEMVs that read
+    them (batch <= 4; separate launches above), the residuals in the epilogues.  ``cache.advance`` must have
     run once for this step.  ``x``, ``out``: ``(B, d_model)`` fp16."""
     B, d = x.shape
     H, E = cache.heads, cache.headdim
     heads = lambda t: t.view(B, H, 1, E)
-    layernorm_(ctx, buf.h, None, None, x, W.ln1_g, W.ln1_b, d, eps)
-    ctx.ws.reset()
-    matmul_(ctx, buf.qkv, W.wqkv, buf.h, W.bqkv)
+    def normed_linear(dst, w, src, g, b_, bias, epi="none"):
+        # every workgroup of the folded form recomputes the row statistics: worth it for a few rows
+        # (one launch less per norm), not for eight
+        ctx.ws.reset()
+        if B <= 4:
+            ln_matmul_(ctx, dst, w, src, g, b_, eps, bias, epi=epi)
+        else:
+            layernorm_(ctx, buf.h, None, None, src, g, b_, d, eps)
+            matmul_(ctx, dst, w, buf.h, bias, epi=epi)
+
+    normed_linear(buf.qkv, W.wqkv, x, W.ln1_g, W.ln1_b, W.bqkv)
     q, k_new, v_new = (buf.qkv[:, i * d:(i + 1) * d].unflatten(1, (H, 1, E)) for i in range(3))
     cache.append(ctx, layer, k_new, v_new)
     ctx.ws.reset()
     sdpa(ctx, q, cache.self_k[layer], cache.self_v[layer], out=heads(buf.att), kv_len=cache.length)
     ctx.ws.reset()
     matmul_(ctx, buf.x1, W.wo, buf.att, W.bo, residual=x)
-    layernorm_(ctx, buf.h, None, None, buf.x1, W.ln2_g, W.ln2_b, d, eps)
-    ctx.ws.reset()
-    matmul_(ctx, buf.qc, W.wq_c, buf.h, W.bq_c)
+    normed_linear(buf.qc, W.wq_c, buf.x1, W.ln2_g, W.ln2_b, W.bq_c)
     ctx.ws.reset()
     sdpa(ctx, heads(buf.qc), cache.cross_k[layer], cache.cross_v[layer], out=heads(buf.catt))
     ctx.ws.reset()
     matmul_(ctx, buf.x2, W.wo_c, buf.catt, W.bo_c, residual=buf.x1)
-    layernorm_(ctx, buf.h, None, None, buf.x2, W.ln3_g, W.ln3_b, d, eps)
-    ctx.ws.reset()
-    matmul_(ctx, buf.f, W.w1, buf.h, W.b1, epi="gelu")
+    normed_linear(buf.f, W.w1, buf.x2, W.ln3_g, W.ln3_b, W.b1, epi="gelu")
     ctx.ws.reset()
     matmul_(ctx, out, W.w2, buf.f, W.b2, residual=buf.x2)
     return out

@@ -230,6 +230,29 @@ def _matmul_run(ctx, plan, out, A, B, bias, epi, residual, bias_mode):
     return out
 
 
+def ln_matmul_(ctx: Ctx, out, A, B, gamma, beta, eps, bias=None, *, epi="none", residual=None):
+    """``out[T,F] = epi(layernorm(B[T,K]) . A[K,F] + bias) (+ residual)`` for ``T <= 8`` in one pass over the weights:
+    ``layernorm_`` (layernorm.jl:125) folded into ``matmul_``'s activation staging, bit-identical to the two calls
+    in sequence.  Larger ``T`` declines (run the two ops)."""
+    plan = mmplan(ctx.dev, out, A, B, bias)
+    if not isinstance(plan, MMSkinnyPlan):
+        raise DeclineError(f"ln_matmul_: only the decode-sized path folds the norm (plan {plan})", L.DECLINE_EXTENT)
+    lib = L.init()
+    K, F = A.shape
+    T = B.shape[0]
+    la, lb, lo = _mat2(A), _mat2(B), _mat2(out)
+    if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
+        raise DeclineError("ln_matmul_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
+    need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1)
+    ws = ctx.ws.scratch(need)
+    rc = lib.mi_ln_gemv_f16(out.data_ptr(), B.data_ptr(), _ptr(gamma), _ptr(beta), float(eps), A.data_ptr(), _ptr(bias), _ptr(residual),
+                            T, K, F, lo[1], lb[1], la[1], plan.w_layout, L.BIAS_NONE if bias is None else L.BIAS_COL, L.EPI[epi],
+                            _dtype_code(out), ws, need, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_ln_gemv_f16", rc)
+    return out
+
+
 def batchedmatmul_(ctx: Ctx, out, A, B):
     """``out[b] = B[b] . A[b]`` over the leading torch axis -- batchedmatmul!, matmul.jl:383.
     ``A``: torch (Bt, K, F), ``B``: torch (Bt, T, K), ``out``: (Bt, T, F); a leading

@@ -153,3 +153,33 @@ def test_split_k_narrow_outputs(ctx, layout):
     _run(ctx, 200, 2048, 256, layout=layout, epi="gelu", residual=True)
     _run(ctx, 200, 2048, 256, layout=layout, out_f32=True)
     _run(ctx, 1500, 5120, 1280, layout=layout, residual=True, seed=7)
+
+
+@pytest.mark.parametrize("layout", ["kf", "fk"])
+@pytest.mark.parametrize("T,K,F", [(1, 1280, 1280), (4, 1280, 3840), (8, 264, 136), (3, 2048, 520)])
+def test_layer_norm_folded_into_decode_sized_gemv(ctx, T, K, F, layout):
+    """ln_matmul_ against the oracle's layernorm -> gemm, and bit for bit against the two device calls in sequence."""
+    import torch
+    import juliavision_amd as jv
+    X = oracle.randn_f16((T, K), 81, 0.3, 2.0)
+    Wkf = oracle.randn_f16((K, F), 82, 0, 1.0 / np.sqrt(K))
+    g, be, b = oracle.randn_f16((K,), 83, 1.0, 0.2), oracle.randn_f16((K,), 84, 0, 0.2), oracle.randn_f16((F,), 85, 0, 0.1)
+    R = oracle.randn_f16((T, F), 86)
+    Wd = to_dev(Wkf) if layout == "kf" else to_dev(np.ascontiguousarray(Wkf.T)).t()
+    dX, dg, dbe, db, dR = to_dev(X), to_dev(g), to_dev(be), to_dev(b), to_dev(R)
+    for (gamma, beta, hg, hb) in ((dg, dbe, g, be), (None, None, None, None), (dg, None, g, None)):
+        h, _, _ = oracle.layernorm_f16(X, hg, hb, 1e-5)
+        want = oracle.gemm_f16(h, Wkf, b, epi="gelu", residual=R)
+        out = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+        ctx.ws.reset()
+        jv.ln_matmul_(ctx, out, Wd, dX, gamma, beta, 1e-5, db, epi="gelu", residual=dR)
+        two = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+        hn = torch.empty_like(dX)
+        jv.layernorm_(ctx, hn, None, None, dX, gamma, beta, K, 1e-5)
+        ctx.ws.reset()
+        jv.matmul_(ctx, two, Wd, hn, db, epi="gelu", residual=dR)
+        torch.cuda.synchronize()
+        assert_parity(to_host(out), want, what=f"ln+gemv T{T} K{K} F{F} {layout}")
+        assert np.array_equal(to_host(out), to_host(two)), "folded norm differs from layernorm_ followed by matmul_"
+    with pytest.raises(jv.DeclineError):
+        jv.ln_matmul_(ctx, torch.empty((16, F), dtype=torch.float16, device="cuda"), Wd, torch.zeros((16, K), dtype=torch.float16, device="cuda"), None, None, 1e-5)
