@@ -263,6 +263,59 @@ def decoder_layer_case(bsz, layout="kf", steps=200):
             "GB/s_graph": round((weights + kv) / replay / 1e9, 1), "frac_hbm_peak_graph": round((weights + kv) / replay / 1e9 / PEAK_HBM_GBS, 4)}
 
 
+def decode_step_case(steps=100):
+    """A whole Whisper-large-v3-turbo-shaped decoder token at batch 1: 4 layers (as decoder_layer_case, [F][K]
+    weights), final layer norm folded into the 1280 -> 51866 vocabulary projection, one graph replay per token.
+    The reference's figure for the same step is 13.5 ms per token in fp32 on its card, against a 2.07 ms floor
+    set by 634 MB of fp32 weights (WhisperRunner/src/decode.jl:18-24); here a token reads 290 MB of fp16."""
+    import time
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd.decode import DecodeBuffers, DecoderLayerWeights, KVCache, StepGraph, decoder_layer_step
+    d, H, E, ffn, NL, V = 1280, 20, 64, 5120, 4, 51866
+    ctx = jv.Ctx("cuda")
+    f16 = torch.float16
+    w = lambda k, f: (torch.randn((f, k), dtype=f16, device="cuda") * 0.02).t()
+    v = lambda n, m=0.0: torch.randn((n,), dtype=f16, device="cuda") * 0.02 + m
+    layers = [DecoderLayerWeights(v(d, 1.0), v(d), w(d, 3 * d), v(3 * d), w(d, d), v(d), v(d, 1.0), v(d), w(d, d), v(d), w(d, d), v(d),
+                                  v(d, 1.0), v(d), w(d, ffn), v(ffn), w(ffn, d), v(d)) for _ in range(NL)]
+    lnf_g, lnf_b, wv = v(d, 1.0), v(d), w(d, V)
+    cache = KVCache(NL, 1, H, E)
+    for t in (cache.self_k, cache.self_v, cache.cross_k, cache.cross_v):
+        t.normal_()
+    buf = DecodeBuffers(1, d, ffn)
+    xs = [torch.randn((1, d), dtype=f16, device="cuda") for _ in range(NL + 1)]
+    logits = torch.empty((1, V), dtype=torch.float32, device="cuda")
+
+    def step():
+        cache.advance(ctx)
+        for i in range(NL):
+            decoder_layer_step(ctx, layers[i], cache, i, xs[i], xs[i + 1], buf)
+        ctx.ws.reset()
+        jv.ln_matmul_(ctx, logits, wv, xs[NL], lnf_g, lnf_b, 1e-5)
+
+    def timed(fn):
+        cache.length.fill_(447)
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    eager = timed(step)
+    graph = StepGraph(step)
+    replay = timed(graph.replay)
+    if not bool(torch.isfinite(logits).all()):
+        raise RuntimeError("decode step produced non-finite logits")
+    nbytes = NL * 2.0 * (3 * d * d + 3 * d * d + 2 * d * ffn) + 2.0 * d * V + NL * 2.0 * 2 * H * E * (448 + 1500)
+    return {"eager_us": round(eager * 1e6, 1), "graph_us": round(replay * 1e6, 1), "launches": 1 + NL * 12 + 1,
+            "MB_per_token": round(nbytes / 1e6, 1), "GB/s_graph": round(nbytes / replay / 1e9, 1),
+            "frac_hbm_peak_graph": round(nbytes / replay / 1e9 / PEAK_HBM_GBS, 4)}
+
+
 def detail_benchmarks(lib, L, stream, only=None):
     import numpy as np
     import torch
@@ -375,6 +428,10 @@ def detail_benchmarks(lib, L, stream, only=None):
             name = f"c5_decoder_layer_b{bsz}_{tag}"
             if only is None or only in name:
                 out[name] = decoder_layer_case(bsz, lay)
+
+    name = "c5_decode_step_4layers_vocab51866_b1"
+    if only is None or only in name:
+        out[name] = decode_step_case()
 
     # config 4: global attention at 4096 and the 3x3 conv
     attn_case("c4_attn_L4096_16x64", 1, 16, 4096, 4096, 64)
