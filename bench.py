@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, vendor figure
 # HBM bytes per launch of the dominant kernel (fc1 GEMM), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of `python bench.py --no-cpu --no-detail`, scaled by the same counters on a plain copy kernel of
 # known size (--calibrate-copy).
-FC1_TRAFFIC_BYTES = 57_253_949       # profiles/fc1_gemm_hbm_traffic.txt: FETCH 20 456 KiB x 2.000 + WRITE 15 000 KiB x 1.000
+FC1_TRAFFIC_BYTES = 57_244_733       # profiles/fc1_gemm_hbm_traffic.txt: FETCH 20 451.5 KiB x 2.000 + WRITE 15 000 KiB x 1.000
 
 
 def parse_args():
