@@ -57,6 +57,7 @@ enum mi_bias_mode { MI_BIAS_NONE = 0, MI_BIAS_COL = 1, MI_BIAS_ROW = 2 };
 enum mi_gemm_path { MI_GEMM_DECLINE = 0, MI_GEMM_MFMA = 1, MI_GEMM_SKINNY = 2, MI_GEMM_SCALAR = 3 };
 enum mi_sdpa_path { MI_SDPA_DECLINE = 0, MI_SDPA_FLASH = 1, MI_SDPA_ROWS = 2 };
 enum mi_conv_path { MI_CONV_DECLINE = 0, MI_CONV_GEMM_1X1 = 1, MI_CONV_IM2COL_GEMM = 2, MI_CONV_DIRECT = 3, MI_CONV_IMPLICIT_GEMM = 4 };
+enum mi_convt_path { MI_CONVT_DECLINE = 0, MI_CONVT_GEMM_SHUFFLE = 1, MI_CONVT_GATHER = 2 };
 
 /* Library / device. */
 int mi_version(void);
@@ -198,6 +199,36 @@ int mi_conv2d_f16_plan(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
                        int64_t dil_x, int64_t dil_y, int64_t groups);
 /* ATen's output extent -- convsize, conv.jl:309. */
 int64_t mi_convsize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d);
+
+/* Transposed convolution.  x as above; w (KW,KH,Cout/groups,Cin) = row-major
+ * [Cin][Cout/groups][KH][KW] (torch's conv_transpose2d weight); out (OW,OH,Cout,N) with
+ * OW = mi_convtransposesize(...); bias[Cout] or NULL.  fp32 accumulation seeded with the
+ * bias, one rounding.  kernel == stride with no padding / dilation / output padding and one
+ * group is one MFMA GEMM (Cout*KH*KW x Cin x H*W per image) followed by a pixel shuffle,
+ * workspace from mi_convtranspose2d_f16_workspace; every other case is the gather kernel
+ * and needs no workspace.
+ * Replaces convolutiontranspose!(ctx, out, x, w, bias, stride, padding, dilation, outpad,
+ * groups) -- conv.jl:226-294 -- with shufflecase / shuffleout (conv.jl:204-222) and the
+ * gather kernel convtranspose2d (conv.jl:149-191). */
+int mi_convtranspose2d_f16(void *out, const void *x, const void *w, const void *bias,
+                           int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                           int64_t KW, int64_t KH, int64_t Cout,
+                           int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                           int64_t dil_x, int64_t dil_y, int64_t outpad_x, int64_t outpad_y,
+                           int64_t groups, void *ws, size_t ws_bytes, void *stream);
+size_t mi_convtranspose2d_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                                        int64_t KW, int64_t KH, int64_t Cout,
+                                        int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                                        int64_t dil_x, int64_t dil_y, int64_t outpad_x, int64_t outpad_y,
+                                        int64_t groups);
+/* Returns an mi_convt_path; replaces shufflecase -- conv.jl:204-209. */
+int mi_convtranspose2d_f16_plan(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                                int64_t KW, int64_t KH, int64_t Cout,
+                                int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                                int64_t dil_x, int64_t dil_y, int64_t outpad_x, int64_t outpad_y,
+                                int64_t groups);
+/* ATen's transposed-convolution output extent -- convtransposesize, conv.jl:201. */
+int64_t mi_convtransposesize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d, int64_t op);
 
 /* ---------------------------------------------------------------- layer norm + glue
  * `groups` rows of C contiguous fp16 elements; mean in fp32, variance about that

@@ -22,6 +22,7 @@ BIAS_NONE, BIAS_COL, BIAS_ROW = 0, 1, 2
 GEMM_PATHS = {0: "decline", 1: "mfma", 2: "skinny", 3: "scalar"}
 SDPA_PATHS = {0: "decline", 1: "flash", 2: "rows"}
 CONV_PATHS = {0: "decline", 1: "gemm_1x1", 2: "im2col_gemm", 3: "direct", 4: "implicit_gemm"}
+CONVT_PATHS = {0: "decline", 1: "gemm_shuffle", 2: "gather"}
 
 _i64, _int, _vp, _sz, _f32 = C.c_int64, C.c_int, C.c_void_p, C.c_size_t, C.c_float
 _i64p = C.POINTER(C.c_int64)
@@ -44,6 +45,10 @@ SIGNATURES = {
     "mi_conv2d_f16_workspace": (_sz, [_i64] * 13),
     "mi_conv2d_f16_plan": (_int, [_i64] * 14),
     "mi_convsize": (_i64, [_i64] * 5),
+    "mi_convtranspose2d_f16": (_int, [_vp] * 4 + [_i64] * 16 + [_vp, _sz, _vp]),
+    "mi_convtranspose2d_f16_workspace": (_sz, [_i64] * 16),
+    "mi_convtranspose2d_f16_plan": (_int, [_i64] * 16),
+    "mi_convtransposesize": (_i64, [_i64] * 6),
     "mi_layernorm_f16": (_int, [_vp] * 6 + [_i64, _i64, _f32, _vp]),
     "mi_add_f16": (_int, [_vp, _vp, _vp, _i64, _vp]),
     "mi_kv_append_f16": (_int, [_vp, _vp, _i64p, _i64, _vp, _vp, _i64p, _vp, _i64, _i64, _i64, _vp]),

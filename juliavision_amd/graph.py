@@ -413,14 +413,25 @@ class Executor:
         raise UnsupportedOp(f"{o['id']}: a stand-alone {o['aten']} (run optimize() so that it folds into its linear)")
 
     def _convolution(self, o):
+        """aten::convolution, ordinary and transposed (arg6), 2-D and -- lifted to a singleton second spatial
+        axis -- 1-D (runop! for convolution.default, ops.jl:1114-1200)."""
         a, ins = o["attrs"], o["in"]
         x, w = self.get(ins[0]), self.get(ins[1])
         bias = self.get(ins[2]) if len(ins) > 2 else None
-        stride, padding, dilation = a["arg3"], a["arg4"], a["arg5"]
-        if a.get("arg6") or any(a.get("arg7", [0, 0])):
-            raise UnsupportedOp(f"{o['id']}: transposed convolution")
+        stride, padding, dilation = list(a["arg3"]), list(a["arg4"]), list(a["arg5"])
+        outpad = list(a.get("arg7") or [0] * len(stride))
+        out = self.t[o["out"]]
+        if len(stride) == 1:                               # (N,C,L) -> (N,C,1,L); the added axis has stride 1, no padding
+            x, w, out = x.unsqueeze(2), w.unsqueeze(2), out.unsqueeze(2)
+            stride, padding, dilation, outpad = [1] + stride, [0] + padding, [1] + dilation, [0] + outpad
+        elif len(stride) != 2:
+            raise UnsupportedOp(f"{o['id']}: {len(stride)}-D convolution")
+        xy = lambda p: tuple(p[::-1])                      # ATen's (h, w) pairs to the kernels' (x, y)
         self.ctx.ws.reset()
-        K.convolution_(self.ctx, self.t[o["out"]], x, w, bias, tuple(stride[::-1]), tuple(padding[::-1]), tuple(dilation[::-1]), a.get("arg8", 1))
+        if a.get("arg6"):
+            K.convolutiontranspose_(self.ctx, out, x, w, bias, xy(stride), xy(padding), xy(dilation), xy(outpad), a.get("arg8", 1))
+        else:
+            K.convolution_(self.ctx, out, x, w, bias, xy(stride), xy(padding), xy(dilation), a.get("arg8", 1))
 
     HANDLERS = {"linear.default": _linear, "addmm.default": _linear, "mm.default": _linear,
                 "scaled_dot_product_attention.default": _sdpa, "layer_norm.default": _layer_norm,

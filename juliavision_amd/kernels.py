@@ -412,6 +412,55 @@ def convolution_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, groups, *
     return out
 
 
+def convtransposesize(n, k, s, p, d, op):
+    """convtransposesize, conv.jl:201."""
+    return (n - 1) * s - 2 * p + d * (k - 1) + op + 1
+
+
+def convtranspose_plan(dev: DeviceCaps, out, x, w, stride=(1, 1), padding=(0, 0), dilation=(1, 1), outpad=(0, 0), groups=1):
+    """Which route a transposed convolution takes: ``gemm_shuffle`` (shufflecase, conv.jl:204-209) or
+    ``gather``.  Pairs are (x, y)."""
+    if not _is_f16_cuda(x, w) or x.dim() != 4 or w.dim() != 4 or not x.is_contiguous() or not w.is_contiguous():
+        return Decline("operands")
+    if not dev.coopmat:
+        return Decline("nocoopmat")
+    N, Cin, Hi, Wi = x.shape
+    cin_w, coutg, KH, KW = w.shape
+    if cin_w != Cin:
+        return Decline("extent")
+    lib = L.load()
+    args = (Wi, Hi, Cin, N, KW, KH, coutg * groups, stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1],
+            outpad[0], outpad[1], groups)
+    path = lib.mi_convtranspose2d_f16_plan(*args)
+    if path == 0:
+        return Decline("extent")
+    return ConvGemmPlan(L.CONVT_PATHS[path], int(lib.mi_convtranspose2d_f16_workspace(*args)))
+
+
+def convolutiontranspose_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, outpad, groups):
+    """convolutiontranspose!(ctx, out, x, w, bias, stride, padding, dilation, outpad, groups) -- conv.jl:226-294.
+    ``x`` torch (N,Cin,H,W), ``w`` torch (Cin,Cout/groups,KH,KW), ``out`` torch (N,Cout,OH,OW), all contiguous
+    fp16; the pairs are ``(x, y)``, the reverse of ATen's ``(h, w)``."""
+    plan = convtranspose_plan(ctx.dev, out, x, w, stride, padding, dilation, outpad, groups)
+    if isinstance(plan, Decline):
+        raise DeclineError(f"convolutiontranspose_ declined ({plan.reason})", L.DECLINE_OPERANDS)
+    lib = L.init()
+    N, Cin, Hi, Wi = x.shape
+    _, coutg, KH, KW = w.shape
+    Cout = coutg * groups
+    OW = convtransposesize(Wi, KW, stride[0], padding[0], dilation[0], outpad[0])
+    OH = convtransposesize(Hi, KH, stride[1], padding[1], dilation[1], outpad[1])
+    if tuple(out.shape) != (N, Cout, OH, OW) or not out.is_contiguous() or out.dtype != torch.float16:
+        raise DeclineError("convolutiontranspose_: out must be dense fp16 (N,Cout,OH,OW)", L.DECLINE_OPERANDS)
+    ws = ctx.ws.scratch(plan.workspace)
+    rc = lib.mi_convtranspose2d_f16(out.data_ptr(), x.data_ptr(), w.data_ptr(), _ptr(bias), Wi, Hi, Cin, N, KW, KH, Cout,
+                                    stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1],
+                                    outpad[0], outpad[1], groups, ws, plan.workspace, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_convtranspose2d_f16", rc)
+    return out
+
+
 # ----------------------------------------------------------------------------- layer norm, add
 
 def layernorm_(ctx: Ctx, out, mean, rstd, a, gamma, beta, C_: int, eps: float):

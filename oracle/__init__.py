@@ -212,6 +212,29 @@ def conv2d_f16(x, w, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1), 
     return out
 
 
+def convtransposesize(n, k, s, p, d, op):
+    return int(lib().orc_convtransposesize(_i64(n), _i64(k), _i64(s), _i64(p), _i64(d), _i64(op)))
+
+
+def convtranspose2d_f16(x, w, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1), output_padding=(0, 0), groups=1, out_f32=False):
+    """x: (N,Cin,H,W) fp16; w: (Cin,Cout/g,KH,KW) (torch's transposed-convolution weight); pairs are (y, x) as in torch."""
+    x = np.ascontiguousarray(x, dtype=np.float16)
+    w = np.ascontiguousarray(w, dtype=np.float16)
+    N, Cin, Hi, Wi = x.shape
+    _, coutg, KH, KW = w.shape
+    Cout = coutg * groups
+    OH = convtransposesize(Hi, KH, stride[0], padding[0], dilation[0], output_padding[0])
+    OW = convtransposesize(Wi, KW, stride[1], padding[1], dilation[1], output_padding[1])
+    out = np.empty((N, Cout, OH, OW), dtype=np.float32 if out_f32 else np.float16)
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, dtype=np.float16)
+    lib().orc_convtranspose2d_f16(_p(out), C.c_int(1 if out_f32 else 0), _p(x), _p(w), _p(bias),
+                                  _i64(Wi), _i64(Hi), _i64(Cin), _i64(N), _i64(KW), _i64(KH), _i64(Cout),
+                                  _i64(stride[1]), _i64(stride[0]), _i64(padding[1]), _i64(padding[0]),
+                                  _i64(dilation[1]), _i64(dilation[0]), _i64(output_padding[1]), _i64(output_padding[0]), _i64(groups))
+    return out
+
+
 def im2col_f16(x, KH, KW, stride=(1, 1), padding=(0, 0), dilation=(1, 1), MP=None, CRSP=None):
     """Returns col as row-major [CRSP][MP] (= the reference's column-major MP x CRSP)."""
     x = np.ascontiguousarray(x, dtype=np.float16)

@@ -22,6 +22,9 @@
  *                        row-sum / masked-row / split-merge invariants
  *   orc_conv2d_f16       torch.nn.functional.conv2d in fp32/fp64; im2col map by
  *                        brute force on tiny shapes
+ *   orc_convtranspose2d_f16  torch.nn.functional.conv_transpose2d in fp64 (stride, padding,
+ *                        dilation, output_padding, groups) and the pixel-shuffle identity of
+ *                        the non-overlapping case (conv.jl:204-222)
  *   orc_layernorm_f16    torch.nn.functional.layer_norm in fp32
  *   unpinned             bit-level accumulation order of Lava.coopmat_gemm!/gemv!
  *                        (third-party, source absent); irrelevant at the 1e-2 /
@@ -398,6 +401,51 @@ ORC_API void orc_conv2d_f16(void *out, int out_f32, const uint16_t *x, const uin
             int64_t o = ((n * Cout + co) * OH + oy) * OW + ox;
             if (out_f32) { ((float *)out)[o] = relu && acc < 0 ? 0.0f : acc; }
             else { float r = h2f(f2h(acc)); ((uint16_t *)out)[o] = f2h(relu && r < 0 ? 0.0f : r); }
+        }
+    }
+}
+
+/* conv.jl:201 (convtransposesize) */
+ORC_API int64_t orc_convtransposesize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d, int64_t op) {
+    return (n - 1) * s - 2 * p + d * (k - 1) + op + 1;
+}
+/* conv.jl:149-191 (convtranspose2d): the gather form -- every output element is computed from the inputs
+ * that reach it (stride divisibility), fp32 accumulator seeded with the bias, one rounding.  w is torch's
+ * transposed-convolution weight [Cin][Cout/groups][KH][KW]. */
+ORC_API void orc_convtranspose2d_f16(void *out, int out_f32, const uint16_t *x, const uint16_t *w, const uint16_t *bias,
+                                     int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                                     int64_t KW, int64_t KH, int64_t Cout,
+                                     int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy,
+                                     int64_t opx, int64_t opy, int64_t groups) {
+    int64_t OW = orc_convtransposesize(Wi, KW, sx, px, dx, opx), OH = orc_convtransposesize(Hi, KH, sy, py, dy, opy);
+    int64_t cing = Cin / groups, coutg = Cout / groups;
+    #pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t n = 0; n < N; n++)
+    for (int64_t co = 0; co < Cout; co++) {
+        int64_t g = co / coutg, cog = co % coutg;
+        for (int64_t oy = 0; oy < OH; oy++)
+        for (int64_t ox = 0; ox < OW; ox++) {
+            float acc = bias ? h2f(bias[co]) : 0.0f;
+            int64_t bx = ox + px, by = oy + py;
+            for (int64_t ci = g * cing; ci < (g + 1) * cing; ci++) {
+                for (int64_t ky = 0; ky < KH; ky++) {
+                    int64_t ty = by - ky * dy;
+                    if (ty < 0 || ty % sy != 0) continue;
+                    int64_t iy = ty / sy;
+                    if (iy >= Hi) continue;
+                    for (int64_t kx = 0; kx < KW; kx++) {
+                        int64_t tx = bx - kx * dx;
+                        if (tx < 0 || tx % sx != 0) continue;
+                        int64_t ix = tx / sx;
+                        if (ix >= Wi) continue;
+                        acc = fmaf(h2f(x[((n * Cin + ci) * Hi + iy) * Wi + ix]),
+                                   h2f(w[((ci * coutg + cog) * KH + ky) * KW + kx]), acc);
+                    }
+                }
+            }
+            int64_t o = ((n * Cout + co) * OH + oy) * OW + ox;
+            if (out_f32) ((float *)out)[o] = acc;
+            else ((uint16_t *)out)[o] = f2h(acc);
         }
     }
 }

@@ -127,6 +127,27 @@ def test_conv_planner_and_extents():
     assert lib.mi_conv2d_f16_workspace(256, 256, 144, 1, 1, 1, 256, 1, 1, 0, 0, 1, 1) == 0
 
 
+def test_convtranspose_planner_takes_only_the_non_overlapping_case():
+    """The case list of test_convtranspose_gemm.jl:64-75."""
+    lib = L.load()
+    plan = lambda *a: L.CONVT_PATHS[lib.mi_convtranspose2d_f16_plan(*a)]
+    #            W  H  Cin N KW KH Cout sx sy px py dx dy ox oy g
+    assert plan(8, 8, 8, 1, 2, 2, 8, 2, 2, 0, 0, 1, 1, 0, 0, 1) == "gemm_shuffle"
+    assert plan(8, 8, 8, 1, 3, 3, 8, 2, 2, 0, 0, 1, 1, 0, 0, 1) == "gather"        # overlapping fields
+    assert plan(8, 8, 8, 1, 2, 2, 8, 2, 2, 1, 1, 1, 1, 0, 0, 1) == "gather"        # padding
+    assert plan(8, 8, 8, 1, 2, 2, 8, 2, 2, 0, 0, 2, 2, 0, 0, 1) == "gather"        # dilation
+    assert plan(8, 8, 8, 1, 2, 2, 8, 2, 2, 0, 0, 1, 1, 1, 1, 1) == "gather"        # output padding
+    assert plan(8, 8, 8, 1, 2, 2, 8, 2, 2, 0, 0, 1, 1, 0, 0, 2) == "gather"        # groups
+    assert plan(8, 8, 8, 1, 2, 2, 8, 2, 2, 0, 0, 1, 1, 2, 0, 1) == "decline"       # output padding >= stride
+    assert plan(8, 8, 9, 1, 2, 2, 8, 2, 2, 0, 0, 1, 1, 0, 0, 2) == "decline"
+    assert lib.mi_convtransposesize(64, 2, 2, 0, 1, 0) == 128 and lib.mi_convtransposesize(8, 3, 2, 0, 1, 0) == 17
+    # scratch of SAM 2's first upsampler (256 -> 64 channels on 64x64, test_convtranspose_gemm.jl:36): the transposed
+    # weights [Cout*4][Cin], the expanded bias, the unshuffled GEMM result [Cout*4][H*W]; the GEMM itself needs none
+    ws = lib.mi_convtranspose2d_f16_workspace(64, 64, 256, 1, 2, 2, 64, 2, 2, 0, 0, 1, 1, 0, 0, 1)
+    assert ws == 256 * 256 * 2 + 256 * 2 + 256 * 4096 * 2 + lib.mi_gemm_f16_workspace(256, 256, 4096, L.W_KF, 1)
+    assert lib.mi_convtranspose2d_f16_workspace(8, 8, 8, 1, 3, 3, 8, 2, 2, 0, 0, 1, 1, 0, 0, 1) == 0
+
+
 def test_host_planners_decline_by_name_on_cpu_tensors():
     import torch
     import juliavision_amd as jv

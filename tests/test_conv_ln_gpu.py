@@ -89,6 +89,83 @@ def test_conv_config4_band(ctx):
     assert_parity(got[:, ch], want, what="config4 conv band")
 
 
+def _convt(ctx, N, Cin, H, W, Cout, KH, KW, s, p=0, d=1, op=0, groups=1, bias=True, expect=None, seed=1):
+    """``s``, ``p``, ``d``, ``op``: one number for both axes or an ``(x, y)`` pair."""
+    import torch
+    import juliavision_amd as jv
+    pair = lambda v: v if isinstance(v, tuple) else (v, v)
+    s, p, d, op = pair(s), pair(p), pair(d), pair(op)
+    x = oracle.randn_f16((N, Cin, H, W), seed, 0, 0.5)
+    w = oracle.randn_f16((Cin, Cout // groups, KH, KW), seed + 1, 0, 0.05)
+    b = oracle.randn_f16((Cout,), seed + 2, 0, 0.5) if bias else None
+    want = oracle.convtranspose2d_f16(x, w, b, s[::-1], p[::-1], d[::-1], op[::-1], groups)
+    out = poison(torch.empty(want.shape, dtype=torch.float16, device="cuda"))
+    dx, dw = to_dev(x), to_dev(w)
+    plan = jv.convtranspose_plan(ctx.dev, out, dx, dw, s, p, d, op, groups)
+    if expect:
+        assert plan.path == expect, plan
+    ctx.ws.reset()
+    jv.convolutiontranspose_(ctx, out, dx, dw, None if b is None else to_dev(b), s, p, d, op, groups)
+    torch.cuda.synchronize()
+    got = to_host(out)
+    assert_parity(got, want, what=f"convT {N},{Cin},{H},{W}->{Cout} k{KH}x{KW} s{s} p{p} d{d} op{op} g{groups}")
+    return got, want
+
+
+@pytest.mark.parametrize("N,Cin,H,W,Cout,KH,KW,kw", [
+    (1, 256, 64, 64, 64, 2, 2, {}),                   # SAM 2's two upsamplers, test_convtranspose_gemm.jl:36
+    (1, 64, 128, 128, 32, 2, 2, {}),
+    (1, 32, 16, 16, 8, 2, 2, {}),                     # channel counts below the GEMM tile
+    (2, 24, 8, 8, 12, 2, 2, {"bias": False}),
+    (3, 40, 5, 7, 10, 3, 2, {}),                      # H*W = 35 and OW = 14: the unaligned GEMM and the scalar shuffle
+    (1, 48, 6, 8, 16, 1, 4, {}),                      # one row of taps
+    (1, 16, 12, 12, 24, 1, 1, {}),                    # 1x1 stride 1: a plain channel mix
+])
+def test_convtranspose_gemm_shuffle(ctx, N, Cin, H, W, Cout, KH, KW, kw):
+    got, _ = _convt(ctx, N, Cin, H, W, Cout, KH, KW, (KW, KH), expect="gemm_shuffle", **kw)
+    # a shuffle that drops a sub-pixel phase leaves a lattice of zeros that an averaged error would hide
+    # (test_convtranspose_gemm.jl:50-58)
+    for ky in range(KH):
+        for kx in range(KW):
+            assert np.any(got[:, :, ky::KH, kx::KW] != 0)
+
+
+@pytest.mark.parametrize("N,Cin,H,W,Cout,KH,KW,s,p,d,op,g", [
+    (1, 16, 8, 8, 8, 3, 3, 2, 0, 1, 0, 1),                         # test_convtranspose_gemm.jl:78-95: overlapping fields
+    (2, 6, 5, 7, 4, 2, 3, (3, 2), (0, 1), (2, 1), (2, 1), 2),      # everything unequal, two groups
+    (1, 8, 6, 6, 8, 4, 4, 2, 1, 1, 0, 8),                          # depthwise 4/2/1 upsampler
+    (1, 3, 1, 9, 5, 1, 5, (3, 1), (2, 0), 1, (2, 0), 1),           # a lifted 1-D layer
+    (1, 16, 8, 8, 8, 2, 2, 2, 0, 1, 1, 1),                         # kernel == stride but with output padding
+])
+def test_convtranspose_gather(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, op, g):
+    _convt(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, op, g, expect="gather")
+
+
+def test_convtranspose_routes_agree_bitwise_on_exact_data(ctx):
+    """Small integers make every product and sum exact in fp16/fp32, so the GEMM + shuffle route, the gather
+    kernel and the oracle must agree bit for bit whatever their summation order."""
+    import torch
+    import juliavision_amd as jv
+    rng = np.random.default_rng(3)
+    x = rng.integers(-3, 4, (2, 32, 8, 16)).astype(np.float16)
+    w = rng.integers(-2, 3, (32, 12, 2, 2)).astype(np.float16)
+    b = rng.integers(-4, 5, (12,)).astype(np.float16)
+    want = oracle.convtranspose2d_f16(x, w, b, (2, 2))
+    out = poison(torch.empty(want.shape, dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.convolutiontranspose_(ctx, out, to_dev(x), to_dev(w), to_dev(b), (2, 2), (0, 0), (1, 1), (0, 0), 1)
+    assert np.array_equal(to_host(out), want)
+    # the same numbers through the gather: two groups of half the channels, summed by hand, is not the same op,
+    # so reach the gather with an output padding instead and compare the part both produce
+    want_op = oracle.convtranspose2d_f16(x, w, b, (2, 2), output_padding=(1, 1))
+    out_op = poison(torch.empty(want_op.shape, dtype=torch.float16, device="cuda"))
+    jv.convolutiontranspose_(ctx, out_op, to_dev(x), to_dev(w), to_dev(b), (2, 2), (0, 0), (1, 1), (1, 1), 1)
+    got_op = to_host(out_op)
+    assert np.array_equal(got_op, want_op)
+    assert np.array_equal(got_op[:, :, :-1, :-1], want)
+    assert np.array_equal(got_op[:, :, -1, :], np.broadcast_to(b[None, :, None], (2, 12, 33)))   # the padded edge is the bias
+
+
 @pytest.mark.parametrize("groups,C", [(1500, 1280), (1370, 384), (7, 144), (5, 37), (3, 4096), (2, 5000)])
 @pytest.mark.parametrize("affine", [True, False])
 def test_layernorm(ctx, groups, C, affine):

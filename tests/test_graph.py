@@ -145,3 +145,38 @@ def test_executor_refuses_what_it_cannot_run(ctx):
     run = G.Executor(g, _block().state_dict(), ctx)
     with pytest.raises(G.UnsupportedOp, match="needs a copy"):
         run(torch.randn(1, 70, 128).half().cuda())
+
+
+@pytest.mark.gpu
+def test_exported_upsampler_runs_transposed_and_lifted_1d_convolutions(ctx):
+    """aten::convolution with arg6 set is the transposed convolution and a one-element stride list is the 1-D
+    layer lifted to a singleton second axis (runop! for convolution.default, ops.jl:1114-1200)."""
+    import torch
+    from juliavision_amd import graph as G
+
+    class Up(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = torch.nn.ConvTranspose2d(32, 16, 2, 2)            # kernel == stride: GEMM + pixel shuffle
+            self.c = torch.nn.Conv2d(16, 16, 3, padding=1)
+            self.u1 = torch.nn.ConvTranspose1d(16, 8, 4, 2, 1)          # overlapping: the gather
+            self.c1 = torch.nn.Conv1d(8, 8, 3, padding=1)
+
+        def forward(self, x):
+            y = self.c(self.up(x))
+            return self.c1(self.u1(y.flatten(2)))
+
+    torch.manual_seed(5)
+    m = Up().eval().half()
+    x = torch.randn(1, 32, 8, 8).half()
+    ep = torch.export.export(m, (x,)).run_decompositions()
+    g = G.Graph.load(G.convert(ep, "up"))
+    assert [o["aten"] for o in g.ops] == ["convolution.default"] * 4
+    assert [bool(o["attrs"]["arg6"]) for o in g.ops] == [True, False, True, False]
+    run = G.Executor(g, m.state_dict(), ctx)
+    with torch.no_grad():
+        want = m.float()(x.float()).numpy()
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == want.shape == (1, 8, 512)
+    assert_parity(got.float().cpu().numpy(), want, what="exported upsampler")

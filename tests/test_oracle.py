@@ -249,6 +249,52 @@ def test_convsize_and_im2col_index_order():
     assert col[c, m] == x[1, 1, 2 * 2 - 1 + 2, 4 * 1 - 0 + 1]
 
 
+# ------------------------------------------------------------------ transposed convolution
+
+@pytest.mark.parametrize("N,Cin,H,W,Cout,KH,KW,s,p,d,op,g", [
+    (1, 16, 8, 8, 8, 2, 2, (2, 2), (0, 0), (1, 1), (0, 0), 1),          # the pixel-shuffle case
+    (1, 16, 8, 8, 8, 3, 3, (2, 2), (0, 0), (1, 1), (0, 0), 1),          # test_convtranspose_gemm.jl:81-84: overlapping fields
+    (2, 6, 5, 7, 4, 3, 2, (2, 3), (1, 0), (1, 2), (1, 2), 2),           # everything unequal, two groups
+    (1, 4, 6, 6, 4, 4, 4, (2, 2), (1, 1), (1, 1), (0, 0), 4),           # depthwise, the usual 4/2/1 upsampler
+    (1, 3, 1, 9, 5, 1, 5, (1, 3), (0, 2), (1, 1), (0, 2), 1),           # a lifted 1-D layer
+    (1, 2, 4, 4, 3, 3, 3, (1, 1), (2, 2), (2, 2), (0, 0), 1),           # stride 1, dilation 2, padding eats the border
+])
+def test_convtranspose_against_torch(N, Cin, H, W, Cout, KH, KW, s, p, d, op, g):
+    x = oracle.randn_f16((N, Cin, H, W), 1)
+    w = oracle.randn_f16((Cin, Cout // g, KH, KW), 2, 0, 0.1)
+    b = oracle.randn_f16((Cout,), 3)
+    t = lambda a: torch.from_numpy(a.astype(np.float64))
+    ref = torch.nn.functional.conv_transpose2d(t(x), t(w), t(b), stride=s, padding=p, output_padding=op, groups=g, dilation=d).numpy()
+    got = oracle.convtranspose2d_f16(x, w, b, s, p, d, op, g, out_f32=True)
+    assert got.shape == ref.shape
+    assert np.max(np.abs(got - ref)) < 1e-4
+    assert np.array_equal(oracle.convtranspose2d_f16(x, w, b, s, p, d, op, g), got.astype(np.float16))
+    nob = oracle.convtranspose2d_f16(x, w, None, s, p, d, op, g, out_f32=True)
+    assert np.max(np.abs(nob + b.astype(np.float32)[None, :, None, None] - got)) < 1e-5
+
+
+def test_convtranspose_size_and_the_pixel_shuffle_identity():
+    # convtransposesize inverts convsize wherever the stride divides evenly (conv.jl:194-201)
+    assert oracle.convtransposesize(64, 2, 2, 0, 1, 0) == 128 and oracle.convtransposesize(8, 3, 2, 0, 1, 0) == 17
+    for n, k, s_, p_, d_ in [(37, 14, 14, 0, 1), (64, 3, 1, 1, 1), (17, 3, 2, 1, 2)]:
+        o = oracle.convtransposesize(n, k, s_, p_, d_, 0)
+        assert oracle.convsize(o, k, s_, p_, d_) == n
+    # kernel == stride: out[co][iy*KH+ky][ix*KW+kx] = sum_ci x[ci][iy][ix] w[ci][co][ky][kx]  (conv.jl:211-222)
+    x = oracle.randn_f16((2, 5, 3, 4), 4)
+    w = oracle.randn_f16((5, 3, 2, 3), 5)
+    got = oracle.convtranspose2d_f16(x, w, None, (2, 3), out_f32=True)
+    y = np.einsum("ncyx,cokl->noykxl", x.astype(np.float64), w.astype(np.float64)).reshape(2, 3, 6, 12)
+    assert got.shape == y.shape and np.max(np.abs(got - y)) < 1e-4
+    # and it is the adjoint of the convolution with the same weights: <conv(u), x> == <u, convT(x)>
+    u = oracle.randn_f16((1, 3, 9, 11), 6)
+    wc = oracle.randn_f16((4, 3, 3, 3), 7)                        # conv weight [Cout=4][Cin=3]; as convT weight: Cin=4 -> Cout=3
+    v = oracle.randn_f16((1, 4, 4, 5), 8)
+    cu = oracle.conv2d_f16(u, wc, None, (2, 2), (0, 0), out_f32=True).astype(np.float64)
+    tv = oracle.convtranspose2d_f16(v, wc, None, (2, 2), out_f32=True).astype(np.float64)
+    assert cu.shape == v.shape and tv.shape == u.shape
+    assert abs(np.sum(cu * v.astype(np.float64)) - np.sum(tv * u.astype(np.float64))) < 1e-3
+
+
 # ------------------------------------------------------------------ layer norm / add
 
 @pytest.mark.parametrize("C", [1280, 384, 37])
