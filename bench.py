@@ -398,6 +398,24 @@ def detail_benchmarks(lib, L, stream, only=None):
         out["c4_conv3x3_256to256_64x64"] = {"us": round(med * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 2),
                                             "frac_mfma_peak": round(flop / med / 1e12 / PEAK_F16_TFLOPS, 4)}
 
+    def convt_case(name, Cin, Hi, Cout):
+        # SAM 2's mask-decoder upsamplers: kernel 2, stride 2 (test_convtranspose_gemm.jl:36)
+        if only is not None and only not in name:
+            return
+        x = torch.randn((1, Cin, Hi, Hi), dtype=f16, device="cuda")
+        w = torch.randn((Cin, Cout, 2, 2), dtype=f16, device="cuda") * 0.05
+        b = torch.randn((Cout,), dtype=f16, device="cuda") * 0.02
+        o = torch.empty((1, Cout, 2 * Hi, 2 * Hi), dtype=f16, device="cuda")
+        geo = (Hi, Hi, Cin, 1, 2, 2, Cout, 2, 2, 0, 0, 1, 1, 0, 0, 1)
+        need = lib.mi_convtranspose2d_f16_workspace(*geo)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        call = Call(lib.mi_convtranspose2d_f16, o.data_ptr(), x.data_ptr(), w.data_ptr(), b.data_ptr(), *geo, ws.data_ptr(), need, stream)
+        med, lo, hi = event_time(call, 10)
+        flop = 2.0 * Hi * Hi * Cin * Cout * 4
+        io = 2.0 * (Cin * Hi * Hi + Cout * 4 * Hi * Hi + Cin * Cout * 4)
+        out[name] = {"us": round(med * 1e6, 2), "us_min": round(lo * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 2),
+                     "io_GB/s": round(io / med / 1e9, 1)}
+
     def decode_cases():
         # config 5: decode-sized linears (HBM-bound on the weights; enough rotating weight sets to exceed the
         # 256 MB last-level cache) and single-query attention over the caches
@@ -437,6 +455,8 @@ def detail_benchmarks(lib, L, stream, only=None):
     attn_case("c4_attn_L4096_16x64", 1, 16, 4096, 4096, 64)
     if only is None or only in "c4_conv3x3_256to256_64x64":
         conv_case()
+    convt_case("sam2_upsample_convT2x2_256to64_64x64", 256, 64, 64)
+    convt_case("sam2_upsample_convT2x2_64to32_128x128", 64, 128, 32)
     decode_cases()
     if only is not None:
         return {k: v for k, v in out.items() if only in k}

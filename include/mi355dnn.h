@@ -230,6 +230,17 @@ int mi_convtranspose2d_f16_plan(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
 /* ATen's transposed-convolution output extent -- convtransposesize, conv.jl:201. */
 int64_t mi_convtransposesize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d, int64_t op);
 
+/* ---------------------------------------------------------------- layout
+ * in is an (E,L,H,B) fp16 operand given by its four element strides (any non-negative
+ * values; a zero broadcasts); out receives it as (L,E,H,B), L contiguous: dense when
+ * out_strides is NULL, else by its own strides (out_strides[0] must be 1).  With H = B = 1
+ * this is the 2-D transpose out[e][l] = in[l][e].
+ * Replaces transposeLE(ctx, a) / toLE_tiled_Float16! -- attention.jl:342-396.  The
+ * reference's other layout pass, padcols_kernel! (matmul.jl:182-185), has no counterpart:
+ * mi_gemm_f16 takes ragged T, K, F as they are. */
+int mi_transpose_le_f16(void *out, const int64_t out_strides[4], const void *in, const int64_t in_strides[4],
+                        int64_t E, int64_t L, int64_t H, int64_t B, void *stream);
+
 /* ---------------------------------------------------------------- layer norm + glue
  * `groups` rows of C contiguous fp16 elements; mean in fp32, variance about that
  * mean in fp32, out = (x-mean)*rstd*gamma + beta rounded to fp16; mean/rstd

@@ -10,7 +10,7 @@ graphs in the reference's JSON schema.
 """
 from . import _lib  # noqa: F401
 from .kernels import (Ctx, Decline, DeclineError, DeviceCaps, MI355X, Workspace, add_, batchedmatmul_, caps, conv_plan,
-                      convolution_, convolutiontranspose_, convsize, convtranspose_plan, convtransposesize, layernorm_, ln_matmul_, matmul_, mmplan, sdpa, sdpaplan)
+                      convolution_, convolutiontranspose_, convsize, convtranspose_plan, convtransposesize, layernorm_, ln_matmul_, matmul_, mmplan, sdpa, sdpaplan, transposeLE_)
 
 __all__ = ["Ctx", "Decline", "DeclineError", "DeviceCaps", "MI355X", "Workspace", "add_", "batchedmatmul_", "caps",
-           "conv_plan", "convolution_", "convolutiontranspose_", "convsize", "convtranspose_plan", "convtransposesize", "layernorm_", "ln_matmul_", "matmul_", "mmplan", "sdpa", "sdpaplan"]
+           "conv_plan", "convolution_", "convolutiontranspose_", "convsize", "convtranspose_plan", "convtransposesize", "layernorm_", "ln_matmul_", "matmul_", "mmplan", "sdpa", "sdpaplan", "transposeLE_"]

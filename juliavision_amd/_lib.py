@@ -49,6 +49,7 @@ SIGNATURES = {
     "mi_convtranspose2d_f16_workspace": (_sz, [_i64] * 16),
     "mi_convtranspose2d_f16_plan": (_int, [_i64] * 16),
     "mi_convtransposesize": (_i64, [_i64] * 6),
+    "mi_transpose_le_f16": (_int, [_vp, _i64p, _vp, _i64p, _i64, _i64, _i64, _i64, _vp]),
     "mi_layernorm_f16": (_int, [_vp] * 6 + [_i64, _i64, _f32, _vp]),
     "mi_add_f16": (_int, [_vp, _vp, _vp, _i64, _vp]),
     "mi_kv_append_f16": (_int, [_vp, _vp, _i64p, _i64, _vp, _vp, _i64p, _vp, _i64, _i64, _i64, _vp]),

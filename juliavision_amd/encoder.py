@@ -1,0 +1,123 @@
+"""Encoder-side compositions of the kernel entry points: a pre-LN transformer block and a
+ViT-style encoder (patch embedding as convolution-as-GEMM, class token, position
+embedding, blocks, final norm).
+
+The reference runs these as exported op graphs (WhisperRunner/src/WhisperRunner.jl's
+``encode``; DepthAnythingRunner's ViT-S/14 backbone); here they are the same op sequence
+issued directly, seven launches per block: layer norm, one GEMM for the three projections,
+fused attention reading q/k/v in place and writing token-major, the output projection with
+the residual in its epilogue, layer norm, the GELU GEMM, and the second MLP GEMM with the
+residual in its epilogue.  Nothing allocates after construction, so a whole encoder can be
+captured and replayed (``decode.StepGraph``).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+from .kernels import Ctx, add_, convolution_, convsize, layernorm_, matmul_, sdpa, transposeLE_
+
+
+@dataclass
+class EncoderLayerWeights:
+    """One pre-LN block.  Linear weights are ``(K, F)`` tensors in either memory layout; ``wqkv`` is the
+    three projections side by side, ``(d, 3d)``."""
+    ln1_g: torch.Tensor
+    ln1_b: torch.Tensor
+    wqkv: torch.Tensor
+    bqkv: torch.Tensor
+    wo: torch.Tensor
+    bo: torch.Tensor
+    ln2_g: torch.Tensor
+    ln2_b: torch.Tensor
+    w1: torch.Tensor
+    b1: torch.Tensor
+    w2: torch.Tensor
+    b2: torch.Tensor
+
+
+class EncoderBuffers:
+    """Activation slots of one block, allocated once and reused by every layer."""
+
+    def __init__(self, tokens: int, d_model: int, ffn: int, device="cuda"):
+        e = lambda n: torch.empty((tokens, n), dtype=torch.float16, device=device)
+        self.h, self.qkv, self.att, self.x1, self.f = e(d_model), e(3 * d_model), e(d_model), e(d_model), e(ffn)
+
+
+def encoder_layer(ctx: Ctx, W: EncoderLayerWeights, x: torch.Tensor, out: torch.Tensor, buf: EncoderBuffers, heads: int,
+                  eps: float = 1e-5, act: str = "gelu"):
+    """``out = x1 + W2 act(W1 LN2(x1))`` with ``x1 = x + Wo attention(LN1(x))``; ``x``, ``out``: ``(T, d)`` fp16
+    (``out`` may be ``x``, which is last read as the output projection's residual)."""
+    T, d = x.shape
+    E = d // heads
+    layernorm_(ctx, buf.h, None, None, x, W.ln1_g, W.ln1_b, d, eps)
+    ctx.ws.reset()
+    matmul_(ctx, buf.qkv, W.wqkv, buf.h, W.bqkv)
+    # q, k, v are column bands of the projection, heads are 64-wide column bands of those: (B,H,L,E) views, no copy
+    q, k, v = (buf.qkv[:, i * d:(i + 1) * d].unflatten(1, (heads, E)).permute(1, 0, 2).unsqueeze(0) for i in range(3))
+    ctx.ws.reset()
+    sdpa(ctx, q, k, v, out=buf.att.unflatten(1, (heads, E)).permute(1, 0, 2).unsqueeze(0))
+    ctx.ws.reset()
+    matmul_(ctx, buf.x1, W.wo, buf.att, W.bo, residual=x)
+    layernorm_(ctx, buf.h, None, None, buf.x1, W.ln2_g, W.ln2_b, d, eps)
+    ctx.ws.reset()
+    matmul_(ctx, buf.f, W.w1, buf.h, W.b1, epi=act)
+    ctx.ws.reset()
+    matmul_(ctx, out, W.w2, buf.f, W.b2, residual=buf.x1)
+    return out
+
+
+@dataclass
+class ViTWeights:
+    """Patch embedding ``patch_w (d, 3, P, P)``, ``patch_b (d,)``; ``cls (1, d)``; ``pos (1 + patches, d)``;
+    the blocks; the final norm."""
+    patch_w: torch.Tensor
+    patch_b: torch.Tensor
+    cls: torch.Tensor
+    pos: torch.Tensor
+    layers: List[EncoderLayerWeights]
+    norm_g: Optional[torch.Tensor] = None
+    norm_b: Optional[torch.Tensor] = None
+
+
+class ViTEncoder:
+    """ViT-style encoder over one image: ``tokens = [cls; patches] + pos`` and the blocks in sequence."""
+
+    def __init__(self, W: ViTWeights, image_hw, heads: int, ffn: int, eps: float = 1e-6, device="cuda"):
+        self.W, self.heads, self.eps = W, heads, eps
+        d, cin, P, _ = W.patch_w.shape
+        self.P = P
+        self.gh, self.gw = convsize(image_hw[0], P, P, 0, 1), convsize(image_hw[1], P, P, 0, 1)
+        self.T = 1 + self.gh * self.gw
+        if tuple(W.pos.shape) != (self.T, d) or tuple(W.cls.shape) != (1, d):
+            raise ValueError(f"pos must be ({self.T}, {d}) and cls (1, {d})")
+        f16 = torch.float16
+        self.patches = torch.empty((1, d, self.gh, self.gw), dtype=f16, device=device)      # channel-major, as the convolution writes
+        self.tokens = [torch.empty((self.T, d), dtype=f16, device=device) for _ in range(2)]
+        self.out = torch.empty((self.T, d), dtype=f16, device=device)
+        self.buf = EncoderBuffers(self.T, d, ffn, device)
+
+    def embed(self, ctx: Ctx, image: torch.Tensor):
+        """``image``: (1, 3, H, W) fp16.  Fills and returns ``tokens[0]``."""
+        W, tok = self.W, self.tokens[0]
+        ctx.ws.reset()
+        convolution_(ctx, self.patches, image, W.patch_w, W.patch_b, (self.P, self.P), (0, 0), (1, 1), 1)
+        # channel-major (d, patches) -> token-major rows 1.. of the token matrix
+        transposeLE_(ctx, tok[1:], self.patches.view(W.patch_w.shape[0], self.T - 1))
+        add_(ctx, tok[1:], tok[1:], W.pos[1:])
+        add_(ctx, tok[:1], W.cls, W.pos[:1])
+        return tok
+
+    def __call__(self, ctx: Ctx, image: torch.Tensor):
+        W = self.W
+        src = self.embed(ctx, image)
+        for i, lw in enumerate(W.layers):
+            dst = self.tokens[(i + 1) % 2]
+            encoder_layer(ctx, lw, src, dst, self.buf, self.heads, self.eps)
+            src = dst
+        if W.norm_g is None:
+            return src
+        layernorm_(ctx, self.out, None, None, src, W.norm_g, W.norm_b, src.shape[1], self.eps)
+        return self.out

@@ -461,6 +461,26 @@ def convolutiontranspose_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, 
     return out
 
 
+# ----------------------------------------------------------------------------- layout
+
+def transposeLE_(ctx: Ctx, out, a):
+    """transposeLE(ctx, a) -- attention.jl:374-396.  ``a`` torch (B,H,L,E) fp16 with any strides (the reference's
+    (E,L,H,B)); ``out`` torch (B,H,E,L) fp16 whose last axis is contiguous.  2-D tensors are taken as H = B = 1:
+    ``out (C,R) = a (R,C)`` transposed."""
+    if a.dim() == 2 and out.dim() == 2:
+        a, out = a[None, None], out[None, None]
+    if not _is_f16_cuda(a, out) or a.dim() != 4 or out.dim() != 4:
+        raise DeclineError("transposeLE_: operands", L.DECLINE_OPERANDS)
+    B, H, Ln, E = a.shape
+    if tuple(out.shape) != (B, H, E, Ln) or (Ln > 1 and out.stride(3) != 1):
+        raise DeclineError("transposeLE_: out must be (B,H,E,L) with L contiguous", L.DECLINE_OPERANDS)
+    ost = L.strides4(1, out.stride(2) if E > 1 else Ln, out.stride(1), out.stride(0))
+    rc = L.init().mi_transpose_le_f16(out.data_ptr(), ost, a.data_ptr(), _strides_elbh(a), E, Ln, H, B, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_transpose_le_f16", rc)
+    return out
+
+
 # ----------------------------------------------------------------------------- layer norm, add
 
 def layernorm_(ctx: Ctx, out, mean, rstd, a, gamma, beta, C_: int, eps: float):

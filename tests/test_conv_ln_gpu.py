@@ -195,3 +195,36 @@ def test_add_bit_exact(ctx):
         jv.add_(ctx, out, to_dev(a), to_dev(b))
         torch.cuda.synchronize()
         assert np.array_equal(to_host(out).view(np.uint16), oracle.add_f16(a, b).view(np.uint16))
+
+
+@pytest.mark.parametrize("B,H,Ln,E", [(1, 1, 384, 1369), (2, 3, 70, 64), (1, 20, 33, 65), (1, 2, 1, 40), (3, 1, 50, 1)])
+@pytest.mark.parametrize("source", ["dense", "token_major", "already_l_fastest"])
+def test_transpose_le_moves_bits(ctx, B, H, Ln, E, source):
+    """(E,L,H,B) strided -> dense (L,E,H,B), the contract of transposeLE (attention.jl:374-396); exact."""
+    import torch
+    import juliavision_amd as jv
+    vals = oracle.randn_f16((B, H, Ln, E), 17)
+    if source == "dense":
+        a = to_dev(vals)
+    elif source == "token_major":                     # a (B,L,H,E) buffer seen as (B,H,L,E): heads are column bands of token rows
+        a = to_dev(np.ascontiguousarray(vals.transpose(0, 2, 1, 3))).permute(0, 2, 1, 3)
+    else:                                             # memory already runs along l: the strided-copy kernel
+        a = to_dev(np.ascontiguousarray(vals.transpose(0, 1, 3, 2))).permute(0, 1, 3, 2)
+    assert np.array_equal(to_host(a), vals)
+    out = poison(torch.empty((B, H, E, Ln), dtype=torch.float16, device="cuda"))
+    jv.transposeLE_(ctx, out, a)
+    assert np.array_equal(to_host(out), vals.transpose(0, 1, 3, 2))
+    # into a wider destination: rows of a larger matrix, the columns beside them untouched
+    wide = poison(torch.empty((B, H, E, Ln + 5), dtype=torch.float16, device="cuda"))
+    jv.transposeLE_(ctx, wide[..., 2:2 + Ln], a)
+    got = to_host(wide)
+    assert np.array_equal(got[..., 2:2 + Ln], vals.transpose(0, 1, 3, 2)) and np.all(np.isnan(got[..., :2])) and np.all(np.isnan(got[..., 2 + Ln:]))
+
+
+def test_transpose_le_2d_is_the_matrix_transpose(ctx):
+    import torch
+    import juliavision_amd as jv
+    w = oracle.randn_f16((100, 37), 3)
+    out = poison(torch.empty((37, 100), dtype=torch.float16, device="cuda"))
+    jv.transposeLE_(ctx, out, to_dev(w))
+    assert np.array_equal(to_host(out), w.T)
