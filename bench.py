@@ -316,6 +316,50 @@ def decode_step_case(steps=100):
             "frac_hbm_peak_graph": round(nbytes / replay / 1e9 / PEAK_HBM_GBS, 4)}
 
 
+def vit_encoder_case(steps=50):
+    """BASELINE config 3 as a whole: ViT-S/14 at 518 x 518 (patch embedding as convolution-as-GEMM, class token and
+    position embedding, 12 pre-LN blocks of 1370 tokens x 384 with 6 x 64 heads and a 1536 MLP, final norm), eager
+    and replayed as one captured graph.  92.78 GFLOP in the blocks + 0.62 in the patch embedding."""
+    import time
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd.decode import StepGraph
+    from juliavision_amd.encoder import EncoderLayerWeights, ViTEncoder, ViTWeights
+    d, H, ffn, P, S, NL = 384, 6, 1536, 14, 518, 12
+    T = 1 + 37 * 37
+    ctx = jv.Ctx("cuda")
+    f16 = torch.float16
+    w = lambda k, f: torch.randn((k, f), dtype=f16, device="cuda") * 0.02
+    v = lambda n, m=0.0: torch.randn((n,), dtype=f16, device="cuda") * 0.02 + m
+    layers = [EncoderLayerWeights(v(d, 1.0), v(d), w(d, 3 * d), v(3 * d), w(d, d), v(d), v(d, 1.0), v(d), w(d, ffn), v(ffn), w(ffn, d), v(d))
+              for _ in range(NL)]
+    W = ViTWeights(torch.randn((d, 3, P, P), dtype=f16, device="cuda") * 0.02, v(d), w(1, d), w(T, d), layers, v(d, 1.0), v(d))
+    enc = ViTEncoder(W, (S, S), H, ffn)
+    image = torch.rand((1, 3, S, S), dtype=f16, device="cuda")
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    run = lambda: enc(ctx, image)
+    eager = timed(run)
+    embed = timed(lambda: enc.embed(ctx, image))
+    graph = StepGraph(run)
+    replay = timed(graph.replay)
+    if not bool(torch.isfinite(enc.out).all()):
+        raise RuntimeError("ViT encoder produced non-finite output")
+    flop = NL * (2.0 * T * d * (3 * d + d + 2 * ffn) + 4.0 * T * T * 64 * H) + 2.0 * (T - 1) * 588 * d
+    return {"eager_ms": round(eager * 1e3, 4), "graph_ms": round(replay * 1e3, 4), "patch_embed_eager_us": round(embed * 1e6, 1),
+            "launches": 5 + 7 * NL + 1, "GFLOP": round(flop / 1e9, 2), "TFLOP/s_graph": round(flop / replay / 1e12, 1),
+            "frac_mfma_peak_graph": round(flop / replay / 1e12 / PEAK_F16_TFLOPS, 4)}
+
+
 def detail_benchmarks(lib, L, stream, only=None):
     import numpy as np
     import torch
@@ -446,6 +490,10 @@ def detail_benchmarks(lib, L, stream, only=None):
             name = f"c5_decoder_layer_b{bsz}_{tag}"
             if only is None or only in name:
                 out[name] = decoder_layer_case(bsz, lay)
+
+    name = "c3_vit_s14_518_encoder_12layers"
+    if only is None or only in name:
+        out[name] = vit_encoder_case()
 
     name = "c5_decode_step_4layers_vocab51866_b1"
     if only is None or only in name:

@@ -912,6 +912,8 @@ bool mfma_addressable(const GemmArgs &a, bool b_kn) {
 
 template <int BM, int BN, int WM, int WN>
 int launch_pipe(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
+    // the kernel always walks at least two 64-deep tiles (its prologue fetches two ahead): one tile would read past K
+    if (a.K < 128 || a.K % 64) return MI_DECLINE_EXTENT;
     a.tiles_m = (int)ceil_div(a.M, BM);
     a.tiles_n = (int)ceil_div(a.N, BN);
     a.group_m = a.tiles_m < 6 ? a.tiles_m : 6;

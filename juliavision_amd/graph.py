@@ -46,6 +46,13 @@ VIEW_OPS = {"view.default", "_unsafe_view.default", "reshape.default", "transpos
 DROP_OPS = {"_assert_tensor_metadata.default", "_assert_scalar.default", "sym_constrain_range_for_size.default"}
 LINEAR_OPS = {"linear.default", "addmm.default", "mm.default"}
 ACTIVATIONS = {"gelu.default": "gelu", "relu.default": "relu"}
+# The fused-attention ops an exported graph can hold: the composite one, and the backend-specific ones it becomes
+# when the program is decomposed on an accelerator (ops.jl:1365-1391).  Value: positions of (dropout_p, is_causal)
+# among the positional arguments; the backend forms return a tuple whose first element is the attention output.
+SDPA_OPS = {"scaled_dot_product_attention.default": (4, 5),
+            "_scaled_dot_product_flash_attention.default": (3, 4),
+            "_scaled_dot_product_flash_attention_for_cpu.default": (3, 4),
+            "_scaled_dot_product_efficient_attention.default": (5, 6)}
 
 
 class UnsupportedOp(NotImplementedError):
@@ -184,14 +191,20 @@ class Graph:
 # ----------------------------------------------------------------------------- rewrites
 
 def fold_activations(g: Graph) -> Graph:
-    """gelu / relu whose only producer is a linear op read by nothing else becomes that op's epilogue
-    (foldrelu.jl:60-125); the activation's buffer then aliases the linear's output."""
+    """gelu / relu whose only producer is a linear op -- directly or through a chain of views, as the
+    decomposed ``addmm`` + ``view`` form of ``linear`` has it -- read by nothing else becomes that op's
+    epilogue (foldrelu.jl:60-125); the activation's buffer then aliases what it used to read.  An
+    elementwise function commutes with any view, so the chain may reshape or permute freely."""
     for act in [o for o in g.ops if o["aten"] in ACTIVATIONS]:
         if act["aten"] == "gelu.default" and act["attrs"].get("approximate", "none") != "none":
             continue                                    # only the erf form is the folded epilogue's arithmetic
         src = act["in"][0]
-        prod = g.op(src)
-        if prod is None or prod["aten"] not in LINEAR_OPS or g.readers(src) != [act["id"]] or src in g.outputs:
+        chain = [src]
+        while g.buffers[chain[-1]]["kind"] == "view":
+            chain.append(g.buffers[chain[-1]]["of"])
+        prod = g.op(chain[-1])
+        single = g.readers(src) == [act["id"]] and all(len(g.readers(c)) == 1 for c in chain[1:]) and not any(c in g.outputs for c in chain)
+        if prod is None or prod["aten"] not in LINEAR_OPS or not single or "epilogue" in prod["attrs"] or "residual" in prod["attrs"]:
             continue
         prod["attrs"]["epilogue"] = ACTIVATIONS[act["aten"]]
         g.ops.remove(act)
@@ -236,9 +249,11 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
     ``permute(0, 2, 1, 3)``): the kernel writes token-major, the swap becomes the view it already is, and
     the ``reshape`` that follows is a free view instead of a copy."""
     for o in g.ops:
-        if o["aten"] != "scaled_dot_product_attention.default":
+        if o["aten"] not in SDPA_OPS:
             continue
         rd = g.readers(o["id"])
+        if len(rd) == 1 and "getitem" in g.buffers[rd[0]].get("op", "") and g.buffers[rd[0]]["attrs"].get("arg1", 0) == 0:
+            rd = g.readers(rd[0])                       # the tuple-returning forms: look past the selection of element 0
         if len(rd) != 1 or g.buffers[rd[0]]["kind"] != "view":
             continue
         v = g.buffers[rd[0]]
@@ -279,14 +294,17 @@ class Executor:
                 raise UnsupportedOp(f"{graph.name}: no kernel on this path for aten.{o['aten']} (op {o['id']})")
         for o in graph.ops:
             b = graph.buffers[o["out"]]
-            if "shape" not in b:
+            if "shape" in b:
+                shape, dtype = list(b["shape"]), b["dtype"]
+            elif o["aten"] in SDPA_OPS:                   # a tuple result: only the attention output is materialised
+                shape, dtype = list(b["shapes"][0]), b["dtypes"][0]
+            else:
                 continue
-            shape = list(b["shape"])
             if o["attrs"].get("token_major"):             # (B, H, L, E) stored as (B, L, H, E)
-                self.t[o["out"]] = torch.empty([shape[0], shape[2], shape[1], shape[3]], dtype=_DTYPES[b["dtype"]],
+                self.t[o["out"]] = torch.empty([shape[0], shape[2], shape[1], shape[3]], dtype=_DTYPES[dtype],
                                                device=self.device).transpose(1, 2)
             else:
-                self.t[o["out"]] = torch.empty(shape, dtype=_DTYPES[b["dtype"]], device=self.device)
+                self.t[o["out"]] = torch.empty(shape, dtype=_DTYPES[dtype], device=self.device)
 
     # -- operands
     def get(self, bid: str) -> torch.Tensor:
@@ -371,10 +389,13 @@ class Executor:
 
     def _sdpa(self, o):
         a = o["attrs"]
-        if a.get("is_causal") or a.get("dropout_p", 0.0) not in (0, 0.0) or a.get("enable_gqa"):
+        pd, pc = SDPA_OPS[o["aten"]]
+        dropout = a.get("dropout_p", a.get(f"arg{pd}", 0.0))
+        causal = a.get("is_causal", a.get(f"arg{pc}", False))
+        if causal or dropout not in (0, 0.0) or a.get("enable_gqa"):
             raise UnsupportedOp(f"{o['id']}: causal flag / dropout / gqa are not exported on this path (masks arrive as attn_mask)")
         q, k, v = (self.get(i) for i in o["in"][:3])
-        bias = self.get(o["in"][3]) if len(o["in"]) > 3 else None
+        bias = self.get(o["in"][3]) if len(o["in"]) > 3 else None       # attn_mask / attn_bias, positional or keyword
         self.ctx.ws.reset()
         K.sdpa(self.ctx, q, k, v, bias, a.get("scale"), out=self.t[o["out"]])
 
@@ -434,7 +455,7 @@ class Executor:
             K.convolution_(self.ctx, out, x, w, bias, xy(stride), xy(padding), xy(dilation), a.get("arg8", 1))
 
     HANDLERS = {"linear.default": _linear, "addmm.default": _linear, "mm.default": _linear,
-                "scaled_dot_product_attention.default": _sdpa, "layer_norm.default": _layer_norm,
+                **dict.fromkeys(SDPA_OPS, _sdpa), "layer_norm.default": _layer_norm,
                 "native_layer_norm.default": _native_layer_norm, "add.Tensor": _add,
                 "gelu.default": _activation, "relu.default": _activation, "convolution.default": _convolution}
 

@@ -180,3 +180,70 @@ def test_exported_upsampler_runs_transposed_and_lifted_1d_convolutions(ctx):
     torch.cuda.synchronize()
     assert tuple(got.shape) == want.shape == (1, 8, 512)
     assert_parity(got.float().cpu().numpy(), want, what="exported upsampler")
+
+
+def _decomposed(m, keep_sdpa=True):
+    """The block exported and lowered to core ops as the reference's exporter does (export_graphs.py:277-279):
+    linear becomes addmm/mm over permuted weights, layer_norm native_layer_norm.  On a CPU the composite
+    attention op would be lowered to its matmul + softmax form; keeping it stands in for the fused op an
+    accelerator export holds."""
+    import torch
+    ep, x = _export(m)
+    table = torch.export.default_decompositions()
+    if keep_sdpa:
+        table.pop(torch.ops.aten.scaled_dot_product_attention.default, None)
+    return ep.run_decompositions(table), x
+
+
+def _as_backend_attention(d, name):
+    """Rewrite the dictionary's composite attention op into a tuple-returning backend form with the same
+    operands, as `_scaled_dot_product_flash_attention` / `_efficient_attention` appear in accelerator exports."""
+    import copy
+    d = copy.deepcopy(d)
+    op = next(o for o in d["ops"] if o["aten"] == "scaled_dot_product_attention.default")
+    old = op["id"]
+    b = next(b for b in d["buffers"] if b["id"] == old)
+    op["aten"] = name
+    op["attrs"] = {"arg3": 0.0, "arg4": False} if "flash" in name else {"arg4": True, "arg5": 0.0, "arg6": False}
+    tup = {"id": old + "_tuple", "kind": "transient", "shapes": [b["shape"], [1, 2, 70], None], "dtypes": [b["dtype"], "float32", None],
+           "live": b.get("live")}
+    op["id"] = op["out"] = tup["id"]
+    b.update(kind="view", of=tup["id"], op="<built-in function getitem>", attrs={"arg1": 0})
+    d["buffers"].append(tup)
+    return d
+
+
+def test_decomposed_export_folds_like_the_composite_one():
+    from juliavision_amd import graph as G
+    ep, _ = _decomposed(_block())
+    d = G.convert(ep, "block")
+    aten = [o["aten"] for o in d["ops"]]
+    assert aten.count("addmm.default") == 5 and aten.count("mm.default") == 1 and aten.count("native_layer_norm.default") == 2
+    g = G.optimize(G.Graph.load(d))
+    assert [o["aten"] for o in g.ops].count("gelu.default") == 0 and len(g.ops) == 9
+    fc1 = next(o for o in g.ops if o["attrs"].get("epilogue") == "gelu")
+    assert fc1["aten"] == "addmm.default" and g.root("gelu") == fc1["id"]       # gelu read the addmm through a view
+    assert sum("residual" in o["attrs"] for o in g.ops) == 2
+    for name in ("_scaled_dot_product_flash_attention.default", "_scaled_dot_product_efficient_attention.default"):
+        g2 = G.optimize(G.Graph.load(_as_backend_attention(d, name)))
+        att = next(o for o in g2.ops if o["aten"] == name)
+        assert att["attrs"]["token_major"] is True and len(g2.ops) == 9
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("attention", ["scaled_dot_product_attention.default", "_scaled_dot_product_flash_attention.default",
+                                       "_scaled_dot_product_efficient_attention.default"])
+def test_decomposed_export_runs_on_the_kernels(ctx, attention):
+    import torch
+    from juliavision_amd import graph as G
+    m = _block(seed=4)
+    ep, x = _decomposed(m)
+    d = G.convert(ep, "block")
+    if attention != "scaled_dot_product_attention.default":
+        d = _as_backend_attention(d, attention)
+    run = G.Executor(G.optimize(G.Graph.load(d)), m.state_dict(), ctx)
+    with torch.no_grad():
+        want = m.float()(x.float()).numpy()
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    assert_parity(got.float().cpu().numpy(), want, what=f"decomposed block, {attention}")
