@@ -5,8 +5,10 @@
 (declared in ``include/mi355dnn.h``).  Importing this package loads nothing; the
 shared object is opened on first use and its absence is an error, never a fallback.
 ``juliavision_amd.decode`` holds the device-resident KV cache and the replayable
-decoder-layer step, ``juliavision_amd.graph`` a loader/executor for exported op
-graphs in the reference's JSON schema.
+decoder-layer step, ``juliavision_amd.encoder`` the encoder block and a ViT-style
+encoder composed from the same entry points, ``juliavision_amd.graph`` a loader/executor
+for exported op graphs in the reference's JSON schema, ``juliavision_amd.safetensors``
+the weight-file reader.
 """
 from . import _lib  # noqa: F401
 from .kernels import (Ctx, Decline, DeclineError, DeviceCaps, MI355X, Workspace, add_, batchedmatmul_, caps, conv_plan,

@@ -16,6 +16,15 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(half_t *out, float *
     const half_t *row = a + g * C;
     float x[NCH][8];
     float s = 0.0f;
+    // gamma and beta are requested together with the row: one trip to memory for the kernel, not two
+    u32x4 graw[NCH], braw[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        graw[i] = (gamma && e0 < C) ? ldg16(gamma + e0) : z;
+        braw[i] = (beta && e0 < C) ? ldg16(beta + e0) : z;
+    }
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
         const int e0 = (lane + 64 * i) * 8;
@@ -47,9 +56,8 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(half_t *out, float *
     for (int i = 0; i < NCH; i++) {
         const int e0 = (lane + 64 * i) * 8;
         if (e0 < C) {
-            half8v gv, bv, o;
-            if (gamma) gv = as_half8(ldg16(gamma + e0));
-            if (beta) bv = as_half8(ldg16(beta + e0));
+            const half8v gv = as_half8(graw[i]), bv = as_half8(braw[i]);
+            half8v o;
 #pragma unroll
             for (int j = 0; j < 8; j++)
                 o[j] = ln_norm1(x[i][j], mu, r, gamma != nullptr, gamma ? (float)gv[j] : 0.0f, beta != nullptr, beta ? (float)bv[j] : 0.0f);

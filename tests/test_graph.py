@@ -247,3 +247,21 @@ def test_decomposed_export_runs_on_the_kernels(ctx, attention):
     got = run(x.cuda())
     torch.cuda.synchronize()
     assert_parity(got.float().cpu().numpy(), want, what=f"decomposed block, {attention}")
+
+
+@pytest.mark.gpu
+def test_executor_takes_weights_from_a_safetensors_file(ctx, tmp_path):
+    """Graph JSON + weights file, the two artifacts the reference's Model(dir, weights) is built from (driver.jl:165-168)."""
+    import torch
+    from safetensors.torch import save_file
+    from juliavision_amd import graph as G
+    from juliavision_amd import safetensors as ST
+    m = _block(seed=6)
+    ep, x = _export(m)
+    (tmp_path / "block.json").write_text(json.dumps(G.convert(ep, "block")))
+    save_file({k: v.float().contiguous() for k, v in m.state_dict().items()}, str(tmp_path / "block.safetensors"))   # stored in fp32
+    g = G.optimize(G.Graph.load(json.loads((tmp_path / "block.json").read_text())))
+    run = G.Executor(g, ST.load_to(str(tmp_path / "block.safetensors"), "cuda", torch.float16), ctx)
+    with torch.no_grad():
+        want = m.float()(x.float()).numpy()
+    assert_parity(run(x.cuda()).float().cpu().numpy(), want, what="block from graph JSON + safetensors")
