@@ -80,22 +80,31 @@ __device__ __forceinline__ void static_for(F &&f) {
 // exponentials (with the next block's first product underneath) the other is in its second product:
 // the matrix pipe and the vector ALU of a SIMD are then busy with different waves instead of both
 // waves wanting the same unit at the same time.  Waves 0-3 do all the global -> LDS staging.
-template <int EP, bool PP>
-__global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
-    constexpr int BC = 64, BR = PP ? 256 : 128, NT = 256;     // NT: threads that stage K and V
+//
+// KH = 2 (grids that leave every CU at most one workgroup): eight waves on 128 queries.  Waves w and w+4 own the
+// same 32 queries and share a SIMD; a stage holds 128 keys, of which waves 0-3 take the first 64 and waves 4-7 the
+// second, so each wave walks half of the keys and a SIMD always has a second wave to run.  The two partial
+// (O, M, l) of a query meet in LDS at the end (the merge identity of flash.jl:1385-1391), waves 0-3 store.
+template <int EP, bool PP, int KH = 1>
+__global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 64 && !PP && KH == 1) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
+    static_assert(KH == 1 || (KH == 2 && !PP), "key halves or ping-pong, not both");
+    constexpr int BC = 64, BR = PP ? 256 : 128, NT = KH == 2 ? 512 : 256;     // NT: threads that stage K and V
+    constexpr int BCS = BC * KH;                                                // keys per LDS stage
     constexpr int KLD = EP + 8, VLD = EP + 32;
     constexpr int KS = EP / 16;       // k16 steps over the head dim
     constexpr int ET = EP / 32;       // 32-wide head-dim tiles of O
     constexpr int KCH = EP / 8;       // 16-byte chunks per key row
-    constexpr int PER = BC * KCH / NT;
+    constexpr int PER = BCS * KCH / NT;
     constexpr float TH = 8.0f;
     extern __shared__ __align__(16) char smem[];
-    half_t (*Ks)[BC * KLD] = reinterpret_cast<half_t (*)[BC * KLD]>(smem);
-    half_t (*Vs)[BC * VLD] = reinterpret_cast<half_t (*)[BC * VLD]>(smem + 3 * BC * KLD * 2);
+    half_t (*Ks)[BCS * KLD] = reinterpret_cast<half_t (*)[BCS * KLD]>(smem);
+    half_t (*Vs)[BCS * VLD] = reinterpret_cast<half_t (*)[BCS * VLD]>(smem + 3 * BCS * KLD * 2);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int tid = threadIdx.x & 255;                       // index among the staging threads
-    const int grp = wave >> 2;                               // PP: 0 = waves 0-3, 1 = waves 4-7
+    const int tid = threadIdx.x & (NT - 1);                  // index among the staging threads
+    const int grp = wave >> 2;                               // PP, KH = 2: 0 = waves 0-3, 1 = waves 4-7
+    const int qw = KH == 2 ? (wave & 3) : wave;              // which 32 queries of the block
+    const int gk = KH == 2 ? grp * BC : 0;                   // this wave's first key within a stage
     const bool loader = !PP || grp == 0;
     const int hl = lane >> 5, l32 = lane & 31;
     // Workgroups are dealt to the 8 XCDs round-robin in launch order; renumbering them so that each XCD
@@ -116,7 +125,7 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     // key blocks and leaves (O, M, l) partials for sdpa_merge_kernel instead of the normalised output.
     const int split = PP ? 0 : qblk % p.nsplit;
     if (!PP) qblk /= p.nsplit;
-    const int q0 = qblk * BR + wave * 32;
+    const int q0 = qblk * BR + qw * 32;
     const half_t *qb = p.q + h * p.qs[2] + b * p.qs[3];
     const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
     const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
@@ -170,7 +179,7 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     }
     auto load_into = [&](u32x4 (&kx)[PER], u32x4 (&vx)[PER], int key0) {
         const u32x4 z = {0u, 0u, 0u, 0u};
-        if (key0 + BC <= LkLoad && p.E == EP) {   // the common case: no predicate, no clamp
+        if (key0 + BCS <= LkLoad && p.E == EP) {   // the common case: no predicate, no clamp
             const long ko = (long)key0 * p.ks[1], vo = (long)key0 * p.vs[1];
 #pragma unroll
             for (int i = 0; i < PER; i++) {
@@ -217,11 +226,11 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     // Three LDS stages: while block j is in its softmax and second product, the first
     // product of block j+1 already runs (its MFMAs fill the matrix pipe under the
     // exponentials), and block j+2 is on its way from memory into the third stage.
-    const int nblk = (Lk + BC - 1) / BC;
+    const int nblk = (Lk + BCS - 1) / BCS;
     {
         u32x4 kr1[PER], vr1[PER];
         if (nblk > 0 && loader) load_kv(0);
-        if (nblk > 1 && loader) load_into(kr1, vr1, BC);
+        if (nblk > 1 && loader) load_into(kr1, vr1, BCS);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             const half8v t = as_half8(qraw[ks]);
@@ -234,8 +243,8 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     __syncthreads();
 
     // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
-    const int vtoff = (4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-    const int ktoff = l32 * KLD + 8 * hl;
+    const int vtoff = (gk + 4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const int ktoff = (gk + l32) * KLD + 8 * hl;
     const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // t = s*scale*log2(e) - M, straight out of the MFMA chain
@@ -272,10 +281,10 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     // One key block: sc holds its scores (computed one iteration earlier), sn receives the next block's.
     auto iter = [&](auto MASK_, float16v (&sc)[2], float16v (&sn)[2], int j) {
         constexpr bool MASK = decltype(MASK_)::value;
-        const int key0 = j * BC;
+        const int key0 = j * BCS + gk;
         const int st = j % 3, st1 = (j + 1) % 3, st2 = (j + 2) % 3;
         const bool next2 = j + 2 < nblk && loader;
-        if (next2) load_kv(key0 + 2 * BC);
+        if (next2) load_kv((j + 2) * BCS);
         if constexpr (MASK) {           // the ragged last block: excluded keys get -inf
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
@@ -294,6 +303,10 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
         half8v pf[2][2];
         float l_new = l_run;
         probs(sc, pf, l_new);
+        // the largest exponent of the block, three at a time: what tells that a probability left fp16 range
+        float tmax = fmaxf(sc[0][0], sc[1][0]);
+#pragma unroll
+        for (int r = 1; r < 16; r++) tmax = fmaxf(fmaxf(tmax, sc[0][r]), sc[1][r]);
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * KS, 0);
 #pragma unroll
         for (int g = 0; g < 2 * KS + 2; g++) {
@@ -301,14 +314,12 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
             __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + 2), 0);     // the remaining vector work trails the last MFMA
         }
         __builtin_amdgcn_sched_barrier(0);
-        // A probability that left fp16 range (t >= 16) shows up as an infinite row sum.  Then, and on
-        // the first block, settle a new reference point: the block maximum, for the rows that outgrew
-        // the old one by 2^TH; rescale what was accumulated; redo the exponentials.
-        if (__any(first || !(l_new < INFINITY))) {
-            float mx = fmaxf(sc[0][0], sc[1][0]);
-#pragma unroll
-            for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sc[0][r]), sc[1][r]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        // A probability leaves fp16 range at t >= 16 (2^16 rounds to infinity; the row sum, kept in fp32 from the
+        // unrounded values, would not show it).  Then, and on the first block, settle a new reference point: the
+        // block maximum, for the rows that outgrew the old one by 2^TH; rescale what was accumulated; redo the
+        // exponentials.
+        if (__any(first || tmax >= 15.9f)) {
+            float mx = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
             const bool grow = (mx > TH || first) && mx != -INFINITY;
             const half_t m16 = (half_t)(m_ref + (grow ? mx : 0.0f));
             const float d = (float)m16 - m_ref;
@@ -359,23 +370,61 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
             __syncthreads();
         }
     };
-    const int nfull = Lk / BC;           // blocks with every key valid
+    // blocks in which every key of this wave is valid (with KH = 2: its half of the stage)
+    const int nfull = KH == 2 ? (Lk - gk + BC) / BCS : Lk / BC;
     if (PP && grp == 1) pp_barrier();    // waves 4-7 run half a block behind waves 0-3
     int j = 0;
     for (; j + 2 <= nfull; j += 2) {
         iter(std::false_type{}, sa, sb, j);
         iter(std::false_type{}, sb, sa, j + 1);
     }
-    if (j < nfull) {
-        iter(std::false_type{}, sa, sb, j);
-        if (j + 1 < nblk) iter(std::true_type{}, sb, sa, j + 1);
-    } else if (j < nblk) {
-        iter(std::true_type{}, sa, sb, j);
+    if constexpr (KH == 1) {
+        if (j < nfull) {
+            iter(std::false_type{}, sa, sb, j);
+            if (j + 1 < nblk) iter(std::true_type{}, sb, sa, j + 1);
+        } else if (j < nblk) {
+            iter(std::true_type{}, sa, sb, j);
+        }
+    } else {
+        // Both halves of the workgroup run all nblk blocks (every block has a workgroup barrier), whatever
+        // share of them is masked for this half: at most one full block is left here, then masked ones.
+        if (j < nblk) { if (j < nfull) iter(std::false_type{}, sa, sb, j); else iter(std::true_type{}, sa, sb, j); j++; }
+        if (j < nblk) { iter(std::true_type{}, sb, sa, j); j++; }
+        if (j < nblk) { iter(std::true_type{}, sa, sb, j); j++; }
     }
 
     if (PP && grp == 0) pp_barrier();    // ... so waves 0-3 meet their last barrier here
     // Both lanes of a query hold half of its row sum.
     l_run += __shfl_xor(l_run, 32, 64);
+
+    if constexpr (KH == 2) {
+        // Waves 4-7 hand their (O, M, l) to the wave that owns the same queries; the last block's barrier has
+        // passed, so the stages are idle.  Lane-major slots: the partner's lane holds the same elements.
+        constexpr int SLOT = (ET * 16 + 2) * 64;
+        float *xo = reinterpret_cast<float *>(smem + 36864) + qw * SLOT;
+        static_assert(36864 + 4 * SLOT * 4 <= 3 * BCS * (KLD + VLD) * 2 && 4 * 32 * (EP + 4) * 4 <= 36864, "merge slots overlap the store staging or leave the stages");
+        if (grp == 1) {
+#pragma unroll
+            for (int t = 0; t < ET; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) xo[(t * 16 + r) * 64 + lane] = o_acc[t][r];
+            xo[(ET * 16) * 64 + lane] = m_ref;
+            xo[(ET * 16 + 1) * 64 + lane] = l_run;
+        }
+        __syncthreads();
+        if (grp == 1) return;
+        const float m1 = xo[(ET * 16) * 64 + lane], l1 = xo[(ET * 16 + 1) * 64 + lane];
+        // a side that saw no valid key has l = 0 and a meaningless reference point
+        const float ma = l_run > 0.0f ? m_ref : -INFINITY, mb = l1 > 0.0f ? m1 : -INFINITY;
+        const float mm = fmaxf(ma, mb);
+        const float a0 = l_run > 0.0f ? __builtin_amdgcn_exp2f(ma - mm) : 0.0f, a1 = l1 > 0.0f ? __builtin_amdgcn_exp2f(mb - mm) : 0.0f;
+#pragma unroll
+        for (int t = 0; t < ET; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o_acc[t][r] = o_acc[t][r] * a0 + xo[(t * 16 + r) * 64 + lane] * a1;
+        l_run = l_run * a0 + l1 * a1;
+        m_ref = mm;
+    }
 
     // out(e, q, h, b); lane owns query q0 + l32 and, per tile t and group g, the four head-dim values
     // e = 32 t + 8 g + 4 hl + 0..3: stored from the registers, a wave's store instruction would touch 32 rows
@@ -385,8 +434,8 @@ __global__ __launch_bounds__(PP ? 512 : 256, (EP <= 64 && !PP) ? 2 : 1) void fla
     const bool partial = !PP && p.nsplit > 1;
     const bool as_f32 = partial || p.out_f32;
     constexpr int SLF = EP + 4, SLH = EP + 8;              // staged row lengths (floats, halves)
-    float *stf = reinterpret_cast<float *>(smem) + wave * 32 * SLF;
-    half_t *sth = reinterpret_cast<half_t *>(smem) + wave * 32 * SLH;
+    float *stf = reinterpret_cast<float *>(smem) + qw * 32 * SLF;
+    half_t *sth = reinterpret_cast<half_t *>(smem) + qw * 32 * SLH;
     const float inv = partial ? 1.0f : (l_run > 0.0f ? 1.0f / l_run : 0.0f);
     const long rows = (long)p.B * p.H * p.Lq;
     if (partial && hl == 0 && q0 + l32 < p.Lq) {
@@ -745,6 +794,7 @@ int mi_sdpa_init() {
     int bad = 0;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     return bad;
 }
@@ -808,7 +858,10 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
                 a.nsplit = 1;
             }
             dim3 grid((unsigned)(ceil_div(Lq, 128) * a.nsplit), (unsigned)H, (unsigned)B);
-            if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false>), grid, dim3(256), flash_lds_bytes(64), st, a);
+            // no CU would hold two workgroups anyway: eight waves per workgroup, each with half of the keys
+            const bool halves = E <= 64 && a.nsplit == 1 && ceil_div(Lq, 128) * H * B <= (int64_t)mi_num_cus() && Lk >= 256;
+            if (halves)       hipLaunchKernelGGL((flash_fwd_kernel<64, false, 2>), grid, dim3(512), 2 * flash_lds_bytes(64), st, a);
+            else if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false>), grid, dim3(256), flash_lds_bytes(64), st, a);
             else         hipLaunchKernelGGL((flash_fwd_kernel<128, false>), grid, dim3(256), flash_lds_bytes(128), st, a);
             if (a.nsplit > 1) {
                 const long total = (long)Lq * H * B * E;

@@ -211,3 +211,58 @@ def test_fused_kernel_splits_keys_on_small_grids(ctx):
     assert rc == 0
     torch.cuda.synchronize()
     assert_parity(to_host(out), oracle.sdpa_ref_f32(q, k, v), what="no workspace: one pass")
+
+
+@pytest.mark.parametrize("Lk", [256, 257, 319, 320, 321, 383, 384, 385, 447, 448, 449, 1000])
+@pytest.mark.parametrize("Lq,E", [(64, 64), (130, 64), (200, 32)])
+def test_fused_kernel_key_halves_on_one_workgroup_per_cu_grids(ctx, Lq, Lk, E):
+    """Grids of at most one workgroup per CU with 256 keys or more run eight waves, each pair of waves sharing its
+    queries and taking alternate 64-key halves of a 128-key stage; the halves merge in LDS.  Key counts around the
+    64- and 128-key boundaries: the second half's last block empty, ragged, exactly full."""
+    q, k, v = _qkv(2, 3, Lq, Lk, E, 211 + Lk)
+    _check(ctx, q, k, v, expect="FlashPlan", what=f"key halves Lq{Lq} Lk{Lk} E{E}")
+
+
+def test_fused_kernel_key_halves_masks_and_layouts(ctx):
+    import torch
+    import juliavision_amd as jv
+    q, k, v = _qkv(6, 2, 150, 300, 64, 251)
+    # kv_len leaves the second half of the keys without a valid one (10, 64), with exactly one (65), a ragged
+    # second stage (129, 200), and a row of the batch with none at all (0)
+    got = _check(ctx, q, k, v, kv_len=[10, 64, 65, 129, 0, 200], out_dtype="f32", expect="FlashPlan", what="key halves with kv_len")
+    assert np.all(got[4] == 0)
+    # large scores: the reference point has to move in one half and not the other
+    q2 = q.copy()
+    q2[:, :, :, :] *= np.float16(6.0)
+    k2 = k.copy()
+    k2[:, :, 64:128] *= np.float16(3.0)
+    _check(ctx, q2, k2, v, expect="FlashPlan", what="key halves, one half with far larger scores")
+    # token-major output and packed strided q/k/v, as the encoder block calls it
+    B, H, L, E = 1, 6, 260, 64
+    qkv = oracle.randn_f16((L, 3 * H * E), 261)
+    dqkv = to_dev(qkv)
+    views = [dqkv[:, i * H * E:(i + 1) * H * E].unflatten(1, (H, E)).permute(1, 0, 2).unsqueeze(0) for i in range(3)]
+    buf = poison(torch.empty((L, H * E), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.sdpa(ctx, *views, None, None, out=buf.unflatten(1, (H, E)).permute(1, 0, 2).unsqueeze(0))
+    torch.cuda.synchronize()
+    hq, hk, hv = (np.ascontiguousarray(qkv[:, i * H * E:(i + 1) * H * E].reshape(L, H, E).transpose(1, 0, 2))[None] for i in range(3))
+    want = oracle.sdpa_ref_f32(hq, hk, hv)
+    assert_parity(to_host(buf).reshape(L, H, E).transpose(1, 0, 2)[None], want, what="key halves, token-major")
+
+
+@pytest.mark.parametrize("B,H,Lq,Lk,which", [(1, 2, 128, 200, "four waves"), (4, 16, 300, 200, "eight waves, 256 queries"),
+                                             (1, 3, 128, 400, "key halves"), (1, 2, 200, 2000, "key splits")])
+def test_reference_point_follows_scores_that_grow_along_the_keys(ctx, B, H, Lq, Lk, which):
+    """The fused kernel exponentiates against a reference point that it moves only when it must.  Keys whose scores
+    exceed everything before them by far more than fp16's exponent range (here by up to ~2^60 from one 64-key block
+    to a later one, for some queries and not for others) must move it; attention then is nearly one-hot on them."""
+    q, k, v = _qkv(B, H, Lq, Lk, 64, 301)
+    q = (q.astype(np.float32) * 3.0).astype(np.float16)
+    k = k.copy()
+    k[:, :, 70:75] *= np.float16(4.0)            # second block
+    k[:, :, 150:152] *= np.float16(8.0)          # third block: dominates for the queries aligned with it
+    if Lk > 330:
+        k[:, :, 330] *= np.float16(10.0)
+    got = _check(ctx, q, k, v, expect="FlashPlan", what=f"growing scores, {which}")
+    assert np.all(np.isfinite(got))
