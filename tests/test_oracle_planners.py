@@ -1,0 +1,66 @@
+"""The reference's integer planner functions (restated in oracle/planners.py) against the reference's own known
+answers, and the one rule of theirs the product keeps: two workgroups per core when splitting keys."""
+from oracle import planners as P
+
+
+def test_shared_memory_budgets_of_the_reference_tilings():
+    # test_flash.jl:84-94
+    assert not P.flashfits(72, 64, 64, 256) and P.flashshared(72, 64, 64) > P.PORTABLE_SHARED_FLOOR
+    assert P.flashfits(72, 64, 32, 256) and P.flashshared(72, 64, 32) <= P.PORTABLE_SHARED_FLOOR
+    assert P.flashfits(72, 32, 32, 256) and P.flashfits(72, 32, 32, 128)
+    # flash.jl:1170-1171: 64x32 at EP = 80 asks 48 904 bytes of the 48 KB budget, 248 to spare; 64x64 is refused
+    assert P.flashcmshared(80, 64, 32) == 48904 and 48 * 1024 - 48904 == 248
+    assert P.flashcmshared(80, 64, 64) > 48 * 1024
+    assert P.flashcmfits(16, 32, 48 * 1024, 80, 64, 32, 256) and not P.flashcmfits(16, 32, 48 * 1024, 80, 64, 64, 256)
+    assert P.flashepad(64) == 8 and P.flashepad(80) == 0
+
+
+def test_crs_padding_table():
+    # conv_coopmat.jl:107-110
+    assert P.crsextent(147) == 160 and P.crs_admitted(147)
+    assert P.crsextent(17) == 32 and not P.crs_admitted(17)
+    assert P.crsextent(257) == 288 and P.crs_admitted(257)
+    assert P.crsextent(769) == 800 and P.crs_admitted(769)
+    assert P.crsextent(48) == 48                      # conv_coopmat.jl:50-53: 64/48 = 1.33 blows the budget, the tile pad is kept
+    assert P.crsextent(588) == 608                    # config 3's patch embedding, 14 x 14 x 3
+
+
+def test_key_split_rule():
+    # two workgroups per core; every split a whole number of key blocks; no split when the grid already fills the device
+    assert P.splitcount(48, 1, 1500, 64, 32, 20) == 4          # 20 head-rows on 48 cores: want 4, 47 blocks -> chunks of 12
+    assert P.splitcount(48, 1500, 1500, 64, 32, 20) == 1
+    assert P.splitcount(48, 1, 32, 64, 32, 20) == 1            # a single key block
+    assert P.splitcount(0, 1, 1500, 64, 32, 20) == 1
+    for (cores, Lq, Lk, BR, BC, nb) in [(256, 1, 1500, 1, 64, 20), (256, 1, 448, 1, 64, 160), (48, 23, 4096, 64, 32, 8)]:
+        n = P.splitcount(cores, Lq, Lk, BR, BC, nb)
+        nkb = P.cld(Lk, BC)
+        chunk = P.cld(nkb, n)
+        assert (n - 1) * chunk < nkb <= n * chunk             # no empty split
+        assert n * P.cld(Lq, BR) * nb <= max(2 * cores, P.cld(Lq, BR) * nb) + P.cld(Lq, BR) * nb
+
+
+def test_decode_attention_keeps_the_two_workgroups_per_core_rule():
+    """mi_sdpa_f16_plan's split count for single-query attention aims, like splitcount (flash.jl:1288-1303), at two
+    workgroups per core (256 CUs, 64-key blocks, one query row per workgroup): min(ceil(2 CUs / rows), blocks, 64).
+    Equal to the reference's count at config 5's batch 1; elsewhere never fewer splits than the reference's rule,
+    which rounds the wanted count down and re-derives it from equal whole-block chunks."""
+    import ctypes as C
+    from juliavision_amd import _lib as L
+    lib = L.load()
+
+    def nsplit(E, Lq, Lk, H, B):
+        ns = C.c_int(0)
+        st = L.strides4(1, E, E * Lq, E * Lq * H)
+        sk = L.strides4(1, E, E * Lk, E * Lk * H)
+        path = lib.mi_sdpa_f16_plan(0x10000, st, 0x20000, sk, 0x30000, sk, 0, 1, E, Lq, Lk, H, B, 0.125, C.byref(ns))
+        assert L.SDPA_PATHS[path] == "rows"
+        return ns.value
+
+    assert nsplit(64, 1, 1500, 20, 1) == P.splitcount(256, 1, 1500, 1, 64, 20) == 24
+    assert nsplit(64, 1, 448, 20, 1) == P.splitcount(256, 1, 448, 1, 64, 20) == 7
+    for (Lq, Lk, H, B) in [(1, 1500, 20, 4), (1, 1500, 20, 8), (1, 448, 20, 4), (1, 448, 20, 8), (1, 4096, 8, 1), (1, 100, 2, 1),
+                           (23, 4096, 8, 1), (5, 100, 2, 1), (1, 17, 4, 1), (1, 64, 1, 1), (1, 100000, 1, 1)]:
+        rows = Lq * H * B
+        mine = nsplit(64, Lq, Lk, H, B)
+        assert mine == max(1, min(P.cld(2 * 256, rows), P.cld(Lk, 64), 64)), (Lq, Lk, H, B)
+        assert mine >= min(64, P.splitcount(256, Lq, Lk, 1, 64, H * B)), (Lq, Lk, H, B)
