@@ -675,6 +675,115 @@ __global__ __launch_bounds__(256) void sdpa_rows_kernel(SdpaArgs p) {
     }
 }
 
+// Single query row per (head, batch), whole key range in one workgroup of 8 waves: nothing to merge in a second
+// launch.  A wave takes keys 8 at a time (8 lanes per key, one 16-byte chunk of the head dim each) with a stride
+// of 64 keys, in rounds of SD_U passes whose K and V loads are all issued before the first is used, the next
+// round's before the current round is consumed: about 190 KB in flight per workgroup.
+constexpr int SD_U = 6;
+__global__ __launch_bounds__(512) void sdpa_decode_kernel(SdpaArgs p) {
+    __shared__ float red_ml[8][2];
+    __shared__ float red_o[8][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = lane >> 3, cl = lane & 7;
+    const int h = blockIdx.x, b = blockIdx.z;
+    int Lk = p.Lk;
+    if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
+    const half_t *qp = p.q + h * p.qs[2] + b * p.qs[3];
+    const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
+    const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
+    const int e0 = cl * 8;
+    const bool eok = e0 < p.E;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    u32x4 kc[2][SD_U], vc[2][SD_U];
+    // pass t of this wave covers keys 64 t + 8 wave + grp
+    auto fetch = [&](int set, int t0) {
+#pragma unroll
+        for (int u = 0; u < SD_U; u++) {
+            const int key = 64 * (t0 + u) + 8 * wave + grp;
+            const int kk = min(key, Lk - 1);
+            const bool on = eok && 64 * (t0 + u) < Lk;           // uniform over the workgroup in its second half
+            kc[set][u] = on ? ldg16(kb + (long)kk * p.ks[1] + e0) : z;
+            vc[set][u] = on ? ldg16(vb + (long)kk * p.vs[1] + e0) : z;
+        }
+    };
+    const int npass = (Lk + 63) / 64;
+    if (npass > 0) fetch(0, 0);
+    if (npass > SD_U) fetch(1, SD_U);
+    float qv[8];
+    {
+        const half8v t = as_half8(eok ? ldg16(qp + e0) : z);
+#pragma unroll
+        for (int j = 0; j < 8; j++) qv[j] = (float)t[j] * p.scale;
+    }
+    float m = -INFINITY, l = 0.0f, acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) acc[j] = 0.0f;
+    auto consume = [&](int set, int t0) {
+#pragma unroll
+        for (int u = 0; u < SD_U; u++) {
+            if (64 * (t0 + u) < Lk) {                            // uniform: the shuffles below need the whole wave
+                const int key = 64 * (t0 + u) + 8 * wave + grp;
+                const half8v kt = as_half8(kc[set][u]), vt = as_half8(vc[set][u]);
+                float d = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; j++) d = fmaf(qv[j], (float)kt[j], d);
+                d += __shfl_xor(d, 1, 64);
+                d += __shfl_xor(d, 2, 64);
+                d += __shfl_xor(d, 4, 64);
+                const float sc = key < Lk ? d : -INFINITY;
+                const float mn = fmaxf(m, sc);
+                const float mu = mn == -INFINITY ? 0.0f : mn;
+                const float al = __expf(m - mu), pw = __expf(sc - mu);
+                l = l * al + pw;
+                m = mn;
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc[j] = fmaf(pw, (float)vt[j], acc[j] * al);
+            }
+        }
+    };
+    for (int t0 = 0; t0 < npass; t0 += 2 * SD_U) {
+        consume(0, t0);
+        if (t0 + 2 * SD_U < npass) fetch(0, t0 + 2 * SD_U);
+        if (t0 + SD_U < npass) consume(1, t0 + SD_U);
+        if (t0 + 3 * SD_U < npass) fetch(1, t0 + 3 * SD_U);
+    }
+    // merge the 8 groups of the wave, then the 8 waves through LDS (flash.jl:1385-1391)
+#pragma unroll
+    for (int o = 8; o < 64; o <<= 1) {
+        const float mo = __shfl_xor(m, o, 64), lo = __shfl_xor(l, o, 64);
+        const float mn = fmaxf(m, mo);
+        const float mu = mn == -INFINITY ? 0.0f : mn;
+        const float a0 = __expf(m - mu), a1 = __expf(mo - mu);
+        l = l * a0 + lo * a1;
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[j] = acc[j] * a0 + __shfl_xor(acc[j], o, 64) * a1;
+        m = mn;
+    }
+    if (lane < 8) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) red_o[wave][cl * 8 + j] = acc[j];
+        if (lane == 0) { red_ml[wave][0] = m; red_ml[wave][1] = l; }
+    }
+    __syncthreads();
+    if (tid < p.E) {
+        float mm = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 8; w++) mm = fmaxf(mm, red_ml[w][0]);
+        const float mu = mm == -INFINITY ? 0.0f : mm;
+        float L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            const float a = __expf(red_ml[w][0] - mu);
+            L += a * red_ml[w][1];
+            O += a * red_o[w][tid];
+        }
+        const float r = L > 0.0f ? O / L : 0.0f;
+        const long oo = (long)b * p.os[3] + (long)h * p.os[2] + (long)tid * p.os[0];
+        if (p.out_f32) reinterpret_cast<float *>(p.out)[oo] = r;
+        else reinterpret_cast<half_t *>(p.out)[oo] = (half_t)r;
+    }
+}
+
 // One thread per (row, e): merges the key splits (attn_flash_cm_merge!, flash.jl:1398-1421).
 __global__ void sdpa_merge_kernel(SdpaArgs p) {
     const long rows = (long)p.B * p.H * p.Lq;
@@ -754,6 +863,14 @@ int flash_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     return (int)want;
 }
 
+// A single query row over a short key range (the decoder's self-attention over its cache) runs in one launch, one
+// workgroup per (head, batch): 7.1 us against 8.2 us for splits + merge at 448 keys, 3.9 us against 6.9 us at 4, and
+// the work follows the device-side kv_len.  Longer ranges need more workgroups than heads to pull on HBM: 1500 keys
+// take 14.7 us this way at batch 1, 10.1 us split 24 ways.
+bool one_pass_decode(const SdpaArgs &a, bool vec) {
+    return a.Lq == 1 && vec && !a.bias && a.E <= 64 && a.Lk >= 1 && a.Lk <= 640;
+}
+
 int sdpa_path(const SdpaArgs &a) {
     if (a.E < 1 || a.E > 256 || a.Lq < 0 || a.Lk < 0 || a.H < 1 || a.B < 1) return MI_SDPA_DECLINE;
     if (a.H > 65535 || a.B > 65535 || (int64_t)a.Lq * a.H * 64 > INT32_MAX) return MI_SDPA_DECLINE;
@@ -821,7 +938,8 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
                   zero4, nullptr, E, Lq, Lk, H, B, scale);
     if (rc != MI_OK) return MI_SDPA_DECLINE;
     int path = sdpa_path(a);
-    if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? rows_splits(Lq, Lk, H, B)
+    const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
+    if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? (one_pass_decode(a, vec) ? 1 : rows_splits(Lq, Lk, H, B))
                                   : path == MI_SDPA_FLASH ? flash_splits(Lq, Lk, H, B) : 1;
     return path;
 }
@@ -873,6 +991,11 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
     }
     // rows path
     bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
+    if (one_pass_decode(a, vec)) {
+        a.nsplit = 1;
+        hipLaunchKernelGGL(sdpa_decode_kernel, dim3((unsigned)H, 1, (unsigned)B), dim3(512), 0, st, a);
+        return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+    }
     a.nsplit = Lq < 64 ? rows_splits(Lq, Lk, H, B) : 1;
     if (a.nsplit > 1) {
         size_t rows = (size_t)Lq * H * B;

@@ -99,7 +99,8 @@ def test_sdpa_planner():
     p1, n1 = _sdpa_plan(64, 1, 1500, 20, 1)
     p8, n8 = _sdpa_plan(64, 1, 1500, 20, 8)
     assert p1 == p8 == "rows" and n1 == 24 and 1 <= n8 < n1
-    assert _sdpa_plan(64, 1, 448, 20, 1)[1] == 7
+    assert _sdpa_plan(64, 1, 448, 20, 1) == ("rows", 1)                      # a short key range: one launch, one workgroup per head
+    assert _sdpa_plan(64, 1, 700, 20, 1)[1] == 11
     assert _sdpa_plan(64, 23, 17, 4, 1)[1] == 1
 
 

@@ -42,8 +42,9 @@ def test_key_split_rule():
 def test_decode_attention_keeps_the_two_workgroups_per_core_rule():
     """mi_sdpa_f16_plan's split count for single-query attention aims, like splitcount (flash.jl:1288-1303), at two
     workgroups per core (256 CUs, 64-key blocks, one query row per workgroup): min(ceil(2 CUs / rows), blocks, 64).
-    Equal to the reference's count at config 5's batch 1; elsewhere never fewer splits than the reference's rule,
-    which rounds the wanted count down and re-derives it from equal whole-block chunks."""
+    Equal to the reference's count at config 5's cross-attention at batch 1; elsewhere never fewer splits than the
+    reference's rule, which rounds the wanted count down and re-derives it from equal whole-block chunks.  A single
+    query over at most 640 keys is not split at all."""
     import ctypes as C
     from juliavision_amd import _lib as L
     lib = L.load()
@@ -57,9 +58,10 @@ def test_decode_attention_keeps_the_two_workgroups_per_core_rule():
         return ns.value
 
     assert nsplit(64, 1, 1500, 20, 1) == P.splitcount(256, 1, 1500, 1, 64, 20) == 24
-    assert nsplit(64, 1, 448, 20, 1) == P.splitcount(256, 1, 448, 1, 64, 20) == 7
-    for (Lq, Lk, H, B) in [(1, 1500, 20, 4), (1, 1500, 20, 8), (1, 448, 20, 4), (1, 448, 20, 8), (1, 4096, 8, 1), (1, 100, 2, 1),
-                           (23, 4096, 8, 1), (5, 100, 2, 1), (1, 17, 4, 1), (1, 64, 1, 1), (1, 100000, 1, 1)]:
+    assert nsplit(64, 1, 700, 20, 1) == P.splitcount(256, 1, 700, 1, 64, 20) == 11
+    assert nsplit(64, 1, 448, 20, 1) == nsplit(64, 1, 448, 20, 8) == 1         # up to 640 keys: a single launch, no splits
+    for (Lq, Lk, H, B) in [(1, 1500, 20, 4), (1, 1500, 20, 8), (1, 700, 20, 4), (1, 1000, 20, 8), (1, 4096, 8, 1), (3, 100, 2, 1),
+                           (23, 4096, 8, 1), (5, 100, 2, 1), (2, 17, 4, 1), (7, 64, 1, 1), (1, 100000, 1, 1)]:
         rows = Lq * H * B
         mine = nsplit(64, Lq, Lk, H, B)
         assert mine == max(1, min(P.cld(2 * 256, rows), P.cld(Lk, 64), 64)), (Lq, Lk, H, B)
