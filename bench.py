@@ -259,7 +259,7 @@ def decoder_layer_case(bsz, layout="kf", steps=200):
     replay = timed(graph.replay)
     weights = 2.0 * (3 * d * d + 3 * d * d + 2 * d * ffn)
     kv = 2.0 * 2 * bsz * H * E * (448 + 1500)
-    return {"eager_us": round(eager * 1e6, 1), "graph_us": round(replay * 1e6, 1), "launches": (18 if layout == "kf" else 12) + (3 if bsz > 4 else 0),
+    return {"eager_us": round(eager * 1e6, 1), "graph_us": round(replay * 1e6, 1), "launches": (16 if layout == "kf" else 10) + (3 if bsz > 4 else 0),
             "GB/s_graph": round((weights + kv) / replay / 1e9, 1), "frac_hbm_peak_graph": round((weights + kv) / replay / 1e9 / PEAK_HBM_GBS, 4)}
 
 
@@ -311,7 +311,7 @@ def decode_step_case(steps=100):
     if not bool(torch.isfinite(logits).all()):
         raise RuntimeError("decode step produced non-finite logits")
     nbytes = NL * 2.0 * (3 * d * d + 3 * d * d + 2 * d * ffn) + 2.0 * d * V + NL * 2.0 * 2 * H * E * (448 + 1500)
-    return {"eager_us": round(eager * 1e6, 1), "graph_us": round(replay * 1e6, 1), "launches": 1 + NL * 12 + 1,
+    return {"eager_us": round(eager * 1e6, 1), "graph_us": round(replay * 1e6, 1), "launches": 1 + NL * 9 + 1,
             "MB_per_token": round(nbytes / 1e6, 1), "GB/s_graph": round(nbytes / replay / 1e9, 1),
             "frac_hbm_peak_graph": round(nbytes / replay / 1e9 / PEAK_HBM_GBS, 4)}
 

@@ -274,6 +274,18 @@ int mi_kv_append_f16(void *cache_k, void *cache_v, const int64_t cache_strides[4
                      const void *k_new, const void *v_new, const int64_t new_strides[4],
                      const int32_t *kv_len, int64_t E, int64_t H, int64_t B, void *stream);
 
+/* mi_kv_append_f16 and mi_sdpa_f16 (Lq = 1) in one launch, for the decoder's self-attention: the key/value row of
+ * the newest token (k_new, v_new: 1 x E per head and batch, element strides new_strides as (E, L, H, B)) is taken
+ * as key kv_len[b] - 1 and written into that slot of the cache on the way; out = attention of q over the first
+ * kv_len[b] keys.  cache_k / cache_v are written to.  Only what the single-launch kernel covers (E <= 64, at most
+ * 640 cache slots, 16-byte addressable rows); MI_DECLINE_UNSUPPORTED otherwise, and the caller makes the two calls.
+ * Replaces index_put + cat + scaled_dot_product_attention of the exported decoder step
+ * (WhisperRunner/src/decode.jl:186-203, tools/export_whisper_decoder.py). */
+int mi_sdpa_append_f16(void *out, int out_dtype, const int64_t out_strides[4],
+                       const void *q, const int64_t q_strides[4],
+                       void *cache_k, const int64_t k_strides[4], void *cache_v, const int64_t v_strides[4],
+                       const void *k_new, const void *v_new, const int64_t new_strides[4],
+                       const int32_t *kv_len, int64_t E, int64_t Lk, int64_t H, int64_t B, float scale, void *stream);
 /* kv_len[b] = clamp(kv_len[b] + delta, 0, cap) for b < B, on the device
  * (KVCache.position += 1, decode.jl:201, without the host in the loop). */
 int mi_kv_advance(int32_t *kv_len, int64_t B, int32_t delta, int32_t cap, void *stream);

@@ -26,6 +26,10 @@ struct SdpaArgs {
     long bs[4];                    // (Lk, Lq, H, B) element strides, 0 = broadcast
     const int *kv_len;
     float *part_o, *part_ml;       // split partials: [split][row][E], [split][row][2]
+    // sdpa_decode_kernel only: the newest key/value row (1 x E per head and batch); when set, key kv_len - 1 is
+    // taken from here instead of the cache and written into the cache on the way (k, v are then written to)
+    const half_t *k_new, *v_new;
+    long ns[4];
     int E, Lq, Lk, H, B;
     int out_f32, bias_f32, nsplit;
     float scale;
@@ -702,8 +706,15 @@ __global__ __launch_bounds__(512) void sdpa_decode_kernel(SdpaArgs p) {
             const int key = 64 * (t0 + u) + 8 * wave + grp;
             const int kk = min(key, Lk - 1);
             const bool on = eok && 64 * (t0 + u) < Lk;           // uniform over the workgroup in its second half
-            kc[set][u] = on ? ldg16(kb + (long)kk * p.ks[1] + e0) : z;
-            vc[set][u] = on ? ldg16(vb + (long)kk * p.vs[1] + e0) : z;
+            const bool fresh = p.k_new && kk == Lk - 1;          // the row that this step appends
+            const half_t *kp = fresh ? p.k_new + h * p.ns[2] + b * p.ns[3] : kb + (long)kk * p.ks[1];
+            const half_t *vp = fresh ? p.v_new + h * p.ns[2] + b * p.ns[3] : vb + (long)kk * p.vs[1];
+            kc[set][u] = on ? ldg16(kp + e0) : z;
+            vc[set][u] = on ? ldg16(vp + e0) : z;
+            if (fresh && on && key == Lk - 1) {                  // exactly eight lanes of the workgroup own it
+                *reinterpret_cast<u32x4 *>(const_cast<half_t *>(kb) + (long)kk * p.ks[1] + e0) = kc[set][u];
+                *reinterpret_cast<u32x4 *>(const_cast<half_t *>(vb) + (long)kk * p.vs[1] + e0) = vc[set][u];
+            }
         }
     };
     const int npass = (Lk + 63) / 64;
@@ -864,8 +875,9 @@ int flash_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
 }
 
 // A single query row over a short key range (the decoder's self-attention over its cache) runs in one launch, one
-// workgroup per (head, batch): 7.1 us against 8.2 us for splits + merge at 448 keys, 3.9 us against 6.9 us at 4, and
-// the work follows the device-side kv_len.  Longer ranges need more workgroups than heads to pull on HBM: 1500 keys
+// workgroup per (head, batch): back to back 7.1 us against 8.2 us for splits + merge at 448 keys, 3.9 us against
+// 6.9 us at 4 (inside a dependent chain at 448 keys the two forms tie, the single launch at about 10 us of its own);
+// the work follows the device-side kv_len and the cache write can ride along (mi_sdpa_append_f16).  Longer ranges need more workgroups than heads to pull on HBM: 1500 keys
 // take 14.7 us this way at batch 1, 10.1 us split 24 ways.
 bool one_pass_decode(const SdpaArgs &a, bool vec) {
     return a.Lq == 1 && vec && !a.bias && a.E <= 64 && a.Lk >= 1 && a.Lk <= 640;
@@ -893,6 +905,8 @@ int fill(SdpaArgs &a, void *out, int out_dtype, const int64_t *os, const void *q
     else { a.os[0] = 1; a.os[1] = E; a.os[2] = E * Lq; a.os[3] = E * Lq * H; }
     a.bias = bias; a.bias_f32 = bias_dtype == MI_F32; a.kv_len = kv_len;
     a.part_o = a.part_ml = nullptr;
+    a.k_new = a.v_new = nullptr;
+    for (int i = 0; i < 4; i++) a.ns[i] = 0;
     a.E = (int)E; a.Lq = (int)Lq; a.Lk = (int)Lk; a.H = (int)H; a.B = (int)B;
     a.out_f32 = out_dtype == MI_F32; a.nsplit = 1; a.scale = scale;
     return MI_OK;
@@ -1014,6 +1028,28 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
         long total = (long)Lq * H * B * E;
         hipLaunchKernelGGL(sdpa_merge_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, a);
     }
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+// Decode step, self-attention: append the newest key/value row to the cache and attend over the cache in one launch.
+int mi_sdpa_append_f16(void *out, int out_dtype, const int64_t out_strides[4],
+                       const void *q, const int64_t q_strides[4],
+                       void *cache_k, const int64_t k_strides[4], void *cache_v, const int64_t v_strides[4],
+                       const void *k_new, const void *v_new, const int64_t new_strides[4],
+                       const int32_t *kv_len, int64_t E, int64_t Lk, int64_t H, int64_t B, float scale, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !k_new || !v_new || !new_strides) return MI_DECLINE_OPERANDS;
+    SdpaArgs a;
+    int rc = fill(a, out, out_dtype, out_strides, q, q_strides, cache_k, k_strides, cache_v, v_strides, nullptr, MI_F16, nullptr, kv_len, E, 1, Lk, H, B, scale);
+    if (rc != MI_OK) return rc;
+    if (H == 0 || B == 0 || E == 0) return MI_OK;
+    a.k_new = (const half_t *)k_new; a.v_new = (const half_t *)v_new;
+    for (int i = 0; i < 4; i++) a.ns[i] = new_strides[i];
+    if (sdpa_path(a) == MI_SDPA_DECLINE) return MI_DECLINE_EXTENT;
+    const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E) &&
+                     vec_addressable(a.k_new, a.ns, a.E) && vec_addressable(a.v_new, a.ns, a.E);
+    if (!one_pass_decode(a, vec)) return MI_DECLINE_UNSUPPORTED;      // the caller appends and attends in two calls
+    hipLaunchKernelGGL(sdpa_decode_kernel, dim3((unsigned)H, 1, (unsigned)B), dim3(512), 0, (hipStream_t)stream, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 

@@ -19,7 +19,11 @@ from typing import Callable, List, Optional
 import torch
 
 from . import _lib as L
-from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, sdpa
+from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, sdpa, sdpa_append
+
+
+# Fold the cache write into the self-attention launch where the one-launch kernel covers the shape.
+FUSE_APPEND = True
 
 
 class KVCache:
@@ -116,9 +120,13 @@ def decoder_layer_step(ctx: Ctx, W: DecoderLayerWeights, cache: KVCache, layer: 
 
     normed_linear(buf.qkv, W.wqkv, x, W.ln1_g, W.ln1_b, W.bqkv)
     q, k_new, v_new = (buf.qkv[:, i * d:(i + 1) * d].unflatten(1, (H, 1, E)) for i in range(3))
-    cache.append(ctx, layer, k_new, v_new)
-    ctx.ws.reset()
-    sdpa(ctx, q, cache.self_k[layer], cache.self_v[layer], out=heads(buf.att), kv_len=cache.length)
+    if FUSE_APPEND and E <= 64 and E % 8 == 0 and cache.max_target <= 640:
+        # one launch: the new row is key length - 1 and goes into its cache slot on the way
+        sdpa_append(ctx, q, cache.self_k[layer], cache.self_v[layer], k_new, v_new, cache.length, out=heads(buf.att))
+    else:
+        cache.append(ctx, layer, k_new, v_new)
+        ctx.ws.reset()
+        sdpa(ctx, q, cache.self_k[layer], cache.self_v[layer], out=heads(buf.att), kv_len=cache.length)
     ctx.ws.reset()
     matmul_(ctx, buf.x1, W.wo, buf.att, W.bo, residual=x)
     normed_linear(buf.qc, W.wq_c, buf.x1, W.ln2_g, W.ln2_b, W.bq_c)

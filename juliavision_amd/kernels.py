@@ -356,6 +356,33 @@ def sdpa(ctx: Ctx, q, k, v, bias=None, scale=None, *, out=None, kv_len=None):
     return out
 
 
+def sdpa_append(ctx: Ctx, q, cache_k, cache_v, k_new, v_new, kv_len, scale=None, *, out):
+    """Self-attention of one new token over its cache with the cache write folded in: ``k_new``/``v_new`` (B,H,1,E)
+    become key ``kv_len[b] - 1`` and are stored into that slot of ``cache_k``/``cache_v`` (B,H,Lmax,E); ``out``
+    (B,H,1,E) = attention of ``q`` (B,H,1,E) over the first ``kv_len[b]`` keys.  One launch in place of the exported
+    step's ``index_put`` + ``cat`` + attention (WhisperRunner/src/decode.jl:186-203).  Raises ``DeclineError`` with
+    ``L.DECLINE_UNSUPPORTED`` for shapes the single-launch kernel does not cover (head dim > 64, more than 640 slots):
+    the caller then appends and attends in two calls."""
+    if not _is_f16_cuda(q, cache_k, cache_v, k_new, v_new) or q.dim() != 4 or cache_k.dim() != 4:
+        raise DeclineError("sdpa_append: operands", L.DECLINE_OPERANDS)
+    Bq, H, Lq, E = q.shape
+    Lk = cache_k.shape[2]
+    if Lq != 1 or tuple(cache_k.shape) != (Bq, H, Lk, E) or tuple(cache_v.shape) != (Bq, H, Lk, E) or \
+            tuple(k_new.shape) != (Bq, H, 1, E) or tuple(v_new.shape) != (Bq, H, 1, E) or k_new.stride() != v_new.stride() or \
+            tuple(out.shape) != (Bq, H, 1, E):
+        raise DeclineError("sdpa_append: shapes", L.DECLINE_OPERANDS)
+    if kv_len.dtype != torch.int32 or not kv_len.is_cuda or kv_len.numel() != Bq:
+        raise DeclineError("sdpa_append: kv_len must be a cuda int32 (B,) tensor", L.DECLINE_OPERANDS)
+    scale = (1.0 / math.sqrt(E)) if scale is None else float(scale)
+    rc = L.init().mi_sdpa_append_f16(out.data_ptr(), _dtype_code(out), (None if out.is_contiguous() else _strides_elbh(out)),
+                                     q.data_ptr(), _strides_elbh(q), cache_k.data_ptr(), _strides_elbh(cache_k),
+                                     cache_v.data_ptr(), _strides_elbh(cache_v), k_new.data_ptr(), v_new.data_ptr(), _strides_elbh(k_new),
+                                     kv_len.data_ptr(), E, Lk, H, Bq, scale, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_sdpa_append_f16", rc)
+    return out
+
+
 # ----------------------------------------------------------------------------- convolution
 
 @dataclass(frozen=True)

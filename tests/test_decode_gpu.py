@@ -165,3 +165,46 @@ def test_step_graph_replays_match_eager(ctx):
         assert np.array_equal(to_host(og[-1]), to_host(oe[-1])), f"replay {t} differs from the eager step"
         assert np.array_equal(to_host(cg.self_k), to_host(ce.self_k))
         assert to_host(cg.length).tolist() == [t + 1] * B
+
+
+@pytest.mark.parametrize("E,Lmax", [(64, 448), (32, 70), (64, 16)])
+def test_fused_append_and_attend_equals_the_two_calls(ctx, E, Lmax):
+    """mi_sdpa_append_f16 against mi_kv_append_f16 followed by mi_sdpa_f16 on a twin cache: the same cache bits, the
+    same output bits (both attend with the one-launch kernel), and the oracle's attention over the updated cache."""
+    import torch
+    import juliavision_amd as jv
+    B, H = 4, 3
+    lens = [1, 5, Lmax, 0]
+    hk, hv = oracle.randn_f16((B, H, Lmax, E), 11), oracle.randn_f16((B, H, Lmax, E), 12)
+    wide = to_dev(oracle.randn_f16((B, 3 * H * E), 13))                 # q, k, v as column bands of one projection
+    q, k_new, v_new = (wide[:, i * H * E:(i + 1) * H * E].unflatten(1, (H, 1, E)) for i in range(3))
+    length = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    ck1, cv1, ck2, cv2 = to_dev(hk), to_dev(hv), to_dev(hk), to_dev(hv)
+    out1 = torch.full((B, H, 1, E), float("nan"), dtype=torch.float16, device="cuda")
+    out2 = out1.clone()
+    jv.sdpa_append(ctx, q, ck1, cv1, k_new, v_new, length, out=out1)
+    strides = lambda t: jv.kernels._strides_elbh(t)
+    rc = jv._lib.init().mi_kv_append_f16(ck2.data_ptr(), cv2.data_ptr(), strides(ck2), Lmax, k_new.data_ptr(), v_new.data_ptr(),
+                                         strides(k_new), length.data_ptr(), E, H, B, ctx.stream)
+    assert rc == 0
+    ctx.ws.reset()
+    jv.sdpa(ctx, q, ck2, cv2, out=out2, kv_len=length)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(ck1), to_host(ck2)) and np.array_equal(to_host(cv1), to_host(cv2))
+    assert np.array_equal(to_host(out1), to_host(out2))
+    assert np.all(to_host(out1)[3] == 0)                               # no live key: zeros, and nothing appended
+    assert np.array_equal(to_host(ck1)[3], hk[3])
+    want = oracle.sdpa_threepass_f16(to_host(q), to_host(ck1), to_host(cv1), kv_len=np.array(lens, dtype=np.int32))
+    assert_parity(to_host(out1), want, what=f"fused append + attention E{E} Lmax{Lmax}")
+
+
+def test_fused_append_declines_what_the_one_launch_kernel_does_not_cover(ctx):
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd import _lib as L
+    B, H, E, Lmax = 1, 2, 64, 700                                       # more than 640 slots
+    z = lambda *s: torch.zeros(s, dtype=torch.float16, device="cuda")
+    with pytest.raises(jv.DeclineError) as e:
+        jv.sdpa_append(ctx, z(B, H, 1, E), z(B, H, Lmax, E), z(B, H, Lmax, E), z(B, H, 1, E), z(B, H, 1, E),
+                       torch.ones((B,), dtype=torch.int32, device="cuda"), out=z(B, H, 1, E))
+    assert e.value.status == L.DECLINE_UNSUPPORTED
