@@ -524,11 +524,6 @@ def main():
     L = jv._lib
     lib = L.init()
     stream = torch.cuda.current_stream().cuda_stream
-    if args.only is not None:
-        print(json.dumps({"only": args.only, "detail": detail_benchmarks(lib, L, stream, args.only)}))
-        return
-    blk = EncoderBlock(lib, stream)
-
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
         dst = torch.empty_like(src)
@@ -536,6 +531,11 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.only is not None:
+        print(json.dumps({"only": args.only, "detail": detail_benchmarks(lib, L, stream, args.only)}))
+        return
+    blk = EncoderBlock(lib, stream)
+
     for _ in range(args.warmup):
         blk.step()
     torch.cuda.synchronize()
