@@ -183,3 +183,30 @@ def test_layer_norm_folded_into_decode_sized_gemv(ctx, T, K, F, layout):
         assert np.array_equal(to_host(out), to_host(two)), "folded norm differs from layernorm_ followed by matmul_"
     with pytest.raises(jv.DeclineError):
         jv.ln_matmul_(ctx, torch.empty((16, F), dtype=torch.float16, device="cuda"), Wd, torch.zeros((16, K), dtype=torch.float16, device="cuda"), None, None, 1e-5)
+
+
+@pytest.mark.parametrize("layout", ["kf", "fk"])
+def test_output_larger_than_2g_elements_is_indexed_in_64_bits(ctx, layout):
+    """70 000 x 32 768 outputs (2.29e9 elements, 4.6 GB of fp16): row offsets pass 2^31.  The oracle checks rows at
+    the start, around the 2^31-element boundary (row 65 536) and at the end; every row is checked for coverage."""
+    import torch
+    import juliavision_amd as jv
+    T, K, F = 70000, 128, 32768
+    Wkf = oracle.randn_f16((K, F), 3, 0, 1.0)
+    b = oracle.randn_f16((F,), 4, 0, 0.5)
+    rows = np.r_[0:4, 65534:65540, T - 4:T]
+    X = torch.empty((T, K), dtype=torch.float16, device="cuda")
+    X.normal_(0, 1.0 / np.sqrt(K))
+    Xs = oracle.randn_f16((len(rows), K), 5, 0, 1.0 / np.sqrt(K))
+    X[torch.from_numpy(rows).cuda()] = to_dev(Xs)
+    Wd = to_dev(Wkf) if layout == "kf" else to_dev(np.ascontiguousarray(Wkf.T)).t()
+    out = torch.empty((T, F), dtype=torch.float16, device="cuda")
+    out.fill_(float("nan"))
+    ctx.ws.reset()
+    jv.matmul_(ctx, out, Wd, X, to_dev(b), epi="gelu")
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())                         # nothing unwritten anywhere
+    want = oracle.gemm_f16(Xs, Wkf, b, epi="gelu")
+    assert_parity(to_host(out[torch.from_numpy(rows).cuda()]), want, what=f"rows across the 2^31 boundary, {layout}")
+    del out, X
+    torch.cuda.empty_cache()
