@@ -123,6 +123,18 @@ int mi_ln_gemv_f16(void *Y, const void *X, const void *gamma, const void *beta, 
                    int w_layout, int bias_mode, int epi, int out_dtype,
                    void *ws, size_t ws_bytes, void *stream);
 
+/* mi_gemm_f16 followed by mi_layernorm_f16 of its output rows: Y[T][F] (fp16, dense rows) as mi_gemm_f16 writes
+ * it, and H[T][F] = layer norm of Y over F with gamma / beta (either may be NULL).  When the GEMM splits K the norm
+ * rides in the pass that sums the planes (one launch less); otherwise the two kernels run back to back.  Either way
+ * Y and H carry the bits of the two separate calls.  The graph shape it serves: a linear op (+ residual) whose
+ * result is both the residual stream and the input of the next block's first norm (layer_norm, ops.jl:575-647,
+ * after addmm + add.Tensor, ops.jl:1347-1363,186-197); the reference runs the three ops one by one.
+ * Workspace as for mi_gemm_f16. */
+int mi_gemm_ln_f16(void *Y, void *H, const void *X, const void *W, const void *bias, const void *residual,
+                   const void *gamma, const void *beta, float eps,
+                   int64_t T, int64_t K, int64_t F, int64_t ldX, int64_t ldW,
+                   int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream);
+
 size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int64_t nbatch);
 /* Returns an mi_gemm_path; never launches.  Replaces mmplan / mm_coopmat_plan /
  * mm_gemv_plan -- matmul.jl:87-95,121-131,172-179. */

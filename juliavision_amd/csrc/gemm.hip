@@ -27,6 +27,11 @@ struct GemmArgs {
     const half_t *ln_gamma, *ln_beta;
     float ln_eps;
     int ln_on;
+    // Output side: when lnout is set, the rows of Y are also layer-normalised over N into lnout (dense rows of N
+    // halves), as mi_layernorm_f16 on Y would write them (the next block's first norm riding in this GEMM's store).
+    half_t *lnout;
+    const half_t *lnout_gamma, *lnout_beta;
+    float lnout_eps;
 };
 
 // ------------------------------------------------------------------------------------------
@@ -870,6 +875,85 @@ __global__ void splitk_epilogue_kernel(GemmArgs p, const float *part, int nsplit
     }
 }
 
+// The same sums, bias, activation and residual as splitk_epilogue_kernel, one wave per output row, followed by the
+// layer norm of that row into p.lnout: lane and chunk order, summation order and rounding are those of
+// layernorm_vec_kernel, so Y and lnout carry the bits the two separate launches would have written.
+template <int NCH>
+__global__ __launch_bounds__(256) void splitk_epilogue_ln_kernel(GemmArgs p, const float *part, int nsplit) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long m = (long)blockIdx.x * 4 + wave;
+    if (m >= p.M) return;
+    const long total = (long)p.M * p.N;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    u32x4 graw[NCH], braw[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        graw[i] = (p.lnout_gamma && e0 < p.N) ? ldg16(p.lnout_gamma + e0) : z;
+        braw[i] = (p.lnout_beta && e0 < p.N) ? ldg16(p.lnout_beta + e0) : z;
+    }
+    float x[NCH][8];
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        if (e0 < p.N) {
+            const float *pp = part + m * p.N + e0;
+            float4v v0 = *reinterpret_cast<const float4v *>(pp), v1 = *reinterpret_cast<const float4v *>(pp + 4);
+            for (int sp = 1; sp < nsplit; sp++) {
+                const float4v w0 = *reinterpret_cast<const float4v *>(pp + (long)sp * total), w1 = *reinterpret_cast<const float4v *>(pp + (long)sp * total + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { v0[e] += w0[e]; v1[e] += w1[e]; }
+            }
+            const long off = m * p.ldY + e0;
+            half8v o;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                float v = e < 4 ? v0[e] : v1[e - 4];
+                v += p.bias_mode == MI_BIAS_COL ? (float)p.bias[e0 + e] : p.bias_mode == MI_BIAS_ROW ? (float)p.bias[m] : 0.0f;
+                o[e] = (half_t)apply_epi((float)(half_t)v, p.epi);
+            }
+            if (p.residual) {
+                const half8v rv = as_half8(ldg16(p.residual + off));
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[e] = (half_t)((float)o[e] + (float)rv[e]);
+            }
+            *reinterpret_cast<half8v *>(reinterpret_cast<half_t *>(p.Y) + off) = o;
+#pragma unroll
+            for (int j = 0; j < 8; j++) { x[i][j] = (float)o[j]; s += x[i][j]; }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) x[i][j] = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    const float mu = s / (float)p.N;
+    float s2 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        if ((lane + 64 * i) * 8 < p.N) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) { const float d = x[i][j] - mu; s2 = fmaf(d, d, s2); }
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+    const float r = 1.0f / sqrtf(s2 / (float)p.N + p.lnout_eps);
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        if (e0 < p.N) {
+            const half8v gv = as_half8(graw[i]), bv = as_half8(braw[i]);
+            half8v o;
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                o[j] = ln_norm1(x[i][j], mu, r, p.lnout_gamma != nullptr, p.lnout_gamma ? (float)gv[j] : 0.0f, p.lnout_beta != nullptr, p.lnout_beta ? (float)bv[j] : 0.0f);
+            *reinterpret_cast<half8v *>(p.lnout + m * p.N + e0) = o;
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 bool g_ready = false;
 int g_cus = 256;
@@ -1018,7 +1102,17 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
     a.cv = ConvGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
+    a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f;
     return MI_OK;
+}
+
+// Internal status: the split-K epilogue has also written a.lnout (the caller must not run the norm again).
+constexpr int MI_LNOUT_DONE = -1;
+
+bool lnout_rowwise_ok(const GemmArgs &a) {
+    return !a.out_f32 && a.N % 8 == 0 && a.N <= 4096 && a.ldY % 8 == 0 && aligned_to(a.Y, 16) && aligned_to(a.lnout, 16) &&
+           (!a.residual || aligned_to(a.residual, 16)) && (!a.lnout_gamma || aligned_to(a.lnout_gamma, 16)) &&
+           (!a.lnout_beta || aligned_to(a.lnout_beta, 16));
 }
 
 int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, hipStream_t st, int force_path) {
@@ -1046,8 +1140,18 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
             if (rc != MI_OK) return rc;
             GemmArgs s2 = a;
             s2.vec_store = !a.out_f32 && a.ldY % 4 == 0 && aligned_to(a.Y, 8);
+            const float *planes = reinterpret_cast<const float *>(ws);
+            if (a.lnout && lnout_rowwise_ok(a)) {
+                // the norm of the finished rows rides in the pass that sums the planes: one wave per row
+                dim3 grid((unsigned)ceil_div(a.M, 4));
+                if (a.N <= 512)       hipLaunchKernelGGL(splitk_epilogue_ln_kernel<1>, grid, dim3(256), 0, st, s2, planes, split);
+                else if (a.N <= 1024) hipLaunchKernelGGL(splitk_epilogue_ln_kernel<2>, grid, dim3(256), 0, st, s2, planes, split);
+                else if (a.N <= 2048) hipLaunchKernelGGL(splitk_epilogue_ln_kernel<4>, grid, dim3(256), 0, st, s2, planes, split);
+                else                  hipLaunchKernelGGL(splitk_epilogue_ln_kernel<8>, grid, dim3(256), 0, st, s2, planes, split);
+                return hipGetLastError() == hipSuccess ? MI_LNOUT_DONE : MI_ERROR_LAUNCH;
+            }
             const long quads = ((long)a.M * a.N) / 4;
-            hipLaunchKernelGGL(splitk_epilogue_kernel, dim3((unsigned)ceil_div(quads, 256)), dim3(256), 0, st, s2, reinterpret_cast<const float *>(ws), split);
+            hipLaunchKernelGGL(splitk_epilogue_kernel, dim3((unsigned)ceil_div(quads, 256)), dim3(256), 0, st, s2, planes, split);
             return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
         }
         // Tile choice: the big tile as soon as the 128 x 128 tiles would outnumber the CUs (some CUs would then
@@ -1081,6 +1185,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     GemmArgs a;
     a.cv = ConvGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
+    a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
@@ -1180,6 +1285,22 @@ int mi_gemm_f16(void *Y, const void *X, const void *W, const void *bias, const v
                 void *ws, size_t ws_bytes, void *stream) {
     return mi_gemm_f16_batched(Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype,
                                1, 0, 0, 0, 0, ws, ws_bytes, stream);
+}
+
+int mi_gemm_ln_f16(void *Y, void *H, const void *X, const void *W, const void *bias, const void *residual,
+                   const void *gamma, const void *beta, float eps,
+                   int64_t T, int64_t K, int64_t F, int64_t ldX, int64_t ldW,
+                   int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream) {
+    if (!H) return MI_DECLINE_OPERANDS;
+    GemmArgs a;
+    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, F, ldX, ldW, w_layout, bias_mode, epi, MI_F16, 0, 0, 0);
+    if (rc != MI_OK) return rc;
+    if (!g_ready) return MI_ERROR_DEVICE;
+    a.lnout = (half_t *)H; a.lnout_gamma = (const half_t *)gamma; a.lnout_beta = (const half_t *)beta; a.lnout_eps = eps;
+    rc = run_gemm(a, w_layout == MI_W_KF, 1, ws, ws_bytes, (hipStream_t)stream, 0);
+    if (rc == MI_LNOUT_DONE) return MI_OK;
+    if (rc != MI_OK) return rc;
+    return mi_layernorm_f16(H, nullptr, nullptr, Y, gamma, beta, F, T, eps, stream);      // rows of Y are dense: ldY = F
 }
 
 int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,

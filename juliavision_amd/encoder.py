@@ -7,7 +7,8 @@ The reference runs these as exported op graphs (WhisperRunner/src/WhisperRunner.
 issued directly, seven launches per block: layer norm, one GEMM for the three projections,
 fused attention reading q/k/v in place and writing token-major, the output projection with
 the residual in its epilogue, layer norm, the GELU GEMM, and the second MLP GEMM with the
-residual in its epilogue.  Nothing allocates after construction, so a whole encoder can be
+residual in its epilogue -- six from the second block on, because that last GEMM also writes
+the next block's first norm (``matmul_ln_``).  Nothing allocates after construction, so a whole encoder can be
 captured and replayed (``decode.StepGraph``).
 """
 from __future__ import annotations
@@ -17,7 +18,7 @@ from typing import List, Optional
 
 import torch
 
-from .kernels import Ctx, add_, convolution_, convsize, layernorm_, matmul_, sdpa, transposeLE_
+from .kernels import Ctx, add_, convolution_, convsize, layernorm_, matmul_, matmul_ln_, sdpa, transposeLE_
 
 
 @dataclass
@@ -47,12 +48,17 @@ class EncoderBuffers:
 
 
 def encoder_layer(ctx: Ctx, W: EncoderLayerWeights, x: torch.Tensor, out: torch.Tensor, buf: EncoderBuffers, heads: int,
-                  eps: float = 1e-5, act: str = "gelu"):
+                  eps: float = 1e-5, act: str = "gelu", *, normed_in: bool = False, next_norm=None):
     """``out = x1 + W2 act(W1 LN2(x1))`` with ``x1 = x + Wo attention(LN1(x))``; ``x``, ``out``: ``(T, d)`` fp16
-    (``out`` may be ``x``, which is last read as the output projection's residual)."""
+    (``out`` may be ``x``, which is last read as the output projection's residual).
+
+    ``next_norm = (gamma, beta, dst)``: the norm that reads ``out`` next (the following layer's first norm, or the
+    encoder's final one) is written to ``dst`` by this layer's last GEMM (``matmul_ln_``).  ``normed_in``: the
+    previous layer did that for this one, ``buf.h`` already holds ``LN1(x)``."""
     T, d = x.shape
     E = d // heads
-    layernorm_(ctx, buf.h, None, None, x, W.ln1_g, W.ln1_b, d, eps)
+    if not normed_in:
+        layernorm_(ctx, buf.h, None, None, x, W.ln1_g, W.ln1_b, d, eps)
     ctx.ws.reset()
     matmul_(ctx, buf.qkv, W.wqkv, buf.h, W.bqkv)
     # q, k, v are column bands of the projection, heads are 64-wide column bands of those: (B,H,L,E) views, no copy
@@ -65,7 +71,10 @@ def encoder_layer(ctx: Ctx, W: EncoderLayerWeights, x: torch.Tensor, out: torch.
     ctx.ws.reset()
     matmul_(ctx, buf.f, W.w1, buf.h, W.b1, epi=act)
     ctx.ws.reset()
-    matmul_(ctx, out, W.w2, buf.f, W.b2, residual=buf.x1)
+    if next_norm is None:
+        matmul_(ctx, out, W.w2, buf.f, W.b2, residual=buf.x1)
+    else:
+        matmul_ln_(ctx, out, next_norm[2], W.w2, buf.f, next_norm[0], next_norm[1], eps, W.b2, residual=buf.x1)
     return out
 
 
@@ -113,11 +122,15 @@ class ViTEncoder:
     def __call__(self, ctx: Ctx, image: torch.Tensor):
         W = self.W
         src = self.embed(ctx, image)
+        n = len(W.layers)
         for i, lw in enumerate(W.layers):
             dst = self.tokens[(i + 1) % 2]
-            encoder_layer(ctx, lw, src, dst, self.buf, self.heads, self.eps)
+            # the norm that reads this layer's output rides in its last GEMM: the next layer's first norm into the
+            # shared slot buf.h, the encoder's final norm into self.out
+            if i + 1 < n:
+                nxt = (W.layers[i + 1].ln1_g, W.layers[i + 1].ln1_b, self.buf.h)
+            else:
+                nxt = None if W.norm_g is None else (W.norm_g, W.norm_b, self.out)
+            encoder_layer(ctx, lw, src, dst, self.buf, self.heads, self.eps, normed_in=i > 0, next_norm=nxt)
             src = dst
-        if W.norm_g is None:
-            return src
-        layernorm_(ctx, self.out, None, None, src, W.norm_g, W.norm_b, src.shape[1], self.eps)
-        return self.out
+        return src if W.norm_g is None else self.out

@@ -244,6 +244,35 @@ def fold_residuals(g: Graph) -> Graph:
     return g
 
 
+RESHAPES = ("view.default", "_unsafe_view.default", "reshape.default", "alias.default", "detach.default")
+
+
+def fold_layernorms(g: Graph) -> Graph:
+    """A layer norm over the last axis whose input is (a reshaping view of) a linear op's output -- the residual
+    stream after ``addmm`` + ``add``, normalised for the next block -- is written by that GEMM as a second result
+    (``matmul_ln_``): one launch less where the GEMM splits K, the same bits everywhere.  The linear's own output
+    stays what it was, so other readers (the next residual add) are untouched."""
+    for ln in [o for o in g.ops if o["aten"] in ("layer_norm.default", "native_layer_norm.default")]:
+        src, a = ln["in"][0], ln["attrs"]
+        chain = [src]
+        while g.buffers[chain[-1]]["kind"] == "view":
+            chain.append(g.buffers[chain[-1]]["of"])
+        prod = g.op(chain[-1])
+        if prod is None or prod["aten"] not in LINEAR_OPS or "ln_out" in prod["attrs"]:
+            continue
+        feat = (g.buffers[chain[-1]].get("shape") or [None])[-1]
+        shapes_ok = all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1])
+        if not shapes_ok or list(a.get("arg1", [])) != [feat]:
+            continue
+        if any(g.op(g.root(i)) is not None and g.ops.index(g.op(g.root(i))) > g.ops.index(prod) for i in ln["in"][1:]):
+            continue                                    # gamma / beta must exist before the GEMM runs (weights always do)
+        prod["attrs"].update(ln_out=ln["out"], ln_gamma=ln["in"][1] if len(ln["in"]) > 1 else None,
+                             ln_beta=ln["in"][2] if len(ln["in"]) > 2 else None, ln_eps=a.get("arg4", a.get("eps", 1e-5)))
+        g.ops.remove(ln)
+        g.notes.append(f"fold {ln['id']} into {prod['id']}")
+    return g
+
+
 def fold_sdpa_transpose(g: Graph) -> Graph:
     """Attention whose only reader swaps the head and token axes back (``transpose(1, 2)`` /
     ``permute(0, 2, 1, 3)``): the kernel writes token-major, the swap becomes the view it already is, and
@@ -266,7 +295,7 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
 
 
 def optimize(g: Graph) -> Graph:
-    return fold_sdpa_transpose(fold_residuals(fold_activations(g)))
+    return fold_sdpa_transpose(fold_layernorms(fold_residuals(fold_activations(g))))
 
 
 # ----------------------------------------------------------------------------- execution
@@ -292,6 +321,12 @@ class Executor:
         for o in graph.ops:                               # check every op has a handler before anything runs
             if o["aten"] not in self.HANDLERS:
                 raise UnsupportedOp(f"{graph.name}: no kernel on this path for aten.{o['aten']} (op {o['id']})")
+        for o in graph.ops:                               # a norm folded into its producer: its result still needs a home
+            nid = o["attrs"].get("ln_out")
+            if nid is not None:
+                nb = graph.buffers[nid]
+                shape, dtype = (nb["shape"], nb["dtype"]) if "shape" in nb else (nb["shapes"][0], nb["dtypes"][0])
+                self.t[nid] = torch.empty(list(shape), dtype=_DTYPES[dtype], device=self.device)
         for o in graph.ops:
             b = graph.buffers[o["out"]]
             if "shape" in b:
@@ -385,6 +420,12 @@ class Executor:
         out = self.t[o["out"]]
         res = self._rows(self.get(res_id)) if res_id else None
         self.ctx.ws.reset()
+        if attrs.get("ln_out") is not None:
+            gamma = self.get(attrs["ln_gamma"]) if attrs.get("ln_gamma") else None
+            beta = self.get(attrs["ln_beta"]) if attrs.get("ln_beta") else None
+            K.matmul_ln_(self.ctx, self._rows(out), self._rows(self.t[attrs["ln_out"]]), w, self._rows(x), gamma, beta,
+                         attrs["ln_eps"], bias, epi=attrs.get("epilogue", "none"), residual=res)
+            return
         K.matmul_(self.ctx, self._rows(out), w, self._rows(x), bias, epi=attrs.get("epilogue", "none"), residual=res)
 
     def _sdpa(self, o):

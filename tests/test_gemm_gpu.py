@@ -210,3 +210,32 @@ def test_output_larger_than_2g_elements_is_indexed_in_64_bits(ctx, layout):
     assert_parity(to_host(out[torch.from_numpy(rows).cuda()]), want, what=f"rows across the 2^31 boundary, {layout}")
     del out, X
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("layout", ["kf", "fk"])
+@pytest.mark.parametrize("T,K,F", [(1370, 1536, 384), (200, 2048, 256), (1500, 5120, 1280), (200, 256, 328), (4, 1280, 1280), (77, 2048, 264)])
+def test_layer_norm_of_the_output_rides_in_the_gemm(ctx, T, K, F, layout):
+    """matmul_ln_ against the oracle's gemm -> layernorm, and bit for bit (both outputs) against matmul_ followed by
+    layernorm_: split-K shapes (the norm is in the plane-summing pass), unsplit and decode-sized ones (two kernels)."""
+    import torch
+    import juliavision_amd as jv
+    X = oracle.randn_f16((T, K), 91, 0, 1.0 / np.sqrt(K))
+    Wkf = oracle.randn_f16((K, F), 92, 0, 1.0)
+    b, R = oracle.randn_f16((F,), 93, 0, 0.1), oracle.randn_f16((T, F), 94, 0.2, 1.0)
+    g, be = oracle.randn_f16((F,), 95, 1.0, 0.2), oracle.randn_f16((F,), 96, 0, 0.2)
+    Wd = to_dev(Wkf) if layout == "kf" else to_dev(np.ascontiguousarray(Wkf.T)).t()
+    dX, db, dR = to_dev(X), to_dev(b), to_dev(R)
+    for (gamma, beta, hg, hb, epi) in ((to_dev(g), to_dev(be), g, be, "none"), (None, None, None, None, "gelu"), (to_dev(g), None, g, None, "relu")):
+        y = oracle.gemm_f16(X, Wkf, b, epi=epi, residual=R)
+        h, _, _ = oracle.layernorm_f16(y, hg, hb, 1e-6)
+        out, normed = (poison(torch.empty((T, F), dtype=torch.float16, device="cuda")) for _ in range(2))
+        ctx.ws.reset()
+        jv.matmul_ln_(ctx, out, normed, Wd, dX, gamma, beta, 1e-6, db, epi=epi, residual=dR)
+        out2, normed2 = (poison(torch.empty((T, F), dtype=torch.float16, device="cuda")) for _ in range(2))
+        ctx.ws.reset()
+        jv.matmul_(ctx, out2, Wd, dX, db, epi=epi, residual=dR)
+        jv.layernorm_(ctx, normed2, None, None, out2, gamma, beta, F, 1e-6)
+        torch.cuda.synchronize()
+        assert_parity(to_host(out), y, what=f"matmul_ln_ output T{T} K{K} F{F} {layout}")
+        assert_parity(to_host(normed), h, what=f"matmul_ln_ norm T{T} K{K} F{F} {layout}")
+        assert np.array_equal(to_host(out), to_host(out2)) and np.array_equal(to_host(normed), to_host(normed2))

@@ -80,8 +80,12 @@ def test_rewrites_fold_activation_residuals_and_attention_layout():
     assert fc1["attrs"]["epilogue"] == "gelu" and g.buffers["gelu"]["kind"] == "view" and g.buffers["gelu"]["of"] == "linear_4"
     assert g.op("linear_3")["attrs"]["residual"] == "$x" and g.op("linear_5")["attrs"]["residual"] == "$add"
     assert g.op("scaled_dot_product_attention")["attrs"]["token_major"] is True
-    assert len(g.ops) == 9                                              # 2 LN + 6 linears + attention
-    assert g.root("add_1") == "linear_5" and len(g.notes) == 4
+    assert len(g.ops) == 8                                              # LN + 6 linears + attention
+    assert g.root("add_1") == "linear_5" and len(g.notes) == 5
+    # the second norm reads the residual stream that the out-projection writes: it became that GEMM's second result
+    proj = g.op("linear_3")
+    assert proj["attrs"]["ln_out"] == "layer_norm_1" and proj["attrs"]["ln_gamma"] == "p_ln2_weight" and proj["attrs"]["ln_eps"] == 1e-5
+    assert g.op("layer_norm_1") is None and g.op("layer_norm") is not None           # the first norm reads the graph's input
     # an activation that something else also reads must stay where it is
     d = G.convert(ep, "block")
     d["outputs"].append("linear_4")
@@ -220,14 +224,15 @@ def test_decomposed_export_folds_like_the_composite_one():
     aten = [o["aten"] for o in d["ops"]]
     assert aten.count("addmm.default") == 5 and aten.count("mm.default") == 1 and aten.count("native_layer_norm.default") == 2
     g = G.optimize(G.Graph.load(d))
-    assert [o["aten"] for o in g.ops].count("gelu.default") == 0 and len(g.ops) == 9
+    assert [o["aten"] for o in g.ops].count("gelu.default") == 0 and len(g.ops) == 8
+    assert [o["aten"] for o in g.ops].count("native_layer_norm.default") == 1         # the second one rides in the out-projection
     fc1 = next(o for o in g.ops if o["attrs"].get("epilogue") == "gelu")
     assert fc1["aten"] == "addmm.default" and g.root("gelu") == fc1["id"]       # gelu read the addmm through a view
     assert sum("residual" in o["attrs"] for o in g.ops) == 2
     for name in ("_scaled_dot_product_flash_attention.default", "_scaled_dot_product_efficient_attention.default"):
         g2 = G.optimize(G.Graph.load(_as_backend_attention(d, name)))
         att = next(o for o in g2.ops if o["aten"] == name)
-        assert att["attrs"]["token_major"] is True and len(g2.ops) == 9
+        assert att["attrs"]["token_major"] is True and len(g2.ops) == 8
 
 
 @pytest.mark.gpu
