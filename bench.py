@@ -360,6 +360,54 @@ def vit_encoder_case(steps=50):
             "frac_mfma_peak_graph": round(flop / replay / 1e12 / PEAK_F16_TFLOPS, 4)}
 
 
+def encoder_stack_case(nl=4, steps=50):
+    """BASELINE config 2's block as it occurs in a stack: `nl` Whisper-shaped blocks in sequence (1500 x 1280, 20 x 64
+    heads, FFN 5120, [K][F] weights), each block's first norm written by the previous block's last GEMM.  Reported per
+    block."""
+    import time
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd.decode import StepGraph
+    from juliavision_amd.encoder import EncoderBuffers, EncoderLayerWeights, encoder_layer
+    T, d, H, ffn = 1500, 1280, 20, 5120
+    ctx = jv.Ctx("cuda")
+    f16 = torch.float16
+    w = lambda k, f: torch.randn((k, f), dtype=f16, device="cuda") * 0.02
+    v = lambda n, m=0.0: torch.randn((n,), dtype=f16, device="cuda") * 0.02 + m
+    layers = [EncoderLayerWeights(v(d, 1.0), v(d), w(d, 3 * d), v(3 * d), w(d, d), v(d), v(d, 1.0), v(d), w(d, ffn), v(ffn), w(ffn, d), v(d))
+              for _ in range(nl)]
+    buf = EncoderBuffers(T, d, ffn)
+    xs = [torch.randn((T, d), dtype=f16, device="cuda") for _ in range(2)]
+    x0 = torch.randn((T, d), dtype=f16, device="cuda")
+
+    def run():
+        src = x0
+        for i, lw in enumerate(layers):
+            dst = xs[i % 2]
+            nxt = (layers[i + 1].ln1_g, layers[i + 1].ln1_b, buf.h) if i + 1 < nl else None
+            encoder_layer(ctx, lw, src, dst, buf, H, 1e-5, normed_in=i > 0, next_norm=nxt)
+            src = dst
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    eager = timed(run)
+    replay = timed(StepGraph(run).replay)
+    if not bool(torch.isfinite(xs[(nl - 1) % 2]).all()):
+        raise RuntimeError("encoder stack produced non-finite output")
+    flop = EncoderBlock.FLOP
+    return {"blocks": nl, "eager_ms_per_block": round(eager / nl * 1e3, 4), "graph_ms_per_block": round(replay / nl * 1e3, 4),
+            "launches": 7 + 6 * (nl - 1), "TFLOP/s_graph": round(flop * nl / replay / 1e12, 1),
+            "frac_mfma_peak_graph": round(flop * nl / replay / 1e12 / PEAK_F16_TFLOPS, 4)}
+
+
 def detail_benchmarks(lib, L, stream, only=None):
     import numpy as np
     import torch
@@ -490,6 +538,10 @@ def detail_benchmarks(lib, L, stream, only=None):
             name = f"c5_decoder_layer_b{bsz}_{tag}"
             if only is None or only in name:
                 out[name] = decoder_layer_case(bsz, lay)
+
+    name = "c2_encoder_stack_4blocks"
+    if only is None or only in name:
+        out[name] = encoder_stack_case()
 
     name = "c3_vit_s14_518_encoder_12layers"
     if only is None or only in name:
