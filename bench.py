@@ -490,6 +490,22 @@ def detail_benchmarks(lib, L, stream, only=None):
         out["c4_conv3x3_256to256_64x64"] = {"us": round(med * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 2),
                                             "frac_mfma_peak": round(flop / med / 1e12 / PEAK_F16_TFLOPS, 4)}
 
+    def conv_nhwc_case():
+        # the same convolution over a channels-last map: the GEMM gathers its A operand from x, nothing is staged
+        x = torch.randn((1, 64, 64, 256), dtype=f16, device="cuda")
+        w = torch.randn((256, 3, 3, 256), dtype=f16, device="cuda") * 0.02
+        b = torch.randn((256,), dtype=f16, device="cuda")
+        o = torch.empty((1, 64, 64, 256), dtype=f16, device="cuda")
+        geo = (64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
+        need = lib.mi_conv2d_nhwc_f16_workspace(*geo)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        conv = Call(lib.mi_conv2d_nhwc_f16, o.data_ptr(), x.data_ptr(), w.data_ptr(), b.data_ptr(), *geo, L.EPI["none"],
+                    ws.data_ptr(), need, stream)
+        med, lo, hi = event_time(conv, 10)
+        flop = 2.0 * 4096 * 2304 * 256
+        out["c4_conv3x3_256to256_64x64_nhwc"] = {"us": round(med * 1e6, 2), "TFLOP/s": round(flop / med / 1e12, 2),
+                                                  "range_us": [round(lo * 1e6, 2), round(hi * 1e6, 2)]}
+
     def convt_case(name, Cin, Hi, Cout):
         # SAM 2's mask-decoder upsamplers: kernel 2, stride 2 (test_convtranspose_gemm.jl:36)
         if only is not None and only not in name:
@@ -555,6 +571,8 @@ def detail_benchmarks(lib, L, stream, only=None):
     attn_case("c4_attn_L4096_16x64", 1, 16, 4096, 4096, 64)
     if only is None or only in "c4_conv3x3_256to256_64x64":
         conv_case()
+    if only is None or only in "c4_conv3x3_256to256_64x64_nhwc":
+        conv_nhwc_case()
     convt_case("sam2_upsample_convT2x2_256to64_64x64", 256, 64, 64)
     convt_case("sam2_upsample_convT2x2_64to32_128x128", 64, 128, 32)
     decode_cases()

@@ -209,6 +209,22 @@ int mi_conv2d_f16_plan(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
                        int64_t KW, int64_t KH, int64_t Cout,
                        int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
                        int64_t dil_x, int64_t dil_y, int64_t groups);
+/* The same convolution over channels-last tensors: x [N][H][W][Cin], w [Cout][KH][KW][Cin], out [N][OH][OW][Cout]
+ * (groups = 1).  An implicit GEMM with nothing staged: out[(n,oh,ow)][Cout] = patch . w^T, the patch matrix gathered
+ * from x by the GEMM's own operand loads, the weights read as they lie; split-K planes in ws where the output tiles
+ * are few.  Needs Cin % 64 == 0 and Cout % 8 == 0 (MI_DECLINE_UNSUPPORTED otherwise: use the layout above).
+ * The reference has no channels-last path -- its arrays are (W,H,C,N) throughout (safetensors.jl:7-12) -- but its
+ * implicit-GEMM kernel walks K the same way, conv2d_igemm!, conv_implicit.jl:53-355. */
+int mi_conv2d_nhwc_f16(void *out, const void *x, const void *w, const void *bias,
+                       int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                       int64_t KW, int64_t KH, int64_t Cout,
+                       int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                       int64_t dil_x, int64_t dil_y, int act,
+                       void *ws, size_t ws_bytes, void *stream);
+size_t mi_conv2d_nhwc_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                                    int64_t KW, int64_t KH, int64_t Cout,
+                                    int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                                    int64_t dil_x, int64_t dil_y);
 /* ATen's output extent -- convsize, conv.jl:309. */
 int64_t mi_convsize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d);
 

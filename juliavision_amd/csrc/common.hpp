@@ -81,6 +81,18 @@ struct ConvGather {
     int split;             // 1: the launch's planes are K-slices of one image, 0: they are images
 };
 
+// Implicit-GEMM convolution over a channels-last input x[N][H][W][C]: how the GEMM finds its [M][K] operand
+// (the patch matrix: row m = output pixel (n, oh, ow), K ordered (kh, kw, ci) with ci fastest) in x itself.
+// A 64-deep tile is 64 consecutive channels of one tap, i.e. 128 contiguous bytes of x per row, at an offset
+// from the row's pixel that is the same for every row; rows whose tap falls outside the image read zeros.
+struct NhwcGather {
+    const half_t *x;       // nullptr = ordinary GEMM
+    int H, W, C, OH, OW;
+    int sx, sy, px, py, dx, dy, KW;
+    int cpt;               // 64-channel tiles per tap: C / 64
+    int split;             // 1: the launch's planes are K-slices
+};
+
 // True once mi_init has run successfully on this process (defined in gemm.hip).
 bool mi_ready();
 int mi_num_cus();
@@ -89,4 +101,4 @@ int mi_sdpa_init();
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
                      long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st,
-                     const ConvGather *gather = nullptr);
+                     const ConvGather *gather = nullptr, const NhwcGather *agather = nullptr);

@@ -281,4 +281,38 @@ int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
                             a.N, (long)a.Cout * PQ, 0, PQP * CRSP, reinterpret_cast<char *>(ws) + col_bytes + wp_bytes, gemm_bytes, st);
 }
 
+// Channels-last convolution as an implicit GEMM with nothing staged: out[(n,oh,ow)][Cout] = patch[(n,oh,ow)][(kh,kw,ci)] .
+// w[Cout][(kh,kw,ci)]^T.  The patch matrix is gathered from x by the GEMM's A-operand loads (64 channels of one tap
+// are 128 contiguous bytes of a pixel; taps outside the image load zeros), the weights are the K-contiguous operand
+// as they lie, the bias is per output column: no padded copy, no re-laid weights, no im2col.
+size_t mi_conv2d_nhwc_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, int64_t KW, int64_t KH, int64_t Cout,
+                                    int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy) {
+    ConvArgs a;
+    if (fill(a, nullptr, nullptr, nullptr, nullptr, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, 1, MI_EPI_NONE) != MI_OK) return 0;
+    return mi_gemm_f16_workspace((int64_t)N * a.OH * a.OW, Cin * KH * KW, Cout, MI_W_FK, 1);
+}
+
+int mi_conv2d_nhwc_f16(void *out, const void *x, const void *w, const void *bias,
+                       int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, int64_t KW, int64_t KH, int64_t Cout,
+                       int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy, int act,
+                       void *ws, size_t ws_bytes, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !x || !w) return MI_DECLINE_OPERANDS;
+    ConvArgs a;
+    int rc = fill(a, out, x, w, bias, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, 1, act);
+    if (rc != MI_OK) return rc;
+    if (N == 0) return MI_OK;
+    const int64_t M = (int64_t)N * a.OH * a.OW, K = Cin * KH * KW;
+    // the gathered operand is read in runs of 64 channels; other channel counts go through the reference layout
+    if (Cin % 64 || K < 128 || M > INT32_MAX || K > INT32_MAX || Cout % 8) return MI_DECLINE_UNSUPPORTED;
+    if (!aligned_to(x, 16) || !aligned_to(w, 16) || !aligned_to(out, 16)) return MI_DECLINE_OPERANDS;
+    NhwcGather g;
+    g.x = (const half_t *)x; g.H = a.Hi; g.W = a.Wi; g.C = a.Cin; g.OH = a.OH; g.OW = a.OW;
+    g.sx = a.sx; g.sy = a.sy; g.px = a.px; g.py = a.py; g.dx = a.dx; g.dy = a.dy; g.KW = a.KW; g.cpt = a.Cin / 64; g.split = 0;
+    const int epi = a.relu ? MI_EPI_RELU : MI_EPI_NONE;
+    // A is never dereferenced through its pointer and leading dimension in this mode; x and K stand in for the operand checks
+    return mi_internal_gemm(out, x, w, bias, (int)M, (int)Cout, (int)Cout, (int)K, Cout, K, K, 0, MI_BIAS_COL, epi, 0,
+                            1, 0, 0, 0, ws, ws_bytes, (hipStream_t)stream, nullptr, &g);
+}
+
 }  // extern "C"

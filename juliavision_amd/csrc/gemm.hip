@@ -22,6 +22,7 @@ struct GemmArgs {
     int tiles_m, tiles_n, group_m;
     int vec_store;          // Y (and residual) rows allow 16-byte accesses
     ConvGather cv;          // cv.xp != nullptr: B is the im2col matrix of a convolution, gathered on the fly
+    NhwcGather ag;          // ag.x != nullptr: A is the patch matrix of a channels-last convolution, gathered on the fly
     // Decode-sized kernels only: the rows of A are layer-normalised over K on their way into LDS
     // (ln_on; gamma, beta may be null), exactly as layernorm_vec_kernel would have written them.
     const half_t *ln_gamma, *ln_beta;
@@ -361,9 +362,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma_kernel(GemmAr
 // where its successor's first fragment read can be hidden behind the last k-step.
 // Two waves per SIMD (8 waves on a 128 x 256 tile) cover each other's waits.
 // BMODE: 0 = B is [N][K], 1 = B is [K][N], 2 = B is [K][N] gathered from a padded image (implicit-GEMM convolution).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BMODE>
+// AMODE 1: A is gathered from a channels-last image (NhwcGather); B is then an ordinary [N][K] or [K][N] operand.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BMODE, int AMODE = 0>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(GemmArgs p) {
     constexpr bool B_KN = BMODE != 0, CONV = BMODE == 2;
+    static_assert(AMODE == 0 || BMODE != 2, "one gathered operand at a time");
     constexpr int BK = 64, LD = BK + 8, NT = WAVES_M * WAVES_N * 64;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
     constexpr int PA = BM * 8 / NT, PB = BN * 8 / NT;     // 16-byte chunks per thread per tile
@@ -408,11 +411,40 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
         cpix = p.cv.xp + (p.cv.split ? 0 : bz * p.cv.img) + (long)oh * p.cv.sy * p.cv.Wp + ow + (long)(tid / CPRB) * p.cv.HpWp;
         ctile0 = p.cv.split ? (int)bz * (p.K / BK) : 0;
     }
+    // Channels-last gather: a thread's rows are fixed output pixels; (iy0, ix0) is where tap (0, 0) of each lands.
+    int aiy0[PA], aix0[PA];
+    int atile0 = 0;
+    if constexpr (AMODE == 1) {
+#pragma unroll
+        for (int i = 0; i < PA; i++) {
+            const int c = tid + i * NT;
+            const int m = min(m0 + (c >> 3), p.M - 1);
+            const int pq = p.ag.OH * p.ag.OW;
+            const int n = m / pq, rem = m - n * pq, oh = rem / p.ag.OW, ow = rem - oh * p.ag.OW;
+            aiy0[i] = oh * p.ag.sy - p.ag.py;
+            aix0[i] = ow * p.ag.sx - p.ag.px;
+            ap[i] = p.ag.x + (long)n * p.ag.H * p.ag.W * p.ag.C + (c & 7) * 8;
+        }
+        atile0 = p.ag.split ? (int)bz * (p.K / BK) : 0;
+    }
     u32x4 ga[2][PA], gb[2][PB];
     auto gload = [&](int set, int kt) {
         const long ko = (long)kt * BK;
+        if constexpr (AMODE == 1) {
+            const int t = atile0 + kt, tap = t / p.ag.cpt, ci0 = (t - tap * p.ag.cpt) * BK;       // the same for every lane
+            const int kh = tap / p.ag.KW, kw = tap - kh * p.ag.KW;
+            const int ddy = kh * p.ag.dy, ddx = kw * p.ag.dx;
 #pragma unroll
-        for (int i = 0; i < PA; i++) ga[set][i] = ldg16(ap[i] + ko);
+            for (int i = 0; i < PA; i++) {
+                const int iy = aiy0[i] + ddy, ix = aix0[i] + ddx;
+                const bool in = (unsigned)iy < (unsigned)p.ag.H && (unsigned)ix < (unsigned)p.ag.W;
+                const u32x4 z = {0u, 0u, 0u, 0u};
+                ga[set][i] = in ? ldg16(ap[i] + ((long)iy * p.ag.W + ix) * p.ag.C + ci0) : z;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < PA; i++) ga[set][i] = ldg16(ap[i] + ko);
+        }
 #pragma unroll
         for (int i = 0; i < PB; i++) {
             if constexpr (CONV) {
@@ -1005,7 +1037,12 @@ int launch_pipe(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
                             : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
     constexpr int lds = gemm_lds_bytes<BM, BN, 64>();
-    if (a.cv.xp)   hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 2>), grid, dim3(WM * WN * 64), lds, st, a);
+    if (a.ag.x) {
+        if (a.cv.xp) return MI_DECLINE_UNSUPPORTED;
+        if (b_kn) hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 1, 1>), grid, dim3(WM * WN * 64), lds, st, a);
+        else      hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 0, 1>), grid, dim3(WM * WN * 64), lds, st, a);
+    }
+    else if (a.cv.xp)   hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 2>), grid, dim3(WM * WN * 64), lds, st, a);
     else if (b_kn) hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 1>), grid, dim3(WM * WN * 64), lds, st, a);
     else           hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 0>), grid, dim3(WM * WN * 64), lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
@@ -1101,6 +1138,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.bias_mode = bias_mode; a.epi = epi; a.out_f32 = out_dtype == MI_F32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
     a.cv = ConvGather{};
+    a.ag = NhwcGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f;
     return MI_OK;
@@ -1134,6 +1172,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
             s1.K = a.K / split;
             s1.sA = s1.K; s1.sB = b_kn ? (long)s1.K * a.ldB : s1.K; s1.sBias = 0;
             s1.cv.split = 1;
+            s1.ag.split = 1;
             // the 128 x 256 tile (two waves per SIMD) when the slices still give most CUs a workgroup
             const bool big_tiles = ceil_div(a.M, 128) * ceil_div(a.N, 256) * split >= (g_cus * 3) / 4;
             int rc = big_tiles ? launch_pipe<128, 256, 2, 4>(s1, b_kn, split, st) : launch_pipe<128, 128, 2, 2>(s1, b_kn, split, st);
@@ -1161,9 +1200,9 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         int64_t big = ceil_div(a.M, 128) * ceil_div(a.N, 256) * nbatch;
         int64_t mid = ceil_div(a.M, 128) * ceil_div(a.N, 128) * nbatch;
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
-        if (a.cv.xp && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
+        if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
         if (big * 2 > g_cus) return pipe ? launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
-        if (mid >= (g_cus * 3) / 8 || a.cv.xp) return pipe ? launch_pipe<128, 128, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
+        if (mid >= (g_cus * 3) / 8 || a.cv.xp || a.ag.x) return pipe ? launch_pipe<128, 128, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
         return launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
     }
     long total = (long)a.M * a.N;
@@ -1181,9 +1220,10 @@ int mi_num_cus() { return g_cus; }
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
                      long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st,
-                     const ConvGather *gather) {
+                     const ConvGather *gather, const NhwcGather *agather) {
     GemmArgs a;
     a.cv = ConvGather{};
+    a.ag = NhwcGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
@@ -1191,8 +1231,9 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;
     if (gather) a.cv = *gather;
+    if (agather) a.ag = *agather;
     const bool addr = mfma_addressable(a, b_kn != 0);
-    if (gather && !addr) return MI_DECLINE_OPERANDS;
+    if ((gather || agather) && !addr) return MI_DECLINE_OPERANDS;
     int path = addr ? MI_GEMM_MFMA : MI_GEMM_SCALAR;
     return run_gemm(a, b_kn != 0, nbatch, ws, ws_bytes, st, path);
 }
@@ -1221,6 +1262,10 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, true>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, false>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 2>, gemm_lds_bytes<128, 256, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 0, 1>, gemm_lds_bytes<128, 256, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 1, 1>, gemm_lds_bytes<128, 256, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, 0, 1>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, 1, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, 2>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(skinny_fk_kernel<1>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<2>, (int)SKINNY_FK_LDS_MAX);

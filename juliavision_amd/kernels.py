@@ -465,6 +465,28 @@ def convolution_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, groups, *
     return out
 
 
+def convolution_nhwc_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, *, act="none"):
+    """The convolution over channels-last tensors: ``x`` (N,H,W,Cin), ``w`` (Cout,KH,KW,Cin), ``out`` (N,OH,OW,Cout), all
+    contiguous fp16; pairs are ``(x, y)``.  An implicit GEMM with no staging pass (``mi_conv2d_nhwc_f16``); needs
+    ``Cin % 64 == 0``, otherwise ``DeclineError`` with ``L.DECLINE_UNSUPPORTED`` (use ``convolution_`` on NCHW views)."""
+    if not _is_f16_cuda(x, w, out) or x.dim() != 4 or w.dim() != 4 or not (x.is_contiguous() and w.is_contiguous() and out.is_contiguous()):
+        raise DeclineError("convolution_nhwc_: operands", L.DECLINE_OPERANDS)
+    lib = L.init()
+    N, Hi, Wi, Cin = x.shape
+    Cout, KH, KW, cin_w = w.shape
+    OW = convsize(Wi, KW, stride[0], padding[0], dilation[0])
+    OH = convsize(Hi, KH, stride[1], padding[1], dilation[1])
+    if cin_w != Cin or tuple(out.shape) != (N, OH, OW, Cout):
+        raise DeclineError("convolution_nhwc_: out must be (N,OH,OW,Cout) and w (Cout,KH,KW,Cin)", L.DECLINE_OPERANDS)
+    args = (Wi, Hi, Cin, N, KW, KH, Cout, stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1])
+    need = lib.mi_conv2d_nhwc_f16_workspace(*args)
+    ws = ctx.ws.scratch(need)
+    rc = lib.mi_conv2d_nhwc_f16(out.data_ptr(), x.data_ptr(), w.data_ptr(), _ptr(bias), *args, L.EPI[act], ws, need, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_conv2d_nhwc_f16", rc)
+    return out
+
+
 def convtransposesize(n, k, s, p, d, op):
     """convtransposesize, conv.jl:201."""
     return (n - 1) * s - 2 * p + d * (k - 1) + op + 1

@@ -89,6 +89,75 @@ def test_conv_config4_band(ctx):
     assert_parity(got[:, ch], want, what="config4 conv band")
 
 
+def _conv_nhwc(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d=1, bias=True, relu=False, seed=1):
+    """The channels-last entry point against the oracle's direct convolution over the same data re-laid to
+    (N,C,H,W): the layouts differ, the sums do not."""
+    import torch
+    import juliavision_amd as jv
+    pair = lambda v: v if isinstance(v, tuple) else (v, v)
+    s, p, d = pair(s), pair(p), pair(d)
+    x = oracle.randn_f16((N, Cin, H, W), seed)
+    w = oracle.randn_f16((Cout, Cin, KH, KW), seed + 1, 0, 0.05)
+    b = oracle.randn_f16((Cout,), seed + 2, 0, 0.5) if bias else None
+    want = oracle.conv2d_f16(x, w, b, s[::-1], p[::-1], d[::-1], 1, relu)
+    xl, wl = np.ascontiguousarray(x.transpose(0, 2, 3, 1)), np.ascontiguousarray(w.transpose(0, 2, 3, 1))
+    out = poison(torch.empty((want.shape[0], want.shape[2], want.shape[3], want.shape[1]), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.convolution_nhwc_(ctx, out, to_dev(xl), to_dev(wl), None if b is None else to_dev(b), s, p, d, act="relu" if relu else "none")
+    torch.cuda.synchronize()
+    assert_parity(to_host(out).transpose(0, 3, 1, 2), want, what=f"conv nhwc {N},{H},{W},{Cin}->{Cout} k{KH}x{KW} s{s} p{p} d{d}")
+
+
+@pytest.mark.parametrize("N,Cin,H,W,Cout,KH,KW,s,p,d,kw", [
+    (1, 256, 16, 16, 256, 3, 3, 1, 1, 1, {}),                      # config 4's 3x3 256->256 on a small map
+    (2, 64, 24, 24, 104, 3, 3, 1, 1, 1, {"relu": True}),           # two images: output rows cross the image boundary inside a tile
+    (1, 64, 40, 40, 64, 7, 7, 1, 3, 1, {"bias": False}),           # 49 taps, three pixels of padding on every side
+    (1, 128, 20, 24, 96, 5, 5, 1, (4, 2), (2, 1), {}),             # dilation 2 along x only, unequal padding; two 64-channel runs per tap
+    (1, 64, 18, 16, 48, 3, 1, (1, 2), (0, 1), 1, {}),              # 3 rows x 1 column of taps, stride 2 along y
+    (3, 64, 30, 30, 256, 5, 5, 2, 2, 1, {"relu": True}),           # stride 2 both ways, M = 675: a ragged last row tile
+    (1, 128, 8, 8, 64, 1, 1, 1, 0, 1, {}),                         # 1x1: the gather degenerates to a plain row-major operand
+    (1, 192, 12, 32, 32, 1, 3, 1, (1, 0), 1, {}),                  # KH = 1, KW = 3, three runs per tap
+    (5, 64, 3, 3, 8, 3, 3, 1, 0, 1, {}),                           # one output pixel per image, M = 5
+])
+def test_conv_nhwc(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, kw):
+    _conv_nhwc(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, **kw)
+
+
+def test_conv_nhwc_config4_is_the_nchw_result(ctx):
+    """3x3 256->256 on 64x64 at full size (M=4096, K=2304, N=256, split over K): the oracle checks 16 output channels,
+    the reference-layout path checks the rest (same products, summed in a different order: fp16 rounding apart)."""
+    import torch
+    import juliavision_amd as jv
+    x = oracle.randn_f16((1, 256, 64, 64), 7)
+    w = oracle.randn_f16((256, 256, 3, 3), 8, 0, 0.02)
+    b = oracle.randn_f16((256,), 9, 0, 0.02)
+    dx, dw, db = to_dev(x), to_dev(w), to_dev(b)
+    out = poison(torch.empty((1, 64, 64, 256), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.convolution_nhwc_(ctx, out, dx.permute(0, 2, 3, 1).contiguous(), dw.permute(0, 2, 3, 1).contiguous(), db, (1, 1), (1, 1), (1, 1))
+    ref = poison(torch.empty((1, 256, 64, 64), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.convolution_(ctx, ref, dx, dw, db, (1, 1), (1, 1), (1, 1), 1)
+    torch.cuda.synchronize()
+    got = to_host(out).transpose(0, 3, 1, 2)
+    ch = np.r_[0:8, 248:256]
+    assert_parity(got[:, ch], oracle.conv2d_f16(x, w[ch], b[ch], (1, 1), (1, 1)), what="config4 nhwc conv band")
+    assert_parity(got, to_host(ref), what="config4 nhwc vs nchw")
+
+
+def test_conv_nhwc_declines(ctx):
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd import _lib as L
+    f = lambda *sh: torch.zeros(sh, dtype=torch.float16, device="cuda")
+    with pytest.raises(jv.DeclineError) as e:      # 32 channels: not a whole 64-channel run
+        jv.convolution_nhwc_(ctx, f(1, 8, 8, 64), f(1, 8, 8, 32), f(64, 3, 3, 32), None, (1, 1), (1, 1), (1, 1))
+    assert e.value.status == L.DECLINE_UNSUPPORTED
+    with pytest.raises(jv.DeclineError) as e:      # output of the wrong extent
+        jv.convolution_nhwc_(ctx, f(1, 8, 8, 64), f(1, 8, 8, 64), f(64, 3, 3, 64), None, (2, 2), (1, 1), (1, 1))
+    assert e.value.status == L.DECLINE_OPERANDS
+
+
 def _convt(ctx, N, Cin, H, W, Cout, KH, KW, s, p=0, d=1, op=0, groups=1, bias=True, expect=None, seed=1):
     """``s``, ``p``, ``d``, ``op``: one number for both axes or an ``(x, y)`` pair."""
     import torch
