@@ -476,6 +476,9 @@ def detail_benchmarks(lib, L, stream, only=None):
     gemm_case("c3_fc2_1370x1536x384", 1370, 1536, 384, L.W_KF)
     attn_case("c3_attn_L1370_6x64", 1, 6, 1370, 1370, 64)
     attn_case("c2_attn_L1500_20x64", 1, 20, 1500, 1500, 64)
+    # the reference's own SAM 2.1 attention shapes, head size 72: global blocks and 16 windows of 256 (tools/attn_lab.jl:8-14)
+    attn_case("sam2_global_attn_L4096_8x72", 1, 8, 4096, 4096, 72)
+    attn_case("sam2_window_attn_L256_8x72_b16", 16, 8, 256, 256, 72)
     def conv_case():
         x = torch.randn((1, 256, 64, 64), dtype=f16, device="cuda")
         w = torch.randn((256, 256, 3, 3), dtype=f16, device="cuda") * 0.02

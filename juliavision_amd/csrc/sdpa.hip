@@ -89,12 +89,16 @@ __device__ __forceinline__ void static_for(F &&f) {
 // same 32 queries and share a SIMD; a stage holds 128 keys, of which waves 0-3 take the first 64 and waves 4-7 the
 // second, so each wave walks half of the keys and a SIMD always has a second wave to run.  The two partial
 // (O, M, l) of a query meet in LDS at the end (the merge identity of flash.jl:1385-1391), waves 0-3 store.
+// Halves per V row in LDS: a multiple of 64 plus 32, so that consecutive key rows start 64 bytes apart modulo the
+// 128 bytes of the banks (96 for head sizes 64 and 96, 160 for 128; 112 measured the same as 96 at 96).
+constexpr int flash_vld(int EP) { return EP == 96 ? EP : EP + 32; }
+
 template <int EP, bool PP, int KH = 1>
-__global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 64 && !PP && KH == 1) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
+__global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH == 1) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
     static_assert(KH == 1 || (KH == 2 && !PP), "key halves or ping-pong, not both");
     constexpr int BC = 64, BR = PP ? 256 : 128, NT = KH == 2 ? 512 : 256;     // NT: threads that stage K and V
     constexpr int BCS = BC * KH;                                                // keys per LDS stage
-    constexpr int KLD = EP + 8, VLD = EP + 32;
+    constexpr int KLD = EP + 8, VLD = flash_vld(EP);
     constexpr int KS = EP / 16;       // k16 steps over the head dim
     constexpr int ET = EP / 32;       // 32-wide head-dim tiles of O
     constexpr int KCH = EP / 8;       // 16-byte chunks per key row
@@ -405,8 +409,9 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 64 && !PP && KH
         // Waves 4-7 hand their (O, M, l) to the wave that owns the same queries; the last block's barrier has
         // passed, so the stages are idle.  Lane-major slots: the partner's lane holds the same elements.
         constexpr int SLOT = (ET * 16 + 2) * 64;
-        float *xo = reinterpret_cast<float *>(smem + 36864) + qw * SLOT;
-        static_assert(36864 + 4 * SLOT * 4 <= 3 * BCS * (KLD + VLD) * 2 && 4 * 32 * (EP + 4) * 4 <= 36864, "merge slots overlap the store staging or leave the stages");
+        constexpr int MOFF = (4 * 32 * (EP + 4) * 4 + 255) / 256 * 256;      // past what the store staging will use
+        float *xo = reinterpret_cast<float *>(smem + MOFF) + qw * SLOT;
+        static_assert(MOFF + 4 * SLOT * 4 <= 3 * BCS * (KLD + VLD) * 2, "merge slots leave the stages");
         if (grp == 1) {
 #pragma unroll
             for (int t = 0; t < ET; t++)
@@ -837,7 +842,7 @@ __global__ void sdpa_merge_kernel(SdpaArgs p) {
 }
 
 // ------------------------------------------------------------------------------------------
-constexpr int flash_lds_bytes(int EP) { return 3 * 64 * (EP + 8) * 2 + 3 * 64 * (EP + 32) * 2; }
+constexpr int flash_lds_bytes(int EP) { return 3 * 64 * (EP + 8) * 2 + 3 * 64 * flash_vld(EP) * 2; }
 
 bool vec_addressable(const half_t *ptr, const long st[4], int E) {
     return st[0] == 1 && E % 8 == 0 && st[1] % 8 == 0 && st[2] % 8 == 0 && st[3] % 8 == 0 && aligned_to(ptr, 16);
@@ -861,9 +866,11 @@ int rows_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
 // and the merge is a second launch of about 6 us, so splitting pays only when the query blocks leave most
 // of the chip idle and every split still walks a dozen blocks (config 3's 66 workgroups x 22 blocks do
 // not: 21.9 us unsplit, 21.1 us at best split three ways).
-int flash_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+int flash_splits(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     const int64_t wgs = ceil_div(Lq, 128) * H * B, cus = mi_num_cus();
-    if (wgs * 2 > cus) return 1;
+    // At head size 64 a grid of up to one workgroup per CU runs the eight-wave key-halves variant instead; wider
+    // heads have no such variant, and two workgroups per CU is what gives their SIMDs a second wave.
+    if (E <= 64 ? wgs * 2 > cus : wgs > cus) return 1;
     int64_t want = ceil_div(cus * 3 / 2, wgs);
     const int64_t blocks = ceil_div(Lk, 64);
     if (want > blocks / 12) want = blocks / 12;
@@ -927,6 +934,7 @@ int mi_sdpa_init() {
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     return bad;
 }
@@ -936,7 +944,7 @@ extern "C" {
 size_t mi_sdpa_f16_workspace(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, int has_bias) {
     // sized for the path the call will most likely take: the fused kernel's key splits for Lq >= 64 without
     // an additive mask (unused if the operands turn out not to be 16-byte addressable), the rows kernel's below
-    int ns = Lq >= 64 ? (has_bias ? 1 : flash_splits(Lq, Lk, H, B)) : rows_splits(Lq, Lk, H, B);
+    int ns = Lq >= 64 ? (has_bias ? 1 : flash_splits(E, Lq, Lk, H, B)) : rows_splits(Lq, Lk, H, B);
     if (ns <= 1) return 0;
     size_t rows = (size_t)Lq * H * B;
     return round_up((size_t)ns * rows * E * sizeof(float), 256) + round_up((size_t)ns * rows * 2 * sizeof(float), 256);
@@ -954,7 +962,7 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
     int path = sdpa_path(a);
     const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
     if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? (one_pass_decode(a, vec) ? 1 : rows_splits(Lq, Lk, H, B))
-                                  : path == MI_SDPA_FLASH ? flash_splits(Lq, Lk, H, B) : 1;
+                                  : path == MI_SDPA_FLASH ? flash_splits(E, Lq, Lk, H, B) : 1;
     return path;
 }
 
@@ -981,7 +989,7 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
             hipLaunchKernelGGL((flash_fwd_kernel<64, true>), grid, dim3(512), flash_lds_bytes(64), st, a);
         } else {
             // few query blocks: split the keys over workgroups too, if the caller brought the workspace for it
-            a.nsplit = flash_splits(Lq, Lk, H, B);
+            a.nsplit = flash_splits(E, Lq, Lk, H, B);
             const size_t rows = (size_t)Lq * H * B;
             const size_t o_bytes = round_up((size_t)a.nsplit * rows * E * sizeof(float), 256);
             if (a.nsplit > 1 && ws && aligned_to(ws, 256) && ws_bytes >= o_bytes + round_up((size_t)a.nsplit * rows * 2 * sizeof(float), 256)) {
@@ -992,9 +1000,12 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
             }
             dim3 grid((unsigned)(ceil_div(Lq, 128) * a.nsplit), (unsigned)H, (unsigned)B);
             // no CU would hold two workgroups anyway: eight waves per workgroup, each with half of the keys
+            // (head size 64 only: the 96-wide instance of this variant measured slower than four waves, 115 us
+            // against 106 us on 8 heads x 4096 x 72)
             const bool halves = E <= 64 && a.nsplit == 1 && ceil_div(Lq, 128) * H * B <= (int64_t)mi_num_cus() && Lk >= 256;
             if (halves)       hipLaunchKernelGGL((flash_fwd_kernel<64, false, 2>), grid, dim3(512), 2 * flash_lds_bytes(64), st, a);
             else if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false>), grid, dim3(256), flash_lds_bytes(64), st, a);
+            else if (E <= 96) hipLaunchKernelGGL((flash_fwd_kernel<96, false>), grid, dim3(256), flash_lds_bytes(96), st, a);
             else         hipLaunchKernelGGL((flash_fwd_kernel<128, false>), grid, dim3(256), flash_lds_bytes(128), st, a);
             if (a.nsplit > 1) {
                 const long total = (long)Lq * H * B * E;

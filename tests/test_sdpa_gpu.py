@@ -52,6 +52,21 @@ def test_flash_shapes(ctx, B, H, Lq, Lk, E):
     _check(ctx, q, k, v, expect="FlashPlan", what=f"flash {B},{H},{Lq},{Lk},{E}")
 
 
+@pytest.mark.parametrize("B,H,Lq,Lk,E,kw", [
+    (1, 2, 256, 256, 72, {}),                              # SAM 2's windowed attention: 256 tokens, head size 72 (tools/attn_lab.jl:8-14)
+    (1, 1, 300, 1000, 72, {}),                             # ragged queries and keys, a masked last block
+    (2, 2, 128, 200, 80, {"kv_len": [200, 77]}),           # per-batch valid keys
+    (1, 2, 130, 129, 88, {"out_dtype": "f32"}),            # one key in the last block; fp32 rows out
+    (1, 1, 192, 320, 96, {}),                              # the variant's full width
+    (1, 1, 128, 2048, 72, {}),                             # one query block over 32 key blocks: the keys are split over workgroups
+])
+def test_flash_head_sizes_65_to_96(ctx, B, H, Lq, Lk, E, kw):
+    """Head sizes in (64, 96] run the 96-wide instance of the fused kernel (six k-steps in the first product, three
+    32-wide output tiles), not the 128-wide one."""
+    q, k, v = _qkv(B, H, Lq, Lk, E, 61)
+    _check(ctx, q, k, v, expect="FlashPlan", what=f"flash {B},{H},{Lq},{Lk},{E}", **kw)
+
+
 def test_flash_small_inputs_and_f32_out(ctx):
     # the reference's own test inputs: randn * 0.2 (test_flash.jl:41-43)
     q, k, v = _qkv(2, 2, 128, 128, 72, 41, std=0.2)
