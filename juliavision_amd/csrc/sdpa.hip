@@ -49,7 +49,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 // Fused kernel.  Workgroup = 4 waves = 128 queries (32 per wave); keys walked in
 // blocks of BC = 64 through three LDS stages, both operands as they lie in memory:
 //   Ks [BC][EP+8]    keys x head-dim   (A operand of S^T = K.Q^T, plain 16-byte reads)
-//   Vs [BC][EP+32]   keys x head-dim   (A operand of O^T = V^T.P^T through
+//   Vs [BC][VLD]     keys x head-dim   (VLD = flash_vld(EP); A operand of O^T = V^T.P^T through
 //                    ds_read_b64_tr_b16, which transposes 4 keys x 16 head-dim
 //                    values per 16 lanes on the way out of LDS)
 //
@@ -70,9 +70,9 @@ __device__ __forceinline__ void static_for(F &&f) {
 //     needs no further arithmetic (M is kept fp16-representable so that what is
 //     subtracted is exactly what the bookkeeping assumes);
 //   * M is a *stale* reference, not the running maximum: it moves on the first
-//     block and when a probability leaves fp16 range (t >= 16, seen as an infinite
-//     row sum), and then to the block maximum.  In between no maximum is computed
-//     at all.  The result is the same softmax -- every term of a row carries the
+//     block and when a probability would leave fp16 range (the block's largest t
+//     reaches 16; one v_max3_f32 per two scores keeps track of it), and then to the
+//     block maximum.  The result is the same softmax -- every term of a row carries the
 //     same factor 2^-M -- with the rescaling of flash.jl:25-38 applied lazily (the
 //     reference's `lazyrescale`, flash.jl:1041-1096, skips it when no maximum grew;
 //     this skips it until fp16 would overflow);

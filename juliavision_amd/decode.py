@@ -19,7 +19,7 @@ from typing import Callable, List, Optional
 import torch
 
 from . import _lib as L
-from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, sdpa, sdpa_append
+from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, matmul_heads_, sdpa, sdpa_append
 
 
 # Fold the cache write into the self-attention launch where the one-launch kernel covers the shape.
@@ -49,6 +49,17 @@ class KVCache:
         rc = L.init().mi_kv_advance(self.length.data_ptr(), self.batch, int(delta), self.max_target, ctx.stream)
         if rc != L.OK:
             raise DeclineError("mi_kv_advance", rc)
+
+    def fill_cross(self, ctx: Ctx, layer: int, enc: torch.Tensor, wk, bk, wv, bv):
+        """Project the encoder output into ``layer``'s cross-attention K/V, once per window (fillcross!, decode.jl:173-177:
+        the ``whispercross`` graph's two matmuls per layer).  ``enc``: ``(B, src_len, d)`` fp16; ``wk``, ``wv``: ``(d, H*E)``
+        weights in either memory layout; ``bk``, ``bv``: ``(H*E,)`` or None.  The GEMMs write the cache's head-major rows
+        themselves: no intermediate, no permute, no copy."""
+        if enc.dim() != 3 or enc.shape[0] != self.batch or enc.shape[1] != self.cross_k.shape[3]:
+            raise DeclineError("fill_cross: enc must be (B, src_len, d)", L.DECLINE_OPERANDS)
+        for store, w, bias in ((self.cross_k, wk, bk), (self.cross_v, wv, bv)):
+            for b in range(self.batch):
+                matmul_heads_(ctx, store[layer, b], w, enc[b], bias)
 
     def append(self, ctx: Ctx, layer: int, k_new: torch.Tensor, v_new: torch.Tensor):
         """Write the new token's K/V rows ``(B,H,1,E)`` into slot ``length-1`` of ``layer``."""

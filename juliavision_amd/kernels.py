@@ -301,6 +301,29 @@ def batchedmatmul_(ctx: Ctx, out, A, B):
     return out
 
 
+def matmul_heads_(ctx: Ctx, out, A, B, bias=None):
+    """A projection written head-major: ``out[h] = B[T,K] . A[:, h*E:(h+1)*E] + bias[h*E:(h+1)*E]`` for ``out`` torch
+    ``(H, T, E)`` with contiguous rows -- the ``(E, L, H)`` operand attention reads, with no permute between the linear
+    op and the cache (the reference's graphs do ``view`` + ``permute`` + ``copyto!``, decode.jl:173-177).  ``A``: torch
+    ``(K, H*E)`` weight in either memory layout.  One batched launch, a head per batch plane."""
+    lib = L.init()
+    la, lb = _mat2(A), _mat2(B)
+    if not _is_f16_cuda(A, B, out) or out.dim() != 3 or la is None or lb is None or lb[0] != 0:
+        raise DeclineError("matmul_heads_: operands", L.DECLINE_OPERANDS)
+    H, T, E = out.shape
+    K, F = A.shape
+    if F != H * E or tuple(B.shape) != (T, K) or out.stride(2) != 1 or (bias is not None and bias.numel() != F):
+        raise DeclineError("matmul_heads_: out must be (H,T,E) with F = H*E", L.DECLINE_OPERANDS)
+    w_layout = L.W_KF if la[0] == 0 else L.W_FK
+    sW = E if w_layout == L.W_KF else E * la[1]
+    rc = lib.mi_gemm_f16_batched(out.data_ptr(), B.data_ptr(), A.data_ptr(), _ptr(bias), None, T, K, E,
+                                 out.stride(1), lb[1], la[1], w_layout, L.BIAS_NONE if bias is None else L.BIAS_COL,
+                                 L.EPI["none"], L.F16, H, out.stride(0), 0, sW, E, None, 0, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_gemm_f16_batched", rc)
+    return out
+
+
 # ----------------------------------------------------------------------------- attention
 
 @dataclass(frozen=True)

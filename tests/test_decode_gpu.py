@@ -208,3 +208,28 @@ def test_fused_append_declines_what_the_one_launch_kernel_does_not_cover(ctx):
         jv.sdpa_append(ctx, z(B, H, 1, E), z(B, H, Lmax, E), z(B, H, Lmax, E), z(B, H, 1, E), z(B, H, 1, E),
                        torch.ones((B,), dtype=torch.int32, device="cuda"), out=z(B, H, 1, E))
     assert e.value.status == L.DECLINE_UNSUPPORTED
+
+
+@pytest.mark.parametrize("layout", ["kf", "fk"])
+@pytest.mark.parametrize("B,S,H,E", [(1, 200, 4, 64), (2, 77, 3, 32)])
+def test_fill_cross_writes_the_projections_head_major(ctx, B, S, H, E, layout):
+    """fillcross! (decode.jl:173-177): cross K/V of a layer = the encoder output through k_proj (no bias in Whisper) and
+    v_proj, laid out (B,H,S,E).  Checked against the oracle's GEMM re-laid on the host; the other layer stays untouched."""
+    import torch
+    from juliavision_amd.decode import KVCache
+    d = H * E
+    enc = oracle.randn_f16((B, S, d), 3)
+    wk, wv = oracle.randn_f16((d, d), 4, std=0.05), oracle.randn_f16((d, d), 5, std=0.05)
+    bv = oracle.randn_f16((d,), 6, std=0.1)
+    dev_w = lambda w: to_dev(w) if layout == "kf" else to_dev(np.ascontiguousarray(w.T)).t()
+    cache = KVCache(2, B, H, E, max_target=8, src_len=S)
+    cache.cross_k.fill_(7.0)
+    cache.cross_v.fill_(7.0)
+    cache.fill_cross(ctx, 1, to_dev(enc), dev_w(wk), None, dev_w(wv), to_dev(bv))
+    torch.cuda.synchronize()
+    for store, w, bias in ((cache.cross_k, wk, None), (cache.cross_v, wv, bv)):
+        got = to_host(store)
+        assert np.all(got[0] == np.float16(7.0))
+        for b in range(B):
+            want = oracle.gemm_f16(enc[b], w, bias).reshape(S, H, E).transpose(1, 0, 2)
+            assert_parity(got[1, b], want, what=f"fill_cross batch {b}")
