@@ -8,9 +8,9 @@ through one handler per ATen op (``runop!``, ``execute.jl:493-539``, ``ops.jl``)
 This module reads the same schema, keeps the handler-per-op shape, and covers
 the ops of the dense-contraction path:
 
-    linear / addmm / mm, scaled_dot_product_attention, layer_norm /
-    native_layer_norm, gelu, relu, add.Tensor, convolution, and the view ops
-    between them.
+    linear / addmm / mm / bmm, scaled_dot_product_attention (also written out
+    as bmm + softmax + bmm), layer_norm / native_layer_norm, gelu, relu,
+    add.Tensor, convolution, and the view ops between them.
 
 Two of the reference's rewrites matter for that path and have counterparts here:
 
@@ -23,7 +23,9 @@ Two of the reference's rewrites matter for that path and have counterparts here:
 and two more fall out of what the kernels accept: the residual ``add.Tensor``
 after a linear rides in its GEMM store (``fold_residuals``; the reference's own
 next item, plans/perf-plan.md:4074-4095), and attention writes its output
-token-major when the graph transposes it straight back (``fold_sdpa_transpose``).
+token-major when the graph transposes it straight back (``fold_sdpa_transpose``);
+attention exported as ``bmm`` + ``_softmax`` + ``bmm`` (DINOv2) is put back together
+(``fold_attention``).
 
 An op outside the list raises :class:`UnsupportedOp`; there is no eager fallback.
 ``convert`` produces the schema from an ``ExportedProgram`` (static shapes only),
@@ -273,6 +275,144 @@ def fold_layernorms(g: Graph) -> Graph:
     return g
 
 
+LAYOUT_VIEWS = RESHAPES + ("expand.default", "contiguous.default")
+SOFTMAX_OPS = ("_softmax.default", "softmax.int")
+
+
+def _layout_source(g: Graph, bid: str, used: List[str]) -> str:
+    """Walk up from ``bid`` through steps that move no values -- reshaping views, expands to the same shape and
+    contiguous ``clone`` ops -- to the buffer they all show; ``used`` collects the clone ops passed."""
+    while True:
+        b = g.buffers[bid]
+        if b["kind"] == "view" and b.get("op") in LAYOUT_VIEWS:
+            if b["op"] == "expand.default" and list(b.get("shape", [])) != list(g.buffers[b["of"]].get("shape", [])):
+                return bid                              # a broadcasting expand does move values
+            bid = b["of"]
+            continue
+        prod = g.op(bid)
+        if prod is not None and prod["aten"] == "clone.default":
+            used.append(prod["id"])
+            bid = prod["in"][0]
+            continue
+        return bid
+
+
+def _consumers(g: Graph, bid: str) -> set:
+    """Ids of the ops that read ``bid`` directly or through any chain of views; ``"<output>"`` if the graph returns it."""
+    seen, todo, ops = set(), [bid], set()
+    while todo:
+        x = todo.pop()
+        if x in seen:
+            continue
+        seen.add(x)
+        if x in g.outputs:
+            ops.add("<output>")
+        for r in g.readers(x):
+            if g.op(r) is not None:
+                ops.add(r)
+            else:
+                todo.append(r)
+    return ops
+
+
+def _scalar_scale(o) -> Optional[float]:
+    """The factor of ``mul.Tensor(x, c)`` / ``div.Tensor(x, c)`` with a constant ``c``; None for anything else."""
+    if o is None or o["aten"] not in ("mul.Tensor", "div.Tensor") or len(o["in"]) != 1:
+        return None
+    c = o["attrs"].get("arg1")
+    if not isinstance(c, (int, float)) or isinstance(c, bool) or c == 0:
+        return None
+    return float(c) if o["aten"] == "mul.Tensor" else 1.0 / float(c)
+
+
+def fold_attention(g: Graph) -> Graph:
+    """Attention written out as ``bmm -> (scale) -> softmax -> bmm`` becomes the fused op.
+
+    Models whose attention does not reach ``scaled_dot_product_attention`` export this way -- DINOv2 inside
+    Depth Anything carries 24 ``bmm`` and 12 ``_softmax`` (DepthAnythingRunner.jl:38-42), which the reference runs
+    through ``batchedmatmul!`` (ops.jl:1393-1399) and its softmax kernel (ops.jl:557-573).  Matched: a softmax over
+    the last axis whose input is ``q3 @ k3^T``, optionally scaled by a constant before (on q) or after (on the
+    scores), and whose only use is ``p3 @ v3``; the 3-D operands are reshapes (with or without the contiguous
+    copies a batch > 1 puts in) of 4-D ``(B, H, L, E)`` tensors.  Everything between disappears: the scores never
+    exist in memory."""
+    for sm in [o for o in g.ops if o["aten"] in SOFTMAX_OPS]:
+        sb = g.buffers[sm["out"]]
+        nd = len(sb.get("shape", []))
+        if nd < 3 or sm["attrs"].get("arg1") not in (-1, nd - 1) or sm["attrs"].get("arg2") not in (None, False):
+            continue
+        dead: List[str] = [sm["id"]]
+        # -- up: the scores
+        scale = 1.0
+        src = _layout_source(g, sm["in"][0], dead)
+        post = g.op(src)
+        if _scalar_scale(post) is not None:
+            scale *= _scalar_scale(post)
+            dead.append(post["id"])
+            src = _layout_source(g, post["in"][0], dead)
+        bmm1 = g.op(src)
+        if bmm1 is None or bmm1["aten"] != "bmm.default":
+            continue
+        dead.append(bmm1["id"])
+        q4 = _layout_source(g, bmm1["in"][0], dead)
+        pre = g.op(q4)
+        if _scalar_scale(pre) is not None:
+            scale *= _scalar_scale(pre)
+            dead.append(pre["id"])
+            q4 = _layout_source(g, pre["in"][0], dead)
+        kt = g.buffers[_layout_source(g, bmm1["in"][1], dead)]
+        swapped = kt["kind"] == "view" and (
+            (kt.get("op") == "permute.default" and [x % 4 for x in kt["attrs"].get("arg1", [])] == [0, 1, 3, 2]) or
+            (kt.get("op") == "transpose.int" and sorted(x % 4 for x in (kt["attrs"].get("arg1"), kt["attrs"].get("arg2"))) == [2, 3]))
+        if not swapped:
+            continue
+        k4 = kt["of"]
+        # -- down: the only use of the probabilities is the second product
+        rd, cur = [], sm["out"]
+        while True:
+            rd = g.readers(cur)
+            if len(rd) != 1:
+                break
+            nxt = g.buffers.get(rd[0])
+            if nxt is not None and nxt["kind"] == "view" and nxt.get("op") in LAYOUT_VIEWS:
+                cur = rd[0]
+                continue
+            o = g.op(rd[0])
+            if o is not None and o["aten"] == "clone.default":
+                dead.append(o["id"])
+                cur = o["out"]
+                continue
+            break
+        bmm2 = g.op(rd[0]) if len(rd) == 1 else None
+        if bmm2 is None or bmm2["aten"] != "bmm.default" or g.root(bmm2["in"][0]) not in (sm["out"], *dead):
+            continue
+        v4 = _layout_source(g, bmm2["in"][1], dead)
+        shapes = [g.buffers[x].get("shape") for x in (q4, k4, v4)]
+        if any(sh is None or len(sh) != 4 for sh in shapes):
+            continue
+        (B, H, Lq, E), (_, _, Lk, _) = shapes[0], shapes[1]
+        if shapes[1] != [B, H, Lk, E] or shapes[2] != [B, H, Lk, E] or g.buffers[bmm2["out"]].get("shape") != [B * H, Lq, E]:
+            continue
+        # every intermediate is read by this chain only, directly or through views, and is no output of the graph
+        mine = set(dead) | {bmm2["id"]}
+        if any(not _consumers(g, g.op(d)["out"]) <= mine for d in dead):
+            continue
+        new_id = bmm2["id"] + "_sdpa"
+        g.buffers[new_id] = {"id": new_id, "kind": "transient", "shape": [B, H, Lq, E], "dtype": g.buffers[bmm2["out"]]["dtype"]}
+        at = g.ops.index(bmm2)
+        g.ops[at] = {"id": new_id, "aten": "scaled_dot_product_attention.default", "in": [q4, k4, v4], "out": new_id,
+                     "attrs": {"scale": scale * 1.0}}
+        g.ops = [o for o in g.ops if o["id"] not in dead]
+        out3 = bmm2["out"]
+        g.buffers[out3].update(kind="view", of=new_id, op="view.default", attrs={"arg1": [B * H, Lq, E]})
+        # a view of the product back to (B, H, Lq, E) reads the fused op's result as it is
+        back = [r for r in g.readers(out3) if g.buffers.get(r, {}).get("kind") == "view" and g.buffers[r].get("shape") == [B, H, Lq, E]]
+        if back and len(g.readers(out3)) == 1 and out3 not in g.outputs:
+            g.buffers[back[0]].update(of=new_id, op="alias.default", attrs={})
+            del g.buffers[out3]
+        g.notes.append(f"fold {bmm1['id']} / {sm['id']} / {bmm2['id']} into {new_id} (scale {scale:g})")
+    return g
+
+
 def fold_sdpa_transpose(g: Graph) -> Graph:
     """Attention whose only reader swaps the head and token axes back (``transpose(1, 2)`` /
     ``permute(0, 2, 1, 3)``): the kernel writes token-major, the swap becomes the view it already is, and
@@ -283,7 +423,9 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
         rd = g.readers(o["id"])
         if len(rd) == 1 and "getitem" in g.buffers[rd[0]].get("op", "") and g.buffers[rd[0]]["attrs"].get("arg1", 0) == 0:
             rd = g.readers(rd[0])                       # the tuple-returning forms: look past the selection of element 0
-        if len(rd) != 1 or g.buffers[rd[0]]["kind"] != "view":
+        while len(rd) == 1 and g.buffers.get(rd[0], {}).get("kind") == "view" and g.buffers[rd[0]].get("op") == "alias.default":
+            rd = g.readers(rd[0])
+        if len(rd) != 1 or g.buffers.get(rd[0], {}).get("kind") != "view":
             continue
         v = g.buffers[rd[0]]
         swap = (v["op"] == "transpose.int" and sorted(x % 4 for x in (v["attrs"].get("arg1"), v["attrs"].get("arg2"))) == [1, 2]) or \
@@ -291,11 +433,19 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
         if swap:
             o["attrs"]["token_major"] = True
             g.notes.append(f"{o['id']} writes token-major")
+            # the contiguous copy a decomposed reshape puts after the swap has nothing left to do
+            vr = g.readers(v["id"])
+            cl = g.op(vr[0]) if len(vr) == 1 else None
+            if cl is not None and cl["aten"] == "clone.default" and cl["attrs"].get("memory_format", "torch.contiguous_format") in (
+                    "torch.contiguous_format", "contiguous_format"):
+                g.ops.remove(cl)
+                g.buffers[cl["out"]].update(kind="view", of=v["id"], op="alias.default", attrs={})
+                g.notes.append(f"{cl['id']} is a view of the token-major result")
     return g
 
 
 def optimize(g: Graph) -> Graph:
-    return fold_sdpa_transpose(fold_layernorms(fold_residuals(fold_activations(g))))
+    return fold_sdpa_transpose(fold_attention(fold_layernorms(fold_residuals(fold_activations(g)))))
 
 
 # ----------------------------------------------------------------------------- execution
@@ -320,7 +470,8 @@ class Executor:
                 self.t[b["id"]] = w.to(self.device, _DTYPES[b["dtype"]]).contiguous()
         for o in graph.ops:                               # check every op has a handler before anything runs
             if o["aten"] not in self.HANDLERS:
-                raise UnsupportedOp(f"{graph.name}: no kernel on this path for aten.{o['aten']} (op {o['id']})")
+                hint = " -- inside bmm + softmax + bmm, optimize() folds it into the fused attention" if o["aten"] in SOFTMAX_OPS else ""
+                raise UnsupportedOp(f"{graph.name}: no kernel on this path for aten.{o['aten']} (op {o['id']}){hint}")
         for o in graph.ops:                               # a norm folded into its producer: its result still needs a home
             nid = o["attrs"].get("ln_out")
             if nid is not None:
@@ -440,6 +591,11 @@ class Executor:
         self.ctx.ws.reset()
         K.sdpa(self.ctx, q, k, v, bias, a.get("scale"), out=self.t[o["out"]])
 
+    def _bmm(self, o):
+        """bmm(a (B,m,k), b (B,k,n)) -- batchedmatmul!, ops.jl:1393-1399."""
+        a, b = self.get(o["in"][0]), self.get(o["in"][1])
+        K.batchedmatmul_(self.ctx, self.t[o["out"]], b, a)
+
     def _layer_norm(self, o):
         ins, a = o["in"], o["attrs"]
         x = self.get(ins[0])
@@ -498,7 +654,8 @@ class Executor:
     HANDLERS = {"linear.default": _linear, "addmm.default": _linear, "mm.default": _linear,
                 **dict.fromkeys(SDPA_OPS, _sdpa), "layer_norm.default": _layer_norm,
                 "native_layer_norm.default": _native_layer_norm, "add.Tensor": _add,
-                "gelu.default": _activation, "relu.default": _activation, "convolution.default": _convolution}
+                "gelu.default": _activation, "relu.default": _activation, "convolution.default": _convolution,
+                "bmm.default": _bmm}
 
     def __call__(self, *inputs: torch.Tensor):
         if len(inputs) != len(self.g.inputs):

@@ -270,3 +270,95 @@ def test_executor_takes_weights_from_a_safetensors_file(ctx, tmp_path):
     with torch.no_grad():
         want = m.float()(x.float()).numpy()
     assert_parity(run(x.cuda()).float().cpu().numpy(), want, what="block from graph JSON + safetensors")
+
+
+def _written_out_attention(style, d=128, heads=2, seed=0, return_probs=False):
+    """Attention as the models that never reach ``scaled_dot_product_attention`` write it: DINOv2's (q scaled
+    first, ``@``, softmax, ``@``; Depth Anything's backbone) or the eager Hugging Face form (scores divided by
+    sqrt(E) after the product)."""
+    import torch
+    import torch.nn as nn
+
+    class Attn(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.h, self.scale = heads, (d // heads) ** -0.5
+            self.qkv, self.proj = nn.Linear(d, 3 * d), nn.Linear(d, d)
+
+        def forward(self, x):
+            B, N, C = x.shape
+            qkv = self.qkv(x).reshape(B, N, 3, self.h, C // self.h).permute(2, 0, 3, 1, 4)
+            if style == "dinov2":
+                q, k, v = qkv[0] * self.scale, qkv[1], qkv[2]
+                attn = (q @ k.transpose(-2, -1)).softmax(dim=-1)
+                y = (attn @ v).transpose(1, 2).reshape(B, N, C)
+            else:
+                attn = torch.matmul(qkv[0], qkv[1].transpose(-1, -2)) / (C // self.h) ** 0.5
+                attn = torch.nn.functional.softmax(attn, dim=-1)
+                y = torch.matmul(attn, qkv[2]).permute(0, 2, 1, 3).contiguous().view(B, N, C)
+            return (self.proj(y), attn) if return_probs else self.proj(y)
+
+    torch.manual_seed(seed)
+    return Attn().eval().half()
+
+
+@pytest.mark.parametrize("style", ["dinov2", "hf_eager"])
+@pytest.mark.parametrize("B", [1, 2])
+def test_written_out_attention_folds_into_the_fused_op(style, B):
+    """24 bmm + 12 _softmax is how the reference's Depth Anything graph holds its attention
+    (DepthAnythingRunner.jl:38-42); with a batch the export also copies the operands contiguous first."""
+    import torch
+    from juliavision_amd import graph as G
+    m = _written_out_attention(style)
+    ep = torch.export.export(m, (torch.randn(B, 70, 128).half(),)).run_decompositions()
+    d = G.convert(ep, "attn")
+    aten = [o["aten"] for o in d["ops"]]
+    assert aten.count("bmm.default") == 2 and aten.count("_softmax.default") == 1
+    g = G.optimize(G.Graph.load(d))
+    assert [o["aten"] for o in g.ops] == ["addmm.default", "scaled_dot_product_attention.default", "addmm.default"], g.notes
+    att = g.ops[1]
+    assert att["attrs"]["scale"] == pytest.approx(0.125) and att["attrs"]["token_major"] is True
+    assert [g.buffers[i]["shape"] for i in att["in"]] == [[B, 2, 70, 64]] * 3
+
+
+def test_attention_whose_probabilities_are_returned_stays_as_it_is():
+    import torch
+    from juliavision_amd import graph as G
+    m = _written_out_attention("hf_eager", return_probs=True)
+    ep = torch.export.export(m, (torch.randn(1, 70, 128).half(),)).run_decompositions()
+    g = G.optimize(G.Graph.load(G.convert(ep, "attn")))
+    assert [o["aten"] for o in g.ops].count("bmm.default") == 2 and not any("sdpa" in n for n in g.notes)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("style,B", [("dinov2", 1), ("dinov2", 2), ("hf_eager", 1)])
+def test_written_out_attention_runs_on_the_fused_kernel(ctx, style, B):
+    import torch
+    from juliavision_amd import graph as G
+    m = _written_out_attention(style, seed=3)
+    x = torch.randn(B, 70, 128).half()
+    ep = torch.export.export(m, (x,)).run_decompositions()
+    run = G.Executor(G.optimize(G.Graph.load(G.convert(ep, "attn"))), m.state_dict(), ctx)
+    with torch.no_grad():
+        want = m.float()(x.float()).numpy()
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    assert_parity(got.float().cpu().numpy(), want, what=f"written-out attention, {style}, batch {B}")
+
+
+@pytest.mark.gpu
+def test_bmm_runs_on_the_batched_gemm(ctx):
+    """aten::bmm on its own (ops.jl:1393-1399 -> batchedmatmul!)."""
+    import torch
+    from juliavision_amd import graph as G
+
+    class M(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.bmm(a, b)
+
+    a, b = torch.randn(6, 70, 64).half(), torch.randn(6, 64, 40).half()
+    ep = torch.export.export(M(), (a, b)).run_decompositions()
+    run = G.Executor(G.Graph.load(G.convert(ep, "bmm")), {}, ctx)
+    got = run(a.cuda(), b.cuda())
+    torch.cuda.synchronize()
+    assert_parity(got.float().cpu().numpy(), torch.bmm(a.float(), b.float()).numpy(), what="bmm")
