@@ -10,7 +10,8 @@ the ops of the dense-contraction path:
 
     linear / addmm / mm / bmm, scaled_dot_product_attention (also written out
     as bmm + softmax + bmm), layer_norm / native_layer_norm, gelu, relu,
-    add.Tensor, convolution, and the view ops between them.
+    add.Tensor, convolution, cat along the token axis, a per-feature
+    mul.Tensor after a linear (LayerScale), and the view ops between them.
 
 Two of the reference's rewrites matter for that path and have counterparts here:
 
@@ -192,6 +193,8 @@ class Graph:
 
 # ----------------------------------------------------------------------------- rewrites
 
+RESHAPES = ("view.default", "_unsafe_view.default", "reshape.default", "alias.default", "detach.default")
+
 def fold_activations(g: Graph) -> Graph:
     """gelu / relu whose only producer is a linear op -- directly or through a chain of views, as the
     decomposed ``addmm`` + ``view`` form of ``linear`` has it -- read by nothing else becomes that op's
@@ -212,6 +215,42 @@ def fold_activations(g: Graph) -> Graph:
         g.ops.remove(act)
         g.buffers[act["id"]].update(kind="view", of=src, op="alias.default", attrs={})
         g.notes.append(f"fold {act['aten']} into {prod['id']}")
+    return g
+
+
+def fold_layerscale(g: Graph) -> Graph:
+    """``mul.Tensor(y, gamma)`` with ``gamma`` a per-feature weight vector and ``y`` (a view chain of) a linear op's
+    output that nothing else reads -- DINOv2's LayerScale after the attention projection and after the MLP -- is
+    applied to the linear's weight columns and bias once, when the executor binds the weights: ``(xW + b) * gamma =
+    x (W gamma) + b gamma``.  The multiplication then costs nothing per run; the rounding moves from the activations
+    to the weights (one fp16 rounding of ``W gamma`` instead of one of the product)."""
+    for mul in [o for o in g.ops if o["aten"] == "mul.Tensor" and len(o["in"]) == 2]:
+        for mine, other in (mul["in"], mul["in"][::-1]):
+            gb = g.buffers[g.root(other)]
+            chain = [mine]
+            while g.buffers[chain[-1]]["kind"] == "view":
+                chain.append(g.buffers[chain[-1]]["of"])
+            prod = g.op(chain[-1])
+            if prod is None or prod["aten"] not in LINEAR_OPS or any(k in prod["attrs"] for k in ("epilogue", "residual", "colscale", "ln_out")):
+                continue
+            feat = (g.buffers[chain[-1]].get("shape") or [None])[-1]
+            gshape = g.buffers[other].get("shape") or []
+            if gb["kind"] != "weight" or not gshape or gshape[-1] != feat or any(d != 1 for d in gshape[:-1]):
+                continue
+            if not all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1]):
+                continue
+            if not (_consumers(g, chain[-1]) <= {mul["id"]}):
+                continue
+            # the linear's own weight and bias must be constants too
+            wpos = {"linear.default": (1, 2), "addmm.default": (2, 0), "mm.default": (1, None)}[prod["aten"]]
+            ids = [prod["in"][wpos[0]]] + ([prod["in"][wpos[1]]] if wpos[1] is not None and len(prod["in"]) > wpos[1] else [])
+            if any(g.buffers[g.root(i)]["kind"] != "weight" for i in ids):
+                continue
+            prod["attrs"]["colscale"] = other
+            g.ops.remove(mul)
+            g.buffers[mul["id"]].update(kind="view", of=mine, op="alias.default", attrs={})
+            g.notes.append(f"fold {mul['id']} (per-feature scale) into the weights of {prod['id']}")
+            break
     return g
 
 
@@ -244,9 +283,6 @@ def fold_residuals(g: Graph) -> Graph:
             g.notes.append(f"fold add {add['id']} into {prod['id']}")
             break
     return g
-
-
-RESHAPES = ("view.default", "_unsafe_view.default", "reshape.default", "alias.default", "detach.default")
 
 
 def fold_layernorms(g: Graph) -> Graph:
@@ -445,7 +481,7 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
 
 
 def optimize(g: Graph) -> Graph:
-    return fold_sdpa_transpose(fold_attention(fold_layernorms(fold_residuals(fold_activations(g)))))
+    return fold_sdpa_transpose(fold_attention(fold_layernorms(fold_residuals(fold_layerscale(fold_activations(g))))))
 
 
 # ----------------------------------------------------------------------------- execution
@@ -462,6 +498,7 @@ class Executor:
         self.ctx = ctx if ctx is not None else K.Ctx(device)
         self.device = torch.device(device)
         self.t: Dict[str, torch.Tensor] = {}
+        self.scaled: Dict[str, Any] = {}                  # op id -> (weight, bias) with a folded per-feature scale
         for b in graph.buffers.values():
             if b["kind"] == "weight":
                 w = weights[b["key"]]
@@ -568,6 +605,11 @@ class Executor:
             bias, x, w = self.get(ins[0]), self.get(ins[1]), self.get(ins[2])
         else:                                            # mm (x, w[K,F])
             x, w, bias = self.get(ins[0]), self.get(ins[1]), None
+        if "colscale" in attrs:                          # LayerScale folded into the constants, once
+            if o["id"] not in self.scaled:
+                gamma = self.get(attrs["colscale"]).reshape(-1).float()
+                self.scaled[o["id"]] = ((w.float() * gamma).to(w.dtype), None if bias is None else (bias.float() * gamma).to(bias.dtype))
+            w, bias = self.scaled[o["id"]]
         out = self.t[o["out"]]
         res = self._rows(self.get(res_id)) if res_id else None
         self.ctx.ws.reset()
@@ -590,6 +632,21 @@ class Executor:
         bias = self.get(o["in"][3]) if len(o["in"]) > 3 else None       # attn_mask / attn_bias, positional or keyword
         self.ctx.ws.reset()
         K.sdpa(self.ctx, q, k, v, bias, a.get("scale"), out=self.t[o["out"]])
+
+    def _cat(self, o):
+        """cat of (B, N_i, C) tensors along the token axis (class token + patch tokens): each operand is copied into its
+        rows of the result with the layout kernel, whatever its strides -- the patch tokens arrive as the transposed
+        view of the convolution's (B, C, N) output, and the copy is that transpose."""
+        ins = [self.get(i) for i in o["in"]]
+        out = self.t[o["out"]]
+        dim = o["attrs"].get("arg1", 0) % out.dim()
+        if out.dim() != 3 or dim != 1 or any(t.dim() != 3 for t in ins):
+            raise UnsupportedOp(f"{o['id']}: cat of {[tuple(t.shape) for t in ins]} along {dim} (only (B, N, C) along N)")
+        at = 0
+        for t in ins:
+            n = t.shape[1]
+            K.transposeLE_(self.ctx, out[:, at:at + n].unsqueeze(1), t.permute(0, 2, 1).unsqueeze(1))
+            at += n
 
     def _bmm(self, o):
         """bmm(a (B,m,k), b (B,k,n)) -- batchedmatmul!, ops.jl:1393-1399."""
@@ -655,7 +712,7 @@ class Executor:
                 **dict.fromkeys(SDPA_OPS, _sdpa), "layer_norm.default": _layer_norm,
                 "native_layer_norm.default": _native_layer_norm, "add.Tensor": _add,
                 "gelu.default": _activation, "relu.default": _activation, "convolution.default": _convolution,
-                "bmm.default": _bmm}
+                "bmm.default": _bmm, "cat.default": _cat}
 
     def __call__(self, *inputs: torch.Tensor):
         if len(inputs) != len(self.g.inputs):

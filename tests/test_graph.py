@@ -362,3 +362,84 @@ def test_bmm_runs_on_the_batched_gemm(ctx):
     got = run(a.cuda(), b.cuda())
     torch.cuda.synchronize()
     assert_parity(got.float().cpu().numpy(), torch.bmm(a.float(), b.float()).numpy(), what="bmm")
+
+
+def _dinov2_like(d=128, heads=2, layers=2, patch=14, image=70, seed=0):
+    """A ViT written the way DINOv2 (the backbone of the reference's Depth Anything model, config 3) is: patch
+    embedding by a strided convolution, class token concatenated in front, learned position embedding, pre-LN blocks
+    with written-out attention and LayerScale on both branches, a final norm."""
+    import torch
+    import torch.nn as nn
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.h, self.scale = heads, (d // heads) ** -0.5
+            self.norm1, self.norm2 = nn.LayerNorm(d, eps=1e-6), nn.LayerNorm(d, eps=1e-6)
+            self.qkv, self.proj = nn.Linear(d, 3 * d), nn.Linear(d, d)
+            self.fc1, self.fc2 = nn.Linear(d, 4 * d), nn.Linear(4 * d, d)
+            self.ls1, self.ls2 = nn.Parameter(torch.rand(d) + 0.5), nn.Parameter(torch.rand(d) + 0.5)
+
+        def attn(self, x):
+            B, N, C = x.shape
+            qkv = self.qkv(x).reshape(B, N, 3, self.h, C // self.h).permute(2, 0, 3, 1, 4)
+            q, k, v = qkv[0] * self.scale, qkv[1], qkv[2]
+            a = (q @ k.transpose(-2, -1)).softmax(dim=-1)
+            return self.proj((a @ v).transpose(1, 2).reshape(B, N, C))
+
+        def forward(self, x):
+            x = x + self.attn(self.norm1(x)) * self.ls1
+            return x + self.fc2(torch.nn.functional.gelu(self.fc1(self.norm2(x)))) * self.ls2
+
+    class ViT(nn.Module):
+        def __init__(self):
+            super().__init__()
+            n = (image // patch) ** 2
+            self.patch_embed = nn.Conv2d(3, d, patch, patch)
+            self.cls_token, self.pos_embed = nn.Parameter(torch.randn(1, 1, d) * 0.1), nn.Parameter(torch.randn(1, n + 1, d) * 0.1)
+            self.blocks = nn.ModuleList([Block() for _ in range(layers)])
+            self.norm = nn.LayerNorm(d, eps=1e-6)
+
+        def forward(self, img):
+            x = self.patch_embed(img).flatten(2).transpose(1, 2)
+            x = torch.cat((self.cls_token.expand(x.shape[0], -1, -1), x), dim=1) + self.pos_embed
+            for b in self.blocks:
+                x = b(x)
+            return self.norm(x)
+
+    torch.manual_seed(seed)
+    return ViT().eval().half()
+
+
+def test_dinov2_like_encoder_folds_to_five_calls_per_block():
+    import torch
+    from juliavision_amd import graph as G
+    m = _dinov2_like()
+    ep = torch.export.export(m, (torch.randn(1, 3, 70, 70).half(),)).run_decompositions()
+    d = G.convert(ep, "vit")
+    aten = [o["aten"] for o in d["ops"]]
+    assert aten.count("bmm.default") == 4 and aten.count("_softmax.default") == 2 and aten.count("cat.default") == 1
+    g = G.optimize(G.Graph.load(d))
+    left = [o["aten"] for o in g.ops]
+    # convolution, cat, + position embedding, first norm; per block: qkv, attention, projection, fc1, fc2 -- the
+    # other norms ride in the GEMM that writes their input, LayerScale in the weights, residuals in the stores
+    assert left == ["convolution.default", "cat.default", "add.Tensor", "native_layer_norm.default"] + \
+        ["addmm.default", "scaled_dot_product_attention.default", "addmm.default", "addmm.default", "addmm.default"] * 2, (left, g.notes)
+    assert sum("colscale" in o["attrs"] for o in g.ops) == 4 and sum("residual" in o["attrs"] for o in g.ops) == 4
+    assert sum("ln_out" in o["attrs"] for o in g.ops) == 4
+
+
+@pytest.mark.gpu
+def test_dinov2_like_encoder_runs_on_the_kernels(ctx):
+    import torch
+    from juliavision_amd import graph as G
+    m = _dinov2_like(seed=5)
+    x = torch.rand(1, 3, 70, 70).half()
+    ep = torch.export.export(m, (x,)).run_decompositions()
+    run = G.Executor(G.optimize(G.Graph.load(G.convert(ep, "vit"))), m.state_dict(), ctx)
+    with torch.no_grad():
+        want = m.float()(x.float()).numpy()
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    assert got.shape == (1, 26, 128)
+    assert_parity(got.float().cpu().numpy(), want, what="DINOv2-like encoder from its exported graph")
