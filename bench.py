@@ -360,6 +360,80 @@ def vit_encoder_case(steps=50):
             "frac_mfma_peak_graph": round(flop / replay / 1e12 / PEAK_F16_TFLOPS, 4)}
 
 
+def vit_graph_case(steps=50):
+    """Config 3's encoder from its exported graph: a ViT-S/14 written the way DINOv2 -- the backbone of the reference's
+    Depth Anything model -- is (class token concatenated in front, written-out attention, LayerScale), exported with
+    torch.export on the host, converted to the reference's JSON schema, rewritten (graph.optimize) and run by the graph
+    executor, eager and replayed as one captured graph.  Random weights; the same 93.39 GFLOP."""
+    import time
+    import torch
+    import torch.nn as nn
+    import juliavision_amd as jv
+    from juliavision_amd import graph as G
+    from juliavision_amd.decode import StepGraph
+    d, H, P, S, NL = 384, 6, 14, 518, 12
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm1, self.norm2 = nn.LayerNorm(d, eps=1e-6), nn.LayerNorm(d, eps=1e-6)
+            self.qkv, self.proj, self.fc1, self.fc2 = nn.Linear(d, 3 * d), nn.Linear(d, d), nn.Linear(d, 4 * d), nn.Linear(4 * d, d)
+            self.ls1, self.ls2 = nn.Parameter(torch.ones(d)), nn.Parameter(torch.ones(d))
+
+        def forward(self, x):
+            B, N, C = x.shape
+            qkv = self.qkv(self.norm1(x)).reshape(B, N, 3, H, C // H).permute(2, 0, 3, 1, 4)
+            a = ((qkv[0] * (C // H) ** -0.5) @ qkv[1].transpose(-2, -1)).softmax(dim=-1)
+            x = x + self.proj((a @ qkv[2]).transpose(1, 2).reshape(B, N, C)) * self.ls1
+            return x + self.fc2(nn.functional.gelu(self.fc1(self.norm2(x)))) * self.ls2
+
+    class ViT(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.patch_embed = nn.Conv2d(3, d, P, P)
+            self.cls_token, self.pos_embed = nn.Parameter(torch.zeros(1, 1, d)), nn.Parameter(torch.randn(1, 1 + (S // P) ** 2, d) * 0.02)
+            self.blocks = nn.ModuleList([Block() for _ in range(NL)])
+            self.norm = nn.LayerNorm(d, eps=1e-6)
+
+        def forward(self, img):
+            x = self.patch_embed(img).flatten(2).transpose(1, 2)
+            x = torch.cat((self.cls_token.expand(x.shape[0], -1, -1), x), dim=1) + self.pos_embed
+            for b in self.blocks:
+                x = b(x)
+            return self.norm(x)
+
+    torch.manual_seed(0)
+    m = ViT().eval().half()
+    t0 = time.perf_counter()
+    ep = torch.export.export(m, (torch.rand(1, 3, S, S).half(),)).run_decompositions()
+    spec = G.convert(ep, "vit_s14")
+    g = G.optimize(G.Graph.load(spec))
+    host_s = time.perf_counter() - t0
+    ctx = jv.Ctx("cuda")
+    run = G.Executor(g, m.state_dict(), ctx)
+    image = torch.rand((1, 3, S, S), dtype=torch.float16, device="cuda")
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / steps
+
+    step = lambda: run(image)
+    eager = timed(step)
+    replay = timed(StepGraph(step).replay)
+    if not bool(torch.isfinite(run(image)).all()):
+        raise RuntimeError("exported ViT produced non-finite output")
+    T = 1 + (S // P) ** 2
+    flop = NL * (2.0 * T * d * (3 * d + d + 8 * d) + 4.0 * T * T * 64 * H) + 2.0 * (T - 1) * 588 * d
+    return {"ops_exported": len(spec["ops"]), "ops_after_rewrites": len(g.ops), "export_and_rewrite_host_s": round(host_s, 2),
+            "eager_ms": round(eager * 1e3, 4), "graph_ms": round(replay * 1e3, 4), "TFLOP/s_graph": round(flop / replay / 1e12, 1)}
+
+
 def encoder_stack_case(nl=4, steps=50):
     """BASELINE config 2's block as it occurs in a stack: `nl` Whisper-shaped blocks in sequence (1500 x 1280, 20 x 64
     heads, FFN 5120, [K][F] weights), each block's first norm written by the previous block's last GEMM.  Reported per
@@ -565,6 +639,10 @@ def detail_benchmarks(lib, L, stream, only=None):
     name = "c3_vit_s14_518_encoder_12layers"
     if only is None or only in name:
         out[name] = vit_encoder_case()
+
+    name = "c3_vit_s14_518_from_exported_graph"
+    if only is None or only in name:
+        out[name] = vit_graph_case()
 
     name = "c5_decode_step_4layers_vocab51866_b1"
     if only is None or only in name:
