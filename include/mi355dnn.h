@@ -278,6 +278,14 @@ int mi_layernorm_f16(void *out, float *mean, float *rstd, const void *a,
                      const void *gamma, const void *beta,
                      int64_t C, int64_t groups, float eps, void *stream);
 
+/* Softmax over the last, contiguous axis of `rows` rows of n elements, fp16 or fp32 (dtype) in and out:
+ * out = exp(scale * a - max) / sum in fp32, one rounding; a row of -inf gives zeros.  The reference's softmax_kernel!
+ * (ops.jl:474-573, aten::_softmax; scale = 1 there) and the softmax of its two-GEMM attention, attn_softmax_rows!
+ * (attention.jl:528-615), which takes the scale. */
+int mi_softmax_f16(void *out, const void *a, int dtype, int64_t n, int64_t rows, float scale, void *stream);
+/* out = fp16(a * c) over n contiguous elements: aten::mul.Tensor / div.Tensor with a constant (the emit() broadcast of
+ * ops.jl's elementwise handlers). */
+int mi_scale_f16(void *out, const void *a, float c, int64_t n, void *stream);
 /* out = fp16(a + b), n elements: the residual add.Tensor in the operand type
  * (ops.jl:186-197), for callers that do not fold it into the GEMM store. */
 int mi_add_f16(void *out, const void *a, const void *b, int64_t n, void *stream);

@@ -1,7 +1,7 @@
-// Layer norm and the residual add: the HBM-bound glue between the contractions
-// of an encoder block.  One wavefront per normalisation group, the row held in
-// registers between the three passes (mean, centred variance, normalise) so it
-// is read from memory once; fp32 statistics (layernorm.jl:53-113).
+// Layer norm, the residual add, row softmax and scaling by a constant: the HBM-bound
+// glue between the contractions of an encoder block.  One wavefront per row or
+// normalisation group, the row held in registers between the passes so that it
+// is read from memory once; fp32 statistics (layernorm.jl:53-113, ops.jl:474-555).
 #include "common.hpp"
 
 namespace {
@@ -99,6 +99,77 @@ __global__ __launch_bounds__(256) void layernorm_any_kernel(half_t *out, float *
     }
 }
 
+// Softmax over rows of n elements (the last, contiguous axis): m = max, s = sum exp(c x - m), out = exp(c x - m) / s in
+// fp32, one rounding (softmax_kernel!, ops.jl:474-555; c = 1 there -- a constant scale ahead of the softmax rides along
+// here).  A row whose maximum is -inf (every element masked) gives zeros, as the attention kernels do.
+template <int NCH>
+__global__ __launch_bounds__(256) void softmax_vec_kernel(half_t *out, const half_t *a, int n, long rows, float c) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long g = (long)blockIdx.x * 4 + wave;
+    if (g >= rows) return;
+    const half_t *row = a + g * n;
+    float x[NCH][8];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        if (e0 < n) {
+            half8v t = as_half8(ldg16(row + e0));
+#pragma unroll
+            for (int j = 0; j < 8; j++) { x[i][j] = (float)t[j] * c; m = fmaxf(m, x[i][j]); }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) x[i][j] = -INFINITY;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    const float mm = m == -INFINITY ? 0.0f : m;
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) { x[i][j] = __expf(x[i][j] - mm); s += x[i][j]; }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    const float inv = s > 0.0f ? 1.0f / s : 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int e0 = (lane + 64 * i) * 8;
+        if (e0 < n) {
+            half8v o;
+#pragma unroll
+            for (int j = 0; j < 8; j++) o[j] = (half_t)(x[i][j] * inv);
+            *reinterpret_cast<half8v *>(out + g * n + e0) = o;
+        }
+    }
+}
+
+// Any n, any alignment, fp16 or fp32 rows: three passes over memory.
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_any_kernel(T *out, const T *a, int n, long rows, float c) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long g = (long)blockIdx.x * 4 + wave;
+    if (g >= rows) return;
+    const T *row = a + g * n;
+    float m = -INFINITY;
+    for (int i = lane; i < n; i += 64) m = fmaxf(m, (float)row[i] * c);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    const float mm = m == -INFINITY ? 0.0f : m;
+    float s = 0.0f;
+    for (int i = lane; i < n; i += 64) s += __expf((float)row[i] * c - mm);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    const float inv = s > 0.0f ? 1.0f / s : 0.0f;
+    for (int i = lane; i < n; i += 64) out[g * n + i] = (T)(__expf((float)row[i] * c - mm) * inv);
+}
+
+__global__ void scale_kernel(half_t *o, const half_t *a, float c, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) o[i] = (half_t)((float)a[i] * c);
+}
+
 __global__ void add_vec_kernel(half_t *o, const half_t *a, const half_t *b, long n8) {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n8) return;
@@ -132,6 +203,38 @@ int mi_layernorm_f16(void *out, float *mean, float *rstd, const void *a, const v
     else if (vec && C <= 2048) hipLaunchKernelGGL(layernorm_vec_kernel<4>, grid, block, 0, st, o, mean, rstd, x, g, b, (int)C, (long)groups, eps);
     else if (vec && C <= 4096) hipLaunchKernelGGL(layernorm_vec_kernel<8>, grid, block, 0, st, o, mean, rstd, x, g, b, (int)C, (long)groups, eps);
     else                       hipLaunchKernelGGL(layernorm_any_kernel, grid, block, 0, st, o, mean, rstd, x, g, b, (int)C, (long)groups, eps);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_softmax_f16(void *out, const void *a, int dtype, int64_t n, int64_t rows, float scale, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !a) return MI_DECLINE_OPERANDS;
+    if (dtype != MI_F16 && dtype != MI_F32) return MI_DECLINE_OPERANDS;
+    if (n < 1 || n > INT32_MAX || rows < 0) return MI_DECLINE_EXTENT;
+    if (rows == 0) return MI_OK;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid((unsigned)ceil_div(rows, 4)), block(256);
+    if (dtype == MI_F32) {
+        hipLaunchKernelGGL(softmax_any_kernel<float>, grid, block, 0, st, (float *)out, (const float *)a, (int)n, (long)rows, scale);
+        return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+    }
+    half_t *o = (half_t *)out;
+    const half_t *x = (const half_t *)a;
+    const bool vec = n % 8 == 0 && aligned_to(a, 16) && aligned_to(out, 16);
+    if (vec && n <= 512)       hipLaunchKernelGGL(softmax_vec_kernel<1>, grid, block, 0, st, o, x, (int)n, (long)rows, scale);
+    else if (vec && n <= 1024) hipLaunchKernelGGL(softmax_vec_kernel<2>, grid, block, 0, st, o, x, (int)n, (long)rows, scale);
+    else if (vec && n <= 2048) hipLaunchKernelGGL(softmax_vec_kernel<4>, grid, block, 0, st, o, x, (int)n, (long)rows, scale);
+    else if (vec && n <= 4096) hipLaunchKernelGGL(softmax_vec_kernel<8>, grid, block, 0, st, o, x, (int)n, (long)rows, scale);
+    else                       hipLaunchKernelGGL(softmax_any_kernel<half_t>, grid, block, 0, st, o, x, (int)n, (long)rows, scale);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_scale_f16(void *out, const void *a, float c, int64_t n, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !a) return MI_DECLINE_OPERANDS;
+    if (n < 0) return MI_DECLINE_EXTENT;
+    if (n == 0) return MI_OK;
+    hipLaunchKernelGGL(scale_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, (half_t *)out, (const half_t *)a, c, (long)n);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 

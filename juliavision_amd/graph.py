@@ -10,8 +10,9 @@ the ops of the dense-contraction path:
 
     linear / addmm / mm / bmm, scaled_dot_product_attention (also written out
     as bmm + softmax + bmm), layer_norm / native_layer_norm, gelu, relu,
-    add.Tensor, convolution, cat along the token axis, a per-feature
-    mul.Tensor after a linear (LayerScale), and the view ops between them.
+    add.Tensor, convolution, cat along the token axis, softmax over the last
+    axis, mul / div by a constant, a per-feature mul.Tensor after a linear
+    (LayerScale), contiguous clone, and the view ops between them.
 
 Two of the reference's rewrites matter for that path and have counterparts here:
 
@@ -507,8 +508,7 @@ class Executor:
                 self.t[b["id"]] = w.to(self.device, _DTYPES[b["dtype"]]).contiguous()
         for o in graph.ops:                               # check every op has a handler before anything runs
             if o["aten"] not in self.HANDLERS:
-                hint = " -- inside bmm + softmax + bmm, optimize() folds it into the fused attention" if o["aten"] in SOFTMAX_OPS else ""
-                raise UnsupportedOp(f"{graph.name}: no kernel on this path for aten.{o['aten']} (op {o['id']}){hint}")
+                raise UnsupportedOp(f"{graph.name}: no kernel on this path for aten.{o['aten']} (op {o['id']})")
         for o in graph.ops:                               # a norm folded into its producer: its result still needs a home
             nid = o["attrs"].get("ln_out")
             if nid is not None:
@@ -648,6 +648,37 @@ class Executor:
             K.transposeLE_(self.ctx, out[:, at:at + n].unsqueeze(1), t.permute(0, 2, 1).unsqueeze(1))
             at += n
 
+    def _softmax(self, o):
+        """aten::_softmax / softmax over the last axis (softmax_kernel!, ops.jl:557-573); inside bmm + softmax + bmm
+        optimize() replaces it, on its own -- or where the probabilities are a result -- it runs as written."""
+        x, out = self.get(o["in"][0]), self.t[o["out"]]
+        if o["attrs"].get("arg1") not in (-1, x.dim() - 1) or o["attrs"].get("arg2") not in (None, False) or not x.is_contiguous():
+            raise UnsupportedOp(f"{o['id']}: softmax over an axis other than the last, or of a strided tensor")
+        K.softmax_(self.ctx, out, x)
+
+    def _scale(self, o):
+        c = _scalar_scale(o)
+        if c is None:
+            raise UnsupportedOp(f"{o['id']}: {o['aten']} other than a tensor times a constant")
+        x, out = self.get(o["in"][0]), self.t[o["out"]]
+        if not x.is_contiguous():                         # a strided operand (a head slice of a packed projection): copy, then scale in place
+            self._copy(o, out, x)
+            x = out
+        K.scale_(self.ctx, out, x, c)
+
+    def _copy(self, o, out, x):
+        """out (contiguous) = x (any strides), up to four axes, with the layout kernel."""
+        if x.dim() > 4 or x.dim() < 2:
+            raise UnsupportedOp(f"{o['id']}: a contiguous copy of a {x.dim()}-axis strided tensor")
+        while x.dim() < 4:
+            x, out = x.unsqueeze(0), out.unsqueeze(0)
+        K.transposeLE_(self.ctx, out, x.transpose(2, 3))
+
+    def _clone(self, o):
+        if o["attrs"].get("memory_format", "torch.contiguous_format") not in ("torch.contiguous_format", "contiguous_format"):
+            raise UnsupportedOp(f"{o['id']}: clone to another memory format")
+        self._copy(o, self.t[o["out"]], self.get(o["in"][0]))
+
     def _bmm(self, o):
         """bmm(a (B,m,k), b (B,k,n)) -- batchedmatmul!, ops.jl:1393-1399."""
         a, b = self.get(o["in"][0]), self.get(o["in"][1])
@@ -712,7 +743,8 @@ class Executor:
                 **dict.fromkeys(SDPA_OPS, _sdpa), "layer_norm.default": _layer_norm,
                 "native_layer_norm.default": _native_layer_norm, "add.Tensor": _add,
                 "gelu.default": _activation, "relu.default": _activation, "convolution.default": _convolution,
-                "bmm.default": _bmm, "cat.default": _cat}
+                "bmm.default": _bmm, "cat.default": _cat, **dict.fromkeys(SOFTMAX_OPS, _softmax),
+                "mul.Tensor": _scale, "div.Tensor": _scale, "clone.default": _clone}
 
     def __call__(self, *inputs: torch.Tensor):
         if len(inputs) != len(self.g.inputs):

@@ -289,12 +289,13 @@ def batchedmatmul_(ctx: Ctx, out, A, B):
     nb = out.shape[0]
     K, F = A.shape[1:]
     T = B.shape[1]
-    if A.stride(2) != 1 or B.stride(2) != 1 or out.stride(2) != 1:
-        raise DeclineError("batchedmatmul_: planes must be row-major", L.DECLINE_OPERANDS)
+    la = _mat2(A[0])                  # the planes of A may be [K][F] or, as a transposed view (k^T of attention), [F][K]
+    if la is None or B.stride(2) != 1 or out.stride(2) != 1:
+        raise DeclineError("batchedmatmul_: planes must be row-major (A's may be transposed views)", L.DECLINE_OPERANDS)
     sA = 0 if A.shape[0] == 1 else A.stride(0)
     sB = 0 if B.shape[0] == 1 else B.stride(0)
     rc = lib.mi_gemm_f16_batched(out.data_ptr(), B.data_ptr(), A.data_ptr(), None, None, T, K, F,
-                                 out.stride(1), B.stride(1), A.stride(1), L.W_KF, L.BIAS_NONE, L.EPI["none"],
+                                 out.stride(1), B.stride(1), la[1], L.W_KF if la[0] == 0 else L.W_FK, L.BIAS_NONE, L.EPI["none"],
                                  _dtype_code(out), nb, out.stride(0), sB, sA, 0, None, 0, ctx.stream)
     if rc != L.OK:
         raise DeclineError("mi_gemm_f16_batched", rc)
@@ -592,6 +593,31 @@ def layernorm_(ctx: Ctx, out, mean, rstd, a, gamma, beta, C_: int, eps: float):
                               C_, groups, float(eps), ctx.stream)
     if rc != L.OK:
         raise DeclineError("mi_layernorm_f16", rc)
+    return out
+
+
+def softmax_(ctx: Ctx, out, a, scale: float = 1.0):
+    """Softmax over the last axis of a contiguous fp16 or fp32 tensor, ``exp(scale * a - max) / sum`` in fp32
+    (softmax_kernel!, ops.jl:474-573; attn_softmax_rows!, attention.jl:528-615)."""
+    lib = L.init()
+    if not (a.is_cuda and out.is_cuda and a.dtype == out.dtype and a.dtype in (torch.float16, torch.float32)) or a.shape != out.shape \
+            or not (a.is_contiguous() and out.is_contiguous()) or a.dim() < 1:
+        raise DeclineError("softmax_: operands", L.DECLINE_OPERANDS)
+    n = a.shape[-1]
+    rc = lib.mi_softmax_f16(out.data_ptr(), a.data_ptr(), _dtype_code(a), n, a.numel() // max(n, 1), float(scale), ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_softmax_f16", rc)
+    return out
+
+
+def scale_(ctx: Ctx, out, a, c: float):
+    """out = fp16(a * c), contiguous fp16 tensors (mul.Tensor / div.Tensor with a constant)."""
+    lib = L.init()
+    if not _is_f16_cuda(a, out) or a.shape != out.shape or not (a.is_contiguous() and out.is_contiguous()):
+        raise DeclineError("scale_: operands", L.DECLINE_OPERANDS)
+    rc = lib.mi_scale_f16(out.data_ptr(), a.data_ptr(), float(c), a.numel(), ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_scale_f16", rc)
     return out
 
 

@@ -265,6 +265,22 @@ def layernorm_f16(a, gamma=None, beta=None, eps=1e-5):
     return out, mean, rstd
 
 
+def softmax_f16(a, scale: float = 1.0):
+    """Softmax over the last axis, fp16 in and out (softmax_kernel!, ops.jl:474-555)."""
+    a = np.ascontiguousarray(a, dtype=np.float16)
+    out = np.empty_like(a)
+    n = a.shape[-1]
+    lib().orc_softmax_f16(_p(out), _p(a), _i64(n), _i64(a.size // max(n, 1)), C.c_float(scale))
+    return out
+
+
+def scale_f16(a, c: float):
+    a = np.ascontiguousarray(a, dtype=np.float16)
+    out = np.empty_like(a)
+    lib().orc_scale_f16(_p(out), _p(a), C.c_float(c), _i64(a.size))
+    return out
+
+
 def add_f16(a, b):
     a = np.ascontiguousarray(a, dtype=np.float16)
     b = np.ascontiguousarray(b, dtype=np.float16)

@@ -26,6 +26,9 @@
  *                        dilation, output_padding, groups) and the pixel-shuffle identity of
  *                        the non-overlapping case (conv.jl:204-222)
  *   orc_layernorm_f16    torch.nn.functional.layer_norm in fp32
+ *   orc_softmax_f16      numpy float64 exp / sum (rows sum to 1, shift invariance, a row of
+ *                        -inf gives zeros); composed with two orc_gemm_f16 it reproduces
+ *                        orc_sdpa_threepass (the two-GEMM attention, attention.jl:675-705)
  *   unpinned             bit-level accumulation order of Lava.coopmat_gemm!/gemv!
  *                        (third-party, source absent); irrelevant at the 1e-2 /
  *                        cosine 0.9999 gate.
@@ -499,6 +502,29 @@ ORC_API void orc_layernorm_f16(uint16_t *out, float *mean, float *rstd, const ui
         if (mean) mean[g] = mu;
         if (rstd) rstd[g] = rs;
     }
+}
+
+/* ops.jl:474-555 softmax_kernel!: per slice m = max, s = sum exp(x - m), out = T(exp(x - m) / s), all in fp32
+ * (the 64-lane strided partial sums are a reduction order, not part of the contract: a double accumulator here).
+ * `scale` multiplies x first, as attn_softmax_rows! does (attention.jl:528-560); 1 for aten::_softmax.
+ * A slice of -inf gives zeros, the attention convention (attention.jl:82-87). */
+ORC_API void orc_softmax_f16(uint16_t *out, const uint16_t *a, int64_t n, int64_t rows, float scale) {
+    #pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < rows; g++) {
+        const uint16_t *r = a + g * n;
+        float m = -INFINITY;
+        for (int64_t i = 0; i < n; i++) { float x = h2f(r[i]) * scale; if (x > m) m = x; }
+        if (m == -INFINITY) { for (int64_t i = 0; i < n; i++) out[g * n + i] = 0; continue; }
+        double s = 0.0;
+        for (int64_t i = 0; i < n; i++) s += (double)expf(h2f(r[i]) * scale - m);
+        float den = (float)s;
+        for (int64_t i = 0; i < n; i++) out[g * n + i] = f2h(expf(h2f(r[i]) * scale - m) / den);
+    }
+}
+
+/* out = fp16(fp32(a) * c): mul.Tensor / div.Tensor with a constant in the operand type. */
+ORC_API void orc_scale_f16(uint16_t *o, const uint16_t *a, float c, int64_t n) {
+    for (int64_t i = 0; i < n; i++) o[i] = f2h(h2f(a[i]) * c);
 }
 
 /* out = fp16(fp32(a) + fp32(b)): the graph's residual add.Tensor in the operand

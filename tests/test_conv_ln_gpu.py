@@ -297,3 +297,47 @@ def test_transpose_le_2d_is_the_matrix_transpose(ctx):
     out = poison(torch.empty((37, 100), dtype=torch.float16, device="cuda"))
     jv.transposeLE_(ctx, out, to_dev(w))
     assert np.array_equal(to_host(out), w.T)
+
+
+@pytest.mark.parametrize("rows,n,scale", [(7, 64, 1.0), (5, 37, 1.0), (9, 1370, 0.125), (6, 1376, 0.125), (3, 4096, 1.0), (2, 5000, 0.5)])
+def test_softmax_rows(ctx, rows, n, scale):
+    """softmax_kernel! (ops.jl:474-573) / attn_softmax_rows! (attention.jl:528-615): register-resident rows up to 4096,
+    the three-pass form beyond and for rows that are not 16-byte addressable."""
+    import torch
+    import juliavision_amd as jv
+    a = oracle.randn_f16((rows, n), 21, std=3.0)
+    a[rows // 2, : n // 3] = -np.inf                      # masked keys: weight exactly 0
+    out = poison(torch.empty((rows, n), dtype=torch.float16, device="cuda"))
+    jv.softmax_(ctx, out, to_dev(a), scale)
+    torch.cuda.synchronize()
+    got = to_host(out)
+    assert np.all(got[rows // 2, : n // 3] == 0)
+    assert_parity(got, oracle.softmax_f16(a, scale), what=f"softmax {rows}x{n}")
+    assert np.allclose(got.astype(np.float64).sum(-1), 1.0, atol=4e-3)
+
+
+def test_softmax_fp32_rows_and_a_fully_masked_row(ctx):
+    import torch
+    import juliavision_amd as jv
+    a = oracle.randn_f32((4, 300), 22, std=4.0)
+    a[1] = -np.inf
+    out = poison(torch.empty((4, 300), dtype=torch.float32, device="cuda"))
+    jv.softmax_(ctx, out, to_dev(a))
+    torch.cuda.synchronize()
+    got = to_host(out)
+    x = a.astype(np.float64)[[0, 2, 3]]
+    e = np.exp(x - x.max(-1, keepdims=True))
+    assert np.all(got[1] == 0) and np.max(np.abs(got[[0, 2, 3]] - e / e.sum(-1, keepdims=True))) < 1e-6
+
+
+def test_scale_bit_exact(ctx):
+    import torch
+    import juliavision_amd as jv
+    a = oracle.randn_f16((3, 1001), 23, std=5.0)
+    out = poison(torch.empty((3, 1001), dtype=torch.float16, device="cuda"))
+    jv.scale_(ctx, out, to_dev(a), 0.125)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(out).view(np.uint16), oracle.scale_f16(a, 0.125).view(np.uint16))
+    jv.scale_(ctx, out, to_dev(a), 1.0 / 3.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(out).view(np.uint16), oracle.scale_f16(a, 1.0 / 3.0).view(np.uint16))

@@ -317,3 +317,30 @@ def test_add_rounds_once():
     a = oracle.randn_f16((1000,), 1)
     b = oracle.randn_f16((1000,), 2)
     assert np.array_equal(oracle.add_f16(a, b), (a.astype(np.float32) + b.astype(np.float32)).astype(np.float16))
+
+
+def test_softmax_and_scale_against_numpy():
+    """orc_softmax_f16 (softmax_kernel!, ops.jl:474-555): float64 closed form, rows summing to one, invariance under a
+    shift of the row, the scale argument equal to scaling the input first, a fully masked row giving zeros; and that
+    two oracle GEMMs around it are the oracle's own three-pass attention (the two-GEMM path, attention.jl:675-705)."""
+    a = oracle.randn_f16((6, 333), 11, std=3.0)
+    got = oracle.softmax_f16(a).astype(np.float64)
+    x = a.astype(np.float64)
+    e = np.exp(x - x.max(-1, keepdims=True))
+    assert np.max(np.abs(got - e / e.sum(-1, keepdims=True))) < 5e-4
+    assert np.allclose(got.sum(-1), 1.0, atol=2e-3)
+    shifted = (a.astype(np.float32) + np.float32(2.0)).astype(np.float16)
+    exact = shifted.astype(np.float32) - a.astype(np.float32) == 2.0          # where the shift is exact in fp16
+    assert np.max(np.abs(oracle.softmax_f16(shifted).astype(np.float64) - got)[exact.all(-1)], initial=0.0) < 1e-3
+    assert np.array_equal(oracle.softmax_f16(a, 0.5), oracle.softmax_f16(oracle.scale_f16(a, 0.5))) or \
+        oracle.max_rel(oracle.softmax_f16(a, 0.5), oracle.softmax_f16(oracle.scale_f16(a, 0.5))) < 2e-3
+    masked = a.copy()
+    masked[2] = -np.inf
+    assert np.all(oracle.softmax_f16(masked)[2] == 0) and np.all(np.isfinite(oracle.softmax_f16(masked)))
+    assert np.array_equal(oracle.scale_f16(a, 0.125), (a.astype(np.float32) * np.float32(0.125)).astype(np.float16))
+    # the two-GEMM attention: S = q k^T, P = softmax(S / sqrt(E)), O = P v, one head
+    q, k, v = oracle.randn_f16((40, 64), 12), oracle.randn_f16((50, 64), 13), oracle.randn_f16((50, 64), 14)
+    s = oracle.gemm_f16(q, np.ascontiguousarray(k.T))
+    o = oracle.gemm_f16(oracle.softmax_f16(s, 0.125), v)
+    ref = oracle.sdpa_threepass_f16(q[None, None], k[None, None], v[None, None])[0, 0]
+    assert oracle.max_rel(o, ref) < 5e-3 and oracle.cosine(o, ref) > 0.99999
