@@ -286,6 +286,11 @@ int mi_softmax_f16(void *out, const void *a, int dtype, int64_t n, int64_t rows,
 /* out = fp16(a * c) over n contiguous elements: aten::mul.Tensor / div.Tensor with a constant (the emit() broadcast of
  * ops.jl's elementwise handlers). */
 int mi_scale_f16(void *out, const void *a, float c, int64_t n, void *stream);
+/* out = fp16(act(a)) over n contiguous elements, act one of enum mi_epilogue: an activation no GEMM or convolution
+ * store could take (aten::gelu / relu after a strided convolution; ops.jl:1698-1702, 1683). */
+int mi_act_f16(void *out, const void *a, int epi, int64_t n, void *stream);
+/* out = min(max(a, lo), hi): aten::clamp, the fp16 overflow guard of exported encoder layers (ops.jl:300-310). */
+int mi_clamp_f16(void *out, const void *a, float lo, float hi, int64_t n, void *stream);
 /* out = fp16(a + b), n elements: the residual add.Tensor in the operand type
  * (ops.jl:186-197), for callers that do not fold it into the GEMM store. */
 int mi_add_f16(void *out, const void *a, const void *b, int64_t n, void *stream);

@@ -56,6 +56,8 @@ SIGNATURES = {
     "mi_layernorm_f16": (_int, [_vp] * 6 + [_i64, _i64, _f32, _vp]),
     "mi_softmax_f16": (_int, [_vp, _vp, _int, _i64, _i64, _f32, _vp]),
     "mi_scale_f16": (_int, [_vp, _vp, _f32, _i64, _vp]),
+    "mi_act_f16": (_int, [_vp, _vp, _int, _i64, _vp]),
+    "mi_clamp_f16": (_int, [_vp, _vp, _f32, _f32, _i64, _vp]),
     "mi_add_f16": (_int, [_vp, _vp, _vp, _i64, _vp]),
     "mi_kv_append_f16": (_int, [_vp, _vp, _i64p, _i64, _vp, _vp, _i64p, _vp, _i64, _i64, _i64, _vp]),
     "mi_sdpa_append_f16": (_int, [_vp, _int, _i64p, _vp, _i64p, _vp, _i64p, _vp, _i64p, _vp, _vp, _i64p, _vp, _i64, _i64, _i64, _i64, _f32, _vp]),

@@ -170,6 +170,16 @@ __global__ void scale_kernel(half_t *o, const half_t *a, float c, long n) {
     if (i < n) o[i] = (half_t)((float)a[i] * c);
 }
 
+// A stand-alone activation (the same functions the GEMM and convolution epilogues apply) and clamp.
+__global__ void act_kernel(half_t *o, const half_t *a, int epi, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) o[i] = (half_t)apply_epi((float)a[i], epi);
+}
+__global__ void clamp_kernel(half_t *o, const half_t *a, float lo, float hi, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) o[i] = (half_t)fminf(fmaxf((float)a[i], lo), hi);
+}
+
 __global__ void add_vec_kernel(half_t *o, const half_t *a, const half_t *b, long n8) {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n8) return;
@@ -235,6 +245,25 @@ int mi_scale_f16(void *out, const void *a, float c, int64_t n, void *stream) {
     if (n < 0) return MI_DECLINE_EXTENT;
     if (n == 0) return MI_OK;
     hipLaunchKernelGGL(scale_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, (half_t *)out, (const half_t *)a, c, (long)n);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_act_f16(void *out, const void *a, int epi, int64_t n, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !a) return MI_DECLINE_OPERANDS;
+    if (epi < MI_EPI_NONE || epi > MI_EPI_RELU) return MI_DECLINE_UNSUPPORTED;
+    if (n < 0) return MI_DECLINE_EXTENT;
+    if (n == 0) return MI_OK;
+    hipLaunchKernelGGL(act_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, (half_t *)out, (const half_t *)a, epi, (long)n);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_clamp_f16(void *out, const void *a, float lo, float hi, int64_t n, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !a) return MI_DECLINE_OPERANDS;
+    if (n < 0 || !(lo <= hi)) return MI_DECLINE_EXTENT;
+    if (n == 0) return MI_OK;
+    hipLaunchKernelGGL(clamp_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, (half_t *)out, (const half_t *)a, lo, hi, (long)n);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 

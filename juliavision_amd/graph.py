@@ -11,8 +11,9 @@ the ops of the dense-contraction path:
     linear / addmm / mm / bmm, scaled_dot_product_attention (also written out
     as bmm + softmax + bmm), layer_norm / native_layer_norm, gelu, relu,
     add.Tensor, convolution, cat along the token axis, softmax over the last
-    axis, mul / div by a constant, a per-feature mul.Tensor after a linear
-    (LayerScale), contiguous clone, and the view ops between them.
+    axis, mul / div by a constant, clamp, a per-feature or constant mul.Tensor
+    after a linear (LayerScale, query scaling), contiguous clone, and the view
+    ops between them.
 
 Two of the reference's rewrites matter for that path and have counterparts here:
 
@@ -220,14 +221,17 @@ def fold_activations(g: Graph) -> Graph:
 
 
 def fold_layerscale(g: Graph) -> Graph:
-    """``mul.Tensor(y, gamma)`` with ``gamma`` a per-feature weight vector and ``y`` (a view chain of) a linear op's
-    output that nothing else reads -- DINOv2's LayerScale after the attention projection and after the MLP -- is
-    applied to the linear's weight columns and bias once, when the executor binds the weights: ``(xW + b) * gamma =
-    x (W gamma) + b gamma``.  The multiplication then costs nothing per run; the rounding moves from the activations
+    """``mul.Tensor(y, gamma)`` with ``gamma`` a per-feature weight vector -- DINOv2's LayerScale after the attention
+    projection and after the MLP -- or a constant -- Whisper's ``q_proj(x) * head_dim ** -0.5`` -- and ``y`` (a view chain
+    of) a linear op's output that nothing else reads is applied to the linear's weight columns and bias once, when
+    the executor binds the weights: ``(xW + b) * gamma = x (W gamma) + b gamma``.  The multiplication then costs nothing per run; the rounding moves from the activations
     to the weights (one fp16 rounding of ``W gamma`` instead of one of the product)."""
-    for mul in [o for o in g.ops if o["aten"] == "mul.Tensor" and len(o["in"]) == 2]:
-        for mine, other in (mul["in"], mul["in"][::-1]):
-            gb = g.buffers[g.root(other)]
+    for mul in [o for o in g.ops if o["aten"] in ("mul.Tensor", "div.Tensor") and len(o["in"]) in (1, 2)]:
+        const = _scalar_scale(mul)                      # x * c or x / c with a constant: the same fold, gamma = c
+        if len(mul["in"]) == 1 and const is None:
+            continue
+        for mine, other in ((mul["in"][0], None),) if const is not None else (mul["in"], mul["in"][::-1]):
+            gb = g.buffers[g.root(other)] if other is not None else None
             chain = [mine]
             while g.buffers[chain[-1]]["kind"] == "view":
                 chain.append(g.buffers[chain[-1]]["of"])
@@ -235,11 +239,12 @@ def fold_layerscale(g: Graph) -> Graph:
             if prod is None or prod["aten"] not in LINEAR_OPS or any(k in prod["attrs"] for k in ("epilogue", "residual", "colscale", "ln_out")):
                 continue
             feat = (g.buffers[chain[-1]].get("shape") or [None])[-1]
-            gshape = g.buffers[other].get("shape") or []
-            if gb["kind"] != "weight" or not gshape or gshape[-1] != feat or any(d != 1 for d in gshape[:-1]):
-                continue
-            if not all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1]):
-                continue
+            if other is not None:
+                gshape = g.buffers[other].get("shape") or []
+                if gb["kind"] != "weight" or not gshape or gshape[-1] != feat or any(d != 1 for d in gshape[:-1]):
+                    continue
+                if not all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1]):
+                    continue
             if not (_consumers(g, chain[-1]) <= {mul["id"]}):
                 continue
             # the linear's own weight and bias must be constants too
@@ -247,7 +252,7 @@ def fold_layerscale(g: Graph) -> Graph:
             ids = [prod["in"][wpos[0]]] + ([prod["in"][wpos[1]]] if wpos[1] is not None and len(prod["in"]) > wpos[1] else [])
             if any(g.buffers[g.root(i)]["kind"] != "weight" for i in ids):
                 continue
-            prod["attrs"]["colscale"] = other
+            prod["attrs"]["colscale"] = other if other is not None else const
             g.ops.remove(mul)
             g.buffers[mul["id"]].update(kind="view", of=mine, op="alias.default", attrs={})
             g.notes.append(f"fold {mul['id']} (per-feature scale) into the weights of {prod['id']}")
@@ -607,7 +612,8 @@ class Executor:
             x, w, bias = self.get(ins[0]), self.get(ins[1]), None
         if "colscale" in attrs:                          # LayerScale folded into the constants, once
             if o["id"] not in self.scaled:
-                gamma = self.get(attrs["colscale"]).reshape(-1).float()
+                cs = attrs["colscale"]
+                gamma = self.get(cs).reshape(-1).float() if isinstance(cs, str) else float(cs)
                 self.scaled[o["id"]] = ((w.float() * gamma).to(w.dtype), None if bias is None else (bias.float() * gamma).to(bias.dtype))
             w, bias = self.scaled[o["id"]]
         out = self.t[o["out"]]
@@ -711,12 +717,36 @@ class Executor:
         if o["attrs"].get("alpha", 1) != 1 or len(o["in"]) != 2:
             raise UnsupportedOp(f"{o['id']}: add with a scalar operand or alpha")
         a, b = self.get(o["in"][0]), self.get(o["in"][1])
-        if a.shape != b.shape:
+        out = self.t[o["out"]]
+        drop1 = lambda t: [d for d in t.shape if d != 1]
+        if a.shape != b.shape and drop1(a) != drop1(b):   # (1, T, D) + (T, D) is the same elements; anything else would broadcast
             raise UnsupportedOp(f"{o['id']}: broadcasting add {tuple(a.shape)} + {tuple(b.shape)}")
-        K.add_(self.ctx, self.t[o["out"]], a, b)
+        if not a.is_contiguous():                         # e.g. the permuted output of a convolution stem + its position embedding
+            self._copy(o, out.view(a.shape), a)
+            a = out
+        if not b.is_contiguous():
+            raise UnsupportedOp(f"{o['id']}: add of two strided tensors")
+        K.add_(self.ctx, out, a, b)
 
     def _activation(self, o):
-        raise UnsupportedOp(f"{o['id']}: a stand-alone {o['aten']} (run optimize() so that it folds into its linear)")
+        """gelu / relu that no linear op could take as its epilogue (after a convolution stem): on its own."""
+        a = o["attrs"]
+        if o["aten"] == "gelu.default" and a.get("approximate", "none") not in ("none", "tanh"):
+            raise UnsupportedOp(f"{o['id']}: gelu approximate={a.get('approximate')}")
+        x, out = self.get(o["in"][0]), self.t[o["out"]]
+        if not x.is_contiguous():
+            self._copy(o, out, x)
+            x = out
+        kind = "relu" if o["aten"] == "relu.default" else ("gelu_tanh" if a.get("approximate") == "tanh" else "gelu")
+        K.act_(self.ctx, out, x, kind)
+
+    def _clamp(self, o):
+        a = o["attrs"]
+        lo, hi = a.get("arg1", a.get("min")), a.get("arg2", a.get("max"))
+        x, out = self.get(o["in"][0]), self.t[o["out"]]
+        if len(o["in"]) != 1 or not x.is_contiguous():
+            raise UnsupportedOp(f"{o['id']}: clamp with tensor bounds or of a strided tensor")
+        K.clamp_(self.ctx, out, x, float("-inf") if lo is None else float(lo), float("inf") if hi is None else float(hi))
 
     def _convolution(self, o):
         """aten::convolution, ordinary and transposed (arg6), 2-D and -- lifted to a singleton second spatial
@@ -744,7 +774,7 @@ class Executor:
                 "native_layer_norm.default": _native_layer_norm, "add.Tensor": _add,
                 "gelu.default": _activation, "relu.default": _activation, "convolution.default": _convolution,
                 "bmm.default": _bmm, "cat.default": _cat, **dict.fromkeys(SOFTMAX_OPS, _softmax),
-                "mul.Tensor": _scale, "div.Tensor": _scale, "clone.default": _clone}
+                "mul.Tensor": _scale, "div.Tensor": _scale, "clone.default": _clone, "clamp.default": _clamp}
 
     def __call__(self, *inputs: torch.Tensor):
         if len(inputs) != len(self.g.inputs):

@@ -621,6 +621,28 @@ def scale_(ctx: Ctx, out, a, c: float):
     return out
 
 
+def act_(ctx: Ctx, out, a, act: str):
+    """out = fp16(act(a)), ``act`` as in ``matmul_``'s ``epi``; contiguous fp16 tensors (may be the same tensor)."""
+    lib = L.init()
+    if not _is_f16_cuda(a, out) or a.shape != out.shape or not (a.is_contiguous() and out.is_contiguous()):
+        raise DeclineError("act_: operands", L.DECLINE_OPERANDS)
+    rc = lib.mi_act_f16(out.data_ptr(), a.data_ptr(), L.EPI[act], a.numel(), ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_act_f16", rc)
+    return out
+
+
+def clamp_(ctx: Ctx, out, a, lo: float, hi: float):
+    """out = min(max(a, lo), hi); contiguous fp16 tensors (clamp, ops.jl:300-310)."""
+    lib = L.init()
+    if not _is_f16_cuda(a, out) or a.shape != out.shape or not (a.is_contiguous() and out.is_contiguous()):
+        raise DeclineError("clamp_: operands", L.DECLINE_OPERANDS)
+    rc = lib.mi_clamp_f16(out.data_ptr(), a.data_ptr(), float(lo), float(hi), a.numel(), ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_clamp_f16", rc)
+    return out
+
+
 def add_(ctx: Ctx, out, a, b):
     """out = fp16(a + b), the residual add.Tensor (ops.jl:186-197)."""
     lib = L.init()

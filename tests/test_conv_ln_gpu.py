@@ -341,3 +341,30 @@ def test_scale_bit_exact(ctx):
     jv.scale_(ctx, out, to_dev(a), 1.0 / 3.0)
     torch.cuda.synchronize()
     assert np.array_equal(to_host(out).view(np.uint16), oracle.scale_f16(a, 1.0 / 3.0).view(np.uint16))
+
+
+@pytest.mark.parametrize("kind", ["gelu", "gelu_tanh", "relu"])
+def test_standalone_activation_is_the_epilogue_function(ctx, kind):
+    """The activation on its own gives what the GEMM epilogue gives: the oracle's erf / tanh / relu forms
+    (ops.jl:161-169, 1665-1685) on fp16 values, one rounding."""
+    import torch
+    import juliavision_amd as jv
+    a = np.concatenate([oracle.randn_f16((2000,), 31, std=2.5), np.arange(-8, 8, 0.01).astype(np.float16)])
+    out = poison(torch.empty(a.shape, dtype=torch.float16, device="cuda"))
+    jv.act_(ctx, out, to_dev(a), kind)
+    torch.cuda.synchronize()
+    got, want = to_host(out).astype(np.float64), oracle.act_f16(a, kind).astype(np.float64)
+    assert np.max(np.abs(got - want)) <= 2e-3 * max(1.0, np.max(np.abs(want)))        # device exp / rcp against libm: an ulp of fp16
+    assert_parity(got, want, what=kind)
+
+
+def test_clamp_bit_exact(ctx):
+    import torch
+    import juliavision_amd as jv
+    a = oracle.randn_f16((4099,), 32, std=3e4)            # many values beyond the guard
+    a[:3] = [np.inf, -np.inf, 65504.0]
+    out = poison(torch.empty(a.shape, dtype=torch.float16, device="cuda"))
+    jv.clamp_(ctx, out, to_dev(a), -64504.0, 64504.0)
+    torch.cuda.synchronize()
+    want = np.clip(a.astype(np.float32), -64504.0, 64504.0).astype(np.float16)
+    assert np.array_equal(to_host(out).view(np.uint16), want.view(np.uint16))

@@ -479,3 +479,87 @@ def test_attention_that_returns_its_probabilities_runs(ctx):
     y, p = run(x.cuda())
     assert_parity(y.float().cpu().numpy(), want_y, what="output")
     assert_parity(p.float().cpu().numpy(), want_p, what="probabilities")
+
+
+def _whisper_like_encoder(d=128, heads=2, layers=2, mels=16, frames=60, seed=0):
+    """An audio encoder written the way Whisper's is (the model of configs 1, 2 and 5): two 1-D convolutions with GELU
+    (the second of stride 2), learned positions, pre-LN layers whose query projection is multiplied by
+    head_dim ** -0.5 ahead of a fused attention with scale 1, k_proj without bias, the fp16 clamp after each layer,
+    a final norm."""
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+
+    class Layer(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.h, self.scaling = heads, (d // heads) ** -0.5
+            self.ln1, self.ln2 = nn.LayerNorm(d), nn.LayerNorm(d)
+            self.q, self.k, self.v, self.o = nn.Linear(d, d), nn.Linear(d, d, bias=False), nn.Linear(d, d), nn.Linear(d, d)
+            self.fc1, self.fc2 = nn.Linear(d, 4 * d), nn.Linear(4 * d, d)
+
+        def forward(self, x):
+            B, T, D = x.shape
+            y = self.ln1(x)
+            sp = lambda t: t.view(B, T, self.h, D // self.h).transpose(1, 2)
+            a = F.scaled_dot_product_attention(sp(self.q(y) * self.scaling), sp(self.k(y)), sp(self.v(y)), scale=1.0)
+            x = x + self.o(a.transpose(1, 2).reshape(B, T, D))
+            x = x + self.fc2(F.gelu(self.fc1(self.ln2(x))))
+            return torch.clamp(x, min=-64504.0, max=64504.0)
+
+    class Encoder(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv1, self.conv2 = nn.Conv1d(mels, d, 3, padding=1), nn.Conv1d(d, d, 3, stride=2, padding=1)
+            self.pos = nn.Parameter(torch.randn(frames // 2, d) * 0.1)
+            self.layers = nn.ModuleList([Layer() for _ in range(layers)])
+            self.ln_post = nn.LayerNorm(d)
+
+        def forward(self, mel):
+            x = F.gelu(self.conv2(F.gelu(self.conv1(mel))))
+            x = x.permute(0, 2, 1) + self.pos
+            for l in self.layers:
+                x = l(x)
+            return self.ln_post(x)
+
+    torch.manual_seed(seed)
+    return Encoder().eval().half()
+
+
+def _export_keeping_sdpa(m, x):
+    import torch
+    table = torch.export.default_decompositions()
+    table.pop(torch.ops.aten.scaled_dot_product_attention.default, None)
+    return torch.export.export(m, (x,)).run_decompositions(table)
+
+
+def test_whisper_like_encoder_rewrites():
+    import torch
+    from juliavision_amd import graph as G
+    m = _whisper_like_encoder()
+    d = G.convert(_export_keeping_sdpa(m, torch.randn(1, 16, 60).half()), "enc")
+    aten = [o["aten"] for o in d["ops"]]
+    assert aten.count("clamp.default") == 2 and aten.count("mul.Tensor") == 2 and aten.count("gelu.default") == 4
+    g = G.optimize(G.Graph.load(d))
+    left = [o["aten"] for o in g.ops]
+    # stem: conv, gelu, conv, gelu, + positions, first norm; per layer q, k, v, attention, out-projection, fc1, fc2, clamp
+    # (a layer's second norm rides in its out-projection; the clamp keeps the next layer's first norm its own launch)
+    assert left.count("mul.Tensor") == 0 and left.count("gelu.default") == 2 and left.count("clamp.default") == 2, (left, g.notes)
+    q = next(o for o in g.ops if o["attrs"].get("colscale") is not None)
+    assert q["attrs"]["colscale"] == pytest.approx(0.125)
+    assert sum(o["attrs"].get("epilogue") == "gelu" for o in g.ops) == 2 and sum("residual" in o["attrs"] for o in g.ops) == 4
+
+
+@pytest.mark.gpu
+def test_whisper_like_encoder_runs_on_the_kernels(ctx):
+    import torch
+    from juliavision_amd import graph as G
+    m = _whisper_like_encoder(seed=9)
+    x = torch.randn(1, 16, 60).half()
+    run = G.Executor(G.optimize(G.Graph.load(G.convert(_export_keeping_sdpa(m, x), "enc"))), m.state_dict(), ctx)
+    with torch.no_grad():
+        want = m.float()(x.float()).numpy()
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    assert got.shape == (1, 30, 128)
+    assert_parity(got.float().cpu().numpy(), want, what="Whisper-like encoder from its exported graph")
