@@ -279,10 +279,11 @@ def ln_matmul_(ctx: Ctx, out, A, B, gamma, beta, eps, bias=None, *, epi="none", 
     return out
 
 
-def batchedmatmul_(ctx: Ctx, out, A, B):
-    """``out[b] = B[b] . A[b]`` over the leading torch axis -- batchedmatmul!, matmul.jl:383.
+def batchedmatmul_(ctx: Ctx, out, A, B, bias=None):
+    """``out[b] = B[b] . A[b] (+ bias[b])`` over the leading torch axis -- batchedmatmul!, matmul.jl:383.
     ``A``: torch (Bt, K, F), ``B``: torch (Bt, T, K), ``out``: (Bt, T, F); a leading
-    extent of 1 on ``A`` or ``B`` shares that operand."""
+    extent of 1 on ``A`` or ``B`` shares that operand.  ``bias``: (Bt, F), one row per plane (several linear ops over
+    the same activations issued as one launch)."""
     lib = L.init()
     if not _is_f16_cuda(A, B) or A.dim() != 3 or B.dim() != 3 or out.dim() != 3:
         raise DeclineError("batchedmatmul_: operands", L.DECLINE_OPERANDS)
@@ -294,9 +295,12 @@ def batchedmatmul_(ctx: Ctx, out, A, B):
         raise DeclineError("batchedmatmul_: planes must be row-major (A's may be transposed views)", L.DECLINE_OPERANDS)
     sA = 0 if A.shape[0] == 1 else A.stride(0)
     sB = 0 if B.shape[0] == 1 else B.stride(0)
-    rc = lib.mi_gemm_f16_batched(out.data_ptr(), B.data_ptr(), A.data_ptr(), None, None, T, K, F,
-                                 out.stride(1), B.stride(1), la[1], L.W_KF if la[0] == 0 else L.W_FK, L.BIAS_NONE, L.EPI["none"],
-                                 _dtype_code(out), nb, out.stride(0), sB, sA, 0, None, 0, ctx.stream)
+    if bias is not None and (not _is_f16_cuda(bias) or tuple(bias.shape) != (nb, F) or bias.stride(1) != 1):
+        raise DeclineError("batchedmatmul_: bias must be (Bt, F) fp16 rows", L.DECLINE_BIAS)
+    rc = lib.mi_gemm_f16_batched(out.data_ptr(), B.data_ptr(), A.data_ptr(), _ptr(bias), None, T, K, F,
+                                 out.stride(1), B.stride(1), la[1], L.W_KF if la[0] == 0 else L.W_FK,
+                                 L.BIAS_NONE if bias is None else L.BIAS_COL, L.EPI["none"],
+                                 _dtype_code(out), nb, out.stride(0), sB, sA, 0 if bias is None else bias.stride(0), None, 0, ctx.stream)
     if rc != L.OK:
         raise DeclineError("mi_gemm_f16_batched", rc)
     return out

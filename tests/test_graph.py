@@ -80,8 +80,10 @@ def test_rewrites_fold_activation_residuals_and_attention_layout():
     assert fc1["attrs"]["epilogue"] == "gelu" and g.buffers["gelu"]["kind"] == "view" and g.buffers["gelu"]["of"] == "linear_4"
     assert g.op("linear_3")["attrs"]["residual"] == "$x" and g.op("linear_5")["attrs"]["residual"] == "$add"
     assert g.op("scaled_dot_product_attention")["attrs"]["token_major"] is True
-    assert len(g.ops) == 8                                              # LN + 6 linears + attention
-    assert g.root("add_1") == "linear_5" and len(g.notes) == 5
+    assert len(g.ops) == 6                                              # LN, q/k/v as one group, attention, 3 linears
+    grp = next(o for o in g.ops if o["aten"] == "linear_group")
+    assert [m["out"] for m in grp["attrs"]["members"]] == ["linear", "linear_1", "linear_2"]
+    assert g.root("add_1") == "linear_5" and len(g.notes) == 6
     # the second norm reads the residual stream that the out-projection writes: it became that GEMM's second result
     proj = g.op("linear_3")
     assert proj["attrs"]["ln_out"] == "layer_norm_1" and proj["attrs"]["ln_gamma"] == "p_ln2_weight" and proj["attrs"]["ln_eps"] == 1e-5
@@ -224,7 +226,7 @@ def test_decomposed_export_folds_like_the_composite_one():
     aten = [o["aten"] for o in d["ops"]]
     assert aten.count("addmm.default") == 5 and aten.count("mm.default") == 1 and aten.count("native_layer_norm.default") == 2
     g = G.optimize(G.Graph.load(d))
-    assert [o["aten"] for o in g.ops].count("gelu.default") == 0 and len(g.ops) == 8
+    assert [o["aten"] for o in g.ops].count("gelu.default") == 0 and len(g.ops) == 6
     assert [o["aten"] for o in g.ops].count("native_layer_norm.default") == 1         # the second one rides in the out-projection
     fc1 = next(o for o in g.ops if o["attrs"].get("epilogue") == "gelu")
     assert fc1["aten"] == "addmm.default" and g.root("gelu") == fc1["id"]       # gelu read the addmm through a view
@@ -232,7 +234,7 @@ def test_decomposed_export_folds_like_the_composite_one():
     for name in ("_scaled_dot_product_flash_attention.default", "_scaled_dot_product_efficient_attention.default"):
         g2 = G.optimize(G.Graph.load(_as_backend_attention(d, name)))
         att = next(o for o in g2.ops if o["aten"] == name)
-        assert att["attrs"]["token_major"] is True and len(g2.ops) == 8
+        assert att["attrs"]["token_major"] is True and len(g2.ops) == 6
 
 
 @pytest.mark.gpu
@@ -545,8 +547,9 @@ def test_whisper_like_encoder_rewrites():
     # stem: conv, gelu, conv, gelu, + positions, first norm; per layer q, k, v, attention, out-projection, fc1, fc2, clamp
     # (a layer's second norm rides in its out-projection; the clamp keeps the next layer's first norm its own launch)
     assert left.count("mul.Tensor") == 0 and left.count("gelu.default") == 2 and left.count("clamp.default") == 2, (left, g.notes)
-    q = next(o for o in g.ops if o["attrs"].get("colscale") is not None)
-    assert q["attrs"]["colscale"] == pytest.approx(0.125)
+    grp = [o for o in g.ops if o["aten"] == "linear_group"]
+    assert len(grp) == 2 and all(len(o["attrs"]["members"]) == 3 for o in grp)                  # q, k, v of each layer: one launch
+    assert [m["colscale"] for m in grp[0]["attrs"]["members"]] == [pytest.approx(0.125), None, None]   # the constant after q_proj
     assert sum(o["attrs"].get("epilogue") == "gelu" for o in g.ops) == 2 and sum("residual" in o["attrs"] for o in g.ops) == 4
 
 
