@@ -434,6 +434,94 @@ def vit_graph_case(steps=50):
             "eager_ms": round(eager * 1e3, 4), "graph_ms": round(replay * 1e3, 4), "TFLOP/s_graph": round(flop / replay / 1e12, 1)}
 
 
+def whisper_graph_case(nl=32, steps=10):
+    """Configs 1/2's model as a whole, from its exported graph: an audio encoder written the way Whisper large-v3's is
+    (128 mel bins x 3000 frames through two 1-D convolutions with GELU, 1500 positions, `nl` pre-LN layers of
+    d_model 1280 with 20 x 64 heads -- q_proj scaled by 1/8 ahead of a fused attention, k_proj without bias -- FFN 5120,
+    the fp16 clamp after every layer, a final norm), exported on the meta device, converted, rewritten and run by the
+    graph executor with random weights.  Reported per layer: what BASELINE's "ms per encoder block" is inside the model."""
+    import time
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+    import juliavision_amd as jv
+    from juliavision_amd import graph as G
+    from juliavision_amd.decode import StepGraph
+    d, heads, mels, frames, ffn = 1280, 20, 128, 3000, 5120
+
+    class Layer(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.ln1, self.ln2 = nn.LayerNorm(d), nn.LayerNorm(d)
+            self.q, self.k, self.v, self.o = nn.Linear(d, d), nn.Linear(d, d, bias=False), nn.Linear(d, d), nn.Linear(d, d)
+            self.fc1, self.fc2 = nn.Linear(d, ffn), nn.Linear(ffn, d)
+
+        def forward(self, x):
+            B, T, D = x.shape
+            y = self.ln1(x)
+            sp = lambda t: t.view(B, T, heads, D // heads).transpose(1, 2)
+            a = F.scaled_dot_product_attention(sp(self.q(y) * (D // heads) ** -0.5), sp(self.k(y)), sp(self.v(y)), scale=1.0)
+            x = x + self.o(a.transpose(1, 2).reshape(B, T, D))
+            x = x + self.fc2(F.gelu(self.fc1(self.ln2(x))))
+            return torch.clamp(x, min=-64504.0, max=64504.0)
+
+    class Encoder(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv1, self.conv2 = nn.Conv1d(mels, d, 3, padding=1), nn.Conv1d(d, d, 3, stride=2, padding=1)
+            self.pos = nn.Parameter(torch.empty(frames // 2, d))
+            self.layers = nn.ModuleList([Layer() for _ in range(nl)])
+            self.ln_post = nn.LayerNorm(d)
+
+        def forward(self, mel):
+            x = F.gelu(self.conv2(F.gelu(self.conv1(mel))))
+            x = x.permute(0, 2, 1) + self.pos
+            for layer in self.layers:
+                x = layer(x)
+            return self.ln_post(x)
+
+    t0 = time.perf_counter()
+    with torch.device("meta"):
+        m = Encoder().eval().half()
+        mel_meta = torch.empty(1, mels, frames, dtype=torch.float16)
+    table = torch.export.default_decompositions()
+    table.pop(torch.ops.aten.scaled_dot_product_attention.default, None)     # an accelerator export keeps the fused op
+    spec = G.convert(torch.export.export(m, (mel_meta,)).run_decompositions(table), "whisper_encoder")
+    g = G.optimize(G.Graph.load(spec))
+    host_s = time.perf_counter() - t0
+    torch.manual_seed(0)
+    weights = {}
+    for k, v in m.state_dict().items():
+        norm_scale = k.endswith("weight") and v.dim() == 1
+        weights[k] = torch.ones(v.shape, dtype=torch.float16, device="cuda") if norm_scale else \
+            torch.randn(v.shape, dtype=torch.float16, device="cuda") * 0.02
+    ctx = jv.Ctx("cuda")
+    run = G.Executor(g, weights, ctx)
+    mel = torch.randn((1, mels, frames), dtype=torch.float16, device="cuda")
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / steps
+
+    step = lambda: run(mel)
+    eager = timed(step)
+    replay = timed(StepGraph(step).replay)
+    if not bool(torch.isfinite(run(mel)).all()):
+        raise RuntimeError("exported Whisper-like encoder produced non-finite output")
+    T = frames // 2
+    flop = nl * (2.0 * T * d * (4 * d + 2 * ffn) + 4.0 * T * T * 64 * heads) + 2.0 * frames * (3 * mels) * d + 2.0 * T * (3 * d) * d
+    return {"layers": nl, "ops_exported": len(spec["ops"]), "ops_after_rewrites": len(g.ops), "export_and_rewrite_host_s": round(host_s, 2),
+            "eager_ms": round(eager * 1e3, 3), "graph_ms": round(replay * 1e3, 3), "graph_ms_per_layer": round(replay * 1e3 / nl, 4),
+            "GFLOP": round(flop / 1e9, 1), "TFLOP/s_graph": round(flop / replay / 1e12, 1),
+            "frac_mfma_peak_graph": round(flop / replay / 1e12 / PEAK_F16_TFLOPS, 4)}
+
+
 def encoder_stack_case(nl=4, steps=50):
     """BASELINE config 2's block as it occurs in a stack: `nl` Whisper-shaped blocks in sequence (1500 x 1280, 20 x 64
     heads, FFN 5120, [K][F] weights), each block's first norm written by the previous block's last GEMM.  Reported per
@@ -639,6 +727,10 @@ def detail_benchmarks(lib, L, stream, only=None):
     name = "c3_vit_s14_518_encoder_12layers"
     if only is None or only in name:
         out[name] = vit_encoder_case()
+
+    name = "c2_whisper_encoder_32layers_from_exported_graph"
+    if only is None or only in name:
+        out[name] = whisper_graph_case()
 
     name = "c3_vit_s14_518_from_exported_graph"
     if only is None or only in name:

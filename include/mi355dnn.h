@@ -134,6 +134,15 @@ int mi_gemm_ln_f16(void *Y, void *H, const void *X, const void *W, const void *b
                    const void *gamma, const void *beta, float eps,
                    int64_t T, int64_t K, int64_t F, int64_t ldX, int64_t ldW,
                    int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream);
+/* mi_gemm_ln_f16 with the result clamped to [-clamp, clamp] (clamp > 0) after the residual add, as a separate
+ * aten::clamp on Y would leave it -- the fp16 overflow guard that exported encoder layers carry after every block
+ * (ops.jl:300-310) -- and H, the layer norm of the clamped rows, optional (null: none).  The tiled kernels and the
+ * split-K plane sum clamp in their stores; decode-sized and unaligned shapes clamp in a pass of their own.  Bits as
+ * the separate ops give them. */
+int mi_gemm_clamp_ln_f16(void *Y, void *H, const void *X, const void *W, const void *bias, const void *residual,
+                         const void *gamma, const void *beta, float eps, float clamp,
+                         int64_t T, int64_t K, int64_t F, int64_t ldX, int64_t ldW,
+                         int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream);
 
 size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int64_t nbatch);
 /* Returns an mi_gemm_path; never launches.  Replaces mmplan / mm_coopmat_plan /

@@ -33,6 +33,9 @@ struct GemmArgs {
     half_t *lnout;
     const half_t *lnout_gamma, *lnout_beta;
     float lnout_eps;
+    // Tiled kernels and the split-K plane sums: > 0 clamps the fp16 result to [-clamp, clamp] after the residual add,
+    // as a separate aten::clamp on Y would (the overflow guard of exported fp16 encoder layers).
+    float clamp;
 };
 
 // ------------------------------------------------------------------------------------------
@@ -239,12 +242,17 @@ __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc
 #pragma unroll
                             for (int e = 0; e < 8; e++) x[e] = (half_t)((float)x[e] + (float)rv[e]);
                         }
+                        if (p.clamp > 0.0f) {
+#pragma unroll
+                            for (int e = 0; e < 8; e++) x[e] = (half_t)fminf(fmaxf((float)x[e], -p.clamp), p.clamp);
+                        }
                         *reinterpret_cast<half8v *>(yp) = x;
                     } else {
                         for (int e = 0; e < 8; e++) {
                             if (n + e < p.N) {
                                 half_t o = x[e];
                                 if (p.residual) o = (half_t)((float)o + (float)p.residual[off + e]);
+                                if (p.clamp > 0.0f) o = (half_t)fminf(fmaxf((float)o, -p.clamp), p.clamp);
                                 yp[e] = o;
                             }
                         }
@@ -899,6 +907,10 @@ __global__ void splitk_epilogue_kernel(GemmArgs p, const float *part, int nsplit
 #pragma unroll
             for (int e = 0; e < 4; e++) o[e] = (half_t)((float)o[e] + (float)p.residual[off + e]);
         }
+        if (p.clamp > 0.0f) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = (half_t)fminf(fmaxf((float)o[e], -p.clamp), p.clamp);
+        }
         if (p.vec_store) *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(p.Y) + off) = o;
         else {
 #pragma unroll
@@ -949,6 +961,10 @@ __global__ __launch_bounds__(256) void splitk_epilogue_ln_kernel(GemmArgs p, con
                 const half8v rv = as_half8(ldg16(p.residual + off));
 #pragma unroll
                 for (int e = 0; e < 8; e++) o[e] = (half_t)((float)o[e] + (float)rv[e]);
+            }
+            if (p.clamp > 0.0f) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[e] = (half_t)fminf(fmaxf((float)o[e], -p.clamp), p.clamp);
             }
             *reinterpret_cast<half8v *>(reinterpret_cast<half_t *>(p.Y) + off) = o;
 #pragma unroll
@@ -1140,7 +1156,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.cv = ConvGather{};
     a.ag = NhwcGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
-    a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f;
+    a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
     return MI_OK;
 }
 
@@ -1167,7 +1183,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         const int split = nbatch == 1 ? splitk_count(a.M, a.N, a.K) : 1;
         if (split > 1 && ws && aligned_to(ws, 256) && ws_bytes >= (size_t)split * a.M * a.N * sizeof(float)) {
             GemmArgs s1 = a;
-            s1.Y = ws; s1.out_f32 = 1; s1.bias = nullptr; s1.bias_mode = MI_BIAS_NONE; s1.epi = MI_EPI_NONE; s1.residual = nullptr;
+            s1.Y = ws; s1.out_f32 = 1; s1.bias = nullptr; s1.bias_mode = MI_BIAS_NONE; s1.epi = MI_EPI_NONE; s1.residual = nullptr; s1.clamp = 0.0f;
             s1.ldY = a.N; s1.sY = (long)a.M * a.N;
             s1.K = a.K / split;
             s1.sA = s1.K; s1.sB = b_kn ? (long)s1.K * a.ldB : s1.K; s1.sBias = 0;
@@ -1225,7 +1241,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     a.cv = ConvGather{};
     a.ag = NhwcGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
-    a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f;
+    a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
@@ -1346,6 +1362,33 @@ int mi_gemm_ln_f16(void *Y, void *H, const void *X, const void *W, const void *b
     if (rc == MI_LNOUT_DONE) return MI_OK;
     if (rc != MI_OK) return rc;
     return mi_layernorm_f16(H, nullptr, nullptr, Y, gamma, beta, F, T, eps, stream);      // rows of Y are dense: ldY = F
+}
+
+int mi_gemm_clamp_ln_f16(void *Y, void *H, const void *X, const void *W, const void *bias, const void *residual,
+                         const void *gamma, const void *beta, float eps, float clamp,
+                         int64_t T, int64_t K, int64_t F, int64_t ldX, int64_t ldW,
+                         int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream) {
+    if (!(clamp > 0.0f)) return MI_DECLINE_OPERANDS;
+    GemmArgs a;
+    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, F, ldX, ldW, w_layout, bias_mode, epi, MI_F16, 0, 0, 0);
+    if (rc != MI_OK) return rc;
+    if (!g_ready) return MI_ERROR_DEVICE;
+    if (T == 0 || F == 0) return MI_OK;
+    const bool b_kn = w_layout == MI_W_KF;
+    // the tiled kernels and the plane sums clamp in their stores; the decode-sized and scalar kernels do not: there the
+    // clamp is a pass of its own over Y
+    const bool in_store = gemm_path(a, b_kn, 1) == MI_GEMM_MFMA;
+    if (in_store) a.clamp = clamp;
+    if (H) { a.lnout = (half_t *)H; a.lnout_gamma = (const half_t *)gamma; a.lnout_beta = (const half_t *)beta; a.lnout_eps = eps; }
+    if (!in_store) a.lnout = nullptr;
+    rc = run_gemm(a, b_kn, 1, ws, ws_bytes, (hipStream_t)stream, 0);
+    if (rc == MI_LNOUT_DONE) return MI_OK;
+    if (rc != MI_OK) return rc;
+    if (!in_store) {
+        rc = mi_clamp_f16(Y, Y, -clamp, clamp, T * F, stream);
+        if (rc != MI_OK) return rc;
+    }
+    return H ? mi_layernorm_f16(H, nullptr, nullptr, Y, gamma, beta, F, T, eps, stream) : MI_OK;
 }
 
 int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,

@@ -270,7 +270,7 @@ def group_linears(g: Graph) -> Graph:
         x, w = o["in"][pos[0]], o["in"][pos[1]]
         b = o["in"][pos[2]] if pos[2] is not None and len(o["in"]) > pos[2] else None
         return x, w, b
-    plain = lambda o: o["aten"] in LINEAR_OPS and not any(k in o["attrs"] for k in ("epilogue", "residual", "ln_out"))
+    plain = lambda o: o["aten"] in LINEAR_OPS and not any(k in o["attrs"] for k in ("epilogue", "residual", "ln_out", "clamp"))
     done = set()
     for first in [o for o in g.ops if plain(o)]:
         if first["id"] in done or first not in g.ops:
@@ -331,6 +331,33 @@ def fold_residuals(g: Graph) -> Graph:
                 g.buffers[chain[-1]]["kind"] = "external"
             g.notes.append(f"fold add {add['id']} into {prod['id']}")
             break
+    return g
+
+
+def fold_clamps(g: Graph) -> Graph:
+    """``clamp(y, -c, c)`` with constant symmetric bounds whose input is (a view chain of) a linear op's result that
+    nothing else reads -- the fp16 overflow guard exported encoder layers carry after their last residual add -- moves
+    into that GEMM's store, after the residual (``matmul_ln_(clamp=)``): the same bits, one pass over the residual
+    stream less, and the norm that reads the clamped stream can then ride in the same GEMM (``fold_layernorms``)."""
+    for cl in [o for o in g.ops if o["aten"] == "clamp.default" and len(o["in"]) == 1]:
+        a = cl["attrs"]
+        lo, hi = a.get("arg1", a.get("min")), a.get("arg2", a.get("max"))
+        if not isinstance(lo, (int, float)) or not isinstance(hi, (int, float)) or hi <= 0 or lo != -hi:
+            continue
+        chain = [cl["in"][0]]
+        while g.buffers[chain[-1]]["kind"] == "view":
+            chain.append(g.buffers[chain[-1]]["of"])
+        prod = g.op(chain[-1])
+        if prod is None or prod["aten"] not in LINEAR_OPS or any(k in prod["attrs"] for k in ("clamp", "ln_out")):
+            continue
+        if g.buffers[chain[-1]].get("dtype") != "float16" or not (_consumers(g, chain[-1]) <= {cl["id"]}):
+            continue
+        prod["attrs"]["clamp"] = float(hi)
+        g.ops.remove(cl)
+        g.buffers[cl["id"]].update(kind="view", of=cl["in"][0], op="alias.default", attrs={})
+        if cl["id"] in g.outputs:
+            g.buffers[chain[-1]]["kind"] = "external"
+        g.notes.append(f"fold {cl['id']} into the store of {prod['id']}")
     return g
 
 
@@ -530,7 +557,7 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
 
 
 def optimize(g: Graph) -> Graph:
-    return group_linears(fold_sdpa_transpose(fold_attention(fold_layernorms(fold_residuals(fold_layerscale(fold_activations(g)))))))
+    return group_linears(fold_sdpa_transpose(fold_attention(fold_layernorms(fold_clamps(fold_residuals(fold_layerscale(fold_activations(g))))))))
 
 
 # ----------------------------------------------------------------------------- execution
@@ -670,11 +697,12 @@ class Executor:
         out = self.t[o["out"]]
         res = self._rows(self.get(res_id)) if res_id else None
         self.ctx.ws.reset()
-        if attrs.get("ln_out") is not None:
-            gamma = self.get(attrs["ln_gamma"]) if attrs.get("ln_gamma") else None
-            beta = self.get(attrs["ln_beta"]) if attrs.get("ln_beta") else None
-            K.matmul_ln_(self.ctx, self._rows(out), self._rows(self.t[attrs["ln_out"]]), w, self._rows(x), gamma, beta,
-                         attrs["ln_eps"], bias, epi=attrs.get("epilogue", "none"), residual=res)
+        if attrs.get("ln_out") is not None or attrs.get("clamp") is not None:
+            has_ln = attrs.get("ln_out") is not None
+            gamma = self.get(attrs["ln_gamma"]) if has_ln and attrs.get("ln_gamma") else None
+            beta = self.get(attrs["ln_beta"]) if has_ln and attrs.get("ln_beta") else None
+            K.matmul_ln_(self.ctx, self._rows(out), self._rows(self.t[attrs["ln_out"]]) if has_ln else None, w, self._rows(x), gamma, beta,
+                         attrs.get("ln_eps", 0.0), bias, epi=attrs.get("epilogue", "none"), residual=res, clamp=attrs.get("clamp"))
             return
         K.matmul_(self.ctx, self._rows(out), w, self._rows(x), bias, epi=attrs.get("epilogue", "none"), residual=res)
 

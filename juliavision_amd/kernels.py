@@ -230,10 +230,12 @@ def _matmul_run(ctx, plan, out, A, B, bias, epi, residual, bias_mode):
     return out
 
 
-def matmul_ln_(ctx: Ctx, out, normed, A, B, gamma, beta, eps, bias=None, *, epi="none", residual=None):
+def matmul_ln_(ctx: Ctx, out, normed, A, B, gamma, beta, eps, bias=None, *, epi="none", residual=None, clamp=None):
     """``out[T,F] = epi(B[T,K] . A[K,F] + bias) (+ residual)`` as ``matmul_`` writes it, and ``normed[T,F]`` = layer norm
     of ``out`` over ``F`` (``layernorm_``, layernorm.jl:125): a linear op whose result is both the residual stream and
-    the input of the next norm.  One launch less than the two calls when the GEMM splits K; the same bits either way."""
+    the input of the next norm.  One launch less than the two calls when the GEMM splits K; the same bits either way.
+    ``clamp``: ``out`` is limited to ``[-clamp, clamp]`` after the residual add (a ``clamp`` op folded in, ops.jl:300-310);
+    with it ``normed`` may be None (no norm)."""
     plan = mmplan(ctx.dev, out, A, B, bias)
     if isinstance(plan, Decline):
         raise DeclineError(f"matmul_ln_ declined ({plan.reason})", L.DECLINE_OPERANDS)
@@ -241,18 +243,26 @@ def matmul_ln_(ctx: Ctx, out, normed, A, B, gamma, beta, eps, bias=None, *, epi=
     K, F = A.shape
     T = B.shape[0]
     la, lb = _mat2(A), _mat2(B)
-    if out.dtype != torch.float16 or not out.is_contiguous() or not _is_f16_cuda(normed) or not normed.is_contiguous() or normed.shape != out.shape:
+    if normed is None and clamp is None:
+        raise DeclineError("matmul_ln_: nothing to add to matmul_ (no norm, no clamp)", L.DECLINE_OPERANDS)
+    if out.dtype != torch.float16 or not out.is_contiguous() or (normed is not None and (
+            not _is_f16_cuda(normed) or not normed.is_contiguous() or normed.shape != out.shape)):
         raise DeclineError("matmul_ln_: out and normed must be dense fp16 (T,F)", L.DECLINE_OPERANDS)
     if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
         raise DeclineError("matmul_ln_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
     bm = L.BIAS_NONE if bias is None else (L.BIAS_COL if bias.numel() == F else L.BIAS_ROW)
     need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1)
     ws = ctx.ws.scratch(need)
-    rc = lib.mi_gemm_ln_f16(out.data_ptr(), normed.data_ptr(), B.data_ptr(), A.data_ptr(), _ptr(bias), _ptr(residual),
-                            _ptr(gamma), _ptr(beta), float(eps), T, K, F, lb[1], la[1], plan.w_layout, bm, L.EPI[epi],
-                            ws, need, ctx.stream)
+    if clamp is not None:
+        rc = lib.mi_gemm_clamp_ln_f16(out.data_ptr(), _ptr(normed), B.data_ptr(), A.data_ptr(), _ptr(bias), _ptr(residual),
+                                      _ptr(gamma), _ptr(beta), float(eps), float(clamp), T, K, F, lb[1], la[1], plan.w_layout, bm,
+                                      L.EPI[epi], ws, need, ctx.stream)
+    else:
+        rc = lib.mi_gemm_ln_f16(out.data_ptr(), normed.data_ptr(), B.data_ptr(), A.data_ptr(), _ptr(bias), _ptr(residual),
+                                _ptr(gamma), _ptr(beta), float(eps), T, K, F, lb[1], la[1], plan.w_layout, bm, L.EPI[epi],
+                                ws, need, ctx.stream)
     if rc != L.OK:
-        raise DeclineError("mi_gemm_ln_f16", rc)
+        raise DeclineError("mi_gemm_clamp_ln_f16" if clamp is not None else "mi_gemm_ln_f16", rc)
     return out
 
 

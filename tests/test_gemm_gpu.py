@@ -239,3 +239,32 @@ def test_layer_norm_of_the_output_rides_in_the_gemm(ctx, T, K, F, layout):
         assert_parity(to_host(out), y, what=f"matmul_ln_ output T{T} K{K} F{F} {layout}")
         assert_parity(to_host(normed), h, what=f"matmul_ln_ norm T{T} K{K} F{F} {layout}")
         assert np.array_equal(to_host(out), to_host(out2)) and np.array_equal(to_host(normed), to_host(normed2))
+
+
+@pytest.mark.parametrize("T,K,F,with_norm", [(300, 256, 384, True), (200, 2048, 256, True), (130, 128, 520, False), (4, 256, 384, True)])
+def test_matmul_with_clamp_in_the_store_is_the_separate_ops(ctx, T, K, F, with_norm):
+    """mi_gemm_clamp_ln_f16: GEMM + residual, then aten::clamp, then the layer norm of the clamped rows -- in the
+    tiled kernel's store, in the split-K plane sum (K = 2048 over few tiles), and as a pass of its own behind the
+    decode-sized kernel (T = 4).  Values are scaled to overflow fp16 in places, so the clamp has something to do."""
+    import torch
+    import juliavision_amd as jv
+    x = to_dev(oracle.randn_f16((T, K), 41, std=30.0))
+    w = to_dev(oracle.randn_f16((K, F), 42, std=1200.0 / K ** 0.5))       # sums of std 36 000 whatever K
+    b = to_dev(oracle.randn_f16((F,), 43))
+    r = to_dev(oracle.randn_f16((T, F), 44, std=1000.0))
+    g, be = to_dev(oracle.randn_f16((F,), 45, mean=1.0, std=0.1)), to_dev(oracle.randn_f16((F,), 46, std=0.1))
+    y0 = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.matmul_(ctx, y0, w, x, b, residual=r)
+    assert bool(torch.isinf(y0).any()) and bool((y0.abs() > 64504).sum() > 100)      # the unclamped result overflows
+    want_y = poison(torch.empty_like(y0))
+    jv.clamp_(ctx, want_y, y0, -64504.0, 64504.0)
+    want_h = poison(torch.empty_like(y0))
+    jv.layernorm_(ctx, want_h, None, None, want_y, g, be, F, 1e-5)
+    y, h = poison(torch.empty_like(y0)), poison(torch.empty_like(y0))
+    ctx.ws.reset()
+    jv.matmul_ln_(ctx, y, h if with_norm else None, w, x, g, be, 1e-5, b, residual=r, clamp=64504.0)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y).all()) and torch.equal(y.view(torch.int16), want_y.view(torch.int16))
+    if with_norm:
+        assert torch.equal(h.view(torch.int16), want_h.view(torch.int16))
