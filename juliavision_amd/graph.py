@@ -224,8 +224,9 @@ def fold_layerscale(g: Graph) -> Graph:
     """``mul.Tensor(y, gamma)`` with ``gamma`` a per-feature weight vector -- DINOv2's LayerScale after the attention
     projection and after the MLP -- or a constant -- Whisper's ``q_proj(x) * head_dim ** -0.5`` -- and ``y`` (a view chain
     of) a linear op's output that nothing else reads is applied to the linear's weight columns and bias once, when
-    the executor binds the weights: ``(xW + b) * gamma = x (W gamma) + b gamma``.  The multiplication then costs nothing per run; the rounding moves from the activations
-    to the weights (one fp16 rounding of ``W gamma`` instead of one of the product)."""
+    the executor binds the weights: ``(xW + b) * gamma = x (W gamma) + b gamma``.  The multiplication then costs
+    nothing per run; the rounding moves from the activations to the weights (one fp16 rounding of ``W gamma``
+    instead of one of the product)."""
     for mul in [o for o in g.ops if o["aten"] in ("mul.Tensor", "div.Tensor") and len(o["in"]) in (1, 2)]:
         const = _scalar_scale(mul)                      # x * c or x / c with a constant: the same fold, gamma = c
         if len(mul["in"]) == 1 and const is None:
@@ -277,18 +278,26 @@ def group_linears(g: Graph) -> Graph:
             continue
         x0, w0, _ = key(first)
         xs = g.buffers[x0]
+
+        def reshaped_root(bid):                          # the root, if only reshapes lie between: then equal shapes mean equal data
+            while g.buffers[bid]["kind"] == "view":
+                if g.buffers[bid].get("op") not in RESHAPES and "getitem" not in g.buffers[bid].get("op", ""):
+                    return None
+                bid = g.buffers[bid]["of"]
+            return bid
         members = []
         for o in g.ops[g.ops.index(first):]:
             if not plain(o) or o["id"] in done:
                 continue
             x, w, b = key(o)
-            same_x = g.root(x) == g.root(x0) and g.buffers[x].get("shape") == xs.get("shape")
+            same_x = x == x0 or (reshaped_root(x) is not None and reshaped_root(x) == reshaped_root(x0) and
+                                 g.buffers[x].get("shape") == xs.get("shape"))
             same_w = g.buffers[w].get("shape") == g.buffers[w0].get("shape") and g.buffers[g.root(w)]["kind"] == "weight"
             if same_x and same_w and (b is None or g.buffers[g.root(b)]["kind"] == "weight") and \
                     g.buffers[o["out"]].get("shape") == g.buffers[first["out"]].get("shape") and o["out"] not in g.outputs:
                 members.append(o)
         # (buffers are written once, so a later member can run where the first one stands: its operands exist there)
-        if len(members) < 2:
+        if len(members) < 2 or members[0] is not first:
             continue
         at = g.ops.index(first)
         spec = []
