@@ -888,6 +888,15 @@ class Executor:
                 "mul.Tensor": _scale, "div.Tensor": _scale, "clone.default": _clone, "clamp.default": _clamp,
                 "linear_group": _linear_group}
 
+    def replayable(self, *inputs: torch.Tensor):
+        """Run once eagerly (binds inputs, sizes the workspace, stacks folded constants), then capture the whole graph as
+        one device graph (the reference's ``Lava.capture/replay``).  Returns ``(replay, outputs)``: ``replay()`` re-runs
+        the captured launches on the same input tensors -- refill them in place -- and ``outputs`` are the tensors it writes."""
+        from .decode import StepGraph
+        outs = self(*inputs)
+        sg = StepGraph(lambda: self(*inputs))
+        return sg.replay, outs
+
     def __call__(self, *inputs: torch.Tensor):
         if len(inputs) != len(self.g.inputs):
             raise ValueError(f"{self.g.name} takes {len(self.g.inputs)} inputs")

@@ -569,3 +569,28 @@ def test_whisper_like_encoder_runs_on_the_kernels(ctx):
     torch.cuda.synchronize()
     assert got.shape == (1, 30, 128)
     assert_parity(got.float().cpu().numpy(), want, what="Whisper-like encoder from its exported graph")
+
+
+@pytest.mark.gpu
+def test_executor_replays_as_one_captured_graph(ctx):
+    """Executor.replayable: the whole op list captured once; replays follow the input tensor's contents and match the
+    eager run every time (several replays with eager work and synchronisations between them)."""
+    import torch
+    from juliavision_amd import graph as G
+    m = _dinov2_like(seed=11)
+    x = torch.rand(1, 3, 70, 70).half().cuda()
+    ep = torch.export.export(m, (x.cpu(),)).run_decompositions()
+    run = G.Executor(G.optimize(G.Graph.load(G.convert(ep, "vit"))), m.state_dict(), ctx)
+    replay, out = run.replayable(x)
+    for seed in (1, 2, 3):
+        torch.manual_seed(seed)
+        x.copy_(torch.rand(1, 3, 70, 70).half())
+        replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = run(x).clone()                       # eager, same tensors
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {seed} differs from the eager run"
+        with torch.no_grad():
+            ref = m.float()(x.float().cpu()).numpy()
+        assert_parity(got.float().cpu().numpy(), ref, what=f"replay {seed}")
