@@ -16,9 +16,10 @@ LIB = os.path.join(HERE, "libmi355dnn.so")
 SOURCES = ["gemm.hip", "sdpa.hip", "conv.hip", "convtranspose.hip", "layernorm.hip", "kvcache.hip", "layout.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
-# -fno-honor-nans: no kernel relies on NaN propagation (infinities stay honoured: they are the masks);
-#   without it every fmaxf operand is first canonicalised with an extra v_max_f32.
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-honor-nans",
+# -Xarch_device -fno-honor-nans: no kernel relies on NaN propagation (infinities stay honoured: they are the masks);
+#   without it every fmaxf operand is first canonicalised with an extra v_max_f32.  Device code only: the host side
+#   checks its arguments with ordinary IEEE comparisons.
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xarch_device", "-fno-honor-nans",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 

@@ -65,6 +65,8 @@ MI_DEVICE half_t ln_norm1(float x, float mu, float r, bool has_g, float g, bool 
 static inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline size_t round_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
+// NaN by its bits: the build tells the compiler that no NaNs occur, which folds comparisons with one away.
+static inline bool is_nan_arg(float x) { uint32_t u; __builtin_memcpy(&u, &x, 4); return (u & 0x7fffffffu) > 0x7f800000u; }
 
 // Implicit-GEMM convolution: how the GEMM finds its [K][N] operand (the im2col matrix) in a
 // zero-padded copy of the input instead of in memory.  The K axis is ordered (kh, kw, ci) with ci

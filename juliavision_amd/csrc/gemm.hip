@@ -1368,7 +1368,7 @@ int mi_gemm_clamp_ln_f16(void *Y, void *H, const void *X, const void *W, const v
                          const void *gamma, const void *beta, float eps, float clamp,
                          int64_t T, int64_t K, int64_t F, int64_t ldX, int64_t ldW,
                          int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream) {
-    if (!(clamp > 0.0f)) return MI_DECLINE_OPERANDS;
+    if (is_nan_arg(clamp) || clamp <= 0.0f) return MI_DECLINE_OPERANDS;
     GemmArgs a;
     int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, F, ldX, ldW, w_layout, bias_mode, epi, MI_F16, 0, 0, 0);
     if (rc != MI_OK) return rc;

@@ -261,7 +261,7 @@ int mi_act_f16(void *out, const void *a, int epi, int64_t n, void *stream) {
 int mi_clamp_f16(void *out, const void *a, float lo, float hi, int64_t n, void *stream) {
     if (!mi_ready()) return MI_ERROR_DEVICE;
     if (!out || !a) return MI_DECLINE_OPERANDS;
-    if (n < 0 || !(lo <= hi)) return MI_DECLINE_EXTENT;
+    if (n < 0 || is_nan_arg(lo) || is_nan_arg(hi) || lo > hi) return MI_DECLINE_EXTENT;
     if (n == 0) return MI_OK;
     hipLaunchKernelGGL(clamp_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, (half_t *)out, (const half_t *)a, lo, hi, (long)n);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;

@@ -368,3 +368,24 @@ def test_clamp_bit_exact(ctx):
     torch.cuda.synchronize()
     want = np.clip(a.astype(np.float32), -64504.0, 64504.0).astype(np.float16)
     assert np.array_equal(to_host(out).view(np.uint16), want.view(np.uint16))
+
+
+def test_rowwise_entry_points_decline_bad_arguments(ctx):
+    """Status codes of the row-wise glue: nothing is launched for a null operand, an empty or negative extent, an
+    unknown activation or an inverted clamp interval."""
+    import torch
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    a = torch.zeros(64, dtype=torch.float16, device="cuda")
+    p, st = a.data_ptr(), ctx.stream
+    assert lib.mi_softmax_f16(None, p, L.F16, 8, 8, 1.0, st) == L.DECLINE_OPERANDS
+    assert lib.mi_softmax_f16(p, p, 7, 8, 8, 1.0, st) == L.DECLINE_OPERANDS          # neither fp16 nor fp32
+    assert lib.mi_softmax_f16(p, p, L.F16, 0, 8, 1.0, st) == L.DECLINE_EXTENT
+    assert lib.mi_softmax_f16(p, p, L.F16, 8, 0, 1.0, st) == L.OK                     # no rows: nothing to do
+    assert lib.mi_scale_f16(p, None, 2.0, 64, st) == L.DECLINE_OPERANDS
+    assert lib.mi_scale_f16(p, p, 2.0, -1, st) == L.DECLINE_EXTENT
+    assert lib.mi_act_f16(p, p, 9, 64, st) == L.DECLINE_UNSUPPORTED
+    assert lib.mi_clamp_f16(p, p, 1.0, -1.0, 64, st) == L.DECLINE_EXTENT
+    assert lib.mi_clamp_f16(p, p, float("nan"), 1.0, 64, st) == L.DECLINE_EXTENT
+    torch.cuda.synchronize()
+    assert bool((a == 0).all())

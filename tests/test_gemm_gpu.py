@@ -268,3 +268,16 @@ def test_matmul_with_clamp_in_the_store_is_the_separate_ops(ctx, T, K, F, with_n
     assert bool(torch.isfinite(y).all()) and torch.equal(y.view(torch.int16), want_y.view(torch.int16))
     if with_norm:
         assert torch.equal(h.view(torch.int16), want_h.view(torch.int16))
+
+
+def test_clamped_gemm_declines_a_clamp_that_is_not_positive(ctx):
+    import torch
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    x = torch.zeros((16, 64), dtype=torch.float16, device="cuda")
+    w = torch.zeros((64, 64), dtype=torch.float16, device="cuda")
+    y = torch.zeros((16, 64), dtype=torch.float16, device="cuda")
+    for bad in (0.0, -1.0, float("nan")):
+        rc = lib.mi_gemm_clamp_ln_f16(y.data_ptr(), None, x.data_ptr(), w.data_ptr(), None, None, None, None, 1e-5, bad,
+                                      16, 64, 64, 64, 64, L.W_KF, L.BIAS_NONE, L.EPI["none"], None, 0, ctx.stream)
+        assert rc == L.DECLINE_OPERANDS
