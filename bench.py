@@ -570,6 +570,60 @@ def encoder_stack_case(nl=4, steps=50):
             "frac_mfma_peak_graph": round(flop * nl / replay / 1e12 / PEAK_F16_TFLOPS, 4)}
 
 
+def vendor_probe():
+    """The same shapes through the libraries this image ships (hipBLASLt / rocBLAS behind torch.addmm and F.linear, the
+    fused attention behind F.scaled_dot_product_attention, MIOpen behind F.conv2d), timed the same way with rotating
+    buffers: context for the figures above, not part of the product path and not a baseline this build is scored on."""
+    import torch
+    import torch.nn.functional as F
+    f16, out = torch.float16, {}
+    r = lambda *sh: torch.randn(sh, dtype=f16, device="cuda")
+
+    def timed(make, n=3, reps=20):
+        fns = [make() for _ in range(n)]
+        state = {"i": 0}
+
+        def fn():
+            fns[state["i"] % n]()
+            state["i"] += 1
+        med, lo, _ = event_time(fn, reps)
+        return round(med * 1e6, 2), round(lo * 1e6, 2)
+
+    def linear_kf():
+        x, w, b = r(1500, 1280) / 36, r(1280, 5120) * 0.02, r(5120) * 0.02
+        y = torch.empty((1500, 5120), dtype=f16, device="cuda")
+        return lambda: torch.addmm(b, x, w, out=y)
+
+    def linear_fk():
+        x, w, b = r(1500, 1280) / 36, r(5120, 1280) * 0.02, r(5120) * 0.02
+        return lambda: F.linear(x, w, b)
+
+    def attn(B, H, Lq, E):
+        def make():
+            q, k, v = r(B, H, Lq, E), r(B, H, Lq, E), r(B, H, Lq, E)
+            return lambda: F.scaled_dot_product_attention(q, k, v)
+        return make
+
+    def conv(channels_last):
+        def make():
+            x, w, b = r(1, 256, 64, 64), r(256, 256, 3, 3) * 0.02, r(256) * 0.02
+            if channels_last:
+                x, w = x.contiguous(memory_format=torch.channels_last), w.contiguous(memory_format=torch.channels_last)
+            return lambda: F.conv2d(x, w, b, padding=1)
+        return make
+
+    for name, make in (("c1_linear_W[K][F]_torch_addmm", linear_kf), ("c1_linear_W[F][K]_torch_linear", linear_fk),
+                       ("c2_attn_L1500_20x64_torch_sdpa", attn(1, 20, 1500, 64)), ("c4_attn_L4096_16x64_torch_sdpa", attn(1, 16, 4096, 64)),
+                       ("sam2_global_attn_L4096_8x72_torch_sdpa", attn(1, 8, 4096, 72)),
+                       ("c4_conv3x3_torch_conv2d_nchw", conv(False)), ("c4_conv3x3_torch_conv2d_channels_last", conv(True))):
+        try:
+            med, lo = timed(make)
+            out[name] = {"us": med, "us_min": lo}
+        except Exception as e:                      # a library that refuses a shape is a result too
+            out[name] = {"error": type(e).__name__}
+    return out
+
+
 def detail_benchmarks(lib, L, stream, only=None):
     import numpy as np
     import torch
@@ -735,6 +789,10 @@ def detail_benchmarks(lib, L, stream, only=None):
     name = "c3_vit_s14_518_from_exported_graph"
     if only is None or only in name:
         out[name] = vit_graph_case()
+
+    name = "vendor_probe_same_shapes_through_torch"
+    if only is None or only in name:
+        out[name] = vendor_probe()
 
     name = "c5_decode_step_4layers_vocab51866_b1"
     if only is None or only in name:
