@@ -428,10 +428,18 @@ def vit_graph_case(steps=50):
     replay = timed(StepGraph(step).replay)
     if not bool(torch.isfinite(run(image)).all()):
         raise RuntimeError("exported ViT produced non-finite output")
+    try:                                              # context: the same module evaluated by torch itself
+        tm = m.cuda()
+        with torch.no_grad():
+            torch_ms = round(timed(lambda: tm(image)) * 1e3, 4)
+            agree = round(float((tm(image).float() - run(image).float()).abs().max() / tm(image).float().abs().max()), 5)
+    except Exception as e:
+        torch_ms, agree = type(e).__name__, None
     T = 1 + (S // P) ** 2
     flop = NL * (2.0 * T * d * (3 * d + d + 8 * d) + 4.0 * T * T * 64 * H) + 2.0 * (T - 1) * 588 * d
     return {"ops_exported": len(spec["ops"]), "ops_after_rewrites": len(g.ops), "export_and_rewrite_host_s": round(host_s, 2),
-            "eager_ms": round(eager * 1e3, 4), "graph_ms": round(replay * 1e3, 4), "TFLOP/s_graph": round(flop / replay / 1e12, 1)}
+            "eager_ms": round(eager * 1e3, 4), "graph_ms": round(replay * 1e3, 4), "TFLOP/s_graph": round(flop / replay / 1e12, 1),
+            "torch_eager_same_module_ms": torch_ms, "max_rel_diff_vs_torch": agree}
 
 
 def whisper_graph_case(nl=32, steps=10):
@@ -514,10 +522,21 @@ def whisper_graph_case(nl=32, steps=10):
     replay = timed(StepGraph(step).replay)
     if not bool(torch.isfinite(run(mel)).all()):
         raise RuntimeError("exported Whisper-like encoder produced non-finite output")
+    # context: the same module with the same weights evaluated by torch itself (vendor kernels, eager dispatch)
+    try:
+        tm = m.to_empty(device="cuda")
+        tm.load_state_dict(weights)
+        with torch.no_grad():
+            torch_ms = round(timed(lambda: tm(mel)) * 1e3, 3)
+            agree = float((tm(mel).float() - run(mel).float()).abs().max() / tm(mel).float().abs().max())
+        del tm
+    except Exception as e:
+        torch_ms, agree = type(e).__name__, None
     T = frames // 2
     flop = nl * (2.0 * T * d * (4 * d + 2 * ffn) + 4.0 * T * T * 64 * heads) + 2.0 * frames * (3 * mels) * d + 2.0 * T * (3 * d) * d
     return {"layers": nl, "ops_exported": len(spec["ops"]), "ops_after_rewrites": len(g.ops), "export_and_rewrite_host_s": round(host_s, 2),
             "eager_ms": round(eager * 1e3, 3), "graph_ms": round(replay * 1e3, 3), "graph_ms_per_layer": round(replay * 1e3 / nl, 4),
+            "torch_eager_same_module_ms": torch_ms, "max_rel_diff_vs_torch": None if agree is None else round(agree, 5),
             "GFLOP": round(flop / 1e9, 1), "TFLOP/s_graph": round(flop / replay / 1e12, 1),
             "frac_mfma_peak_graph": round(flop / replay / 1e12 / PEAK_F16_TFLOPS, 4)}
 
