@@ -302,15 +302,21 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
                     if (key >= Lk) sc[kt][r] = -INFINITY;
                 }
         }
-        // Fast path: exponentiate against the current reference point while the next block's
-        // first product runs underneath.  (After the last block that product multiplies a stale
-        // stage: wasted, harmless, and it keeps this stretch free of branches so that the two
-        // instruction streams can be interleaved: one MFMA, then a handful of vector instructions.)
+        // Fast path: exponentiate against the current reference point.  Without the ping-pong the next block's
+        // first product is issued here as well, to run underneath.  (After the last block that product multiplies a
+        // stale stage: wasted, harmless, and it keeps this stretch free of branches.)  With the ping-pong it moves
+        // behind the second product: a block is then a vector half (the exponentials, ~610 cycles of issue) and a
+        // matrix half (both products, 18 MFMAs = 576 cycles) of about equal length, and the two wave groups, half a
+        // block apart, always want different units -- 90.7 -> 83.5 us on 16 heads x 4096 x 64; with the first product
+        // in the vector half that half was twice as long as the other and set the pace of both.
         __builtin_amdgcn_sched_barrier(0);
-        // The stretch that mixes exponentials with the next block's first product issues ahead of the other wave of
-        // the SIMD, the second product behind it (1-4 % on the measured shapes; the opposite assignment loses 4 %).
-        __builtin_amdgcn_s_setprio(1);
-        qk(sn, st1);
+        // Without the ping-pong the stretch that mixes exponentials with the next block's first product issues ahead
+        // of the other wave of the SIMD, the second product behind it (1-4 % on the measured shapes; the opposite
+        // assignment loses 4 %).  Between the ping-pong's halves priorities change nothing.
+        if constexpr (!PP) {
+            __builtin_amdgcn_s_setprio(1);
+            qk(sn, st1);
+        }
         half8v pf[2][2];
         float l_new = l_run;
         probs(sc, pf, l_new);
@@ -341,7 +347,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) { sc[kt][r] -= d; sn[kt][r] -= d; }   // sn was formed against the old M
+                for (int r = 0; r < 16; r++) { sc[kt][r] -= d; if constexpr (!PP) sn[kt][r] -= d; }   // sn was formed against the old M
 #pragma unroll
             for (int t = 0; t < ET; t++)
 #pragma unroll
@@ -359,7 +365,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
             if (next2) store_kv(st2);
         }
         // O^T += V^T . P^T
-        __builtin_amdgcn_s_setprio(0);
+        if constexpr (!PP) __builtin_amdgcn_s_setprio(0);
         const half_t *vbase = &Vs[st][vtoff];
 #pragma unroll
         for (int t = 0; t < ET; t++) {
@@ -376,6 +382,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
                 }
         }
         if constexpr (PP) {
+            qk(sn, st1);         // the next block's scores, against the reference point as it stands now
             pp_barrier();
         } else {
             if (next2) store_kv(st2);
