@@ -81,7 +81,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 //
 // PP ("ping-pong"): eight waves per workgroup, 256 queries.  Waves w and w+4 share a SIMD and are kept
 // half a key block apart by two workgroup barriers per block, so that while one of them is in its
-// exponentials (with the next block's first product underneath) the other is in its second product:
+// exponentials the other is in its matrix half (the block's second product and the next block's first):
 // the matrix pipe and the vector ALU of a SIMD are then busy with different waves instead of both
 // waves wanting the same unit at the same time.  Waves 0-3 do all the global -> LDS staging.
 //
@@ -89,14 +89,16 @@ __device__ __forceinline__ void static_for(F &&f) {
 // same 32 queries and share a SIMD; a stage holds 128 keys, of which waves 0-3 take the first 64 and waves 4-7 the
 // second, so each wave walks half of the keys and a SIMD always has a second wave to run.  The two partial
 // (O, M, l) of a query meet in LDS at the end (the merge identity of flash.jl:1385-1391), waves 0-3 store.
+// It runs with PP as well: its two key-half groups then take turns like the two query groups above; all waves stage.
 // Halves per V row in LDS: a multiple of 64 plus 32, so that consecutive key rows start 64 bytes apart modulo the
 // 128 bytes of the banks (96 for head sizes 64 and 96, 160 for 128; 112 measured the same as 96 at 96).
 constexpr int flash_vld(int EP) { return EP == 96 ? EP : EP + 32; }
 
 template <int EP, bool PP, int KH = 1>
 __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH == 1) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
-    static_assert(KH == 1 || (KH == 2 && !PP), "key halves or ping-pong, not both");
-    constexpr int BC = 64, BR = PP ? 256 : 128, NT = KH == 2 ? 512 : 256;     // NT: threads that stage K and V
+    // PP with KH = 2: the two key-half groups of the eight-wave form (same 128 queries) take turns at the vector
+    // and matrix units like the two query groups of the 256-query form do; every thread stages.
+    constexpr int BC = 64, BR = (PP && KH == 1) ? 256 : 128, NT = KH == 2 ? 512 : 256;     // NT: threads that stage K and V
     constexpr int BCS = BC * KH;                                                // keys per LDS stage
     constexpr int KLD = EP + 8, VLD = flash_vld(EP);
     constexpr int KS = EP / 16;       // k16 steps over the head dim
@@ -113,7 +115,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     const int grp = wave >> 2;                               // PP, KH = 2: 0 = waves 0-3, 1 = waves 4-7
     const int qw = KH == 2 ? (wave & 3) : wave;              // which 32 queries of the block
     const int gk = KH == 2 ? grp * BC : 0;                   // this wave's first key within a stage
-    const bool loader = !PP || grp == 0;
+    const bool loader = !PP || KH == 2 || grp == 0;
     const int hl = lane >> 5, l32 = lane & 31;
     // Workgroups are dealt to the 8 XCDs round-robin in launch order; renumbering them so that each XCD
     // owns a contiguous run keeps all query blocks of a head on one XCD, whose L2 then holds that head's
@@ -464,7 +466,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         float2v ml = {l_run > 0.0f ? m_ref * 0.6931471805599453f : -INFINITY, l_run};
         *reinterpret_cast<float2v *>(p.part_ml + ((long)split * rows + row) * 2) = ml;
     }
-    if (PP && as_f32) {
+    if (PP && KH == 1 && as_f32) {
         // eight waves of fp32 rows do not fit the operand LDS: this combination stores from the registers
         const int qi = q0 + l32;
         if (qi < p.Lq) {
@@ -944,7 +946,7 @@ int mi_sdpa_init() {
     int bad = 0;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
-    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     return bad;
@@ -1014,7 +1016,8 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
             // (head size 64 only: the 96-wide instance of this variant measured slower than four waves, 115 us
             // against 106 us on 8 heads x 4096 x 72)
             const bool halves = E <= 64 && a.nsplit == 1 && ceil_div(Lq, 128) * H * B <= (int64_t)mi_num_cus() && Lk >= 256;
-            if (halves)       hipLaunchKernelGGL((flash_fwd_kernel<64, false, 2>), grid, dim3(512), 2 * flash_lds_bytes(64), st, a);
+            // (its two key-half groups in ping-pong: 25.1 -> 23.8 us on 20 heads x 1500, 20.1 -> 19.4 us on 6 heads x 1370)
+            if (halves)       hipLaunchKernelGGL((flash_fwd_kernel<64, true, 2>), grid, dim3(512), 2 * flash_lds_bytes(64), st, a);
             else if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false>), grid, dim3(256), flash_lds_bytes(64), st, a);
             else if (E <= 96) hipLaunchKernelGGL((flash_fwd_kernel<96, false>), grid, dim3(256), flash_lds_bytes(96), st, a);
             else         hipLaunchKernelGGL((flash_fwd_kernel<128, false>), grid, dim3(256), flash_lds_bytes(128), st, a);
