@@ -193,6 +193,20 @@ def test_eight_wave_kernel_on_large_grids(ctx):
     _check(ctx, q, k[:, :, :129], v[:, :, :129], out_dtype="f32", expect="FlashPlan", what="8-wave three blocks f32")
 
 
+@pytest.mark.parametrize("B,H,Lq,Lk,E", [(4, 16, 768, 65, 64), (4, 12, 1024, 257, 32), (2, 48, 520, 129, 64),
+                                         (4, 16, 768, 1, 64), (3, 22, 770, 300, 48)])
+def test_eight_wave_kernel_odd_key_counts_and_random_lengths(ctx, B, H, Lq, Lk, E):
+    """The 8-wave variant alternates its two groups between a vector half and a matrix half, the next block's
+    scores being formed one half ahead: key counts that end inside, on and one past a block, a single key, a
+    head size below 64 and per-batch lengths drawn at random (0 and Lk included by the seed) must not show."""
+    q, k, v = _qkv(B, H, Lq, Lk, E, 7000 + Lk, std=1.5)
+    _check(ctx, q, k, v, expect="FlashPlan", what="8-wave odd keys")
+    lens = np.random.default_rng(Lk).integers(0, Lk + 1, size=B)
+    lens[0], lens[-1] = Lk, 0
+    got = _check(ctx, q, k, v, kv_len=[int(x) for x in lens], expect="FlashPlan", what="8-wave random kv_len")
+    assert np.all(got[-1] == 0)
+
+
 def test_fused_kernel_splits_keys_on_small_grids(ctx):
     """Few query blocks and very many keys: the fused kernel also splits the keys over workgroups and a merge joins
     the partials.  Ragged last split, per-batch kv_len that leaves the later split without a key (one row of the
