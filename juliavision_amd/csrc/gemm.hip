@@ -408,12 +408,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
         else       bp[i] = B + (long)(c / CPRB) * p.ldB + min(n0 + (c % CPRB) * 8, p.NB - 8);
     }
     // Implicit GEMM: every chunk of this thread lies in the same eight columns (NT is a multiple of
-    // CPRB), i.e. at one pixel offset, in channels 16 apart; which tap and which 64 channels a tile
+    // CPRB), i.e. at one pixel offset, in channels NT / CPRB apart; which tap and which 64 channels a tile
     // covers is the same for the whole workgroup.
     const half_t *cpix = nullptr;
     int ctile0 = 0;
     if constexpr (CONV) {
-        static_assert(NT % CPRB == 0 && NT / CPRB == 16, "a thread's chunks share their columns, 16 rows apart");
+        static_assert(NT % CPRB == 0 && PB * (NT / CPRB) == BK, "a thread's chunks share their columns, NT / CPRB rows apart");
         const int ncol = min(n0 + (tid % CPRB) * 8, p.NB - 8);
         const int oh = ncol / p.cv.OW, ow = ncol % p.cv.OW;
         cpix = p.cv.xp + (p.cv.split ? 0 : bz * p.cv.img) + (long)oh * p.cv.sy * p.cv.Wp + ow + (long)(tid / CPRB) * p.cv.HpWp;
@@ -462,7 +462,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
                 // The eight halves start kw*dx elements into an aligned row, i.e. at a 2-byte boundary, and
                 // vector loads want 4-byte alignment: odd starts are read from the second copy of the padded
                 // input, which is the first shifted by one element (the choice is the same for every lane).
-                const uint32_t *src = reinterpret_cast<const uint32_t *>(cpix + toff + ((toff & 1) ? p.cv.odd : 0L) + (long)i * 16 * p.cv.HpWp);
+                const uint32_t *src = reinterpret_cast<const uint32_t *>(cpix + toff + ((toff & 1) ? p.cv.odd : 0L) + (long)i * (NT / CPRB) * p.cv.HpWp);
                 uint32_t w4[4];
                 __builtin_memcpy(w4, src, 16);
 #pragma unroll
@@ -1080,7 +1080,7 @@ int launch_mfma(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
 
 // K-slices for a GEMM whose 128 x 128 output tiles number fewer than the CUs: as many as fit two
 // workgroups per CU, each slice a multiple of 64 and deep enough; N must allow 4-wide rows.
-int splitk_count(int64_t M, int64_t N, int64_t K) {
+int splitk_count(int64_t M, int64_t N, int64_t K, bool gathered = false) {
     if (M <= 8 || N % 4 || K % 64) return 1;
     const int64_t tiles = ceil_div(M, 128) * ceil_div(N, 128);
     if (ceil_div(M, 128) * ceil_div(N, 256) >= (g_cus * 3) / 4 || tiles * 2 > g_cus) return 1;
@@ -1090,6 +1090,11 @@ int splitk_count(int64_t M, int64_t N, int64_t K) {
     // the tiles would otherwise leave three quarters of the chip idle.
     const int64_t kmin = tiles * 4 <= g_cus ? 512 : 1024;
     while (s > 1 && (K % (s * 64) != 0 || K / s < kmin)) s--;
+    // Few tiles (and no gathered operand, which only the 128-wide tiles take): unsplit they run on the 64 x 64 tile, one per CU whatever their number, about 0.28 us per 64 of K
+    // after 3.5 us of launch and prologue; split, the 128 x 128 tile takes 0.47 us per 64 of a slice, and the fp32
+    // planes with the second launch that sums them about 11 us (1370 x 1536 -> 384: 9.4 us unsplit, 14.1 us in
+    // three slices; 300 x 5120 -> 1280: 24.8 us unsplit, 17.4 us in eight).
+    if (s > 1 && !gathered && tiles < (g_cus * 3) / 8 && 350 + 28 * (K / 64) <= 1100 + 47 * (K / (s * 64))) return 1;
     return (int)s;
 }
 
@@ -1180,7 +1185,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         // Split K over workgroups when the output alone cannot fill the chip: each K-slice is one plane
         // of a batched launch (plane strides: A advances along k, Y one fp32 M x N plane in ws), and a
         // second small kernel sums the planes and applies bias, activation and residual.
-        const int split = nbatch == 1 ? splitk_count(a.M, a.N, a.K) : 1;
+        const int split = nbatch == 1 ? splitk_count(a.M, a.N, a.K, a.cv.xp || a.ag.x) : 1;
         if (split > 1 && ws && aligned_to(ws, 256) && ws_bytes >= (size_t)split * a.M * a.N * sizeof(float)) {
             GemmArgs s1 = a;
             s1.Y = ws; s1.out_f32 = 1; s1.bias = nullptr; s1.bias_mode = MI_BIAS_NONE; s1.epi = MI_EPI_NONE; s1.residual = nullptr; s1.clamp = 0.0f;
@@ -1191,7 +1196,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
             s1.ag.split = 1;
             // the 128 x 256 tile (two waves per SIMD) when the slices still give most CUs a workgroup
             const bool big_tiles = ceil_div(a.M, 128) * ceil_div(a.N, 256) * split >= (g_cus * 3) / 4;
-            int rc = big_tiles ? launch_pipe<128, 256, 2, 4>(s1, b_kn, split, st) : launch_pipe<128, 128, 2, 2>(s1, b_kn, split, st);
+            int rc = big_tiles ? launch_pipe<128, 256, 2, 4>(s1, b_kn, split, st) : launch_pipe<128, 128, 2, 4>(s1, b_kn, split, st);
             if (rc != MI_OK) return rc;
             GemmArgs s2 = a;
             s2.vec_store = !a.out_f32 && a.ldY % 4 == 0 && aligned_to(a.Y, 8);
@@ -1218,8 +1223,8 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
         if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
         if (big * 2 > g_cus) return pipe ? launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
-        if (mid >= (g_cus * 3) / 8 || a.cv.xp || a.ag.x) return pipe ? launch_pipe<128, 128, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
-        return launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
+        if (mid >= (g_cus * 3) / 8 || a.cv.xp || a.ag.x) return pipe ? launch_pipe<128, 128, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
+        return pipe ? launch_pipe<64, 64, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
     }
     long total = (long)a.M * a.N;
     hipLaunchKernelGGL(gemm_scalar_kernel, dim3((unsigned)ceil_div(total, 256), (unsigned)nbatch), dim3(256), 0, st, a, b_kn ? 1 : 0);
@@ -1230,6 +1235,14 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
 
 bool mi_ready() { return g_ready; }
 int mi_num_cus() { return g_cus; }
+
+// Split-K planes of a GEMM one of whose operands the kernel gathers (implicit convolution): mi_gemm_f16_workspace
+// for the launches that conv.hip makes through mi_internal_gemm with a gather descriptor.
+size_t mi_internal_gemm_gathered_workspace(int64_t T, int64_t K, int64_t F, int64_t nbatch) {
+    if (T <= 8 || nbatch > 1) return 0;
+    const int split = splitk_count(T, F, K, true);
+    return split > 1 ? round_up((size_t)split * T * F * sizeof(float), 256) : 0;
+}
 
 // Internal entry used by the convolution path (conv.hip): Y[M x N] = A . B with
 // every GemmArgs field meaningful.
@@ -1275,14 +1288,14 @@ int mi_init(void) {
     bad |= raise_lds(gemm_mfma_kernel<GEMM_SMALL, false>, gemm_lds_bytes<64, 64, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, true>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, false>, gemm_lds_bytes<128, 256, 64>());
-    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, true>, gemm_lds_bytes<128, 128, 64>());
-    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, false>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, true>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, false>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 2>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 0, 1>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 1, 1>, gemm_lds_bytes<128, 256, 64>());
-    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, 0, 1>, gemm_lds_bytes<128, 128, 64>());
-    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, 1, 1>, gemm_lds_bytes<128, 128, 64>());
-    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 2, 2>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 0, 1>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 1, 1>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 2>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(skinny_fk_kernel<1>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<2>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<4>, (int)SKINNY_FK_LDS_MAX);
