@@ -1086,6 +1086,9 @@ int splitk_count(int64_t M, int64_t N, int64_t K, bool gathered = false) {
     if (ceil_div(M, 128) * ceil_div(N, 256) >= (g_cus * 3) / 4 || tiles * 2 > g_cus) return 1;
     int64_t s = (2 * (int64_t)g_cus) / tiles;
     if (s > 8) s = 8;
+    // More than a quarter of the CUs in tiles: two slices of 128 x 128 tiles rather than four of 128 x 256, half the
+    // fp32 planes to write and read back (1500 x 5120 -> 1280: 35.0-35.9 us against 36.2-39.6 us).
+    if (tiles * 4 > g_cus && s > 2) s = 2;
     // A slice must be deep enough to pay for the second pass over the output: 1024, or 512 when
     // the tiles would otherwise leave three quarters of the chip idle.
     const int64_t kmin = tiles * 4 <= g_cus ? 512 : 1024;
@@ -1223,6 +1226,10 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
         if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
         if (big * 2 > g_cus) return pipe ? launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
+        // Between the two, 64 x 128 tiles of eight waves (32 x 32 each): twice the workgroups, two to a CU, each a shorter
+        // chain of prologue, K loop and store (1500 x 1280 x 1280: 11.8 us against 14.2 us on 128 x 128 tiles of eight
+        // waves and 16.3 us on 128 x 128 tiles of four).  Gathered operands stay on the 128 x 128 tile.
+        if (mid >= (g_cus * 3) / 8 && !a.cv.xp && !a.ag.x && pipe) return launch_pipe<64, 128, 2, 4>(a, b_kn, nbatch, st);
         if (mid >= (g_cus * 3) / 8 || a.cv.xp || a.ag.x) return pipe ? launch_pipe<128, 128, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
         return pipe ? launch_pipe<64, 64, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
     }
@@ -1290,6 +1297,8 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, false>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, true>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, false>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 1>, gemm_lds_bytes<64, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 0>, gemm_lds_bytes<64, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 2>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 0, 1>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 1, 1>, gemm_lds_bytes<128, 256, 64>());
