@@ -104,6 +104,3 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
                      long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st,
                      const ConvGather *gather = nullptr, const NhwcGather *agather = nullptr);
-// Workspace bytes of such a call when a gather descriptor is passed (the split-K decision differs: gathered
-// operands only run on the 128-wide tiles); without one, mi_gemm_f16_workspace.
-size_t mi_internal_gemm_gathered_workspace(int64_t T, int64_t K, int64_t F, int64_t nbatch);

@@ -1080,7 +1080,7 @@ int launch_mfma(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
 
 // K-slices for a GEMM whose 128 x 128 output tiles number fewer than the CUs: as many as fit two
 // workgroups per CU, each slice a multiple of 64 and deep enough; N must allow 4-wide rows.
-int splitk_count(int64_t M, int64_t N, int64_t K, bool gathered = false) {
+int splitk_count(int64_t M, int64_t N, int64_t K) {
     if (M <= 8 || N % 4 || K % 64) return 1;
     const int64_t tiles = ceil_div(M, 128) * ceil_div(N, 128);
     if (ceil_div(M, 128) * ceil_div(N, 256) >= (g_cus * 3) / 4 || tiles * 2 > g_cus) return 1;
@@ -1093,11 +1093,11 @@ int splitk_count(int64_t M, int64_t N, int64_t K, bool gathered = false) {
     // the tiles would otherwise leave three quarters of the chip idle.
     const int64_t kmin = tiles * 4 <= g_cus ? 512 : 1024;
     while (s > 1 && (K % (s * 64) != 0 || K / s < kmin)) s--;
-    // Few tiles (and no gathered operand, which only the 128-wide tiles take): unsplit they run on the 64 x 64 tile, one per CU whatever their number, about 0.28 us per 64 of K
+    // Few tiles: unsplit they run on the 64 x 64 tile, one per CU whatever their number, about 0.28 us per 64 of K
     // after 3.5 us of launch and prologue; split, the 128 x 128 tile takes 0.47 us per 64 of a slice, and the fp32
     // planes with the second launch that sums them about 11 us (1370 x 1536 -> 384: 9.4 us unsplit, 14.1 us in
     // three slices; 300 x 5120 -> 1280: 24.8 us unsplit, 17.4 us in eight).
-    if (s > 1 && !gathered && tiles < (g_cus * 3) / 8 && 350 + 28 * (K / 64) <= 1100 + 47 * (K / (s * 64))) return 1;
+    if (s > 1 && tiles < (g_cus * 3) / 8 && 350 + 28 * (K / 64) <= 1100 + 47 * (K / (s * 64))) return 1;
     return (int)s;
 }
 
@@ -1188,7 +1188,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         // Split K over workgroups when the output alone cannot fill the chip: each K-slice is one plane
         // of a batched launch (plane strides: A advances along k, Y one fp32 M x N plane in ws), and a
         // second small kernel sums the planes and applies bias, activation and residual.
-        const int split = nbatch == 1 ? splitk_count(a.M, a.N, a.K, a.cv.xp || a.ag.x) : 1;
+        const int split = nbatch == 1 ? splitk_count(a.M, a.N, a.K) : 1;
         if (split > 1 && ws && aligned_to(ws, 256) && ws_bytes >= (size_t)split * a.M * a.N * sizeof(float)) {
             GemmArgs s1 = a;
             s1.Y = ws; s1.out_f32 = 1; s1.bias = nullptr; s1.bias_mode = MI_BIAS_NONE; s1.epi = MI_EPI_NONE; s1.residual = nullptr; s1.clamp = 0.0f;
@@ -1225,12 +1225,14 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         int64_t mid = ceil_div(a.M, 128) * ceil_div(a.N, 128) * nbatch;
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
         if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
+        // At most 64 columns: half of a 128-wide tile would multiply padding.
+        if (a.N <= 64 && pipe) return launch_pipe<64, 64, 2, 2>(a, b_kn, nbatch, st);
         if (big * 2 > g_cus) return pipe ? launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
         // Between the two, 64 x 128 tiles of eight waves (32 x 32 each): twice the workgroups, two to a CU, each a shorter
         // chain of prologue, K loop and store (1500 x 1280 x 1280: 11.8 us against 14.2 us on 128 x 128 tiles of eight
-        // waves and 16.3 us on 128 x 128 tiles of four).  Gathered operands stay on the 128 x 128 tile.
+        // waves and 16.3 us on 128 x 128 tiles of four).  Gathered operands take the 128 x 128 tile here.
         if (mid >= (g_cus * 3) / 8 && !a.cv.xp && !a.ag.x && pipe) return launch_pipe<64, 128, 2, 4>(a, b_kn, nbatch, st);
-        if (mid >= (g_cus * 3) / 8 || a.cv.xp || a.ag.x) return pipe ? launch_pipe<128, 128, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
+        if (mid >= (g_cus * 3) / 8) return pipe ? launch_pipe<128, 128, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
         return pipe ? launch_pipe<64, 64, 2, 2>(a, b_kn, nbatch, st) : launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
     }
     long total = (long)a.M * a.N;
@@ -1242,14 +1244,6 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
 
 bool mi_ready() { return g_ready; }
 int mi_num_cus() { return g_cus; }
-
-// Split-K planes of a GEMM one of whose operands the kernel gathers (implicit convolution): mi_gemm_f16_workspace
-// for the launches that conv.hip makes through mi_internal_gemm with a gather descriptor.
-size_t mi_internal_gemm_gathered_workspace(int64_t T, int64_t K, int64_t F, int64_t nbatch) {
-    if (T <= 8 || nbatch > 1) return 0;
-    const int split = splitk_count(T, F, K, true);
-    return split > 1 ? round_up((size_t)split * T * F * sizeof(float), 256) : 0;
-}
 
 // Internal entry used by the convolution path (conv.hip): Y[M x N] = A . B with
 // every GemmArgs field meaningful.

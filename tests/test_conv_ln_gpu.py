@@ -51,6 +51,7 @@ def test_conv_im2col(ctx, N, Cin, H, W, Cout, K, s, p):
     (1, 64, 18, 16, 48, 3, 1, (1, 2), (0, 1), 1, {}),              # 3 rows x 1 column, stride 2 along y, no x padding
     (1, 192, 12, 32, 32, 1, 3, 1, (1, 0), 1, {}),                  # KH = 1, KW = 3
     (3, 64, 9, 10, 40, 3, 3, 1, (0, 2), 1, {"relu": True}),        # OW = 8 without x padding, three images
+    (1, 512, 32, 32, 128, 3, 3, 1, 1, 1, {"relu": True}),          # K = 4608 over eight output tiles: split into fp32 planes
 ])
 def test_conv_implicit_gemm(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, kw):
     _conv(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, expect="implicit_gemm", **kw)
@@ -118,13 +119,14 @@ def _conv_nhwc(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d=1, bias=True, relu=False
     (1, 128, 8, 8, 64, 1, 1, 1, 0, 1, {}),                         # 1x1: the gather degenerates to a plain row-major operand
     (1, 192, 12, 32, 32, 1, 3, 1, (1, 0), 1, {}),                  # KH = 1, KW = 3, three runs per tap
     (5, 64, 3, 3, 8, 3, 3, 1, 0, 1, {}),                           # one output pixel per image, M = 5
+    (1, 512, 32, 32, 128, 3, 3, 1, 1, 1, {"relu": True}),          # K = 4608 over eight output tiles: split into fp32 planes
 ])
 def test_conv_nhwc(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, kw):
     _conv_nhwc(ctx, N, Cin, H, W, Cout, KH, KW, s, p, d, **kw)
 
 
 def test_conv_nhwc_config4_is_the_nchw_result(ctx):
-    """3x3 256->256 on 64x64 at full size (M=4096, K=2304, N=256, split over K): the oracle checks 16 output channels,
+    """3x3 256->256 on 64x64 at full size (M=4096, K=2304, N=256): the oracle checks 16 output channels,
     the reference-layout path checks the rest (same products, summed in a different order: fp16 rounding apart)."""
     import torch
     import juliavision_amd as jv
