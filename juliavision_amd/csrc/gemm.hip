@@ -1227,6 +1227,12 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
         // At most 64 columns: half of a 128-wide tile would multiply padding.
         if (a.N <= 64 && pipe) return launch_pipe<64, 64, 2, 2>(a, b_kn, nbatch, st);
+        // Big tiles on half to three quarters of the CUs: 192 x 128 tiles (eight waves of 96 x 32) when they put more
+        // workgroups on the chip and still at most one per CU -- the three batched 1500 x 1280 x 1280 projections on 240
+        // workgroups instead of 180: 21.4 us against 24.3 us.
+        const int64_t t192 = ceil_div(a.M, 192) * ceil_div(a.N, 128) * nbatch;
+        if (pipe && !a.cv.xp && !a.ag.x && big * 2 > g_cus && big * 4 < g_cus * 3 && t192 > big && t192 <= g_cus)
+            return launch_pipe<192, 128, 2, 4>(a, b_kn, nbatch, st);
         if (big * 2 > g_cus) return pipe ? launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st) : launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
         // Between the two, 64 x 128 tiles of eight waves (32 x 32 each): twice the workgroups, two to a CU, each a shorter
         // chain of prologue, K loop and store (1500 x 1280 x 1280: 11.8 us against 14.2 us on 128 x 128 tiles of eight
@@ -1293,6 +1299,8 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, false>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 1>, gemm_lds_bytes<64, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 0>, gemm_lds_bytes<64, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<192, 128, 2, 4, 1>, gemm_lds_bytes<192, 128, 64>());
+    bad |= raise_lds(gemm_pipe_kernel<192, 128, 2, 4, 0>, gemm_lds_bytes<192, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 2>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 0, 1>, gemm_lds_bytes<128, 256, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 256, 2, 4, 1, 1>, gemm_lds_bytes<128, 256, 64>());

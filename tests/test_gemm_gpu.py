@@ -143,6 +143,18 @@ def test_batched_shared_activations_with_per_plane_bias(ctx):
 
 
 @pytest.mark.parametrize("layout", ["kf", "fk"])
+def test_tile_shapes_between_the_big_and_the_small_tile(ctx, layout):
+    """The tile is chosen from the grid it gives: 192 x 128 where 128 x 256 tiles would cover half to three quarters
+    of the CUs (ragged last row and column tiles), 64 x 128 on mid-sized outputs, 64 x 64 on few tiles and on
+    outputs of at most 64 columns."""
+    _run(ctx, 1500, 128, 3000, layout=layout, epi="gelu", residual=True, seed=31)      # 144 big tiles -> 8 x 24 of 192 x 128
+    _run(ctx, 1500, 192, 1288, layout=layout, residual=True, seed=32)                  # 132 tiles of 128 x 128 -> 24 x 11 of 64 x 128
+    _run(ctx, 700, 256, 392, layout=layout, epi="relu", seed=33)                       # 24 tiles -> 11 x 7 of 64 x 64
+    _run(ctx, 20000, 128, 64, layout=layout, seed=34)                                  # 64 columns: 64 x 64 tiles, not half-empty 128-wide ones
+    _run(ctx, 3000, 128, 40, layout=layout, out_f32=True, seed=35)
+
+
+@pytest.mark.parametrize("layout", ["kf", "fk"])
 def test_split_k_narrow_outputs(ctx, layout):
     """Few output tiles and a deep K: the library splits K over workgroups (fp32 planes in the workspace,
     summed by a second kernel that applies bias, activation and residual)."""
