@@ -104,3 +104,5 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
                      long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st,
                      const ConvGather *gather = nullptr, const NhwcGather *agather = nullptr);
+// Workspace bytes such a call needs (fp32 planes when it splits K); T > 8 rows.
+size_t mi_internal_gemm_workspace(int64_t T, int64_t K, int64_t F, int64_t nbatch);

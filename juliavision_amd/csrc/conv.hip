@@ -204,14 +204,14 @@ size_t mi_conv2d_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, i
         int Hp, Wp;
         padded_extents(a, Hp, Wp);
         return 2 * round_up((size_t)N * Cin * Hp * Wp * 2, 256) + round_up((size_t)Cout * Cin * KH * KW * 2, 256) +
-               mi_gemm_f16_workspace(Cout, Cin * KH * KW, (int64_t)a.OW * a.OH, MI_W_KF, N);
+               mi_internal_gemm_workspace(Cout, Cin * KH * KW, (int64_t)a.OW * a.OH, N);
     }
     if (conv_path(a) != MI_CONV_IM2COL_GEMM) return 0;
     int64_t PQP, CRSP;
     im2col_extents(a, PQP, CRSP);
     size_t col = round_up((size_t)N * PQP * CRSP * 2, 256);
     size_t wp = CRSP != (int64_t)Cin * KH * KW ? round_up((size_t)Cout * CRSP * 2, 256) : 0;
-    return col + wp + mi_gemm_f16_workspace(Cout, CRSP, (int64_t)a.OW * a.OH, MI_W_KF, N);
+    return col + wp + mi_internal_gemm_workspace(Cout, CRSP, (int64_t)a.OW * a.OH, N);
 }
 
 int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
@@ -245,7 +245,7 @@ int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
         const int CRS = a.Cin * a.KH * a.KW;
         const size_t xp1 = round_up((size_t)a.N * a.Cin * Hp * Wp * 2, 256), xp_bytes = 2 * xp1;     // the copy and its shifted twin
         const size_t w2_bytes = round_up((size_t)a.Cout * CRS * 2, 256);
-        const size_t gemm_bytes = mi_gemm_f16_workspace(a.Cout, CRS, PQ, MI_W_KF, a.N);
+        const size_t gemm_bytes = mi_internal_gemm_workspace(a.Cout, CRS, PQ, a.N);
         if (!ws || ws_bytes < xp_bytes + w2_bytes + gemm_bytes || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
         if ((long)a.Cin * Hp * Wp > INT32_MAX || (long)a.Cout * CRS > INT32_MAX) return MI_DECLINE_EXTENT;
         half_t *xp = reinterpret_cast<half_t *>(ws);
@@ -265,7 +265,7 @@ int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
     const int CRS = a.Cin * a.KH * a.KW;
     size_t col_bytes = round_up((size_t)N * PQP * CRSP * 2, 256);
     size_t wp_bytes = CRSP != CRS ? round_up((size_t)Cout * CRSP * 2, 256) : 0;
-    const size_t gemm_bytes = mi_gemm_f16_workspace(Cout, CRSP, PQ, MI_W_KF, N);
+    const size_t gemm_bytes = mi_internal_gemm_workspace(Cout, CRSP, PQ, N);
     if (!ws || ws_bytes < col_bytes + wp_bytes + gemm_bytes || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
     if (PQP * CRSP > INT32_MAX) return MI_DECLINE_EXTENT;
     half_t *col = reinterpret_cast<half_t *>(ws);
@@ -289,7 +289,7 @@ size_t mi_conv2d_nhwc_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t
                                     int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy) {
     ConvArgs a;
     if (fill(a, nullptr, nullptr, nullptr, nullptr, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, 1, MI_EPI_NONE) != MI_OK) return 0;
-    return mi_gemm_f16_workspace((int64_t)N * a.OH * a.OW, Cin * KH * KW, Cout, MI_W_FK, 1);
+    return mi_internal_gemm_workspace((int64_t)N * a.OH * a.OW, Cin * KH * KW, Cout, 1);
 }
 
 int mi_conv2d_nhwc_f16(void *out, const void *x, const void *w, const void *bias,

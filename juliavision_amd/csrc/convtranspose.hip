@@ -142,7 +142,7 @@ CtScratch scratch_of(const CtArgs &a) {
     s.w2 = round_up((size_t)M * a.Cin * 2, 256);
     s.bias2 = round_up((size_t)M * 2, 256);
     s.y = round_up((size_t)a.N * M * HW * 2, 256);
-    s.gemm = mi_gemm_f16_workspace(M, a.Cin, HW, MI_W_KF, a.N);
+    s.gemm = mi_internal_gemm_workspace(M, a.Cin, HW, a.N);
     return s;
 }
 

@@ -119,11 +119,12 @@ def test_conv_planner_and_extents():
     assert lib.mi_convsize(518, 14, 14, 0, 1) == 37 and lib.mi_convsize(256, 7, 4, 3, 1) == 64
     # implicit GEMM scratch: the zero-padded input [Cin][H+2][W+2 -> 72] fp16 twice (the second copy shifted by one
     # element, for taps that start at an odd column), the weights re-laid tap-major; K = 2304 is shallow enough for
-    # one pass of 64 x 64 tiles, K = 9216 is split into eight fp32 planes of the 256 x 4096 output
+    # one pass of 64 x 64 tiles, K = 9216 is split into fp32 planes of the 256 x 4096 output
     ws = lib.mi_conv2d_f16_workspace(64, 64, 256, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
     assert ws == 2 * 256 * 66 * 72 * 2 + 256 * 2304 * 2
     ws = lib.mi_conv2d_f16_workspace(64, 64, 1024, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
-    assert ws == 2 * 1024 * 66 * 72 * 2 + 256 * 9216 * 2 + 8 * 256 * 4096 * 4
+    planes = ws - (2 * 1024 * 66 * 72 * 2 + 256 * 9216 * 2)
+    assert planes >= 2 * 256 * 4096 * 4 and planes % (256 * 4096 * 4) == 0
     # im2col scratch: col[CRS->8][PQ->8] fp16 (+ padded weights when CRS % 8 != 0)
     ws3 = lib.mi_conv2d_f16_workspace(518, 518, 3, 1, 14, 14, 384, 14, 14, 0, 0, 1, 1)
     assert ws3 == -(-(592 * 1376 * 2) // 256) * 256 + 384 * 592 * 2

@@ -161,8 +161,10 @@ def test_split_k_narrow_outputs(ctx, layout):
     from juliavision_amd import _lib as L
     lib = L.load()
     assert lib.mi_gemm_f16_workspace(1500, 5120, 1280, L.W_KF, 1) >= 2 * 1500 * 1280 * 4
-    assert lib.mi_gemm_f16_workspace(200, 4096, 256, L.W_KF, 1) == 8 * 200 * 256 * 4
-    assert lib.mi_gemm_f16_workspace(200, 2048, 256, L.W_KF, 1) == 0     # shallow enough for one pass of 64 x 64 tiles
+    ws = lib.mi_gemm_f16_workspace(200, 4096, 256, L.W_KF, 1)
+    assert ws >= 2 * 200 * 256 * 4 and ws % (200 * 256 * 4) == 0         # whole fp32 planes of the output
+    assert lib.mi_gemm_f16_workspace(200, 128, 256, L.W_KF, 1) == 0      # two 64-deep steps: nothing to split
+    assert lib.mi_gemm_f16_workspace(1370, 1536, 384, L.W_KF, 1) == 0    # one pass of 64 x 64 tiles is cheaper than planes
     _run(ctx, 200, 4096, 256, layout=layout, epi="gelu", residual=True)
     _run(ctx, 200, 4096, 256, layout=layout, out_f32=True)
     _run(ctx, 200, 2048, 256, layout=layout, epi="gelu", residual=True)
