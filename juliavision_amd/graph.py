@@ -231,6 +231,8 @@ def fold_layerscale(g: Graph) -> Graph:
         const = _scalar_scale(mul)                      # x * c or x / c with a constant: the same fold, gamma = c
         if len(mul["in"]) == 1 and const is None:
             continue
+        if const is None and mul["aten"] != "mul.Tensor":
+            continue                                    # y / gamma and gamma / y are not a multiplication by gamma: left as written
         for mine, other in ((mul["in"][0], None),) if const is not None else (mul["in"], mul["in"][::-1]):
             gb = g.buffers[g.root(other)] if other is not None else None
             chain = [mine]

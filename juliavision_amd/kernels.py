@@ -135,6 +135,33 @@ def _is_f16_cuda(*ts) -> bool:
     return all(isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float16 for t in ts)
 
 
+def _vec_problem(name: str, t, n: int, dtype=torch.float16, *, require_cuda: bool = True) -> Optional[str]:
+    """Why a small per-feature / per-row operand (bias, gamma, beta, mean, rstd) cannot be handed to a kernel as a raw
+    pointer, or None if it can: the kernels read exactly ``n`` contiguous elements of ``dtype`` from it, so a shorter,
+    strided or differently typed tensor would be an out-of-bounds or misinterpreted device read."""
+    if t is None:
+        return None
+    if not isinstance(t, torch.Tensor):
+        return f"{name} is not a tensor"
+    if require_cuda and not t.is_cuda:
+        return f"{name} is not on the GPU"
+    if t.dtype != dtype:
+        return f"{name} is {t.dtype}, the kernel reads {dtype}"
+    if t.numel() != n:
+        return f"{name} has {t.numel()} elements, the kernel reads {n}"
+    if not t.is_contiguous():
+        return f"{name} is not contiguous"
+    return None
+
+
+def _check_vecs(what: str, status: int, *specs):
+    """specs: (name, tensor, n[, dtype]); raises DeclineError naming the first operand a kernel could not read."""
+    for spec in specs:
+        why = _vec_problem(*spec)
+        if why is not None:
+            raise DeclineError(f"{what}: {why}", status)
+
+
 def _dtype_code(t: torch.Tensor) -> int:
     if t.dtype == torch.float16:
         return L.F16
@@ -186,8 +213,8 @@ def mmplan(dev: DeviceCaps, out, A, B, bias=None):
     T = B.shape[0]
     if B.shape[1] != K or tuple(out.shape) != (T, F):
         return Decline("extent")
-    if bias is not None and not (bias.dim() == 1 and bias.numel() in (F, T)):
-        return Decline("bias")
+    if bias is not None and not (bias.dim() == 1 and bias.numel() in (F, T) and _vec_problem("bias", bias, bias.numel()) is None):
+        return Decline("bias")                          # e.g. an fp32 bias of a mixed-precision export: not read as fp16
     if not dev.coopmat:
         return Decline("nocoopmat")
     w_layout = L.W_KF if la[0] == 0 else L.W_FK
@@ -218,6 +245,8 @@ def _matmul_run(ctx, plan, out, A, B, bias, epi, residual, bias_mode):
         bm = {"col": L.BIAS_COL, "row": L.BIAS_ROW}[bias_mode]
     else:
         bm = L.BIAS_COL if bias.numel() == F else L.BIAS_ROW
+    if bias is not None and bias.numel() != (F if bm == L.BIAS_COL else T):
+        raise DeclineError("matmul_: bias length does not match its mode (col: F values, row: T values)", L.DECLINE_BIAS)
     if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
         raise DeclineError("matmul_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
     need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1)
@@ -250,6 +279,7 @@ def matmul_ln_(ctx: Ctx, out, normed, A, B, gamma, beta, eps, bias=None, *, epi=
         raise DeclineError("matmul_ln_: out and normed must be dense fp16 (T,F)", L.DECLINE_OPERANDS)
     if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
         raise DeclineError("matmul_ln_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
+    _check_vecs("matmul_ln_", L.DECLINE_OPERANDS, ("gamma", gamma, F), ("beta", beta, F))
     bm = L.BIAS_NONE if bias is None else (L.BIAS_COL if bias.numel() == F else L.BIAS_ROW)
     need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1)
     ws = ctx.ws.scratch(need)
@@ -279,6 +309,9 @@ def ln_matmul_(ctx: Ctx, out, A, B, gamma, beta, eps, bias=None, *, epi="none", 
     la, lb, lo = _mat2(A), _mat2(B), _mat2(out)
     if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
         raise DeclineError("ln_matmul_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
+    _check_vecs("ln_matmul_", L.DECLINE_OPERANDS, ("gamma", gamma, K), ("beta", beta, K))
+    if bias is not None and bias.numel() != F:
+        raise DeclineError("ln_matmul_: bias must have one value per output feature", L.DECLINE_BIAS)
     need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1)
     ws = ctx.ws.scratch(need)
     rc = lib.mi_ln_gemv_f16(out.data_ptr(), B.data_ptr(), _ptr(gamma), _ptr(beta), float(eps), A.data_ptr(), _ptr(bias), _ptr(residual),
@@ -602,7 +635,11 @@ def layernorm_(ctx: Ctx, out, mean, rstd, a, gamma, beta, C_: int, eps: float):
     lib = L.init()
     if not _is_f16_cuda(a, out) or not a.is_contiguous() or not out.is_contiguous():
         raise DeclineError("layernorm_: operands", L.DECLINE_OPERANDS)
+    if C_ < 1 or a.numel() % C_ or out.shape != a.shape:
+        raise DeclineError("layernorm_: the normalised extent must divide the operand, out must have a's shape", L.DECLINE_EXTENT)
     groups = a.numel() // C_
+    _check_vecs("layernorm_", L.DECLINE_OPERANDS, ("gamma", gamma, C_), ("beta", beta, C_),
+                ("mean", mean, groups, torch.float32), ("rstd", rstd, groups, torch.float32))
     rc = lib.mi_layernorm_f16(out.data_ptr(), _ptr(mean), _ptr(rstd), a.data_ptr(), _ptr(gamma), _ptr(beta),
                               C_, groups, float(eps), ctx.stream)
     if rc != L.OK:
@@ -662,6 +699,10 @@ def add_(ctx: Ctx, out, a, b):
     lib = L.init()
     if not _is_f16_cuda(a, b, out) or not (a.is_contiguous() and b.is_contiguous() and out.is_contiguous()):
         raise DeclineError("add_: operands", L.DECLINE_OPERANDS)
+    drop1 = lambda t: [d for d in t.shape if d != 1]       # (1, T, D) + (T, D) are the same elements
+    if not (drop1(a) == drop1(b) == drop1(out)):
+        raise DeclineError(f"add_: shapes differ ({tuple(a.shape)}, {tuple(b.shape)}, {tuple(out.shape)}); nothing is broadcast",
+                           L.DECLINE_EXTENT)
     rc = lib.mi_add_f16(out.data_ptr(), a.data_ptr(), b.data_ptr(), a.numel(), ctx.stream)
     if rc != L.OK:
         raise DeclineError("mi_add_f16", rc)

@@ -161,3 +161,26 @@ def test_host_planners_decline_by_name_on_cpu_tensors():
     x = torch.zeros((1, 8, 8, 8), dtype=torch.float16)
     assert jv.conv_plan(jv.MI355X, x, x, x) == jv.Decline("operands")
     assert jv.convsize(518, 14, 14, 0, 1) == 37
+
+
+def test_small_operands_are_validated_before_their_pointer_is_taken():
+    """bias / gamma / beta / mean / rstd reach the kernels as raw pointers read at a fixed length and type: the host
+    wrappers refuse a wrong dtype, length or stride by name instead of launching an out-of-bounds read."""
+    import torch
+    from juliavision_amd import kernels as K
+    f16 = torch.float16
+    ok = torch.zeros(16, dtype=f16)
+    assert K._vec_problem("bias", ok, 16, require_cuda=False) is None
+    assert K._vec_problem("bias", None, 16) is None
+    assert "GPU" in K._vec_problem("bias", ok, 16)
+    assert "float32" in K._vec_problem("bias", torch.zeros(16), 16, require_cuda=False)          # fp32 bias of a mixed-precision export
+    assert "16 elements" in K._vec_problem("gamma", ok, 24, require_cuda=False)                  # shorter than the row
+    assert "contiguous" in K._vec_problem("beta", torch.zeros(32, dtype=f16)[::2], 16, require_cuda=False)
+    assert K._vec_problem("mean", torch.zeros(4), 4, torch.float32, require_cuda=False) is None
+    assert "float16" in K._vec_problem("mean", torch.zeros(4, dtype=f16), 4, torch.float32, require_cuda=False)
+    with pytest.raises(K.DeclineError, match="layernorm_: gamma is not on the GPU"):
+        K._check_vecs("layernorm_", L.DECLINE_OPERANDS, ("beta", None, 24), ("gamma", ok, 24))
+    # the planner turns an unreadable bias into a decline (on the CPU every operand declines first, so only the order
+    # of the checks is visible here: operands, then extents, then the bias)
+    dev = K.MI355X
+    assert K.mmplan(dev, torch.zeros(4, 8, dtype=f16), torch.zeros(8, 8, dtype=f16), torch.zeros(4, 8, dtype=f16)).reason == "operands"

@@ -431,6 +431,33 @@ def test_dinov2_like_encoder_folds_to_five_calls_per_block():
     assert sum("ln_out" in o["attrs"] for o in g.ops) == 4
 
 
+def test_division_by_a_weight_vector_is_not_folded_as_layerscale():
+    """Only ``linear(x) * g`` is a column scale of the weights; ``linear(x) / g`` and ``g / linear(x)`` are not, and
+    stay in the graph as written (there the executor refuses them by name instead of computing ``W * g``)."""
+    import torch
+    import torch.nn as nn
+    from juliavision_amd import graph as G
+
+    class M(nn.Module):
+        def __init__(self, mode):
+            super().__init__()
+            self.lin, self.g, self.mode = nn.Linear(16, 24), nn.Parameter(torch.rand(24) + 0.5), mode
+
+        def forward(self, x):
+            y = self.lin(x)
+            return y * self.g if self.mode == "mul" else y / self.g if self.mode == "div" else self.g / y
+
+    for mode in ("mul", "div", "rdiv"):
+        ep = torch.export.export(M(mode).eval().half(), (torch.randn(5, 16).half(),)).run_decompositions()
+        g = G.optimize(G.Graph.load(G.convert(ep, mode)))
+        folded = [o for o in g.ops if "colscale" in o["attrs"]]
+        left = [o["aten"] for o in g.ops]
+        if mode == "mul":
+            assert len(folded) == 1 and "mul.Tensor" not in left, (left, g.notes)
+        else:
+            assert not folded and "div.Tensor" in left, (mode, left, g.notes)
+
+
 @pytest.mark.gpu
 def test_dinov2_like_encoder_runs_on_the_kernels(ctx):
     import torch
