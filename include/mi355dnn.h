@@ -44,7 +44,8 @@ enum mi_status {
     MI_DECLINE_BIAS = 4,        /* a bias/mask shape the call cannot apply       (Decline(:bias))     */
     MI_DECLINE_UNSUPPORTED = 5, /* e.g. grouped convolution                                            */
     MI_ERROR_LAUNCH = 6,        /* HIP reported an error at launch                                     */
-    MI_ERROR_DEVICE = 7         /* no gfx950 device / library not initialised                          */
+    MI_ERROR_DEVICE = 7,        /* no gfx950 device / library not initialised                          */
+    MI_DECLINE_SCRATCH_LIMIT = 8 /* mi_gemm_f16_noalloc: the call needs more than MI_NOALLOC_SCRATCH_BYTES */
 };
 
 enum mi_epilogue { MI_EPI_NONE = 0, MI_EPI_GELU_ERF = 1, MI_EPI_GELU_TANH = 2, MI_EPI_RELU = 3 };
@@ -145,6 +146,20 @@ int mi_gemm_clamp_ln_f16(void *Y, void *H, const void *X, const void *W, const v
                          int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream);
 
 size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int64_t nbatch);
+
+/* mi_gemm_f16 without the workspace arguments, for callers that cannot allocate device memory and have no
+ * workspace to hand over: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference (whose kernels always draw scratch from the caller's bump workspace,
+ * workspace.jl:63-106).  The split-K / decode planes go to a static device array of MI_NOALLOC_SCRATCH_BYTES that
+ * every GPU the library runs on holds until the process ends; a call that would need more (what
+ * mi_gemm_f16_workspace(T, K, F, w_layout, 1) returns) is refused with MI_DECLINE_SCRATCH_LIMIT and enqueues
+ * nothing.  Calls no hipMalloc / hipFree / allocating routine.  Same kernels, same plan and same bits as
+ * mi_gemm_f16.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams
+ * without ordering between them) race on it. */
+#define MI_NOALLOC_SCRATCH_BYTES (32 * 1024 * 1024)
+int mi_gemm_f16_noalloc(void *Y, const void *X, const void *W, const void *bias, const void *residual,
+                        int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                        int w_layout, int bias_mode, int epi, int out_dtype, void *stream);
 /* Returns an mi_gemm_path; never launches.  Replaces mmplan / mm_coopmat_plan /
  * mm_gemv_plan -- matmul.jl:87-95,121-131,172-179. */
 int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,

@@ -13,8 +13,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi355dnn.so")
 
 # enum mi_status
-OK, DECLINE_OPERANDS, DECLINE_EXTENT, DECLINE_WORKSPACE, DECLINE_BIAS, DECLINE_UNSUPPORTED, ERROR_LAUNCH, ERROR_DEVICE = range(8)
-STATUS_NAMES = {0: "ok", 1: "operands", 2: "extent", 3: "workspace", 4: "bias", 5: "unsupported", 6: "launch", 7: "device"}
+OK, DECLINE_OPERANDS, DECLINE_EXTENT, DECLINE_WORKSPACE, DECLINE_BIAS, DECLINE_UNSUPPORTED, ERROR_LAUNCH, ERROR_DEVICE, DECLINE_SCRATCH_LIMIT = range(9)
+STATUS_NAMES = {0: "ok", 1: "operands", 2: "extent", 3: "workspace", 4: "bias", 5: "unsupported", 6: "launch", 7: "device", 8: "scratch_limit"}
+NOALLOC_SCRATCH_BYTES = 32 * 1024 * 1024
 EPI = {"none": 0, "identity": 0, "gelu": 1, "gelu_erf": 1, "gelu_tanh": 2, "relu": 3}
 F16, F32 = 0, 1
 W_KF, W_FK = 0, 1
@@ -39,6 +40,7 @@ SIGNATURES = {
     "mi_gemm_ln_f16": (_int, [_vp] * 8 + [_f32] + [_i64] * 5 + [_int] * 3 + [_vp, _sz, _vp]),
     "mi_gemm_clamp_ln_f16": (_int, [_vp] * 8 + [_f32, _f32] + [_i64] * 5 + [_int] * 3 + [_vp, _sz, _vp]),
     "mi_gemm_f16_workspace": (_sz, [_i64, _i64, _i64, _int, _i64]),
+    "mi_gemm_f16_noalloc": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp]),
     "mi_gemm_f16_plan": (_int, [_vp] * 3 + [_i64] * 6 + [_int] * 2 + [_i64] * 4),
     "mi_sdpa_f16": (_int, [_vp, _int, _i64p, _vp, _i64p, _vp, _i64p, _vp, _i64p, _vp, _int, _i64p, _vp] + [_i64] * 5 + [_f32, _vp, _sz, _vp]),
     "mi_sdpa_f16_workspace": (_sz, [_i64] * 5 + [_int]),

@@ -9,6 +9,9 @@
 #include "common.hpp"
 #include <type_traits>
 
+// Static device scratch of the allocation-free entry point (see mi_gemm_f16_noalloc).
+static __device__ __align__(256) unsigned char scratch[MI_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 struct GemmArgs {
@@ -1006,6 +1009,24 @@ __global__ __launch_bounds__(256) void splitk_epilogue_ln_kernel(GemmArgs p, con
 bool g_ready = false;
 int g_cus = 256;
 
+// Scratch of mi_gemm_f16_noalloc: every GPU the library runs on holds its own copy of this array, at its own
+// address, until the process ends.  Host code never uses the name as a pointer; g_scratch_ptr[device] is the
+// address hipGetSymbolAddress gave with that device current.
+constexpr int MAX_DEVICES = 64;
+void *g_scratch_ptr[MAX_DEVICES] = {};
+
+// The current device's copy of `scratch`; resolved once per device, with that device current.  Null on failure.
+void *scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
 template <typename KernelT>
 int raise_lds(KernelT kern, int bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? 0 : 1;
@@ -1345,6 +1366,7 @@ int mi_init(void) {
     bad |= raise_lds(skinny_fk_kernel<4>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<8>, (int)SKINNY_FK_LDS_MAX);
     bad |= mi_sdpa_init();
+    bad |= scratch_of_current_device() == nullptr;
     if (bad) return MI_ERROR_DEVICE;
     g_ready = true;
     return MI_OK;
@@ -1447,6 +1469,24 @@ int mi_gemm_clamp_ln_f16(void *Y, void *H, const void *X, const void *W, const v
         if (rc != MI_OK) return rc;
     }
     return H ? mi_layernorm_f16(H, nullptr, nullptr, Y, gamma, beta, F, T, eps, stream) : MI_OK;
+}
+
+// mi_gemm_f16 for callers that cannot allocate: the split-K / decode planes go to `scratch`, a file-scope
+// device array, reached through the per-device address that hipGetSymbolAddress returns (the array's name is only a
+// host-side stand-in).  The planes are written in full before they are summed, so nothing needs clearing between calls.
+int mi_gemm_f16_noalloc(void *Y, const void *X, const void *W, const void *bias, const void *residual,
+                        int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                        int w_layout, int bias_mode, int epi, int out_dtype, void *stream) {
+    if (!g_ready) return MI_ERROR_DEVICE;
+    const size_t need = mi_gemm_f16_workspace(T, K, F, w_layout, 1);
+    if (need > (size_t)MI_NOALLOC_SCRATCH_BYTES) return MI_DECLINE_SCRATCH_LIMIT;
+    void *planes = nullptr;
+    if (need) {
+        planes = scratch_of_current_device();
+        if (!planes) return MI_ERROR_DEVICE;
+    }
+    return mi_gemm_f16(Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype,
+                       planes, need ? (size_t)MI_NOALLOC_SCRATCH_BYTES : 0, stream);
 }
 
 int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,
