@@ -37,10 +37,29 @@ if ROOT not in sys.path:
 PEAK_F16_TFLOPS = 2500.0       # MI355X dense fp16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, vendor figure
 
-# HBM bytes per launch of the dominant kernel (fc1 GEMM), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of `python bench.py --no-cpu --no-detail`, scaled by the same counters on a plain copy kernel of
-# known size (--calibrate-copy).
-FC1_TRAFFIC_BYTES = 57_244_733       # profiles/fc1_gemm_hbm_traffic.txt: FETCH 20 451.5 KiB x 2.000 + WRITE 15 000 KiB x 1.000
+# HBM bytes per launch of the dominant kernel (fc1 GEMM) come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `python bench.py --no-cpu --no-detail`, scaled by the same counters on a plain copy kernel of known size
+# (--calibrate-copy).  The committed summary of those runs carries the figure on a line of its own; it is read from
+# there, not restated here.
+FC1_TRAFFIC_FILE = os.path.join("profiles", "fc1_gemm_hbm_traffic.txt")
+MFMA_FLOP_PER_CLK_PER_CU = 4 * 1024     # four SIMDs, one v_mfma_f32_32x32x16_f16 (32 768 flop) per 32 cycles each
+
+
+def fc1_traffic_bytes():
+    """``traffic_bytes_per_launch: N`` from the committed rocprofv3 summary, or None if it is not there."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, FC1_TRAFFIC_FILE)).read()
+    except OSError:
+        return None
+    m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
+    return int(m.group(1)) if m else None
+
+
+def randn_f16(shape, seed, mean=0.0, std=1.0):
+    """Seeded synthetic fp16 data (numpy's PCG64); the same host arrays feed the GPU step and the CPU baseline."""
+    import numpy as np
+    return (np.random.default_rng(seed).standard_normal(shape, dtype=np.float32) * std + mean).astype(np.float16)
 
 
 def parse_args():
@@ -114,24 +133,23 @@ class EncoderBlock:
     def __init__(self, lib, stream, seed=1000):
         import numpy as np
         import torch
-        import oracle
         L = self.L = __import__("juliavision_amd")._lib
         T, D, H, E, FF = self.T, self.D, self.H, self.E, self.FF
         f16 = torch.float16
         self.host = {}
         h = self.host
-        h["x"] = oracle.randn_f16((T, D), seed)
-        h["wqkv"] = oracle.randn_f16((3, D, D), seed + 1, 0, 0.02)      # Wq, Wk, Wv, each [K][F]
-        h["wo"] = oracle.randn_f16((D, D), seed + 4, 0, 0.02)
-        h["w1"] = oracle.randn_f16((D, FF), seed + 5, 0, 0.02)
-        h["w2"] = oracle.randn_f16((FF, D), seed + 6, 0, 0.02)
-        h["bqkv"] = oracle.randn_f16((3, D), seed + 10, 0, 0.02)
+        h["x"] = randn_f16((T, D), seed)
+        h["wqkv"] = randn_f16((3, D, D), seed + 1, 0, 0.02)      # Wq, Wk, Wv, each [K][F]
+        h["wo"] = randn_f16((D, D), seed + 4, 0, 0.02)
+        h["w1"] = randn_f16((D, FF), seed + 5, 0, 0.02)
+        h["w2"] = randn_f16((FF, D), seed + 6, 0, 0.02)
+        h["bqkv"] = randn_f16((3, D), seed + 10, 0, 0.02)
         for i, (n, m) in enumerate((("bo", D), ("b1", FF), ("b2", D))):
-            h[n] = oracle.randn_f16((m,), seed + 13 + i, 0, 0.02)
+            h[n] = randn_f16((m,), seed + 13 + i, 0, 0.02)
         for i, n in enumerate(("g1", "g2")):
-            h[n] = oracle.randn_f16((D,), seed + 20 + i, 1.0, 0.02)
+            h[n] = randn_f16((D,), seed + 20 + i, 1.0, 0.02)
         for i, n in enumerate(("be1", "be2")):
-            h[n] = oracle.randn_f16((D,), seed + 22 + i, 0.0, 0.02)
+            h[n] = randn_f16((D,), seed + 22 + i, 0.0, 0.02)
         d = self.d = {k: dev(v) for k, v in h.items()}
         for n in ("h1", "a", "o", "h2", "y"):
             d[n] = torch.empty((T, D), dtype=f16, device="cuda")
@@ -185,9 +203,7 @@ class EncoderBlock:
         # the three-pass attention at full length (a few seconds on 16 threads), repeated `reps` times.
         reps = 3
         rows, heads = T, H
-        qa = oracle.randn_f16((1, heads, T, E), 5)
-        ka = oracle.randn_f16((1, heads, T, E), 6)
-        va = oracle.randn_f16((1, heads, T, E), 7)
+        qa, ka, va = (randn_f16((1, heads, T, E), sd) for sd in (5, 6, 7))
         t_lin = t_att = 0.0
         for _ in range(reps):
             t0 = time.perf_counter()
@@ -861,6 +877,26 @@ def main():
     torch.cuda.synchronize()
     # The roofline kernel is bracketed by events inside the timed steps, but only in every EV_EVERY-th step: one
     # event marker costs about 5 us of queue time, and three of them in every step would be a tenth of the step.
+    # Shader clock during the fc1 launch: workgroup 0 of the kernel stores {shader clock, 100 MHz clock} at its start
+    # and end (mi_set_clock_probe); read after a few untimed steps so that the timed region carries no extra stores.
+    clk = torch.zeros(4, dtype=torch.int64, device="cuda")
+    blk.step()
+    torch.cuda.synchronize()
+    lib.mi_set_clock_probe(clk.data_ptr())
+    mhz = []
+    for _ in range(8):
+        for c in blk.calls_before_fc1:
+            c()
+        blk.fc1()
+        torch.cuda.synchronize()
+        c0, r0, c1, r1 = (int(v) for v in clk.tolist())
+        if r1 > r0:
+            mhz.append((c1 - c0) / (r1 - r0) * 100.0)
+        for c in blk.calls_after_fc1:
+            c()
+    lib.mi_set_clock_probe(None)
+    torch.cuda.synchronize()
+    shader_mhz = sorted(mhz)[len(mhz) // 2] if mhz else None
     EV_EVERY = 8 if args.steps >= 16 else 1
     evs = [tuple(torch.cuda.Event(enable_timing=True) for _ in range(3)) for _ in range((args.steps + EV_EVERY - 1) // EV_EVERY)]
     torch.cuda.synchronize()
@@ -881,6 +917,8 @@ def main():
         raise RuntimeError("encoder block produced non-finite or empty output")
 
     achieved = blk.FC1_FLOP / fc1_avg / 1e12
+    cus = int(jv.caps().cores)
+    peak_at_clock = cus * MFMA_FLOP_PER_CLK_PER_CU * shader_mhz * 1e6 / 1e12 if shader_mhz else None
     res = {
         "metric": "fp16 GEMM/attention TFLOP/s + % of MFMA peak; ms per encoder block",
         "value": round(blk.FLOP / sec / 1e12, 2),
@@ -895,9 +933,15 @@ def main():
                    "tokens": 1500, "d_model": 1280, "heads": 20, "head_dim": 64, "ffn": 5120,
                    "weight_layout": "[K][F] (the reference's hoisted layout)"},
         "frac_mfma_peak": round(blk.FLOP / sec / 1e12 / PEAK_F16_TFLOPS, 4),
-        "roofline": {"kernel": "gemm_pipe_kernel<128,256,2,4,KN> fc1: Y[1500x5120] = gelu(X[1500x1280].W[1280x5120] + b)",
+        "roofline": {"kernel": "gemm_pp_kernel<128,256,64,3,2,4,KN> fc1: Y[1500x5120] = gelu(X[1500x1280].W[1280x5120] + b)",
                      "bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": FC1_TRAFFIC_BYTES,
+                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": fc1_traffic_bytes(),
+                     "traffic_source": FC1_TRAFFIC_FILE,
+                     # next to the vendor-peak fraction, never instead of it: the same rate against what the MFMA
+                     # units can deliver at the shader clock measured inside this launch
+                     "shader_clock_mhz": round(shader_mhz, 1) if shader_mhz else None,
+                     "peak_at_measured_clock": round(peak_at_clock, 1) if peak_at_clock else None,
+                     "frac_at_measured_clock": round(achieved / peak_at_clock, 4) if peak_at_clock else None,
                      "flop_per_launch": blk.FC1_FLOP, "avg_launch_us": round(fc1_avg * 1e6, 2),
                      "median_launch_us": round(fc1_ms[len(fc1_ms) // 2] * 1e3, 2),
                      "avg_event_bracket_us": round(sum(bracket_ms) / len(bracket_ms) * 1e3, 2),

@@ -71,6 +71,13 @@ int mi_init(void);
  * [3]=LDS bytes per workgroup, [4]=max workgroup size, [5]=compute units. */
 int mi_device_caps(int64_t out[6]);
 
+/* Measurement aid (no counterpart in the reference).  While a device buffer of four uint64 is registered (NULL
+ * clears it), workgroup 0 of every launch of the ping-pong GEMM kernels (the 128 x 256 and 256 x 256 tiles of
+ * mi_gemm_f16 and its variants) stores {shader clock, constant 100 MHz clock} there when it starts and again after
+ * its last store: buf = {clk0, ref0, clk1, ref1}, and (clk1 - clk0) / (ref1 - ref0) x 100 MHz is the shader clock the
+ * launch ran at.  The caller keeps the buffer alive while it is registered.  Process-wide, not thread safe. */
+int mi_set_clock_probe(void *dev_u64x4);
+
 /* ---------------------------------------------------------------- GEMM
  * Y[T x F] = epi(round(X[T x K] . W + bias)) (+ residual)
  *   X   fp16 [T][K], ldX.

@@ -33,6 +33,7 @@ SIGNATURES = {
     "mi_version": (_int, []),
     "mi_init": (_int, []),
     "mi_device_caps": (_int, [_i64p]),
+    "mi_set_clock_probe": (_int, [_vp]),
     "mi_gemm_f16": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
     "mi_gemm_f16_batched": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_i64] * 5 + [_vp, _sz, _vp]),
     "mi_gemv_f16": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),

@@ -8,6 +8,7 @@
 //   [N][K].  For a linear layer M = tokens, N = features, A = X, B = W.
 #include "common.hpp"
 #include <type_traits>
+#include <cstdlib>
 
 // Static device scratch of the allocation-free entry point (see mi_gemm_f16_noalloc).
 static __device__ __align__(256) unsigned char scratch[MI_NOALLOC_SCRATCH_BYTES];
@@ -39,6 +40,9 @@ struct GemmArgs {
     // Tiled kernels and the split-K plane sums: > 0 clamps the fp16 result to [-clamp, clamp] after the residual add,
     // as a separate aten::clamp on Y would (the overflow guard of exported fp16 encoder layers).
     float clamp;
+    // Measurement only (mi_set_clock_probe): workgroup 0 of a ping-pong launch stores {shader clock, 100 MHz clock}
+    // here when it starts and again after its last store.  Null in ordinary use.
+    unsigned long long *clk;
 };
 
 // ------------------------------------------------------------------------------------------
@@ -599,6 +603,201 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
 }
 
 // ------------------------------------------------------------------------------------------
+// The ping-pong kernel: K % BK == 0, ordinary (ungathered) operands, eight waves.
+//
+// Operand tiles travel global -> LDS without passing through registers (global_load_lds_dwordx4: every lane
+// of a wave hands over 16 bytes, the wave's 1 KB lands contiguously at the LDS address in M0), STAGES BK-deep
+// stages deep, so a tile's loads are issued STAGES - 1 tiles ahead of its use and cost no VGPRs and no LDS-write
+// issue slots.  Unpadded rows would put every row of a fragment read on the same banks, and a direct load cannot pad
+// inside its 1 KB, so the 16-byte chunks are permuted instead: the chunk a lane fetches is chosen so that LDS
+// position `pos` of row r holds chunk pos ^ swz(r) (K-contiguous operands: swz = (r & 7) ^ ((r >> 3) & 1) for
+// 128-byte rows, (r >> 2) & 3 for 64-byte rows; the [K][N] operand: chunk ^ ((k & 3) << 2)), and the fragment
+// reads apply the same permutation.
+//
+// The two waves of a SIMD alternate between a memory phase (all fragment reads of a BK-deep tile plus the wave's
+// share of the loads of tile kt + STAGES - 1) and a matrix phase (the tile's 16 MFMAs): waves 0-3 (one per
+// SIMD) run one phase ahead of waves 4-7, a workgroup barrier closes every phase, and so one wave of each SIMD
+// always has a full phase of MFMAs queued while the other waits on LDS.  Every wave executes the same number of
+// barriers: the trailing group takes one extra at the start and none after its last matrix phase.
+//
+// Stage of tile t: t % STAGES.  A stage is free again once both groups have read it, i.e. after the barrier that
+// closes the trailing group's memory phase; tile t + STAGES is requested into it during the following memory phases
+// and has to have landed 2 (STAGES - 1) phases later: each wave waits for its own share (s_waitcnt vmcnt) ahead of the barrier that
+// precedes the leading group's first read of that tile.
+template <int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool B_KN, bool PINGPONG>
+__global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
+    static_assert(WAVES_M * WAVES_N == 8, "two groups of four waves");
+    static_assert(BK == 64 || BK == 32, "rows of 128 or 64 bytes");
+    constexpr int NT = 512, KS = BK / 16, CPR = BK / 8, ROWB = BK * 2;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
+    constexpr int PA = BM * CPR / NT, PB = BN * CPR / NT;          // 1 KB load instructions per wave and tile
+    constexpr int NL = PA + PB;
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE_BYTES = A_BYTES + B_BYTES;
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && PA >= 1 && PB >= 1 && STAGES >= 3 && STAGES <= 4, "tile shape");
+    static_assert(!B_KN || BN >= 128, "the [K][N] permutation moves a chunk by up to 12 places inside its row");
+    static_assert((STAGES - 2) * NL <= 63, "vmcnt is a 6-bit counter");
+    extern __shared__ __align__(16) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = PINGPONG ? wave >> 2 : 0;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    int tm_, tn_;
+    tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
+    const int m0 = tm_ * BM, n0 = tn_ * BN;
+    const long bz = blockIdx.y;
+    // tile origins; the per-lane part of every load address is a 32-bit byte offset from these
+    const half_t *Ag = p.A + bz * p.sA + (long)m0 * p.ldA;
+    const half_t *Bg = p.B + bz * p.sB + (B_KN ? (long)n0 : (long)n0 * p.ldB);
+    const long a_step = BK * 2, b_step = B_KN ? (long)BK * p.ldB * 2 : BK * 2;       // bytes per BK-deep tile
+
+    // K-contiguous rows: LDS position pos of row r holds chunk pos ^ rowswz(r)
+    auto rowswz = [](int r) { return BK == 64 ? (r & 7) ^ ((r >> 3) & 1) : (r >> 2) & 3; };
+    uint32_t aoffg[PA], boffg[PB];
+#pragma unroll
+    for (int i = 0; i < PA; i++) {
+        const int q = (i * 8 + wave) * 64 + lane, r = q / CPR, pos = q % CPR;
+        const int c = pos ^ rowswz(r);
+        aoffg[i] = (uint32_t)(((long)(min(m0 + r, p.M - 1) - m0) * p.ldA + c * 8) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < PB; i++) {
+        const int q = (i * 8 + wave) * 64 + lane;
+        if (!B_KN) {
+            const int r = q / CPR, pos = q % CPR;
+            const int c = pos ^ rowswz(r);
+            boffg[i] = (uint32_t)(((long)(min(n0 + r, p.N - 1) - n0) * p.ldB + c * 8) * 2);
+        } else {
+            constexpr int CPRB = BN / 8;
+            const int k = q / CPRB, pos = q % CPRB;
+            const int j = pos ^ ((k & 3) << 2);
+            boffg[i] = (uint32_t)(((long)k * p.ldB + (min(n0 + j * 8, p.NB - 8) - n0)) * 2);
+        }
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
+    // the wave's 1 KB slots inside a stage
+    auto issue = [&](int kt, int stage) {
+        const char *ab = reinterpret_cast<const char *>(Ag) + (long)kt * a_step;
+        const char *bb = reinterpret_cast<const char *>(Bg) + (long)kt * b_step;
+        const uint32_t sa = lds0 + stage * STAGE_BYTES + wave * 1024, sb = sa + A_BYTES;
+#pragma unroll
+        for (int i = 0; i < PA; i++) {
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(sa + i * 8192);
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(aoffg[i]), "s"(ab), "s"(dst) : "memory");
+        }
+#pragma unroll
+        for (int i = 0; i < PB; i++) {
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(sb + i * 8192);
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(boffg[i]), "s"(bb), "s"(dst) : "memory");
+        }
+    };
+
+    // fragment read offsets inside a stage (bytes)
+    const int frow = lane & 31, fhi = lane >> 5;
+    const int swz = rowswz(lane & 15);
+    int a_rd[KS], b_rd[KS], bt_rd[TN];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        const int cc = ((2 * ks + fhi) ^ swz) << 4;
+        a_rd[ks] = (wm * WTM + frow) * ROWB + cc;
+        b_rd[ks] = A_BYTES + (wn * WTN + frow) * ROWB + cc;
+    }
+    {
+        const int kk = (lane >> 2) & 3;
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+            const int col = (wn * WTN + i * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4) ^ (kk << 5);
+            bt_rd[i] = A_BYTES + ((fhi * 8 + kk) * BN + col) * 2;
+        }
+    }
+    half8v fa[KS][TM], fb[KS][TN];
+    auto fread = [&](int stage) {
+        const char *st = smem + stage * STAGE_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+#pragma unroll
+            for (int j = 0; j < TM; j++) fa[ks][j] = *reinterpret_cast<const half8v *>(st + a_rd[ks] + j * 32 * ROWB);
+            if (!B_KN) {
+#pragma unroll
+                for (int i = 0; i < TN; i++) fb[ks][i] = *reinterpret_cast<const half8v *>(st + b_rd[ks] + i * 32 * ROWB);
+            } else {
+#pragma unroll
+                for (int i = 0; i < TN; i++) {
+                    const char *bs = st + bt_rd[i] + ks * 16 * BN * 2;
+                    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(bs));
+                    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(bs + 4 * BN * 2));
+                    short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    fb[ks][i] = __builtin_bit_cast(half8v, both);
+                }
+            }
+        }
+    };
+    float16v acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    auto mma = [&]() {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int j = 0; j < TM; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks][i], fa[ks][j], acc[i][j], 0, 0, 0);
+    };
+    const bool probe = p.clk && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0;
+    if (probe) { p.clk[0] = clock64(); p.clk[1] = wall_clock64(); }
+    const int nk = p.K / BK;      // the launcher guarantees K % BK == 0 and K >= BK
+    // this wave's loads of tile kt + 1 have landed: only the tiles requested after it may still be in flight
+    auto wait_next = [&](int kt) {
+        const int newer = min(kt + STAGES - 1, nk - 1) - (kt + 1);
+        if (newer >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NL) : "memory");
+        else if (newer == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    auto barrier = [&]() {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; t++)
+        if (t < nk) issue(t, t);
+    wait_next(-1);                // tile 0
+    barrier();
+    if (grp == 1) barrier();
+    half4v cb[TN][4];
+    int stage = 0;
+    for (int kt = 0; kt < nk; kt++) {
+        // memory phase
+#ifdef ABL_NOREAD
+        if (kt == 0)
+#endif
+        fread(stage);
+#ifndef ABL_NOLOAD
+        if (kt + STAGES - 1 < nk) issue(kt + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
+#endif
+        if (kt + 1 == nk) load_col_bias<TN, WTN>(p, cb, n0, wn, lane, bz);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (grp == 1) wait_next(kt);
+        barrier();
+        // matrix phase
+        __builtin_amdgcn_s_setprio(1);
+        mma();
+        __builtin_amdgcn_s_setprio(0);
+        if (grp == 0) wait_next(kt);
+        // the trailing group's last matrix phase closes with no barrier (the leading group is already storing its
+        // tile): with the extra one it took at the start, both groups have then executed 2 nk + 1
+        if (!(PINGPONG && grp == 1 && kt + 1 == nk)) barrier();
+        stage = stage == STAGES - 1 ? 0 : stage + 1;
+    }
+    store_tile<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz);
+    if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
+}
+
+// ------------------------------------------------------------------------------------------
 // Scalar kernel: one thread per output, fp32 accumulation seeded with the bias,
 // any strides.  The arithmetic of the reference's mm2 (matmul.jl:17-27).
 __global__ void gemm_scalar_kernel(GemmArgs p, int b_kn) {
@@ -1008,6 +1207,7 @@ __global__ __launch_bounds__(256) void splitk_epilogue_ln_kernel(GemmArgs p, con
 // ------------------------------------------------------------------------------------------
 bool g_ready = false;
 int g_cus = 256;
+unsigned long long *g_clock_probe = nullptr;      // mi_set_clock_probe
 
 // Scratch of mi_gemm_f16_noalloc: every GPU the library runs on holds its own copy of this array, at its own
 // address, until the process ends.  Host code never uses the name as a pointer; g_scratch_ptr[device] is the
@@ -1030,6 +1230,12 @@ void *scratch_of_current_device() {
 template <typename KernelT>
 int raise_lds(KernelT kern, int bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? 0 : 1;
+}
+
+template <int BM, int BN, int BK, int STAGES>
+constexpr int pp_lds_bytes() {
+    constexpr int stages = STAGES * (BM + BN) * BK * 2, epi = 8 * 32 * (BN / 4 + 4) * 4;      // operand ring; epilogue staging of 8 waves
+    return stages > epi ? stages : epi;
 }
 
 template <int BM, int BN, int BK>
@@ -1085,13 +1291,39 @@ int launch_pipe(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
-// tile: index into TILE_MODELS
+template <int BM, int BN, int BK, int STAGES, int WM, int WN, bool PP>
+int launch_pp(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
+    if (a.K < BK || a.K % BK || a.cv.xp || a.ag.x) return MI_DECLINE_EXTENT;
+    a.tiles_m = (int)ceil_div(a.M, BM);
+    a.tiles_n = (int)ceil_div(a.N, BN);
+    a.group_m = a.tiles_m < 6 ? a.tiles_m : 6;
+    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
+                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
+    // per-lane load offsets are 32-bit byte offsets from the tile origin
+    if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? BK : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;
+    a.clk = g_clock_probe;
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
+    constexpr int lds = pp_lds_bytes<BM, BN, BK, STAGES>();
+    if (b_kn) hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, BK, STAGES, WM, WN, true, PP>), grid, dim3(512), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, BK, STAGES, WM, WN, false, PP>), grid, dim3(512), lds, st, a);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+// tile: index into TILE_MODELS.  The ping-pong kernels take ordinary operands only; a gathered operand (implicit-GEMM
+// convolution) planned onto one of their tiles runs the pipelined kernel's 128 x 256 tile instead: same K order per
+// output, same bits, and the plan (hence the workspace) stays a function of the extents alone.
 int launch_tile(int tile, const GemmArgs &a, bool b_kn, int64_t nbatch, hipStream_t st) {
+    const bool plain = !a.cv.xp && !a.ag.x;
+#ifdef MI_LAB
+    if (tile == 6) return launch_pp<128, 256, 64, 3, 2, 4, false>(a, b_kn, nbatch, st);
+    if (tile == 7) return launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
+#endif
     switch (tile) {
-        case 0: return launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
+        case 0: return plain ? launch_pp<128, 256, 64, 3, 2, 4, true>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
         case 1: return launch_pipe<192, 128, 2, 4>(a, b_kn, nbatch, st);
         case 2: return launch_pipe<128, 128, 2, 4>(a, b_kn, nbatch, st);
         case 3: return launch_pipe<64, 128, 2, 4>(a, b_kn, nbatch, st);
+        case 5: return plain ? launch_pp<256, 256, 32, 4, 2, 4, true>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
         default: return launch_pipe<64, 64, 2, 2>(a, b_kn, nbatch, st);
     }
 }
@@ -1118,12 +1350,16 @@ int launch_mfma(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
 // the second launch (about 4 us) and the fp32 planes (0.25 us per MB).  Picking the cheapest estimate lands within
 // 1 % of the best measured choice on average over those shapes and within 6 % on 95 % of them.
 struct TileModel { int bm, bn; double step_lo, step_full, round, fixed; };
-constexpr TileModel TILE_MODELS[5] = {
+constexpr int NTILES = 6;
+constexpr TileModel TILE_MODELS[NTILES] = {
     {128, 256, 0.660, 0.970, 0.97, 5.6},
     {192, 128, 0.545, 0.800, 0.93, 4.8},
     {128, 128, 0.428, 0.600, 1.00, 4.0},
     {64, 128, 0.318, 0.430, 0.90, 3.1},
     {64, 64, 0.235, 0.315, 0.73, 3.0},
+    // 256 x 256 (ping-pong kernel, 32-deep stages): 4096^3 in 120-123 us on one round of 256 workgroups, 8192^3 in
+    // 884-938 us on four; the lightly loaded step is scaled from the 128 x 256 tile's ratio
+    {256, 256, 1.200, 1.770, 1.00, 9.0},
 };
 struct TilePlan { int tile, split; };
 
@@ -1146,7 +1382,7 @@ TilePlan plan_tiles(int64_t M, int64_t N, int64_t K, int64_t nbatch, bool may_sp
     const int max_split = (may_split && nbatch == 1 && M > 8 && N % 4 == 0 && K % 64 == 0) ? 8 : 1;
     for (int split = 1; split <= max_split; split++) {
         if (K % (64 * split) != 0 || (split > 1 && K / split < 128)) continue;
-        for (int tile = 0; tile < 5; tile++) {
+        for (int tile = 0; tile < NTILES; tile++) {
             const double us = tile_cost_us(M, N, K, nbatch, tile, split);
             if (us < best_us) { best_us = us; best = {tile, split}; }
         }
@@ -1218,6 +1454,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.ag = NhwcGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
+    a.clk = nullptr;
     return MI_OK;
 }
 
@@ -1244,7 +1481,16 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
         if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
         TilePlan tp = {4, 1};
+#ifdef MI_LAB
+        // timing builds only: MI_FORCE_TILE = 1 + tile index (7: ping-pong 128 x 256 with both wave groups in phase,
+        // 8: the pipelined kernel's 128 x 256), MI_FORCE_SPLIT = K-slices
+        const char *ft = getenv("MI_FORCE_TILE"), *fs = getenv("MI_FORCE_SPLIT");
+        const bool forced = pipe && ft && atoi(ft) > 0;
+        if (forced) tp = {atoi(ft) - 1, fs ? atoi(fs) : 1};
+        if (pipe && !forced) {
+#else
         if (pipe) {
+#endif
             tp = plan_tiles(a.M, a.N, a.K, nbatch, true);
             if (tp.split > 1 && !(ws && aligned_to(ws, 256) && ws_bytes >= (size_t)tp.split * a.M * a.N * sizeof(float)))
                 tp = plan_tiles(a.M, a.N, a.K, nbatch, false);
@@ -1313,6 +1559,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     a.ag = NhwcGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
+    a.clk = nullptr;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
@@ -1361,6 +1608,14 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 0, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 1, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 2>, gemm_lds_bytes<128, 128, 64>());
+    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true>, pp_lds_bytes<128, 256, 64, 3>());
+    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, true>, pp_lds_bytes<128, 256, 64, 3>());
+#ifdef MI_LAB
+    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, false>, pp_lds_bytes<128, 256, 64, 3>());
+    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, false>, pp_lds_bytes<128, 256, 64, 3>());
+#endif
+    bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, true, true>, pp_lds_bytes<256, 256, 32, 4>());
+    bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, false, true>, pp_lds_bytes<256, 256, 32, 4>());
     bad |= raise_lds(skinny_fk_kernel<1>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<2>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<4>, (int)SKINNY_FK_LDS_MAX);
@@ -1369,6 +1624,12 @@ int mi_init(void) {
     bad |= scratch_of_current_device() == nullptr;
     if (bad) return MI_ERROR_DEVICE;
     g_ready = true;
+    return MI_OK;
+}
+
+int mi_set_clock_probe(void *dev_u64x4) {
+    if (dev_u64x4 && !aligned_to(dev_u64x4, 8)) return MI_DECLINE_OPERANDS;
+    g_clock_probe = reinterpret_cast<unsigned long long *>(dev_u64x4);
     return MI_OK;
 }
 
