@@ -131,6 +131,19 @@ int mi_ln_gemv_f16(void *Y, const void *X, const void *gamma, const void *beta, 
                    int w_layout, int bias_mode, int epi, int out_dtype,
                    void *ws, size_t ws_bytes, void *stream);
 
+/* The same fold for any T: Y = epi(layernorm(X) . W + bias) (+ residual), bit-identical to mi_layernorm_f16 followed
+ * by mi_gemm_f16 on its result.  T <= 8 is mi_ln_gemv_f16.  Larger T runs the tiled MFMA kernel with the norm as its
+ * prologue: every workgroup normalises its 64 rows of X into an LDS panel (one wave per row, the lane / summation
+ * order of mi_layernorm_f16) and then streams W alone; this needs 128 <= K <= 512 and K % 64 == 0 (a ViT-S block's
+ * d = 384), anything else returns MI_DECLINE_EXTENT and the caller runs the two ops.  No workspace is used for T > 8.
+ * The reference runs layernorm! (layernorm.jl:125) and matmul! (matmul.jl:78-79) as separate ops; the fold is item 3
+ * of its plans/kernels-to-port.md. */
+int mi_ln_gemm_f16(void *Y, const void *X, const void *gamma, const void *beta, float eps,
+                   const void *W, const void *bias, const void *residual,
+                   int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                   int w_layout, int bias_mode, int epi, int out_dtype,
+                   void *ws, size_t ws_bytes, void *stream);
+
 /* mi_gemm_f16 followed by mi_layernorm_f16 of its output rows: Y[T][F] (fp16, dense rows) as mi_gemm_f16 writes
  * it, and H[T][F] = layer norm of Y over F with gamma / beta (either may be NULL).  When the GEMM splits K the norm
  * rides in the pass that sums the planes (one launch less); otherwise the two kernels run back to back.  Either way

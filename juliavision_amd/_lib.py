@@ -38,6 +38,7 @@ SIGNATURES = {
     "mi_gemm_f16_batched": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_i64] * 5 + [_vp, _sz, _vp]),
     "mi_gemv_f16": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
     "mi_ln_gemv_f16": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp] + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
+    "mi_ln_gemm_f16": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp] + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
     "mi_gemm_ln_f16": (_int, [_vp] * 8 + [_f32] + [_i64] * 5 + [_int] * 3 + [_vp, _sz, _vp]),
     "mi_gemm_clamp_ln_f16": (_int, [_vp] * 8 + [_f32, _f32] + [_i64] * 5 + [_int] * 3 + [_vp, _sz, _vp]),
     "mi_gemm_f16_workspace": (_sz, [_i64, _i64, _i64, _int, _i64]),

@@ -27,6 +27,50 @@ MI_DEVICE uint32_t pack_hi(uint32_t x, uint32_t y) { return __builtin_amdgcn_per
 
 MI_DEVICE half8v as_half8(u32x4 v) { return __builtin_bit_cast(half8v, v); }
 
+// Lane exchanges without the LDS crossbar.  lane_xor<O>(v) is v of lane (lane ^ O) for O = 1, 2, 4, 8: data-parallel
+// primitives riding on the consuming VALU instruction (quad permutes, a rotation by 8 inside each row of 16, and for 4
+// the mirror of 8 lanes followed by the mirror of 4: lane ^ 7 ^ 3).  Across rows gfx950 has v_permlane16_swap /
+// v_permlane32_swap, which exchange the odd rows of one register with the even rows of another: from two copies of v
+// they leave (even rows twice, odd rows twice), whose sum or maximum is op(v[lane], v[lane ^ 16]) in every lane.
+// wave_sum / wave_max are the butterflies over 32, 16, 8, 4, 2, 1 built from these: the pairs, the order and therefore
+// the bits are those of the same butterfly written with __shfl_xor (six ds_bpermute round trips).
+template <int CTRL>
+MI_DEVICE float dpp_mov(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true)); }
+template <int O>
+MI_DEVICE float lane_xor(float v) {
+    static_assert(O == 1 || O == 2 || O == 4 || O == 8, "inside a row of 16 lanes");
+    if constexpr (O == 1) return dpp_mov<0xB1>(v);             // quad_perm [1,0,3,2]
+    else if constexpr (O == 2) return dpp_mov<0x4E>(v);        // quad_perm [2,3,0,1]
+    else if constexpr (O == 4) return dpp_mov<0x1B>(dpp_mov<0x141>(v));   // row_half_mirror, then quad_perm [3,2,1,0]
+    else return dpp_mov<0x128>(v);                              // row_ror:8
+}
+// (x, y) <- (even 32-lane halves of both, odd halves of both); the instruction is written out because the builtin's
+// second result is miscompiled when both operands hold the same value.
+MI_DEVICE void swap_rows32(float &x, float &y) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y)); }
+MI_DEVICE void swap_rows16(float &x, float &y) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y)); }
+MI_DEVICE float wave_sum(float a) {
+    float x = a, y = a;
+    swap_rows32(x, y); a = x + y;
+    x = a; y = a;
+    swap_rows16(x, y); a = x + y;
+    a += lane_xor<8>(a);
+    a += lane_xor<4>(a);
+    a += lane_xor<2>(a);
+    a += lane_xor<1>(a);
+    return a;
+}
+MI_DEVICE float wave_max(float a) {
+    float x = a, y = a;
+    swap_rows32(x, y); a = fmaxf(x, y);
+    x = a; y = a;
+    swap_rows16(x, y); a = fmaxf(x, y);
+    a = fmaxf(a, lane_xor<8>(a));
+    a = fmaxf(a, lane_xor<4>(a));
+    a = fmaxf(a, lane_xor<2>(a));
+    a = fmaxf(a, lane_xor<1>(a));
+    return a;
+}
+
 // Abramowitz & Stegun 7.1.26 in fp32: the same expression as the reference's
 // `erf` (DNNKernels/src/ops.jl:161-169), so a folded gelu is the graph's gelu.
 MI_DEVICE float erf_as(float x) {
@@ -35,10 +79,27 @@ MI_DEVICE float erf_as(float x) {
     float y = 1.0f - (((((1.061405429f * t - 1.453152027f) * t) + 1.421413741f) * t - 0.284496736f) * t + 0.254829592f) * t * __expf(-a * a);
     return x < 0.0f ? -y : y;
 }
+// geluexact (DNNKernels/src/ops.jl:1665-1669) = 0.5 v (1 + erf(v / sqrt 2)) with the erf above, written so that it
+// costs 11 vector instructions and two transcendentals instead of 17 and two (the GEMM store is bound by them: 32 768
+// outputs per workgroup).  With u = |v|, t = 1 / (1 + p u / sqrt 2) and q = 0.5 P(t) exp(-v^2 / 2):
+//   v >= 0:  0.5 v (2 - P e) = v - v q        v < 0:  0.5 v (P e) = v q        both:  max(v, 0) - u q.
+// Same polynomial, same coefficients; the difference from the textbook order is rounding in the last fp32 place
+// (and, for v < -3, none of the cancellation in 1 - (1 - P e)), far below the fp16 result's resolution.
+MI_DEVICE float gelu_erf(float v) {
+    const float u = fabsf(v);
+    const float t = __builtin_amdgcn_rcpf(fmaf(u, 0.3275911f * 0.70710678118654752440f, 1.0f));
+    float pl = fmaf(0.5f * 1.061405429f, t, -0.5f * 1.453152027f);
+    pl = fmaf(pl, t, 0.5f * 1.421413741f);
+    pl = fmaf(pl, t, -0.5f * 0.284496736f);
+    pl = fmaf(pl, t, 0.5f * 0.254829592f);
+    pl *= t;
+    const float e = __builtin_amdgcn_exp2f((v * v) * (-0.5f * 1.44269504088896340736f));
+    return fmaf(-u, pl * e, fmaxf(v, 0.0f));
+}
 // ops.jl:1665-1669 (geluexact), 1677-1682 (gelutanh), 1683 (relu_epi)
 MI_DEVICE float apply_epi(float v, int epi) {
     switch (epi) {
-    case MI_EPI_GELU_ERF: return 0.5f * v * (1.0f + erf_as(v * 0.70710678118654752440f));
+    case MI_EPI_GELU_ERF: return gelu_erf(v);
     case MI_EPI_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
     case MI_EPI_RELU: return fmaxf(v, 0.0f);
     default: return v;
@@ -47,7 +108,7 @@ MI_DEVICE float apply_epi(float v, int epi) {
 
 template <int EPI>
 MI_DEVICE float apply_epi_c(float v) {
-    if constexpr (EPI == MI_EPI_GELU_ERF) return 0.5f * v * (1.0f + erf_as(v * 0.70710678118654752440f));
+    if constexpr (EPI == MI_EPI_GELU_ERF) return gelu_erf(v);
     else if constexpr (EPI == MI_EPI_GELU_TANH) return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
     else if constexpr (EPI == MI_EPI_RELU) return fmaxf(v, 0.0f);
     else return v;

@@ -378,9 +378,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_mfma_kernel(GemmAr
 // Two waves per SIMD (8 waves on a 128 x 256 tile) cover each other's waits.
 // BMODE: 0 = B is [N][K], 1 = B is [K][N], 2 = B is [K][N] gathered from a padded image (implicit-GEMM convolution).
 // AMODE 1: A is gathered from a channels-last image (NhwcGather); B is then an ordinary [N][K] or [K][N] operand.
+// AMODE 2: the rows of A are layer-normalised over K on their way in (K <= 512): before the K loop every wave
+// normalises rows of the tile's A panel -- one wave per row, a lane holding eight consecutive k, statistics,
+// arithmetic and rounding exactly those of layernorm_vec_kernel -- into an LDS panel [BM][K + 8] that stays resident;
+// the K loop then streams B alone and reads its A fragments from the panel.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BMODE, int AMODE = 0>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(GemmArgs p) {
-    constexpr bool B_KN = BMODE != 0, CONV = BMODE == 2;
+    constexpr bool B_KN = BMODE != 0, CONV = BMODE == 2, LNA = AMODE == 2;
     static_assert(AMODE == 0 || BMODE != 2, "one gathered operand at a time");
     constexpr int BK = 64, LD = BK + 8, NT = WAVES_M * WAVES_N * 64;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
@@ -392,8 +396,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
     static_assert(PA >= 1 && PB >= 1, "tile too small for this workgroup");
     constexpr int BSZ = B_KN ? BK * BLD : BN * LD;      // halves per B buffer
     extern __shared__ __align__(16) char smem[];
-    half_t *As = reinterpret_cast<half_t *>(smem);   // [2][BM][LD]
-    half_t *Bs = As + 2 * BM * LD;                   // [2][BN][LD] or [2][BK][BLD]
+    half_t *As = reinterpret_cast<half_t *>(smem);   // [2][BM][LD]; AMODE 2: the normalised panel [BM][K + 8]
+    const int KP = p.K + 8;                          // panel row (halves): 16 bytes off a multiple of 128, like LD
+    half_t *Bs = As + (LNA ? BM * KP : 2 * BM * LD); // [2][BN][LD] or [2][BK][BLD]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     int tm_, tn_;
@@ -456,7 +461,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
                 const u32x4 z = {0u, 0u, 0u, 0u};
                 ga[set][i] = in ? ldg16(ap[i] + ((long)iy * p.ag.W + ix) * p.ag.C + ci0) : z;
             }
-        } else {
+        } else if constexpr (!LNA) {
 #pragma unroll
             for (int i = 0; i < PA; i++) ga[set][i] = ldg16(ap[i] + ko);
         }
@@ -480,6 +485,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
         }
     };
     auto lwrite_a = [&](int set, int buf) {
+        if constexpr (LNA) return;                     // the panel is already there
 #pragma unroll
         for (int i = 0; i < PA; i++) { const int c = tid + i * NT; *reinterpret_cast<u32x4 *>(As + buf * BM * LD + (c >> 3) * LD + (c & 7) * 8) = ga[set][i]; }
     };
@@ -501,17 +507,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     const int frow = lane & 31, fk = (lane >> 5) * 8;
-    const int aoff = (wm * WTM + frow) * LD + fk, boff = (wn * WTN + frow) * LD + fk;
+    const int aoff = (wm * WTM + frow) * (LNA ? KP : LD) + fk, boff = (wn * WTN + frow) * LD + fk;
     // [K][N] fragments: within each block of 16 lanes, lane i of ds_read_b64_tr_b16
     // receives, for j = 0..3, element i%4 of the 8 bytes addressed by lane 4j + i/4.
     // Pointing lane s at row (k0 + s/4), columns (n0 + 4 (s%4) .. +3) therefore hands
     // lane i the four consecutive k of column n0 + i: the MFMA operand layout.
     const int tboff = (fk + ((lane & 15) >> 2)) * BLD + wn * WTN + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
     half8v fa[2][TM], fb[2][TN];
-    auto fread = [&](int fs, int buf, int ks) {
-        const half_t *as = As + buf * BM * LD + aoff + ks * 16;
+    auto fread = [&](int fs, int buf, int ks, int kt) {
+        const half_t *as = LNA ? As + aoff + kt * BK + ks * 16 : As + buf * BM * LD + aoff + ks * 16;
+        const int jstep = 32 * (LNA ? KP : LD);
 #pragma unroll
-        for (int j = 0; j < TM; j++) fa[fs][j] = *reinterpret_cast<const half8v *>(as + j * 32 * LD);
+        for (int j = 0; j < TM; j++) fa[fs][j] = *reinterpret_cast<const half8v *>(as + j * jstep);
         if (!B_KN) {
             const half_t *bs = Bs + buf * BSZ + boff + ks * 16;
 #pragma unroll
@@ -537,10 +544,48 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
     const int nk = p.K / BK;   // the launcher guarantees K % 64 == 0 and nk >= 2
     gload(0, 0);
     gload(1, 1);
+    if constexpr (LNA) {
+        // One wave per row, all rows of a wave in flight at once (one trip to memory).  Rows past M repeat the last one.
+        constexpr int NW = NT / 64, RB = BM / NW;
+        static_assert(RB >= 1 && RB <= 16 && BM % NW == 0, "a wave's rows fit its registers");
+        const int e0 = lane * 8;
+        const bool mine = e0 < p.K;
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        const half8v gv = as_half8((p.ln_gamma && mine) ? ldg16(p.ln_gamma + e0) : z);
+        const half8v bv = as_half8((p.ln_beta && mine) ? ldg16(p.ln_beta + e0) : z);
+        for (int r0 = wave * (BM / NW); r0 < (wave + 1) * (BM / NW); r0 += RB) {
+            u32x4 raw[RB];
+#pragma unroll
+            for (int q = 0; q < RB; q++) raw[q] = mine ? ldg16(A + (long)min(m0 + r0 + q, p.M - 1) * p.ldA + e0) : z;
+#pragma unroll
+            for (int q = 0; q < RB; q++) {
+                const half8v t = as_half8(raw[q]);
+                float x[8], sum = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; j++) { x[j] = mine ? (float)t[j] : 0.0f; if (mine) sum += x[j]; }
+                sum = wave_sum(sum);
+                const float mu = sum / (float)p.K;
+                float s2 = 0.0f;
+                if (mine) {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) { const float d = x[j] - mu; s2 = fmaf(d, d, s2); }
+                }
+                s2 = wave_sum(s2);
+                const float rs = 1.0f / sqrtf(s2 / (float)p.K + p.ln_eps);
+                if (mine) {
+                    half8v o8;
+#pragma unroll
+                    for (int j = 0; j < 8; j++)
+                        o8[j] = ln_norm1(x[j], mu, rs, p.ln_gamma != nullptr, p.ln_gamma ? (float)gv[j] : 0.0f, p.ln_beta != nullptr, p.ln_beta ? (float)bv[j] : 0.0f);
+                    *reinterpret_cast<half8v *>(As + (r0 + q) * KP + e0) = o8;
+                }
+            }
+        }
+    }
     lwrite_a(0, 0);
     lwrite_b(0, 0);
     __syncthreads();
-    fread(0, 0, 0);
+    fread(0, 0, 0, 0);
 
     // MODE 0: steady state; 1: second-to-last tile (nothing left to fetch); 2: last tile.
     // Tile kt is computed from LDS buffer `cur`; register set `gw` holds tile kt+1, set `gl` receives tile kt+2.
@@ -552,20 +597,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
         // memory instructions dealt out between them, so that neither the LDS pipe nor the
         // vector-memory path sees a burst.
         if constexpr (MODE == 0) gload(gl, kt + 2);
-        fread(1, cur, 1);
+        fread(1, cur, 1, kt);
         mma(0);
         __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
 #pragma unroll
         for (int g = 0; g < NM; g++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x020, (PA + PB + NM - 1) / NM, 0); }
         __builtin_amdgcn_sched_barrier(0);
-        fread(0, cur, 2);
+        fread(0, cur, 2, kt);
         mma(1);
         if constexpr (MODE < 2) lwrite_a(gw, cur ^ 1);
         __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
 #pragma unroll
         for (int g = 0; g < NM; g++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x200, (PA + NM - 1) / NM, 0); }
         __builtin_amdgcn_sched_barrier(0);
-        fread(1, cur, 3);
+        fread(1, cur, 3, kt);
         mma(0);
         if constexpr (MODE < 2) lwrite_b(gw, cur ^ 1);
         __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
@@ -573,7 +618,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
         for (int g = 0; g < NM; g++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x200, (PB + NM - 1) / NM, 0); }
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
-        if constexpr (MODE < 2) fread(0, cur ^ 1, 0);
+        if constexpr (MODE < 2) fread(0, cur ^ 1, 0, kt + 1);
         mma(1);
         __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -767,6 +812,9 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         if (t < nk) issue(t, t);
     wait_next(-1);                // tile 0
     barrier();
+#ifdef MI_LAB_TS
+    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 4; t[0] = clock64(); }
+#endif
     if (grp == 1) barrier();
     half4v cb[TN][4];
     int stage = 0;
@@ -793,7 +841,13 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         if (!(PINGPONG && grp == 1 && kt + 1 == nk)) barrier();
         stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
+#ifdef MI_LAB_TS
+    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 4; t[1] = clock64(); }
+#endif
     store_tile<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz);
+#ifdef MI_LAB_TS
+    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 4; t[2] = clock64(); t[3] = wall_clock64(); }
+#endif
     if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
 }
 
@@ -856,8 +910,7 @@ __device__ __forceinline__ void ln_row_stats(const GemmArgs &p, float (*stats)[2
                     for (int j = 0; j < 8; j++) s += (float)t[j];
                 }
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+            s = wave_sum(s);
             const float mu = s / (float)p.K;
 #pragma unroll
             for (int i = 0; i < NCH; i++) {
@@ -867,8 +920,7 @@ __device__ __forceinline__ void ln_row_stats(const GemmArgs &p, float (*stats)[2
                     for (int j = 0; j < 8; j++) { const float d = (float)t[j] - mu; s2 = fmaf(d, d, s2); }
                 }
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+            s2 = wave_sum(s2);
             if (lane == 0) { stats[m][0] = mu; stats[m][1] = 1.0f / sqrtf(s2 / (float)p.K + p.ln_eps); }
         } else {
             for (int e0 = lane * 8; e0 < p.K; e0 += 512) {
@@ -876,16 +928,14 @@ __device__ __forceinline__ void ln_row_stats(const GemmArgs &p, float (*stats)[2
 #pragma unroll
                 for (int j = 0; j < 8; j++) s += (float)t[j];
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+            s = wave_sum(s);
             const float mu = s / (float)p.K;
             for (int e0 = lane * 8; e0 < p.K; e0 += 512) {
                 const half8v t = as_half8(ldg16(row + e0));
 #pragma unroll
                 for (int j = 0; j < 8; j++) { const float d = (float)t[j] - mu; s2 = fmaf(d, d, s2); }
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+            s2 = wave_sum(s2);
             if (lane == 0) { stats[m][0] = mu; stats[m][1] = 1.0f / sqrtf(s2 / (float)p.K + p.ln_eps); }
         }
     }
@@ -971,8 +1021,10 @@ __global__ __launch_bounds__(256) void skinny_kn_kernel(GemmArgs p, float *part,
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             float v = acc[m][e];
-            v += __shfl_xor(v, 16, 64);
-            v += __shfl_xor(v, 32, 64);
+            float x0 = v, y0 = v;
+            swap_rows16(x0, y0); v = x0 + y0;            // v[lane] + v[lane ^ 16]
+            x0 = v; y0 = v;
+            swap_rows32(x0, y0); v = x0 + y0;            // ... + the same of lane ^ 32
             if (lane < 16) red[wave][m][cx * 8 + e] = v;
         }
     __syncthreads();
@@ -1063,8 +1115,7 @@ __global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p, int rows_per
 #pragma unroll
         for (int m = 0; m < MT; m++) {
             float sres = acc[m];
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) sres += __shfl_xor(sres, o, 64);
+            sres = wave_sum(sres);
             if (lane == m) mine = sres;
         }
         if (lane < p.M) {
@@ -1176,8 +1227,7 @@ __global__ __launch_bounds__(256) void splitk_epilogue_ln_kernel(GemmArgs p, con
             for (int j = 0; j < 8; j++) x[i][j] = 0.0f;
         }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    s = wave_sum(s);
     const float mu = s / (float)p.N;
     float s2 = 0.0f;
 #pragma unroll
@@ -1187,8 +1237,7 @@ __global__ __launch_bounds__(256) void splitk_epilogue_ln_kernel(GemmArgs p, con
             for (int j = 0; j < 8; j++) { const float d = x[i][j] - mu; s2 = fmaf(d, d, s2); }
         }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+    s2 = wave_sum(s2);
     const float r = 1.0f / sqrtf(s2 / (float)p.N + p.lnout_eps);
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
@@ -1288,6 +1337,28 @@ int launch_pipe(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     else if (a.cv.xp)   hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 2>), grid, dim3(WM * WN * 64), lds, st, a);
     else if (b_kn) hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 1>), grid, dim3(WM * WN * 64), lds, st, a);
     else           hipLaunchKernelGGL((gemm_pipe_kernel<BM, BN, WM, WN, 0>), grid, dim3(WM * WN * 64), lds, st, a);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+// The pipelined kernel with the layer norm of A's rows as its prologue (AMODE 2): 64-row tiles, 128 <= K <= 512.
+constexpr int LNA_KMAX = 512;
+template <int BN, int WM, int WN>
+constexpr int lna_lds_bytes(int K) {
+    constexpr int kc = BN * (64 + 8), kn = 64 * (BN + 32);
+    return (64 * (K + 8) + 2 * (kc > kn ? kc : kn)) * 2;
+}
+template <int BN, int WM, int WN>
+int launch_pipe_ln(GemmArgs a, bool b_kn, hipStream_t st) {
+    if (a.K < 128 || a.K % 64 || a.K > LNA_KMAX || a.cv.xp || a.ag.x) return MI_DECLINE_EXTENT;
+    a.tiles_m = (int)ceil_div(a.M, 64);
+    a.tiles_n = (int)ceil_div(a.N, BN);
+    a.group_m = a.tiles_m < 6 ? a.tiles_m : 6;
+    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
+                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), 1);
+    const int lds = lna_lds_bytes<BN, WM, WN>(a.K);
+    if (b_kn) hipLaunchKernelGGL((gemm_pipe_kernel<64, BN, WM, WN, 1, 2>), grid, dim3(WM * WN * 64), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_pipe_kernel<64, BN, WM, WN, 0, 2>), grid, dim3(WM * WN * 64), lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
@@ -1616,6 +1687,10 @@ int mi_init(void) {
 #endif
     bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, true, true>, pp_lds_bytes<256, 256, 32, 4>());
     bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, false, true>, pp_lds_bytes<256, 256, 32, 4>());
+    bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 1, 2>, lna_lds_bytes<128, 2, 4>(LNA_KMAX));
+    bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 0, 2>, lna_lds_bytes<128, 2, 4>(LNA_KMAX));
+    bad |= raise_lds(gemm_pipe_kernel<64, 64, 2, 2, 1, 2>, lna_lds_bytes<64, 2, 2>(LNA_KMAX));
+    bad |= raise_lds(gemm_pipe_kernel<64, 64, 2, 2, 0, 2>, lna_lds_bytes<64, 2, 2>(LNA_KMAX));
     bad |= raise_lds(skinny_fk_kernel<1>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<2>, (int)SKINNY_FK_LDS_MAX);
     bad |= raise_lds(skinny_fk_kernel<4>, (int)SKINNY_FK_LDS_MAX);
@@ -1761,6 +1836,32 @@ int mi_gemv_f16(void *Y, const void *X, const void *W, const void *bias, const v
     if (T < 1 || T > 8) return MI_DECLINE_EXTENT;
     if (!mfma_addressable(a, w_layout == MI_W_KF)) return MI_DECLINE_OPERANDS;
     return run_skinny(a, w_layout == MI_W_KF, ws, ws_bytes, (hipStream_t)stream);
+}
+
+int mi_ln_gemm_f16(void *Y, const void *X, const void *gamma, const void *beta, float eps,
+                   const void *W, const void *bias, const void *residual,
+                   int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                   int w_layout, int bias_mode, int epi, int out_dtype,
+                   void *ws, size_t ws_bytes, void *stream) {
+    if (T >= 1 && T <= 8)
+        return mi_ln_gemv_f16(Y, X, gamma, beta, eps, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi,
+                              out_dtype, ws, ws_bytes, stream);
+    GemmArgs a;
+    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, ldY, ldX, ldW, w_layout, bias_mode, epi, out_dtype, 0, 0, 0);
+    if (rc != MI_OK) return rc;
+    if (!g_ready) return MI_ERROR_DEVICE;
+    if (T == 0 || F == 0) return MI_OK;
+    const bool b_kn = w_layout == MI_W_KF;
+    if (!mfma_addressable(a, b_kn)) return MI_DECLINE_OPERANDS;
+    if ((gamma && !aligned_to(gamma, 16)) || (beta && !aligned_to(beta, 16))) return MI_DECLINE_OPERANDS;
+    if (K < 128 || K % 64 || K > LNA_KMAX) return MI_DECLINE_EXTENT;      // the caller runs the two ops
+    // a shape whose plain GEMM would split K sums in another order: keep the promise of identical bits, decline
+    if (plan_tiles(T, F, K, 1, true).split != 1) return MI_DECLINE_EXTENT;
+    a.ln_on = 1; a.ln_gamma = (const half_t *)gamma; a.ln_beta = (const half_t *)beta; a.ln_eps = eps;
+    // 64-row tiles only (the normalised panel of a workgroup stays in LDS); which width, by the same estimate as
+    // every other tiled launch
+    const bool wide = tile_cost_us(T, F, K, 1, 3, 1) <= tile_cost_us(T, F, K, 1, 4, 1);
+    return wide ? launch_pipe_ln<128, 2, 4>(a, b_kn, (hipStream_t)stream) : launch_pipe_ln<64, 2, 2>(a, b_kn, (hipStream_t)stream);
 }
 
 int mi_ln_gemv_f16(void *Y, const void *X, const void *gamma, const void *beta, float eps,

@@ -37,8 +37,7 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(half_t *out, float *
             for (int j = 0; j < 8; j++) x[i][j] = 0.0f;
         }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    s = wave_sum(s);
     const float mu = s / (float)C;
     float s2 = 0.0f;
 #pragma unroll
@@ -49,8 +48,7 @@ __global__ __launch_bounds__(256) void layernorm_vec_kernel(half_t *out, float *
             for (int j = 0; j < 8; j++) { const float d = x[i][j] - mu; s2 = fmaf(d, d, s2); }
         }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+    s2 = wave_sum(s2);
     const float r = 1.0f / sqrtf(s2 / (float)C + eps);
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
@@ -79,13 +77,11 @@ __global__ __launch_bounds__(256) void layernorm_any_kernel(half_t *out, float *
     const half_t *row = a + g * C;
     float s = 0.0f;
     for (int i = lane; i < C; i += 64) s += (float)row[i];
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    s = wave_sum(s);
     const float mu = s / (float)C;
     float s2 = 0.0f;
     for (int i = lane; i < C; i += 64) { const float d = (float)row[i] - mu; s2 = fmaf(d, d, s2); }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+    s2 = wave_sum(s2);
     const float r = 1.0f / sqrtf(s2 / (float)C + eps);
     for (int i = lane; i < C; i += 64) {
         float y = ((float)row[i] - mu) * r;
@@ -122,16 +118,14 @@ __global__ __launch_bounds__(256) void softmax_vec_kernel(half_t *out, const hal
             for (int j = 0; j < 8; j++) x[i][j] = -INFINITY;
         }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    m = wave_max(m);
     const float mm = m == -INFINITY ? 0.0f : m;
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < NCH; i++)
 #pragma unroll
         for (int j = 0; j < 8; j++) { x[i][j] = __expf(x[i][j] - mm); s += x[i][j]; }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    s = wave_sum(s);
     const float inv = s > 0.0f ? 1.0f / s : 0.0f;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
@@ -154,13 +148,11 @@ __global__ __launch_bounds__(256) void softmax_any_kernel(T *out, const T *a, in
     const T *row = a + g * n;
     float m = -INFINITY;
     for (int i = lane; i < n; i += 64) m = fmaxf(m, (float)row[i] * c);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    m = wave_max(m);
     const float mm = m == -INFINITY ? 0.0f : m;
     float s = 0.0f;
     for (int i = lane; i < n; i += 64) s += __expf((float)row[i] * c - mm);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    s = wave_sum(s);
     const float inv = s > 0.0f ? 1.0f / s : 0.0f;
     for (int i = lane; i < n; i += 64) out[g * n + i] = (T)(__expf((float)row[i] * c - mm) * inv);
 }

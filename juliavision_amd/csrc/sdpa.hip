@@ -619,9 +619,9 @@ __global__ __launch_bounds__(256) void sdpa_rows_kernel(SdpaArgs p) {
                     if (e0 + j < p.E) d = fmaf(qv[ci][j], (float)kp[(long)(e0 + j) * p.ks[0]], d);
             }
         }
-        d += __shfl_xor(d, 1, 64);
-        d += __shfl_xor(d, 2, 64);
-        d += __shfl_xor(d, 4, 64);
+        d += lane_xor<1>(d);
+        d += lane_xor<2>(d);
+        d += lane_xor<4>(d);
         float sc = d * p.scale;
         if (p.bias && live) {
             const long bo = (long)kk * p.bs[0] + (long)lq * p.bs[1] + (long)h * p.bs[2] + (long)b * p.bs[3];
@@ -767,9 +767,9 @@ __global__ __launch_bounds__(512) void sdpa_decode_kernel(SdpaArgs p) {
                 float d = 0.0f;
 #pragma unroll
                 for (int j = 0; j < 8; j++) d = fmaf(qv[j], (float)kt[j], d);
-                d += __shfl_xor(d, 1, 64);
-                d += __shfl_xor(d, 2, 64);
-                d += __shfl_xor(d, 4, 64);
+                d += lane_xor<1>(d);
+                d += lane_xor<2>(d);
+                d += lane_xor<4>(d);
                 const float sc = key < Lk ? d : -INFINITY;
                 const float mn = fmaxf(m, sc);
                 const float mu = mn == -INFINITY ? 0.0f : mn;

@@ -18,7 +18,7 @@ from typing import List, Optional
 
 import torch
 
-from .kernels import Ctx, add_, convolution_, convsize, layernorm_, matmul_, matmul_ln_, sdpa, transposeLE_
+from .kernels import Ctx, add_, convolution_, convsize, layernorm_, ln_matmul_, ln_matmul_folds, ln_matmul_pays, matmul_, matmul_ln_, sdpa, transposeLE_
 
 
 @dataclass
@@ -57,19 +57,28 @@ def encoder_layer(ctx: Ctx, W: EncoderLayerWeights, x: torch.Tensor, out: torch.
     previous layer did that for this one, ``buf.h`` already holds ``LN1(x)``."""
     T, d = x.shape
     E = d // heads
-    if not normed_in:
+    # where the norm is cheaper as the prologue of the GEMM that reads it (today: at most 8 token rows), it is one
+    fold1 = not normed_in and ln_matmul_folds(T, d, 3 * d) and ln_matmul_pays(T, d, 3 * d)
+    fold2 = ln_matmul_folds(T, d, W.w1.shape[1]) and ln_matmul_pays(T, d, W.w1.shape[1])
+    if not normed_in and not fold1:
         layernorm_(ctx, buf.h, None, None, x, W.ln1_g, W.ln1_b, d, eps)
     ctx.ws.reset()
-    matmul_(ctx, buf.qkv, W.wqkv, buf.h, W.bqkv)
+    if fold1:
+        ln_matmul_(ctx, buf.qkv, W.wqkv, x, W.ln1_g, W.ln1_b, eps, W.bqkv)
+    else:
+        matmul_(ctx, buf.qkv, W.wqkv, buf.h, W.bqkv)
     # q, k, v are column bands of the projection, heads are 64-wide column bands of those: (B,H,L,E) views, no copy
     q, k, v = (buf.qkv[:, i * d:(i + 1) * d].unflatten(1, (heads, E)).permute(1, 0, 2).unsqueeze(0) for i in range(3))
     ctx.ws.reset()
     sdpa(ctx, q, k, v, out=buf.att.unflatten(1, (heads, E)).permute(1, 0, 2).unsqueeze(0))
     ctx.ws.reset()
     matmul_(ctx, buf.x1, W.wo, buf.att, W.bo, residual=x)
-    layernorm_(ctx, buf.h, None, None, buf.x1, W.ln2_g, W.ln2_b, d, eps)
     ctx.ws.reset()
-    matmul_(ctx, buf.f, W.w1, buf.h, W.b1, epi=act)
+    if fold2:
+        ln_matmul_(ctx, buf.f, W.w1, buf.x1, W.ln2_g, W.ln2_b, eps, W.b1, epi=act)
+    else:
+        layernorm_(ctx, buf.h, None, None, buf.x1, W.ln2_g, W.ln2_b, d, eps)
+        matmul_(ctx, buf.f, W.w1, buf.h, W.b1, epi=act)
     ctx.ws.reset()
     if next_norm is None:
         matmul_(ctx, out, W.w2, buf.f, W.b2, residual=buf.x1)
@@ -127,10 +136,11 @@ class ViTEncoder:
             dst = self.tokens[(i + 1) % 2]
             # the norm that reads this layer's output rides in its last GEMM: the next layer's first norm into the
             # shared slot buf.h, the encoder's final norm into self.out
+            folds = ln_matmul_folds(self.T, lw.wqkv.shape[0], lw.wqkv.shape[1]) and ln_matmul_pays(self.T, lw.wqkv.shape[0], lw.wqkv.shape[1])
             if i + 1 < n:
-                nxt = (W.layers[i + 1].ln1_g, W.layers[i + 1].ln1_b, self.buf.h)
+                nxt = None if folds else (W.layers[i + 1].ln1_g, W.layers[i + 1].ln1_b, self.buf.h)
             else:
                 nxt = None if W.norm_g is None else (W.norm_g, W.norm_b, self.out)
-            encoder_layer(ctx, lw, src, dst, self.buf, self.heads, self.eps, normed_in=i > 0, next_norm=nxt)
+            encoder_layer(ctx, lw, src, dst, self.buf, self.heads, self.eps, normed_in=i > 0 and not folds, next_norm=nxt)
             src = dst
         return src if W.norm_g is None else self.out

@@ -273,7 +273,7 @@ def group_linears(g: Graph) -> Graph:
         x, w = o["in"][pos[0]], o["in"][pos[1]]
         b = o["in"][pos[2]] if pos[2] is not None and len(o["in"]) > pos[2] else None
         return x, w, b
-    plain = lambda o: o["aten"] in LINEAR_OPS and not any(k in o["attrs"] for k in ("epilogue", "residual", "ln_out", "clamp"))
+    plain = lambda o: o["aten"] in LINEAR_OPS and not any(k in o["attrs"] for k in ("epilogue", "residual", "ln_out", "ln_in", "clamp"))
     done = set()
     for first in [o for o in g.ops if plain(o)]:
         if first["id"] in done or first not in g.ops:
@@ -359,7 +359,7 @@ def fold_clamps(g: Graph) -> Graph:
         while g.buffers[chain[-1]]["kind"] == "view":
             chain.append(g.buffers[chain[-1]]["of"])
         prod = g.op(chain[-1])
-        if prod is None or prod["aten"] not in LINEAR_OPS or any(k in prod["attrs"] for k in ("clamp", "ln_out")):
+        if prod is None or prod["aten"] not in LINEAR_OPS or any(k in prod["attrs"] for k in ("clamp", "ln_out", "ln_in")):
             continue
         if g.buffers[chain[-1]].get("dtype") != "float16" or not (_consumers(g, chain[-1]) <= {cl["id"]}):
             continue
@@ -369,6 +369,58 @@ def fold_clamps(g: Graph) -> Graph:
         if cl["id"] in g.outputs:
             g.buffers[chain[-1]]["kind"] = "external"
         g.notes.append(f"fold {cl['id']} into the store of {prod['id']}")
+    return g
+
+
+def fold_layernorm_prologues(g: Graph) -> Graph:
+    """A layer norm over the last axis that only one linear op reads (through reshapes at most) becomes that GEMM's
+    prologue (``ln_matmul_``) where the kernels can take it and it is the faster choice (``kernels.ln_matmul_folds``,
+    ``ln_matmul_pays``): the rows are normalised on their way into LDS, so the normalised activations never exist in
+    memory and the norm costs no launch.  Today that is the decode-sized case (at most 8 rows: a decoder step's norms);
+    the tiled kernel's prologue exists (rows of at most 512) but is slower than the norm's own launch, so wider
+    batches stay with ``fold_layernorms``.  The reference's plans/kernels-to-port.md, item 3."""
+    for ln in [o for o in g.ops if o["aten"] in ("layer_norm.default", "native_layer_norm.default")]:
+        a = ln["attrs"]
+        xb = g.buffers[ln["in"][0]]
+        feat = (xb.get("shape") or [None])[-1]
+        if feat is None or list(a.get("arg1", [])) != [feat] or xb.get("dtype") != "float16":
+            continue
+        readers = _consumers(g, ln["out"])
+        if len(readers) != 1 or "<output>" in readers:
+            continue
+        lin = g.op(next(iter(readers)))
+        if lin is None or lin["aten"] not in LINEAR_OPS or any(k in lin["attrs"] for k in ("ln_in", "ln_out", "clamp")):
+            continue
+        xpos = {"linear.default": 0, "addmm.default": 1, "mm.default": 0}[lin["aten"]]
+        wpos = {"linear.default": 1, "addmm.default": 2, "mm.default": 1}[lin["aten"]]
+        chain = [lin["in"][xpos]]
+        ok = True
+        while chain[-1] != ln["out"]:
+            b = g.buffers[chain[-1]]
+            if b["kind"] != "view" or not (b.get("op") in RESHAPES or "getitem" in b.get("op", "")) or \
+                    ("getitem" not in b.get("op", "") and (b.get("shape") or [None])[-1] != feat):
+                ok = False
+                break
+            chain.append(b["of"])
+        if not ok or sum(1 for i in lin["in"] if i == lin["in"][xpos]) != 1:
+            continue
+        wshape = g.buffers[lin["in"][wpos]].get("shape") or []
+        if len(wshape) != 2 or g.buffers[g.root(lin["in"][wpos])]["kind"] != "weight":
+            continue
+        F = wshape[0] if lin["aten"] == "linear.default" else wshape[1]
+        T = 1
+        for d in (xb.get("shape") or [])[:-1]:
+            T *= d
+        if not (K.ln_matmul_folds(T, feat, F) and K.ln_matmul_pays(T, feat, F)):
+            continue
+        if any(g.op(g.root(i)) is not None for i in ln["in"][1:]):
+            continue                                    # gamma / beta must be constants
+        lin["attrs"].update(ln_in=True, ln_in_gamma=ln["in"][1] if len(ln["in"]) > 1 else None,
+                            ln_in_beta=ln["in"][2] if len(ln["in"]) > 2 else None, ln_in_eps=a.get("arg4", a.get("eps", 1e-5)))
+        g.ops.remove(ln)
+        ob = g.buffers[ln["out"]]
+        ob.update(kind="view", of=ln["in"][0], op="alias.default", attrs={})
+        g.notes.append(f"fold {ln['id']} into the prologue of {lin['id']}")
     return g
 
 
@@ -383,7 +435,7 @@ def fold_layernorms(g: Graph) -> Graph:
         while g.buffers[chain[-1]]["kind"] == "view":
             chain.append(g.buffers[chain[-1]]["of"])
         prod = g.op(chain[-1])
-        if prod is None or prod["aten"] not in LINEAR_OPS or "ln_out" in prod["attrs"]:
+        if prod is None or prod["aten"] not in LINEAR_OPS or "ln_out" in prod["attrs"] or "ln_in" in prod["attrs"]:
             continue
         feat = (g.buffers[chain[-1]].get("shape") or [None])[-1]
         shapes_ok = all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1])
@@ -568,7 +620,8 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
 
 
 def optimize(g: Graph) -> Graph:
-    return group_linears(fold_sdpa_transpose(fold_attention(fold_layernorms(fold_clamps(fold_residuals(fold_layerscale(fold_activations(g))))))))
+    return group_linears(fold_sdpa_transpose(fold_attention(fold_layernorms(fold_layernorm_prologues(
+        fold_clamps(fold_residuals(fold_layerscale(fold_activations(g)))))))))
 
 
 # ----------------------------------------------------------------------------- execution
@@ -714,6 +767,12 @@ class Executor:
             beta = self.get(attrs["ln_beta"]) if has_ln and attrs.get("ln_beta") else None
             K.matmul_ln_(self.ctx, self._rows(out), self._rows(self.t[attrs["ln_out"]]) if has_ln else None, w, self._rows(x), gamma, beta,
                          attrs.get("ln_eps", 0.0), bias, epi=attrs.get("epilogue", "none"), residual=res, clamp=attrs.get("clamp"))
+            return
+        if attrs.get("ln_in"):
+            gamma = self.get(attrs["ln_in_gamma"]) if attrs.get("ln_in_gamma") else None
+            beta = self.get(attrs["ln_in_beta"]) if attrs.get("ln_in_beta") else None
+            K.ln_matmul_(self.ctx, self._rows(out), w, self._rows(x), gamma, beta, attrs.get("ln_in_eps", 1e-5), bias,
+                         epi=attrs.get("epilogue", "none"), residual=res)
             return
         K.matmul_(self.ctx, self._rows(out), w, self._rows(x), bias, epi=attrs.get("epilogue", "none"), residual=res)
 

@@ -296,29 +296,53 @@ def matmul_ln_(ctx: Ctx, out, normed, A, B, gamma, beta, eps, bias=None, *, epi=
     return out
 
 
+LN_GEMM_KMAX = 512
+
+
+def ln_matmul_folds(T: int, K: int, F: int, w_layout: int = L.W_KF) -> bool:
+    """Whether ``ln_matmul_`` takes these extents (no GPU needed): decode-sized ``T``, or a tiled launch whose
+    workgroups can hold their normalised 64 x K panel in LDS and whose plain GEMM would not split K."""
+    if 1 <= T <= 8:
+        return True
+    return 128 <= K <= LN_GEMM_KMAX and K % 64 == 0 and L.load().mi_gemm_f16_workspace(T, K, F, w_layout, 1) == 0
+
+
+def ln_matmul_pays(T: int, K: int, F: int) -> bool:
+    """Whether folding the norm is also the faster choice.  Decode-sized rows: yes (one launch less, the statistics are
+    a few KB).  Tiled launches: measured, no -- every workgroup of a row of tiles repeats the norm of its 64 rows, about
+    120 vector instructions per row on a single wave, 6.5 us before its first MFMA (1370 x 384 -> 1152: 11.2 us folded
+    against 2.6 + 5.7 us for the two launches, and the same 6.5 us at every other extent tried), which is more than the
+    norm's own launch costs.  The rewrites and the encoder compositions ask this; ``ln_matmul_`` itself takes any
+    call ``ln_matmul_folds`` admits."""
+    return 1 <= T <= 8
+
+
 def ln_matmul_(ctx: Ctx, out, A, B, gamma, beta, eps, bias=None, *, epi="none", residual=None):
-    """``out[T,F] = epi(layernorm(B[T,K]) . A[K,F] + bias) (+ residual)`` for ``T <= 8`` in one pass over the weights:
-    ``layernorm_`` (layernorm.jl:125) folded into ``matmul_``'s activation staging, bit-identical to the two calls
-    in sequence.  Larger ``T`` declines (run the two ops)."""
+    """``out[T,F] = epi(layernorm(B[T,K]) . A[K,F] + bias) (+ residual)`` in one launch: ``layernorm_``
+    (layernorm.jl:125) folded into ``matmul_``'s activation staging, bit-identical to the two calls in sequence.
+    ``T <= 8``: one pass over the weights (the decode-sized kernels).  Larger ``T``: the tiled kernel with the norm as
+    its prologue, for ``128 <= K <= 512`` (``ln_matmul_folds``); anything else declines (run the two ops)."""
     plan = mmplan(ctx.dev, out, A, B, bias)
-    if not isinstance(plan, MMSkinnyPlan):
-        raise DeclineError(f"ln_matmul_: only the decode-sized path folds the norm (plan {plan})", L.DECLINE_EXTENT)
+    if not isinstance(plan, (MMSkinnyPlan, MMMfmaPlan)):
+        raise DeclineError(f"ln_matmul_: no kernel folds the norm for this call (plan {plan})", L.DECLINE_EXTENT)
     lib = L.init()
     K, F = A.shape
     T = B.shape[0]
     la, lb, lo = _mat2(A), _mat2(B), _mat2(out)
+    if isinstance(plan, MMMfmaPlan) and not ln_matmul_folds(T, K, F, plan.w_layout):
+        raise DeclineError(f"ln_matmul_: T={T} K={K} F={F} does not fold (tiled launches need 128 <= K <= {LN_GEMM_KMAX})", L.DECLINE_EXTENT)
     if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
         raise DeclineError("ln_matmul_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
     _check_vecs("ln_matmul_", L.DECLINE_OPERANDS, ("gamma", gamma, K), ("beta", beta, K))
     if bias is not None and bias.numel() != F:
         raise DeclineError("ln_matmul_: bias must have one value per output feature", L.DECLINE_BIAS)
-    need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1)
+    need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1) if T <= 8 else 0
     ws = ctx.ws.scratch(need)
-    rc = lib.mi_ln_gemv_f16(out.data_ptr(), B.data_ptr(), _ptr(gamma), _ptr(beta), float(eps), A.data_ptr(), _ptr(bias), _ptr(residual),
+    rc = lib.mi_ln_gemm_f16(out.data_ptr(), B.data_ptr(), _ptr(gamma), _ptr(beta), float(eps), A.data_ptr(), _ptr(bias), _ptr(residual),
                             T, K, F, lo[1], lb[1], la[1], plan.w_layout, L.BIAS_NONE if bias is None else L.BIAS_COL, L.EPI[epi],
                             _dtype_code(out), ws, need, ctx.stream)
     if rc != L.OK:
-        raise DeclineError("mi_ln_gemv_f16", rc)
+        raise DeclineError("mi_ln_gemm_f16", rc)
     return out
 
 

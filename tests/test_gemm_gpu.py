@@ -202,6 +202,50 @@ def test_layer_norm_folded_into_decode_sized_gemv(ctx, T, K, F, layout):
 
 
 @pytest.mark.parametrize("layout", ["kf", "fk"])
+@pytest.mark.parametrize("T,K,F", [(1370, 384, 1152), (1370, 384, 1536), (300, 512, 200), (65, 128, 72), (1000, 256, 3000), (64, 448, 64)])
+def test_layer_norm_as_prologue_of_the_tiled_gemm(ctx, T, K, F, layout):
+    """ln_matmul_ for T > 8 (the tiled kernel normalises its 64-row panel of X in LDS before the K loop): against the
+    oracle's layernorm -> gemm, and bit for bit against layernorm_ followed by matmul_.  Config 3's qkv and fc1
+    shapes, ragged last row and column tiles, both tile widths, K at both ends of the supported range."""
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd.kernels import ln_matmul_folds
+    assert ln_matmul_folds(T, K, F)
+    X = oracle.randn_f16((T, K), 91, 0.3, 2.0)
+    Wkf = oracle.randn_f16((K, F), 92, 0, 1.0 / np.sqrt(K))
+    g, be, b = oracle.randn_f16((K,), 93, 1.0, 0.2), oracle.randn_f16((K,), 94, 0, 0.2), oracle.randn_f16((F,), 95, 0, 0.1)
+    R = oracle.randn_f16((T, F), 96)
+    Wd = to_dev(Wkf) if layout == "kf" else to_dev(np.ascontiguousarray(Wkf.T)).t()
+    dX, dg, dbe, db, dR = to_dev(X), to_dev(g), to_dev(be), to_dev(b), to_dev(R)
+    for (gamma, beta, hg, hb, epi, res) in ((dg, dbe, g, be, "gelu", True), (None, None, None, None, "none", False), (dg, None, g, None, "relu", True)):
+        h, _, _ = oracle.layernorm_f16(X, hg, hb, 1e-6)
+        want = oracle.gemm_f16(h, Wkf, b, epi=epi, residual=R if res else None)
+        out = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+        ctx.ws.reset()
+        jv.ln_matmul_(ctx, out, Wd, dX, gamma, beta, 1e-6, db, epi=epi, residual=dR if res else None)
+        two = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+        hn = torch.empty_like(dX)
+        jv.layernorm_(ctx, hn, None, None, dX, gamma, beta, K, 1e-6)
+        ctx.ws.reset()
+        jv.matmul_(ctx, two, Wd, hn, db, epi=epi, residual=dR if res else None)
+        torch.cuda.synchronize()
+        assert_parity(to_host(out), want, what=f"ln+gemm T{T} K{K} F{F} {layout} {epi}")
+        assert np.array_equal(to_host(out), to_host(two)), "norm prologue differs from layernorm_ followed by matmul_"
+
+
+def test_layer_norm_prologue_declines_what_it_cannot_hold(ctx):
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd.kernels import ln_matmul_folds
+    assert not ln_matmul_folds(1500, 1280, 1280) and not ln_matmul_folds(100, 576, 128) and not ln_matmul_folds(100, 200, 128)
+    assert ln_matmul_folds(4, 1280, 1280) and ln_matmul_folds(1370, 384, 1152)
+    z = lambda *sh: torch.zeros(sh, dtype=torch.float16, device="cuda")
+    for (T, K, F) in ((100, 576, 128), (100, 1280, 128)):
+        with pytest.raises(jv.DeclineError):
+            jv.ln_matmul_(ctx, z(T, F), z(K, F), z(T, K), None, None, 1e-5)
+
+
+@pytest.mark.parametrize("layout", ["kf", "fk"])
 def test_output_larger_than_2g_elements_is_indexed_in_64_bits(ctx, layout):
     """70 000 x 32 768 outputs (2.29e9 elements, 4.6 GB of fp16): row offsets pass 2^31.  The oracle checks rows at
     the start, around the 2^31-element boundary (row 65 536) and at the end; every row is checked for coverage."""

@@ -134,6 +134,58 @@ def test_exported_block_runs_on_the_kernels(ctx, fold):
     assert_parity(run(x2.cuda()).float().cpu().numpy(), want2, what="second call")
 
 
+def _mlp(d=256, ffn=512, seed=0):
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+
+    class MLP(nn.Module):
+        """The feed-forward half of a pre-LN decoder layer, as a decoder step sees it: a handful of token rows."""
+
+        def __init__(self):
+            super().__init__()
+            self.ln, self.fc1, self.fc2 = nn.LayerNorm(d), nn.Linear(d, ffn), nn.Linear(ffn, d)
+
+        def forward(self, x):
+            return x + self.fc2(F.gelu(self.fc1(self.ln(x))))
+
+    torch.manual_seed(seed)
+    return MLP().eval().half()
+
+
+def test_decode_sized_norm_becomes_the_prologue_of_the_linear_that_reads_it():
+    import torch
+    from juliavision_amd import graph as G
+    m = _mlp()
+    for rows, folded in ((4, True), (300, False)):
+        ep = torch.export.export(m, (torch.randn(1, rows, 256).half(),))
+        g = G.optimize(G.Graph.load(G.convert(ep, "mlp")))
+        fc1 = g.op("linear")
+        if folded:      # norm -> fc1's prologue, gelu -> its epilogue, add -> fc2's store: two launches
+            assert [o["aten"] for o in g.ops] == ["linear.default", "linear.default"], g.notes
+            assert fc1["attrs"]["ln_in"] is True and fc1["attrs"]["ln_in_gamma"] == "p_ln_weight" and fc1["attrs"]["epilogue"] == "gelu"
+            assert g.root(fc1["in"][0]) == "x"
+        else:           # a wide batch keeps the norm's own launch (the tiled kernel's prologue is the slower choice)
+            assert [o["aten"] for o in g.ops] == ["layer_norm.default", "linear.default", "linear.default"] and "ln_in" not in fc1["attrs"]
+
+
+@pytest.mark.gpu
+def test_decode_sized_norm_prologue_runs_on_the_kernels(ctx):
+    import torch
+    from juliavision_amd import graph as G
+    m = _mlp(seed=2)
+    x = torch.randn(1, 4, 256).half()
+    ep = torch.export.export(m, (x,))
+    g = G.optimize(G.Graph.load(G.convert(ep, "mlp")))
+    assert g.op("linear")["attrs"].get("ln_in") is True
+    run = G.Executor(g, {k: v for k, v in m.state_dict().items()}, ctx)
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        want = m.float()(x.float())
+    assert_parity(got.float().cpu().numpy(), want.numpy(), what="decode-sized norm prologue from an exported graph")
+
+
 @pytest.mark.gpu
 def test_executor_refuses_what_it_cannot_run(ctx):
     import torch
