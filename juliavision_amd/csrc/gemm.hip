@@ -9,6 +9,13 @@
 #include "common.hpp"
 #include <type_traits>
 #include <cstdlib>
+#include <atomic>
+
+// Arrival flags of the split-K peer reduction (gemm_pp_kernel, SK): SK_BANKS banks of SK_FLAGS words; a launch uses
+// the bank its epoch selects and writes the epoch itself, so flags are never cleared and launches that overlap on one
+// GPU (up to SK_BANKS of them) do not see each other's.  Zero when the module loads; epochs start at 1.
+constexpr int SK_BANKS = 16, SK_FLAGS = 4096;
+static __device__ unsigned sk_flag_words[SK_BANKS * SK_FLAGS];
 
 // Static device scratch of the allocation-free entry point (see mi_gemm_f16_noalloc).
 static __device__ __align__(256) unsigned char scratch[MI_NOALLOC_SCRATCH_BYTES];
@@ -43,6 +50,13 @@ struct GemmArgs {
     // Measurement only (mi_set_clock_probe): workgroup 0 of a ping-pong launch stores {shader clock, 100 MHz clock}
     // here when it starts and again after its last store.  Null in ordinary use.
     unsigned long long *clk;
+    // Split-K with the partial tiles exchanged between the workgroups of a tile instead of written as planes
+    // (ping-pong kernel, SK instances): sk_S workgroups per tile, tiles dealt sk_tpx per XCD; partials in sk_part,
+    // per-wave arrival flags in sk_flags (they carry sk_epoch, unique per launch: nothing is ever cleared).
+    int sk_S, sk_tpx;
+    float *sk_part;
+    unsigned *sk_flags;
+    unsigned sk_epoch;
 };
 
 // ------------------------------------------------------------------------------------------
@@ -669,7 +683,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
 // closes the trailing group's memory phase; tile t + STAGES is requested into it during the following memory phases
 // and has to have landed 2 (STAGES - 1) phases later: each wave waits for its own share (s_waitcnt vmcnt) ahead of the barrier that
 // precedes the leading group's first read of that tile.
-template <int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool B_KN, bool PINGPONG>
+//
+// SK instances split K over the sk_S (2 or 4) workgroups of a tile without fp32 planes and without a second launch.
+// Workgroup pid runs on XCD pid % 8 (workgroups are dealt to the XCDs round robin; mi_init checks that this device
+// does so and the path stays off otherwise): pid = (slot * S + s) * 8 + xcd computes K-slice s of tile xcd * tpx + slot,
+// so the partners of a tile share an XCD, i.e. one L2, and are dispatched together.  After its K loop every wave owns
+// a quarter (S = 4) or half (S = 2) of its 64 x 64 accumulators -- the 32 x 32 sub-tiles q with q % S == s -- writes the
+// others into its partners' slots of sk_part (plain stores: they stay in the shared L2), waits for them to be
+// acknowledged, and raises its flag; it then waits (bounded) for the same wave of every partner, adds what they sent
+// in slice order (the result does not depend on which workgroup sums), and stores its share through the usual
+// epilogue.  Every workgroup publishes before it waits, and the grid fits the device in one round (the launcher
+// checks), so the waits cannot be circular.
+template <int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool B_KN, bool PINGPONG, bool SK = false>
 __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
     static_assert(WAVES_M * WAVES_N == 8, "two groups of four waves");
     static_assert(BK == 64 || BK == 32, "rows of 128 or 64 bytes");
@@ -686,14 +711,24 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = PINGPONG ? wave >> 2 : 0;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-    int tm_, tn_;
-    tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
+    int tm_, tn_, sk_s = 0, sk_tile = 0;
+    if constexpr (SK) {
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        sk_s = idx % p.sk_S;
+        sk_tile = xcd * p.sk_tpx + idx / p.sk_S;
+        if (sk_tile >= p.tiles_m * p.tiles_n) return;          // the whole workgroup: the last XCD's run may be short
+        tm_ = sk_tile % p.tiles_m;
+        tn_ = sk_tile / p.tiles_m;
+    } else {
+        tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
+    }
     const int m0 = tm_ * BM, n0 = tn_ * BN;
     const long bz = blockIdx.y;
+    const int nk = SK ? p.K / BK / p.sk_S : p.K / BK;      // the launcher guarantees whole BK-deep tiles per slice
     // tile origins; the per-lane part of every load address is a 32-bit byte offset from these
-    const half_t *Ag = p.A + bz * p.sA + (long)m0 * p.ldA;
-    const half_t *Bg = p.B + bz * p.sB + (B_KN ? (long)n0 : (long)n0 * p.ldB);
     const long a_step = BK * 2, b_step = B_KN ? (long)BK * p.ldB * 2 : BK * 2;       // bytes per BK-deep tile
+    const half_t *Ag = p.A + bz * p.sA + (long)m0 * p.ldA + (SK ? (long)sk_s * nk * (a_step / 2) : 0L);
+    const half_t *Bg = p.B + bz * p.sB + (B_KN ? (long)n0 : (long)n0 * p.ldB) + (SK ? (long)sk_s * nk * (b_step / 2) : 0L);
 
     // K-contiguous rows: LDS position pos of row r holds chunk pos ^ rowswz(r)
     auto rowswz = [](int r) { return BK == 64 ? (r & 7) ^ ((r >> 3) & 1) : (r >> 2) & 3; };
@@ -793,7 +828,6 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
     };
     const bool probe = p.clk && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0;
     if (probe) { p.clk[0] = clock64(); p.clk[1] = wall_clock64(); }
-    const int nk = p.K / BK;      // the launcher guarantees K % BK == 0 and K >= BK
     // this wave's loads of tile kt + 1 have landed: only the tiles requested after it may still be in flight
     auto wait_next = [&](int kt) {
         const int newer = min(kt + STAGES - 1, nk - 1) - (kt + 1);
@@ -813,7 +847,7 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
     wait_next(-1);                // tile 0
     barrier();
 #ifdef MI_LAB_TS
-    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 4; t[0] = clock64(); }
+    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[0] = clock64(); }
 #endif
     if (grp == 1) barrier();
     half4v cb[TN][4];
@@ -842,11 +876,112 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
 #ifdef MI_LAB_TS
-    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 4; t[1] = clock64(); }
+    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[1] = clock64(); }
 #endif
+    if constexpr (SK) {
+        // A wave's accumulators are NQ = TM * TN sub-tiles of 32 x 32, q = i * TM + j; sub-tile q goes to slice q % S.
+        constexpr int NQ = TM * TN;
+        static_assert(TM == 2 && (TN == 1 || TN == 2), "two or four 32 x 32 sub-tiles per wave");
+        const int S = p.sk_S, NSL = NQ / S;                    // slices (2, or 4 when NQ = 4); sub-tiles a wave keeps
+        // sk_part[tile][owner][source][wave][slot][4][64 lanes][4]: four registers per lane and access, 1 KB per wave instruction
+        auto part_of = [&](int owner, int src) { return p.sk_part + ((((long)sk_tile * S + owner) * S + src) * 8 + wave) * (long)(NSL * 1024) + lane * 4; };
+        static_for<NQ>([&](auto Q) {
+            constexpr int q = decltype(Q)::value, i = q / TM, j = q % TM;
+            if (q % S != sk_s) {                               // uniform
+                float *dst = part_of(q % S, sk_s) + (q / S) * 1024;
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    const float4v v = {acc[i][j][4 * r4], acc[i][j][4 * r4 + 1], acc[i][j][4 * r4 + 2], acc[i][j][4 * r4 + 3]};
+                    *reinterpret_cast<float4v *>(dst + r4 * 256) = v;
+                }
+            }
+        });
+        // the partials must have reached L2 before the flag can be seen
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned *myflag = p.sk_flags + ((long)sk_tile * S + sk_s) * 8 + wave;
+        if (lane == 0) __hip_atomic_store(myflag, p.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#ifdef MI_LAB_TS
+        if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[4] = clock64(); }
+#endif
+        // the sub-tiles this wave keeps (slot 0, and slot 1 when it keeps two)
+        float16v own[2];
+        static_for<NQ>([&](auto Q) {
+            constexpr int q = decltype(Q)::value, i = q / TM, j = q % TM;
+            if (q % S == sk_s) {                               // uniform
+                if (q / S == 0) own[0] = acc[i][j]; else own[1] = acc[i][j];
+            }
+        });
+        // Wait (bounded) for the same wave of every partner, then fetch everything they sent in one trip: at most three
+        // blocks of sixteen registers (three partners' one sub-tile, or one partner's one or two).  The three polls of a
+        // round are in flight together: a poll is a trip past the L1.
+        {
+            const unsigned *f[3];
+#pragma unroll
+            for (int bi = 0; bi < 3; bi++) {
+                const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;
+                f[bi] = p.sk_flags + ((long)sk_tile * S + src) * 8 + wave;
+            }
+            for (int spins = 0; spins < (1 << 18); spins++) {
+                const unsigned u0 = __hip_atomic_load(f[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const unsigned u1 = __hip_atomic_load(f[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const unsigned u2 = __hip_atomic_load(f[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (u0 == p.sk_epoch && u1 == p.sk_epoch && u2 == p.sk_epoch) break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        asm volatile("" ::: "memory");
+        // Ordinary loads: this CU has not touched these lines since the kernel began (its L1 was invalidated then), so
+        // they come from the L2 the partners' acknowledged stores are in.
+        float4v blk[3][4];
+#pragma unroll
+        for (int bi = 0; bi < 3; bi++) {
+            const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;      // S = 4: the bi-th partner in slice order
+            if (S == 4 || bi < NSL) {
+                const float *from = part_of(sk_s, src) + (S == 4 ? 0 : bi * 1024);
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) blk[bi][r4] = *reinterpret_cast<const float4v *>(from + r4 * 256);
+            }
+        }
+        float16v tot[2];                                       // summed in slice order, whoever does the summing
+        if (S == 4) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float x0 = blk[0][r >> 2][r & 3], x1 = blk[1][r >> 2][r & 3], x2 = blk[2][r >> 2][r & 3], o = own[0][r];
+                tot[0][r] = sk_s == 0 ? ((o + x0) + x1) + x2 : sk_s == 1 ? ((x0 + o) + x1) + x2 : sk_s == 2 ? ((x0 + x1) + o) + x2 : ((x0 + x1) + x2) + o;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                tot[0][r] = sk_s == 0 ? own[0][r] + blk[0][r >> 2][r & 3] : blk[0][r >> 2][r & 3] + own[0][r];
+                if (NQ == 4) tot[1][r] = sk_s == 0 ? own[1][r] + blk[1][r >> 2][r & 3] : blk[1][r >> 2][r & 3] + own[1][r];
+            }
+        }
+#ifdef MI_LAB_TS
+        if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[5] = clock64(); }
+#endif
+        // One kept sub-tile (S = NQ): q = s.  Two (S = 2 of four): q = s and s + 2, the 32-row half j = s at both
+        // 32-column halves.
+        if (NSL == 1) {
+            const int i = sk_s / TM, j = sk_s % TM;
+            float16v one[1][1] = {{tot[0]}};
+            half4v cb1[1][4];
+            // a 32-column store: the wave's column origin goes into n0 (the staging rows are as wide as the stored tile)
+            const int nw = n0 + wn * WTN + 32 * i;
+            load_col_bias<1, 32>(p, cb1, nw, 0, lane, bz);
+            store_tile<1, 1, WTM, 32, 8, STAGES * STAGE_BYTES>(p, one, cb1, smem, m0 + 32 * j, nw, wm, 0, wave, lane, bz);
+        } else if constexpr (TN == 2) {
+            float16v two[2][1] = {{tot[0]}, {tot[1]}};
+            store_tile<1, 2, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, two, cb, smem, m0 + 32 * sk_s, n0, wm, wn, wave, lane, bz);
+        }
+#ifdef MI_LAB_TS
+        if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[2] = clock64(); t[3] = wall_clock64(); }
+#endif
+        if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
+        return;
+    }
     store_tile<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz);
 #ifdef MI_LAB_TS
-    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 4; t[2] = clock64(); t[3] = wall_clock64(); }
+    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[2] = clock64(); t[3] = wall_clock64(); }
 #endif
     if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
 }
@@ -1264,6 +1399,39 @@ unsigned long long *g_clock_probe = nullptr;      // mi_set_clock_probe
 constexpr int MAX_DEVICES = 64;
 void *g_scratch_ptr[MAX_DEVICES] = {};
 
+unsigned *g_sk_flags_ptr[MAX_DEVICES] = {};
+int g_sk_state[MAX_DEVICES] = {};            // 0: not probed, 1: usable, -1: this device does not deal workgroups round robin
+std::atomic<unsigned> g_sk_epoch{0};
+
+// Workgroup -> XCD: every workgroup of a 1024-workgroup probe writes the id of the XCD it runs on (HW_REG_XCC_ID).
+__global__ void xcc_probe_kernel(unsigned *out) {
+    if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((3 << 11) | 20);      // XCC_ID, bits 3:0
+}
+
+// The split-K peer reduction relies on workgroups pid, pid + 8, pid + 16, ... sharing an XCD (one L2).  Checked once
+// per device on a probe launch: all workgroups with the same pid % 8 must report one XCD.  Uses the flag words as the
+// probe's output (they are zeroed again) and synchronises the device: call from mi_init only.
+int sk_probe_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return -1;
+    if (g_sk_state[dev]) return g_sk_state[dev];
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(sk_flag_words)) != hipSuccess || !ptr) return g_sk_state[dev] = -1;
+    g_sk_flags_ptr[dev] = reinterpret_cast<unsigned *>(ptr);
+    constexpr int NP = 1024;
+    static_assert(NP <= SK_BANKS * SK_FLAGS, "probe output fits the flag words");
+    unsigned host[NP];
+    hipLaunchKernelGGL(xcc_probe_kernel, dim3(NP), dim3(64), 0, 0, g_sk_flags_ptr[dev]);
+    bool ok = hipGetLastError() == hipSuccess && hipMemcpy(host, g_sk_flags_ptr[dev], sizeof(host), hipMemcpyDeviceToHost) == hipSuccess;
+    ok = ok && hipMemset(g_sk_flags_ptr[dev], 0, sizeof(host)) == hipSuccess && hipDeviceSynchronize() == hipSuccess;
+    for (int i = 8; ok && i < NP; i++) ok = host[i] == host[i & 7];
+    return g_sk_state[dev] = ok ? 1 : -1;
+}
+bool sk_usable() {
+    int dev = -1;
+    return hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MAX_DEVICES && g_sk_state[dev] == 1;
+}
+
 // The current device's copy of `scratch`; resolved once per device, with that device current.  Null on failure.
 void *scratch_of_current_device() {
     int dev = -1;
@@ -1380,6 +1548,36 @@ int launch_pp(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
+bool sk_fits(int64_t M, int64_t N, int64_t K, int bm, int bn, int split);
+
+// The ping-pong kernel with `split` workgroups per tile exchanging their partial tiles (see the kernel).
+template <int BM, int BN>
+int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
+    if (a.cv.xp || a.ag.x || !sk_usable() || !sk_fits(a.M, a.N, a.K, BM, BN, split)) return MI_DECLINE_EXTENT;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MI_ERROR_DEVICE;
+    a.tiles_m = (int)ceil_div(a.M, BM);
+    a.tiles_n = (int)ceil_div(a.N, BN);
+    a.group_m = 1;
+    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
+                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
+    if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? 64 : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;
+    const int tiles = a.tiles_m * a.tiles_n;
+    a.sk_S = split;
+    a.sk_tpx = (int)ceil_div(tiles, 8);
+    a.sk_part = reinterpret_cast<float *>(ws);
+    unsigned epoch = ++g_sk_epoch;
+    if (epoch == 0) epoch = ++g_sk_epoch;               // zero is what untouched flags hold
+    a.sk_epoch = epoch;
+    a.sk_flags = g_sk_flags_ptr[dev] + (size_t)(epoch % SK_BANKS) * SK_FLAGS;
+    a.clk = g_clock_probe;
+    dim3 grid((unsigned)(8 * a.sk_tpx * split), 1);
+    constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
+    if (b_kn) hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, 64, 3, 2, 4, true, true, true>), grid, dim3(512), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, 64, 3, 2, 4, false, true, true>), grid, dim3(512), lds, st, a);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
 // tile: index into TILE_MODELS.  The ping-pong kernels take ordinary operands only; a gathered operand (implicit-GEMM
 // convolution) planned onto one of their tiles runs the pipelined kernel's 128 x 256 tile instead: same K order per
 // output, same bits, and the plan (hence the workspace) stays a function of the extents alone.
@@ -1388,6 +1586,7 @@ int launch_tile(int tile, const GemmArgs &a, bool b_kn, int64_t nbatch, hipStrea
 #ifdef MI_LAB
     if (tile == 6) return launch_pp<128, 256, 64, 3, 2, 4, false>(a, b_kn, nbatch, st);
     if (tile == 7) return launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
+    if (tile == 8) return launch_pp<128, 128, 64, 3, 2, 4, true>(a, b_kn, nbatch, st);
 #endif
     switch (tile) {
         case 0: return plain ? launch_pp<128, 256, 64, 3, 2, 4, true>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
@@ -1432,7 +1631,7 @@ constexpr TileModel TILE_MODELS[NTILES] = {
     // 884-938 us on four; the lightly loaded step is scaled from the 128 x 256 tile's ratio
     {256, 256, 1.200, 1.770, 1.00, 9.0},
 };
-struct TilePlan { int tile, split; };
+struct TilePlan { int tile, split; bool peer; };      // peer: the K-slices exchange partial tiles in the kernel (no planes)
 
 double tile_cost_us(int64_t M, int64_t N, int64_t K, int64_t nbatch, int tile, int split) {
     const TileModel &t = TILE_MODELS[tile];
@@ -1446,19 +1645,66 @@ double tile_cost_us(int64_t M, int64_t N, int64_t K, int64_t nbatch, int tile, i
     return us;
 }
 
+// Split-K with the partials exchanged inside the launch (ping-pong kernel; 128 x 256 tiles in 2 or 4 K-slices, or
+// 128 x 128 tiles in 2; every workgroup resident at once): the tile's own estimate at that many workgroups, no planes
+// and no second launch, plus the exchange.  A workgroup writes and reads (S - 1) / S of its accumulators; what that
+// costs is set by how fast the burst drains -- 23 MB from 240 workgroups of 128 x 256 in four slices take 5 to 10 us
+// end to end (stores acknowledged after 1 to 10 us, every wave waiting for its slowest partner), 7.7 MB from 120 or 240
+// workgroups in two slices 2 to 3 us.
+constexpr int SK_TILES[2] = {0, 2};      // indices into TILE_MODELS: 128 x 256, 128 x 128
+double sk_exchange_us(int64_t wg, int bm, int bn, int split) {
+    const double mb = (double)wg * bm * bn * 4.0 * (split - 1) / split / 1e6;
+    return 3.0 + 0.45 * mb;      // fitted: 33.6 us measured on 1500 x 5120 -> 1280 (128 x 128, two slices), 37.8 (128 x 256, four)
+}
+size_t sk_workspace_bytes(int64_t M, int64_t N, int bm, int bn, int split) { return (size_t)(ceil_div(M, bm) * ceil_div(N, bn)) * split * bm * bn * 4; }
+bool sk_fits(int64_t M, int64_t N, int64_t K, int bm, int bn, int split) {
+    const int64_t tiles = ceil_div(M, bm) * ceil_div(N, bn), tpx = ceil_div(tiles, 8);
+    return (split == 2 || (split == 4 && bn == 256)) && K % (64 * split) == 0 && K / split >= 128 && 8 * tpx * split <= g_cus &&
+           8 * tpx * split * 8 <= SK_FLAGS;
+}
+// Before mi_init (planner queries without a device) the path is assumed: a workspace sized for it also holds the planes
+// the same split falls back to.
+bool sk_planned() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return true;
+    return g_sk_state[dev] != -1;
+}
+double sk_cost_us(int64_t M, int64_t N, int64_t K, int tile, int split) {
+    const TileModel &t = TILE_MODELS[tile];
+    const int64_t wg = ceil_div(M, t.bm) * ceil_div(N, t.bn) * split;
+    const double load = (double)wg / (double)g_cus;
+    const double step = t.step_lo + (t.step_full - t.step_lo) * load;
+    return 2.0 + (t.fixed - 2.0) * (0.4 + 0.6 / (double)split) + (t.fixed - 2.0) * 0.4 * load + (double)(K / (64 * split)) * step +
+           sk_exchange_us(wg, t.bm, t.bn, split);
+}
+
 // The plan depends on the extents alone, so a GEMM gives the same bits whichever entry point issues it.
 TilePlan plan_tiles(int64_t M, int64_t N, int64_t K, int64_t nbatch, bool may_split) {
-    TilePlan best = {4, 1};
+    TilePlan best = {4, 1, false};
     double best_us = 1e30;
     const int max_split = (may_split && nbatch == 1 && M > 8 && N % 4 == 0 && K % 64 == 0) ? 8 : 1;
     for (int split = 1; split <= max_split; split++) {
         if (K % (64 * split) != 0 || (split > 1 && K / split < 128)) continue;
         for (int tile = 0; tile < NTILES; tile++) {
             const double us = tile_cost_us(M, N, K, nbatch, tile, split);
-            if (us < best_us) { best_us = us; best = {tile, split}; }
+            if (us < best_us) { best_us = us; best = {tile, split, false}; }
+        }
+        if (max_split > 1 && sk_planned()) {
+            for (int tile : SK_TILES) {
+                if (!sk_fits(M, N, K, TILE_MODELS[tile].bm, TILE_MODELS[tile].bn, split)) continue;
+                const double us = sk_cost_us(M, N, K, tile, split);
+                if (us < best_us) { best_us = us; best = {tile, split, true}; }
+            }
         }
     }
     return best;
+}
+
+// Workspace of a planned split: the planes, or the exchanged partials of the peer reduction (never less than the planes,
+// so a launch that cannot take the peer path -- a gathered operand -- falls back to planes in the same workspace).
+size_t plan_workspace_bytes(const TilePlan &tp, int64_t M, int64_t N) {
+    if (tp.split <= 1) return 0;
+    return round_up(tp.peer ? sk_workspace_bytes(M, N, TILE_MODELS[tp.tile].bm, TILE_MODELS[tp.tile].bn, tp.split) : (size_t)tp.split * M * N * sizeof(float), 256);
 }
 
 int gemm_path(const GemmArgs &a, bool b_kn, int64_t nbatch) {
@@ -1526,6 +1772,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
     a.clk = nullptr;
+    a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
     return MI_OK;
 }
 
@@ -1551,22 +1798,28 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         // second small kernel sums the planes and applies bias, activation and residual.
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
         if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
-        TilePlan tp = {4, 1};
+        TilePlan tp = {4, 1, false};
 #ifdef MI_LAB
         // timing builds only: MI_FORCE_TILE = 1 + tile index (7: ping-pong 128 x 256 with both wave groups in phase,
         // 8: the pipelined kernel's 128 x 256), MI_FORCE_SPLIT = K-slices
         const char *ft = getenv("MI_FORCE_TILE"), *fs = getenv("MI_FORCE_SPLIT");
         const bool forced = pipe && ft && atoi(ft) > 0;
-        if (forced) tp = {atoi(ft) - 1, fs ? atoi(fs) : 1};
+        if (forced) tp = {atoi(ft) - 1, fs ? atoi(fs) : 1, false};
+        if (forced && atoi(ft) == 20) tp = {0, fs ? atoi(fs) : 2, true};      // 20, 21: the peer reduction on 128 x 256, 128 x 128
+        if (forced && atoi(ft) == 21) tp = {2, 2, true};
         if (pipe && !forced) {
 #else
         if (pipe) {
 #endif
             tp = plan_tiles(a.M, a.N, a.K, nbatch, true);
-            if (tp.split > 1 && !(ws && aligned_to(ws, 256) && ws_bytes >= (size_t)tp.split * a.M * a.N * sizeof(float)))
+            if (tp.split > 1 && !(ws && aligned_to(ws, 256) && ws_bytes >= plan_workspace_bytes(tp, a.M, a.N)))
                 tp = plan_tiles(a.M, a.N, a.K, nbatch, false);
         }
         const int split = tp.split;
+        if (split > 1 && tp.peer && ws && aligned_to(ws, 256) && ws_bytes >= plan_workspace_bytes(tp, a.M, a.N)) {
+            const int rc = tp.tile == 0 ? launch_pp_peer<128, 256>(a, b_kn, split, ws, st) : launch_pp_peer<128, 128>(a, b_kn, split, ws, st);
+            if (rc != MI_DECLINE_EXTENT) return rc;     // declined (a gathered operand, a device that failed the probe): planes
+        }
         if (split > 1 && ws && aligned_to(ws, 256) && ws_bytes >= (size_t)split * a.M * a.N * sizeof(float)) {
             GemmArgs s1 = a;
             s1.Y = ws; s1.out_f32 = 1; s1.bias = nullptr; s1.bias_mode = MI_BIAS_NONE; s1.epi = MI_EPI_NONE; s1.residual = nullptr; s1.clamp = 0.0f;
@@ -1615,8 +1868,7 @@ int mi_num_cus() { return g_cus; }
 size_t mi_internal_gemm_workspace(int64_t T, int64_t K, int64_t F, int64_t nbatch) {
     if (T <= 8) return mi_gemm_f16_workspace(T, K, F, MI_W_KF, nbatch);      // decode-sized: the [K][F] kernel's planes
     if (nbatch > 1 || K % 64 || K < 128) return 0;
-    const int split = plan_tiles(T, F, K, 1, true).split;
-    return split > 1 ? round_up((size_t)split * T * F * sizeof(float), 256) : 0;
+    return plan_workspace_bytes(plan_tiles(T, F, K, 1, true), T, F);
 }
 
 // Internal entry used by the convolution path (conv.hip): Y[M x N] = A . B with
@@ -1631,6 +1883,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
     a.clk = nullptr;
+    a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
@@ -1682,9 +1935,15 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true>, pp_lds_bytes<128, 256, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, true>, pp_lds_bytes<128, 256, 64, 3>());
 #ifdef MI_LAB
+    bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, true, true>, pp_lds_bytes<128, 128, 64, 3>());
+    bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, false, true>, pp_lds_bytes<128, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, false>, pp_lds_bytes<128, 256, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, false>, pp_lds_bytes<128, 256, 64, 3>());
 #endif
+    bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 128, 64, 3>());
+    bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, false, true, true>, pp_lds_bytes<128, 128, 64, 3>());
+    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 256, 64, 3>());
+    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, true, true>, pp_lds_bytes<128, 256, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, true, true>, pp_lds_bytes<256, 256, 32, 4>());
     bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, false, true>, pp_lds_bytes<256, 256, 32, 4>());
     bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 1, 2>, lna_lds_bytes<128, 2, 4>(LNA_KMAX));
@@ -1697,6 +1956,7 @@ int mi_init(void) {
     bad |= raise_lds(skinny_fk_kernel<8>, (int)SKINNY_FK_LDS_MAX);
     bad |= mi_sdpa_init();
     bad |= scratch_of_current_device() == nullptr;
+    sk_probe_current_device();      // a device that fails the probe only loses that path
     if (bad) return MI_ERROR_DEVICE;
     g_ready = true;
     return MI_OK;
@@ -1726,8 +1986,7 @@ size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int6
     if (T < 1 || nbatch > 1) return 0;
     if (T > 8) {
         if (K % 64 || K < 128) return 0;
-        const int split = plan_tiles(T, F, K, 1, true).split;
-        return split > 1 ? round_up((size_t)split * T * F * sizeof(float), 256) : 0;
+        return plan_workspace_bytes(plan_tiles(T, F, K, 1, true), T, F);
     }
     if (w_layout != MI_W_KF) return 0;      // the [F][K] skinny kernel finishes its outputs itself
     return round_up((size_t)skinny_splits(K, F) * T * F * sizeof(float), 256);

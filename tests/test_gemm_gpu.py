@@ -171,6 +171,41 @@ def test_split_k_narrow_outputs(ctx, layout):
     _run(ctx, 1500, 5120, 1280, layout=layout, residual=True, seed=7)
 
 
+def test_split_k_partials_exchanged_inside_the_launch(ctx):
+    """Config 2's second MLP linear (1500 x 5120 -> 1280) splits K over two workgroups per 128 x 128 tile that exchange
+    their partial tiles through L2 and per-wave arrival flags instead of writing fp32 planes.  The flags carry a
+    per-launch epoch and are never cleared: forty launches back to back on one stream, alternating two problems in one
+    workspace, must each give the bits of the first launch of that problem; and the result meets the oracle."""
+    import torch
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    st = torch.cuda.current_stream().cuda_stream
+    cases = []
+    for (T, K, F, seed) in ((1500, 5120, 1280, 3), (700, 2560, 640, 4)):
+        X = oracle.randn_f16((T, K), seed, 0, 1.0 / np.sqrt(K))
+        W = oracle.randn_f16((K, F), seed + 10)
+        b = oracle.randn_f16((F,), seed + 20, 0, 0.02)
+        R = oracle.randn_f16((T, F), seed + 30)
+        need = lib.mi_gemm_f16_workspace(T, K, F, L.W_KF, 1)
+        assert need > 0
+        cases.append((T, K, F, X, W, b, R, to_dev(X), to_dev(W), to_dev(b), to_dev(R), need))
+    ws = torch.empty(max(c[-1] for c in cases), dtype=torch.uint8, device="cuda")
+    outs = [[], []]
+    for rep in range(20):
+        for ci, (T, K, F, X, W, b, R, dX, dW, db, dR, need) in enumerate(cases):
+            y = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+            rc = lib.mi_gemm_f16(y.data_ptr(), dX.data_ptr(), dW.data_ptr(), db.data_ptr(), dR.data_ptr(), T, K, F, F, K, F,
+                                 L.W_KF, L.BIAS_COL, L.EPI["gelu"], L.F16, ws.data_ptr(), need, st)
+            assert rc == L.OK
+            outs[ci].append(y)
+    torch.cuda.synchronize()
+    for ci, (T, K, F, X, W, b, R, *_rest) in enumerate(cases):
+        first = to_host(outs[ci][0])
+        assert_parity(first, oracle.gemm_f16(X, W, b, epi="gelu", residual=R), what=f"peer split-K {T}x{K}x{F}")
+        for y in outs[ci][1:]:
+            assert np.array_equal(to_host(y).view(np.uint16), first.view(np.uint16)), "a later launch differs from the first"
+
+
 @pytest.mark.parametrize("layout", ["kf", "fk"])
 @pytest.mark.parametrize("T,K,F", [(1, 1280, 1280), (4, 1280, 3840), (8, 264, 136), (3, 2048, 520)])
 def test_layer_norm_folded_into_decode_sized_gemv(ctx, T, K, F, layout):
