@@ -690,7 +690,8 @@ def detail_benchmarks(lib, L, stream, only=None):
                      "weight_GB/s": round(wbytes / med / 1e9, 1)}
         return out[name]
 
-    def attn_case(name, B, H, Lq, Lk, E, kv_len=None, sets=NB, reps=10):
+    def attn_case(name, B, H, Lq, Lk, E, kv_len=None, sets=NB, reps=10, mask=None):
+        """mask: None, "pad" ((B,1,1,Lk) fp16 0 / finfo.min padding mask) or "full" (dense fp16 (B,H,Lq,Lk))."""
         if only is not None and only not in name:
             return
         qs = [torch.randn((B, H, Lq, E), dtype=f16, device="cuda") for _ in range(sets)]
@@ -701,8 +702,16 @@ def detail_benchmarks(lib, L, stream, only=None):
         need = lib.mi_sdpa_f16_workspace(E, Lq, Lk, H, B, 0)
         ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
         dq, dk = L.strides4(1, E, E * Lq, E * Lq * H), L.strides4(1, E, E * Lk, E * Lk * H)
+        mk, mst = None, None
+        if mask == "pad":
+            mk = torch.zeros((B, 1, 1, Lk), dtype=f16, device="cuda")
+            mk[..., Lk - 100:] = torch.finfo(f16).min
+            mst = L.strides4(1, 0, 0, Lk)
+        elif mask == "full":
+            mk = torch.randn((B, H, Lq, Lk), dtype=f16, device="cuda")
+            mst = L.strides4(1, Lk, Lk * Lq, Lk * Lq * H)
         calls = [Call(lib.mi_sdpa_f16, o.data_ptr(), L.F16, None, qs[i].data_ptr(), dq, ks[i].data_ptr(), dk, vs[i].data_ptr(), dk,
-                      None, 0, None, (kl.data_ptr() if kl is not None else None), E, Lq, Lk, H, B, 1.0 / np.sqrt(E),
+                      (mk.data_ptr() if mk is not None else None), L.F16, mst, (kl.data_ptr() if kl is not None else None), E, Lq, Lk, H, B, 1.0 / np.sqrt(E),
                       ws.data_ptr(), need, stream) for i in range(sets)]
         state = {"i": 0}
 
@@ -727,6 +736,9 @@ def detail_benchmarks(lib, L, stream, only=None):
     gemm_case("c3_fc2_1370x1536x384", 1370, 1536, 384, L.W_KF)
     attn_case("c3_attn_L1370_6x64", 1, 6, 1370, 1370, 64)
     attn_case("c2_attn_L1500_20x64", 1, 20, 1500, 1500, 64)
+    # the same attention with an additive mask: it stays in the fused kernel (the reference's fused plan declines masks)
+    attn_case("c2_attn_L1500_20x64_padding_mask", 1, 20, 1500, 1500, 64, mask="pad")
+    attn_case("c2_attn_L1500_20x64_dense_fp16_mask", 1, 20, 1500, 1500, 64, mask="full")
     # the reference's own SAM 2.1 attention shapes, head size 72: global blocks and 16 windows of 256 (tools/attn_lab.jl:8-14)
     attn_case("sam2_global_attn_L4096_8x72", 1, 8, 4096, 4096, 72)
     attn_case("sam2_window_attn_L256_8x72_b16", 16, 8, 256, 256, 72)

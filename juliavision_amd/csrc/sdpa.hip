@@ -94,8 +94,15 @@ __device__ __forceinline__ void static_for(F &&f) {
 // 128 bytes of the banks (96 for head sizes 64 and 96, 160 for 128; 112 measured the same as 96 at 96).
 constexpr int flash_vld(int EP) { return EP == 96 ? EP : EP + 32; }
 
-template <int EP, bool PP, int KH = 1>
+//
+// BIAS (four-wave form only): an additive mask (Lk, Lq, H, B), keys contiguous, fp16 or fp32, any of the other axes
+// broadcast.  A lane owns one query and, per block, eight runs of four consecutive keys: its 32 mask values of block
+// j + 1 are requested while block j is worked on (two register sets, like the scores) and join the scores, times
+// log2(e), ahead of the exponentials -- the reference's bias term of attention.jl:55-59, which its own fused kernel
+// declines (flash.jl:1327).
+template <int EP, bool PP, int KH = 1, int BIAS = 0>      // BIAS: 0 none, 1 fp16, 2 fp32
 __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH == 1) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
+    static_assert(BIAS == 0 || (!PP && KH == 1), "the mask rides in the four-wave form");
     // PP with KH = 2: the two key-half groups of the eight-wave form (same 128 queries) take turns at the vector
     // and matrix units like the two query groups of the 256-query form do; every thread stages.
     constexpr int BC = 64, BR = (PP && KH == 1) ? 256 : 128, NT = KH == 2 ? 512 : 256;     // NT: threads that stage K and V
@@ -285,16 +292,80 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
             }
     };
 
+    // The lane's mask values of one key block: eight runs of four keys (tile kt, register group g: keys
+    // key0 + 32 kt + 8 g + 4 hl .. +3), raw as they lie in memory.  Runs past the last key read nothing.
+    struct BiasRegs { u32x4 w[BIAS == 2 ? 8 : (BIAS == 1 ? 4 : 1)]; };
+    const char *brow = nullptr;
+    if constexpr (BIAS != 0) {
+        const int qr = min(q0 + l32, p.Lq - 1);
+        brow = reinterpret_cast<const char *>(p.bias) + ((long)qr * p.bs[1] + (long)h * p.bs[2] + (long)b * p.bs[3]) * (BIAS == 2 ? 4 : 2);
+    }
+    auto load_bias = [&](BiasRegs &br, int j) {
+        if constexpr (BIAS != 0) {
+            const int key0 = j * BCS + gk;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int key = key0 + 32 * kt + 8 * g + 4 * hl, idx = kt * 4 + g;
+                    if constexpr (BIAS == 2) {
+                        float4v v = {0.f, 0.f, 0.f, 0.f};
+                        const float *src = reinterpret_cast<const float *>(brow) + key;
+                        if (key + 3 < p.Lk) v = *reinterpret_cast<const float4v *>(src);
+                        else for (int e = 0; e < 4; e++) if (key + e < p.Lk) v[e] = src[e];
+                        br.w[idx] = __builtin_bit_cast(u32x4, v);
+                    } else {
+                        u32x2 v = {0u, 0u};
+                        const half_t *src = reinterpret_cast<const half_t *>(brow) + key;
+                        if (key + 3 < p.Lk) v = *reinterpret_cast<const u32x2 *>(src);
+                        else {
+                            half4v t = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+                            for (int e = 0; e < 4; e++) if (key + e < p.Lk) t[e] = src[e];
+                            v = __builtin_bit_cast(u32x2, t);
+                        }
+                        br.w[idx >> 1][(idx & 1) * 2] = v[0];
+                        br.w[idx >> 1][(idx & 1) * 2 + 1] = v[1];
+                    }
+                }
+        }
+    };
+    auto add_bias = [&](float16v (&sc)[2], const BiasRegs &br) {
+        if constexpr (BIAS != 0) {
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int idx = kt * 4 + g;
+                    if constexpr (BIAS == 2) {
+                        const float4v v = __builtin_bit_cast(float4v, br.w[idx]);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) sc[kt][4 * g + e] = fmaf(v[e], LOG2E, sc[kt][4 * g + e]);
+                    } else {
+                        const u32x2 raw = {br.w[idx >> 1][(idx & 1) * 2], br.w[idx >> 1][(idx & 1) * 2 + 1]};
+                        const half4v v = __builtin_bit_cast(half4v, raw);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) sc[kt][4 * g + e] = fmaf((float)v[e], LOG2E, sc[kt][4 * g + e]);
+                    }
+                }
+        }
+    };
+    BiasRegs ba, bb;
+    if (nblk > 0) load_bias(ba, 0);
+
     float16v sa[2], sb[2];
     if (nblk > 0) qk(sa, 0);
 
     // One key block: sc holds its scores (computed one iteration earlier), sn receives the next block's.
-    auto iter = [&](auto MASK_, float16v (&sc)[2], float16v (&sn)[2], int j) {
+    auto iter = [&](auto MASK_, float16v (&sc)[2], float16v (&sn)[2], BiasRegs &bc, BiasRegs &bn, int j) {
         constexpr bool MASK = decltype(MASK_)::value;
         const int key0 = j * BCS + gk;
         const int st = j % 3, st1 = (j + 1) % 3, st2 = (j + 2) % 3;
         const bool next2 = j + 2 < nblk && loader;
         if (next2) load_kv((j + 2) * BCS);
+        if constexpr (BIAS != 0) {
+            if (j + 1 < nblk) load_bias(bn, j + 1);
+            add_bias(sc, bc);
+        }
         if constexpr (MASK) {           // the ragged last block: excluded keys get -inf
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
@@ -407,22 +478,22 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     if (PP && grp == 1) pp_barrier();    // waves 4-7 run half a block behind waves 0-3
     int j = 0;
     for (; j + 2 <= nfull; j += 2) {
-        iter(std::false_type{}, sa, sb, j);
-        iter(std::false_type{}, sb, sa, j + 1);
+        iter(std::false_type{}, sa, sb, ba, bb, j);
+        iter(std::false_type{}, sb, sa, bb, ba, j + 1);
     }
     if constexpr (KH == 1) {
         if (j < nfull) {
-            iter(std::false_type{}, sa, sb, j);
-            if (j + 1 < nblk) iter(std::true_type{}, sb, sa, j + 1);
+            iter(std::false_type{}, sa, sb, ba, bb, j);
+            if (j + 1 < nblk) iter(std::true_type{}, sb, sa, bb, ba, j + 1);
         } else if (j < nblk) {
-            iter(std::true_type{}, sa, sb, j);
+            iter(std::true_type{}, sa, sb, ba, bb, j);
         }
     } else {
         // Both halves of the workgroup run all nblk blocks (every block has a workgroup barrier), whatever
         // share of them is masked for this half: at most one full block is left here, then masked ones.
-        if (j < nblk) { if (j < nfull) iter(std::false_type{}, sa, sb, j); else iter(std::true_type{}, sa, sb, j); j++; }
-        if (j < nblk) { iter(std::true_type{}, sb, sa, j); j++; }
-        if (j < nblk) { iter(std::true_type{}, sa, sb, j); j++; }
+        if (j < nblk) { if (j < nfull) iter(std::false_type{}, sa, sb, ba, bb, j); else iter(std::true_type{}, sa, sb, ba, bb, j); j++; }
+        if (j < nblk) { iter(std::true_type{}, sb, sa, bb, ba, j); j++; }
+        if (j < nblk) { iter(std::true_type{}, sa, sb, ba, bb, j); j++; }
     }
 
     if (PP && grp == 0) pp_barrier();    // ... so waves 0-3 meet their last barrier here
@@ -914,12 +985,20 @@ bool one_pass_decode(const SdpaArgs &a, bool vec) {
     return a.Lq == 1 && vec && !a.bias && a.E <= 64 && a.Lk >= 1 && a.Lk <= 640;
 }
 
+// A mask the fused kernel can carry: keys contiguous (a lane reads runs of four), the other axes any stride including
+// broadcast; fp16 runs are read as two dwords, so every row must start on a 4-byte boundary.
+bool flash_bias_ok(const SdpaArgs &a) {
+    if (a.bs[0] != 1 && a.Lk != 1) return false;
+    if (a.bias_f32) return aligned_to(a.bias, 4);
+    return aligned_to(a.bias, 4) && a.bs[1] % 2 == 0 && a.bs[2] % 2 == 0 && a.bs[3] % 2 == 0;
+}
+
 int sdpa_path(const SdpaArgs &a) {
     if (a.E < 1 || a.E > 256 || a.Lq < 0 || a.Lk < 0 || a.H < 1 || a.B < 1) return MI_SDPA_DECLINE;
     if (a.H > 65535 || a.B > 65535 || (int64_t)a.Lq * a.H * 64 > INT32_MAX) return MI_SDPA_DECLINE;
     bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
     bool out_ok = (aligned_to(a.out, 16) || a.out == nullptr) && a.os[0] == 1 && a.os[1] % 8 == 0 && a.os[2] % 8 == 0 && a.os[3] % 8 == 0;
-    if (vec && out_ok && !a.bias && a.scale > 0.0f && a.E <= 128 && a.Lq >= 64 && a.Lk >= 1) return MI_SDPA_FLASH;
+    if (vec && out_ok && (!a.bias || flash_bias_ok(a)) && a.scale > 0.0f && a.E <= 128 && a.Lq >= 64 && a.Lk >= 1) return MI_SDPA_FLASH;
     return MI_SDPA_ROWS;
 }
 
@@ -960,6 +1039,12 @@ int mi_sdpa_init() {
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false, 1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false, 1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false, 1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false, 1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     return bad;
 }
 
@@ -980,13 +1065,15 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
     (void)has_kv_len;
     SdpaArgs a;
     static const int64_t zero4[4] = {0, 0, 0, 0};
+    // a mask is planned as a dense fp16 (Lk, Lq, H, B) array: what an exported graph hands over
+    const int64_t dense4[4] = {1, Lk, Lk * Lq, Lk * Lq * H};
     int rc = fill(a, nullptr, MI_F16, nullptr, q, q_strides, k, k_strides, v, v_strides, has_bias ? (const void *)q : nullptr, MI_F16,
-                  zero4, nullptr, E, Lq, Lk, H, B, scale);
+                  has_bias ? dense4 : zero4, nullptr, E, Lq, Lk, H, B, scale);
     if (rc != MI_OK) return MI_SDPA_DECLINE;
     int path = sdpa_path(a);
     const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
     if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? (one_pass_decode(a, vec) ? 1 : rows_splits(Lq, Lk, H, B))
-                                  : path == MI_SDPA_FLASH ? flash_splits(E, Lq, Lk, H, B) : 1;
+                                  : (path == MI_SDPA_FLASH && !has_bias) ? flash_splits(E, Lq, Lk, H, B) : 1;
     return path;
 }
 
@@ -1007,8 +1094,19 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
     if (path == MI_SDPA_DECLINE) return MI_DECLINE_EXTENT;
     if (path == MI_SDPA_FLASH) {
         // The 8-wave ping-pong kernel when 256-query workgroups still cover most of the chip.
-        const bool pp = E <= 64 && ceil_div(Lq, 256) * H * B * 4 >= (int64_t)mi_num_cus() * 3;
-        if (pp) {
+        const bool pp = !a.bias && E <= 64 && ceil_div(Lq, 256) * H * B * 4 >= (int64_t)mi_num_cus() * 3;
+        if (a.bias) {
+            // the mask rides in the four-wave form, keys unsplit
+            a.nsplit = 1;
+            dim3 grid((unsigned)ceil_div(Lq, 128), (unsigned)H, (unsigned)B);
+            const bool f32 = a.bias_f32 != 0;
+            if (E <= 64)      { if (f32) hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 2>), grid, dim3(256), flash_lds_bytes(64), st, a);
+                                else     hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 1>), grid, dim3(256), flash_lds_bytes(64), st, a); }
+            else if (E <= 96) { if (f32) hipLaunchKernelGGL((flash_fwd_kernel<96, false, 1, 2>), grid, dim3(256), flash_lds_bytes(96), st, a);
+                                else     hipLaunchKernelGGL((flash_fwd_kernel<96, false, 1, 1>), grid, dim3(256), flash_lds_bytes(96), st, a); }
+            else              { if (f32) hipLaunchKernelGGL((flash_fwd_kernel<128, false, 1, 2>), grid, dim3(256), flash_lds_bytes(128), st, a);
+                                else     hipLaunchKernelGGL((flash_fwd_kernel<128, false, 1, 1>), grid, dim3(256), flash_lds_bytes(128), st, a); }
+        } else if (pp) {
             dim3 grid((unsigned)ceil_div(Lq, 256), (unsigned)H, (unsigned)B);
             hipLaunchKernelGGL((flash_fwd_kernel<64, true>), grid, dim3(512), flash_lds_bytes(64), st, a);
         } else {

@@ -441,7 +441,20 @@ def sdpaplan(ctx: Ctx, q, k, v, bias=None, scale=None, kv_len=None):
     scale = (1.0 / math.sqrt(E)) if scale is None else float(scale)
     ns = C.c_int(1)
     path = L.load().mi_sdpa_f16_plan(q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k), v.data_ptr(), _strides_elbh(v),
-                                     int(bias is not None), int(kv_len is not None), E, Lq, Lk, H, Bq, scale, C.byref(ns))
+                                     0, int(kv_len is not None), E, Lq, Lk, H, Bq, scale, C.byref(ns))
+    if bias is not None:
+        # The fused kernel carries a mask whose keys are contiguous and whose fp16 rows start on 4-byte boundaries (any
+        # other axis may broadcast); everything else is the rows kernel's.  The C planner sees only "a mask" and plans a
+        # dense fp16 one, so the mask's own layout is judged here, as mi_sdpa_f16 judges it at the call.
+        bst = list(_bias_strides(bias, Lk, Lq, H, Bq))
+        fused = path == 1 and (bst[0] == 1 or Lk == 1) and bias.data_ptr() % 4 == 0 and \
+            (bias.dtype == torch.float32 or all(x % 2 == 0 for x in bst[1:]))
+        if fused:
+            return FlashPlan(1)
+        ns1 = C.c_int(1)
+        L.load().mi_sdpa_f16_plan(q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k), v.data_ptr(), _strides_elbh(v),
+                                  1, int(kv_len is not None), E, Lq, Lk, H, Bq, scale, C.byref(ns1))
+        return RowsSDPAPlan(ns1.value if Lq < 64 else 1) if path in (1, 2) else Decline("extent")
     if path == 1:
         return FlashPlan(ns.value)
     if path == 2:

@@ -118,7 +118,47 @@ def test_full_bias_f32(ctx):
     B, H, Lq, Lk, E = 1, 2, 70, 90, 64
     q, k, v = _qkv(B, H, Lq, Lk, E, 81)
     bias = oracle.randn_f32((B, H, Lq, Lk), 84)
-    _check(ctx, q, k, v, bias=bias, expect="RowsSDPAPlan", what="full f32 bias")
+    _check(ctx, q, k, v, bias=bias, expect="FlashPlan", what="full f32 bias")
+    _check(ctx, q[:, :, :40], k, v, bias=bias[:, :, :40].copy(), expect="RowsSDPAPlan", what="full f32 bias, 40 query rows")
+
+
+@pytest.mark.parametrize("B,H,Lq,Lk,E,kind", [
+    (2, 3, 200, 136, 64, "pad16"),        # (B,1,1,Lk) fp16 0 / finfo.min padding mask, broadcast over heads and queries
+    (1, 2, 130, 260, 64, "full16"),       # dense fp16 (B,H,Lq,Lk), ragged last key block (260 = 4 x 64 + 4)
+    (1, 2, 300, 333, 64, "full32"),       # dense fp32, an odd row length (fp32 rows are always dword aligned)
+    (2, 2, 128, 130, 72, "causal16"),     # 0 / -inf lower-triangular mask (Lq, Lk) broadcast over batch and heads, head size 72
+    (1, 1, 192, 320, 128, "full32"),      # the 128-wide instance
+    (1, 20, 1500, 1500, 64, "pad16"),     # config 2's attention with a padding mask
+])
+def test_additive_mask_rides_in_the_fused_kernel(ctx, B, H, Lq, Lk, E, kind):
+    """Encoder-sized attention with an additive mask: the mask tile joins the scores inside the fused kernel (the
+    reference's own fused plan declines masks, flash.jl:1327, and falls to its three-pass form, attention.jl:55-59)."""
+    q, k, v = _qkv(B, H, Lq, Lk, E, 87)
+    if kind == "pad16":
+        valid = [Lk - 7 * (b + 1) for b in range(B)]
+        bias = np.zeros((B, 1, 1, Lk), dtype=np.float16)
+        for b in range(B):
+            bias[b, :, :, valid[b]:] = np.finfo(np.float16).min
+    elif kind == "full16":
+        bias = oracle.randn_f16((B, H, Lq, Lk), 88)
+    elif kind == "full32":
+        bias = oracle.randn_f32((B, H, Lq, Lk), 89)
+    else:
+        bias = np.where(np.arange(Lk)[None, :] <= np.arange(Lq)[:, None] + (Lk - Lq), 0.0, -np.inf).astype(np.float16).reshape(1, 1, Lq, Lk)
+    got = _check(ctx, q, k, v, bias=bias, expect="FlashPlan", what=f"fused mask {kind} {B},{H},{Lq},{Lk},{E}")
+    if kind == "pad16":       # the same thing said with kv_len
+        other = _check(ctx, q, k, v, kv_len=valid, expect="FlashPlan", what="kv_len twin")
+        np.testing.assert_allclose(got.astype(np.float32), other.astype(np.float32), rtol=2e-3, atol=2e-3)
+
+
+def test_mask_the_fused_kernel_cannot_read_takes_the_rows_kernel(ctx):
+    q, k, v = _qkv(1, 2, 128, 129, 64, 90)
+    bias = oracle.randn_f16((1, 2, 128, 129), 91)                     # fp16 rows of 129: every other row at a 2-byte offset
+    _check(ctx, q, k, v, bias=bias, expect="RowsSDPAPlan", what="odd fp16 rows")
+    import torch
+    bt = to_dev(oracle.randn_f16((1, 2, 136, 128), 92)).transpose(2, 3)      # (B,H,Lq=128,Lk=136) with the queries contiguous
+    _check(ctx, q[:, :, :, :], oracle.randn_f16((1, 2, 136, 64), 93), oracle.randn_f16((1, 2, 136, 64), 94), bias=None, what="sanity")
+    assert type(__import__("juliavision_amd").sdpaplan(ctx, to_dev(q), to_dev(oracle.randn_f16((1, 2, 136, 64), 93)), to_dev(oracle.randn_f16((1, 2, 136, 64), 94)), bt)).__name__ == "RowsSDPAPlan"
 
 
 def test_all_masked_rows_give_zeros(ctx):
