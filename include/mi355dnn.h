@@ -354,7 +354,10 @@ int mi_add_f16(void *out, const void *a, const void *b, int64_t n, void *stream)
  *
  * cache_k/cache_v: (E, Lmax, H, B) with element strides cache_strides, E contiguous.
  * k_new/v_new: (E, 1, H, B) with element strides new_strides (the L stride is unused).
- * A row whose kv_len is 0 or exceeds Lmax is left untouched. */
+ * A row whose kv_len is 0 or exceeds Lmax is left untouched: a caller that advances with cap = Lmax + 1 gets
+ * "length Lmax + 1" as the mark of a step that found the cache full -- nothing stored (here and in
+ * mi_sdpa_append_f16), attention over the Lmax stored keys -- and can read it back; with cap = Lmax the counter
+ * saturates silently and each further step overwrites the last slot. */
 int mi_kv_append_f16(void *cache_k, void *cache_v, const int64_t cache_strides[4], int64_t Lmax,
                      const void *k_new, const void *v_new, const int64_t new_strides[4],
                      const int32_t *kv_len, int64_t E, int64_t H, int64_t B, void *stream);
@@ -374,6 +377,21 @@ int mi_sdpa_append_f16(void *out, int out_dtype, const int64_t out_strides[4],
 /* kv_len[b] = clamp(kv_len[b] + delta, 0, cap) for b < B, on the device
  * (KVCache.position += 1, decode.jl:201, without the host in the loop). */
 int mi_kv_advance(int32_t *kv_len, int64_t B, int32_t delta, int32_t cap, void *stream);
+/* kv_len[b] = clamp(position[b] + 1, 0, cap) for b < B, on the device; npos = 1 (one position for every row, as
+ * the exported step's cache_position input has it) or B.  The exported decoder step names the slot its new token
+ * is written to (cache_position, int64; tools/export_whisper_decoder.py:158-181, decode.jl:186-203); the kernels
+ * here count valid keys, which is that slot + 1.  mi_kv_advance saturates at cap, and so does this: a caller that
+ * steps past the capacity overwrites the last slot, unless cap = capacity + 1 is passed (see mi_kv_append_f16). */
+int mi_kv_len_from_position(int32_t *kv_len, const int64_t *position, int64_t npos, int64_t B, int32_t cap, void *stream);
+
+/* out[i, :] = table[ids[i], :] (+ table2[ids2[i], :], or table2[ids2[0], :] when n2 = 1) for i < n: rows of D
+ * contiguous fp16 elements, int64 ids, tables V x D and V2 x D, table2 = NULL for a plain gather; the sum is fp32,
+ * rounded once.  aten::embedding (embedding_kernel!, ops.jl:1754-1783), the row gather of aten::index.Tensor along
+ * the first axis (ops.jl:1524-1640), and -- with both tables -- the decoder step's token embedding + position
+ * embedding (tools/export_whisper_decoder.py:150-152) in one launch.  An id outside its table contributes a row
+ * of zeros (torch raises there; the reference reads out of bounds). */
+int mi_embedding_f16(void *out, const void *table, const int64_t *ids, int64_t n, int64_t D, int64_t V,
+                     const void *table2, const int64_t *ids2, int64_t n2, int64_t V2, void *stream);
 
 #ifdef __cplusplus
 }

@@ -67,6 +67,8 @@ SIGNATURES = {
     "mi_kv_append_f16": (_int, [_vp, _vp, _i64p, _i64, _vp, _vp, _i64p, _vp, _i64, _i64, _i64, _vp]),
     "mi_sdpa_append_f16": (_int, [_vp, _int, _i64p, _vp, _i64p, _vp, _i64p, _vp, _i64p, _vp, _vp, _i64p, _vp, _i64, _i64, _i64, _i64, _f32, _vp]),
     "mi_kv_advance": (_int, [_vp, _i64, C.c_int32, C.c_int32, _vp]),
+    "mi_kv_len_from_position": (_int, [_vp, _vp, _i64, _i64, C.c_int32, _vp]),
+    "mi_embedding_f16": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _vp]),
 }
 
 _lib = None

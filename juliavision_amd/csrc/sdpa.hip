@@ -791,7 +791,8 @@ __global__ __launch_bounds__(512) void sdpa_decode_kernel(SdpaArgs p) {
     const int grp = lane >> 3, cl = lane & 7;
     const int h = blockIdx.x, b = blockIdx.z;
     int Lk = p.Lk;
-    if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
+    bool room = true;                          // a length past the capacity: the cache is full, the new row is not stored
+    if (p.kv_len) { const int n = p.kv_len[b]; room = n <= Lk; Lk = max(0, min(Lk, n)); }
     const half_t *qp = p.q + h * p.qs[2] + b * p.qs[3];
     const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
     const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
@@ -806,7 +807,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_kernel(SdpaArgs p) {
             const int key = 64 * (t0 + u) + 8 * wave + grp;
             const int kk = min(key, Lk - 1);
             const bool on = eok && 64 * (t0 + u) < Lk;           // uniform over the workgroup in its second half
-            const bool fresh = p.k_new && kk == Lk - 1;          // the row that this step appends
+            const bool fresh = p.k_new && room && kk == Lk - 1;  // the row that this step appends
             const half_t *kp = fresh ? p.k_new + h * p.ns[2] + b * p.ns[3] : kb + (long)kk * p.ks[1];
             const half_t *vp = fresh ? p.v_new + h * p.ns[2] + b * p.ns[3] : vb + (long)kk * p.vs[1];
             kc[set][u] = on ? ldg16(kp + e0) : z;

@@ -45,10 +45,17 @@ class KVCache:
         self.length.zero_()
 
     def advance(self, ctx: Ctx, delta: int = 1):
-        """length += delta on the device (``c.position += 1``, decode.jl:201)."""
-        rc = L.init().mi_kv_advance(self.length.data_ptr(), self.batch, int(delta), self.max_target, ctx.stream)
+        """length += delta on the device (``c.position += 1``, decode.jl:201).  The counter stops at ``max_target + 1``:
+        a step that finds the cache full stores nothing, attends over the stored keys and leaves that mark, which
+        ``overflowed()`` reads back (the reference's greedy loop bounds its token count on the host, decode.jl:206-230; a
+        replayed graph has no host in the loop, so the device keeps the evidence instead)."""
+        rc = L.init().mi_kv_advance(self.length.data_ptr(), self.batch, int(delta), self.max_target + 1, ctx.stream)
         if rc != L.OK:
             raise DeclineError("mi_kv_advance", rc)
+
+    def overflowed(self) -> bool:
+        """True if some row was stepped past ``max_target`` since the last ``reset()`` (synchronises with the device)."""
+        return bool((self.length > self.max_target).any().item())
 
     def fill_cross(self, ctx: Ctx, layer: int, enc: torch.Tensor, wk, bk, wv, bv):
         """Project the encoder output into ``layer``'s cross-attention K/V, once per window (fillcross!, decode.jl:173-177:

@@ -30,14 +30,30 @@ token-major when the graph transposes it straight back (``fold_sdpa_transpose``)
 attention exported as ``bmm`` + ``_softmax`` + ``bmm`` (DINOv2) is put back together
 (``fold_attention``).
 
+The decoder step (tools/export_whisper_decoder.py:90-240) is functional: it takes
+the self-attention cache, writes the new token's rows with ``index_copy`` /
+``index_put``, masks the unwritten slots with ``arange <= cache_position`` and
+returns the whole cache through ``stack`` / ``cat``; the reference copies the tensor
+once per write and once more on the host (ops.jl:1018-1023, decode.jl:186-203).
+``fold_cache_step`` turns that into an in-place write on the input cache fused with
+the attention launch, the mask into a device-side count of valid keys, and the
+returned cache into an alias of the input -- the "output aliases input" the
+reference's schema cannot say.  ``embedding`` and the first-axis ``index.Tensor``
+gather run as one kernel (``fold_embedding_sum`` joins the token and position rows).
+
 An op outside the list raises :class:`UnsupportedOp`; there is no eager fallback.
-``convert`` produces the schema from an ``ExportedProgram`` (static shapes only),
-so a graph can be built and run without the reference's tooling.
+``convert`` produces the schema from an ``ExportedProgram`` -- extents that
+``torch.export`` left symbolic are written as expressions in the base symbols, as
+the reference's exporter writes them (export_graphs.py:75-90) -- and ``Graph.load``
+binds them to integers (``evalshape``, graph.jl:150-205), so a graph can be built
+and run without the reference's tooling.
 """
 from __future__ import annotations
 
+import ast
 import json
 import math
+from fractions import Fraction
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 
@@ -60,6 +76,15 @@ SDPA_OPS = {"scaled_dot_product_attention.default": (4, 5),
             "_scaled_dot_product_efficient_attention.default": (5, 6)}
 
 
+def _mentions(text: str, names: set) -> bool:
+    """Does ``text`` parse as an expression that uses one of ``names``?  (An attribute such as ``"float16"`` does not.)"""
+    try:
+        tree = ast.parse(text, mode="eval")
+    except SyntaxError:
+        return False
+    return any(isinstance(n, ast.Name) and n.id in names for n in ast.walk(tree))
+
+
 class UnsupportedOp(NotImplementedError):
     """An ATen op with no kernel on this path (the reference would route it to one of its other kernels)."""
 
@@ -80,11 +105,69 @@ def _const(x):
     return str(x)
 
 
+def _dim(d, symbols: set):
+    """One extent: an int, or -- where the export left it symbolic -- its expression in the base symbols as text."""
+    if isinstance(d, (int, bool)):
+        return int(d)
+    expr = d.node.expr if hasattr(d, "node") else d
+    if getattr(expr, "is_Integer", False):
+        return int(expr)
+    symbols.update(str(x) for x in getattr(expr, "free_symbols", ()))
+    return str(expr)
+
+
+def _note_symbols(x, symbols: set):
+    if isinstance(x, (list, tuple)):
+        for v in x:
+            _note_symbols(v, symbols)
+    elif isinstance(x, (torch.SymInt, torch.SymFloat, torch.SymBool)):
+        _dim(x, symbols)
+
+
+_BINOPS = {ast.Add: lambda a, b: a + b, ast.Sub: lambda a, b: a - b, ast.Mult: lambda a, b: a * b,
+           ast.FloorDiv: lambda a, b: a // b, ast.Div: lambda a, b: Fraction(a) / Fraction(b), ast.Mod: lambda a, b: a % b,
+           ast.Pow: lambda a, b: a ** b}
+_CALLS = {"Mod": lambda a, b: a % b, "Max": max, "Min": min, "Pow": lambda a, b: a ** b,
+          "floor": lambda a, *b: math.floor(Fraction(a) / Fraction(b[0])) if b else math.floor(a),
+          "floordiv": lambda a, b: a // b, "FloorDiv": lambda a, b: a // b,
+          "ceiling": lambda a, *b: math.ceil(Fraction(a) / Fraction(b[0])) if b else math.ceil(a),
+          "CeilDiv": lambda a, b: math.ceil(Fraction(a) / Fraction(b))}
+
+
+def evalexpr(expr, dims: Dict[str, int]) -> int:
+    """An extent expression -- sums, products, quotients, remainders and the function forms sympy prints (``Mod``,
+    ``Max``, ``Min``, ``floor``, ``ceiling``, ``Pow``) over the base symbols -- as an integer under ``dims``; the
+    operator set of ``evalexpr``, graph.jl:185-207.  ``/`` is the exact quotient while the expression is walked
+    (``ceiling(h/3)`` is the ceiling of the fraction) and a value that is still fractional at the end is floored,
+    which for a lone ``h/2`` is the floor division the reference applies.  Parsed with ``ast`` and walked by hand;
+    nothing is ever handed to ``eval``."""
+    if isinstance(expr, (int, bool)):
+        return int(expr)
+
+    def walk(n):
+        if isinstance(n, ast.Constant) and isinstance(n.value, int):
+            return int(n.value)
+        if isinstance(n, ast.Name):
+            if n.id not in dims:
+                raise KeyError(f"extent expression {expr!r}: no value bound for symbol {n.id!r}")
+            return int(dims[n.id])
+        if isinstance(n, ast.UnaryOp) and isinstance(n.op, (ast.USub, ast.UAdd)):
+            return -walk(n.operand) if isinstance(n.op, ast.USub) else walk(n.operand)
+        if isinstance(n, ast.BinOp) and type(n.op) in _BINOPS:
+            return _BINOPS[type(n.op)](walk(n.left), walk(n.right))
+        if isinstance(n, ast.Call) and isinstance(n.func, ast.Name) and n.func.id in _CALLS and not n.keywords:
+            return _CALLS[n.func.id](*[walk(a) for a in n.args])
+        raise UnsupportedOp(f"unsupported shape expression: {expr!r}")
+
+    return int(math.floor(walk(ast.parse(str(expr), mode="eval").body)))
+
+
 def convert(ep, name: str = "graph") -> Dict[str, Any]:
-    """``ExportedProgram`` -> the buffers/ops dictionary (the schema of export_graphs.py:111-230, static
-    shapes).  Parameters and buffers become ``weight`` buffers keyed by their state-dict name, user inputs
-    and outputs ``external``, view ops ``view`` buffers that alias their parent, everything else an op
-    with a ``transient`` result and a ``live`` interval in op indices."""
+    """``ExportedProgram`` -> the buffers/ops dictionary (the schema of export_graphs.py:111-230).  Parameters
+    and buffers become ``weight`` buffers keyed by their state-dict name, user inputs and outputs ``external``,
+    view ops ``view`` buffers that alias their parent, sizes computed on the host ``host`` scalars, everything
+    else an op with a ``transient`` result and a ``live`` interval in op indices.  Symbolic extents stay
+    expressions in torch's own symbol names (``s0`` ...), listed under ``symbols``."""
     import torch.fx as fx
     sig = ep.graph_signature
     key_of = dict(sig.inputs_to_parameters)
@@ -94,6 +177,7 @@ def convert(ep, name: str = "graph") -> Dict[str, Any]:
     ops: List[Dict[str, Any]] = []
     inputs, outputs = [], []
     born, last = {}, {}
+    symbols: set = set()
 
     def describe(nid, val, kind, **extra):
         b = {"id": nid, "kind": kind}
@@ -101,7 +185,7 @@ def convert(ep, name: str = "graph") -> Dict[str, Any]:
             b["shapes"] = [list(v.shape) if hasattr(v, "shape") else None for v in val]
             b["dtypes"] = [str(v.dtype).replace("torch.", "") if hasattr(v, "dtype") else None for v in val]
         elif val is not None and hasattr(val, "shape"):
-            b["shape"] = [int(d) for d in val.shape]
+            b["shape"] = [_dim(d, symbols) for d in val.shape]
             b["dtype"] = str(val.dtype).replace("torch.", "")
         b.update(extra)
         buffers[nid] = b
@@ -131,6 +215,7 @@ def convert(ep, name: str = "graph") -> Dict[str, Any]:
                     attrs[f"arg{j}"] = [f"${v.name}" if isinstance(v, fx.Node) else _const(v) for v in a]
                 else:
                     attrs[f"arg{j}"] = _const(a)
+                    _note_symbols(a, symbols)
             for k, v in n.kwargs.items():
                 if isinstance(v, fx.Node):
                     args.append(v.name)
@@ -139,6 +224,10 @@ def convert(ep, name: str = "graph") -> Dict[str, Any]:
                     attrs[k] = _const(v)
             val = n.meta.get("val")
             born[n.name] = at
+            if isinstance(val, (int, bool, float, torch.SymInt, torch.SymBool, torch.SymFloat)):
+                # a size computed on the host (sym_size, h * w): a named scalar the views that use it refer to as "$name"
+                buffers[n.name] = {"id": n.name, "kind": "host", "expr": _dim(val, symbols)}
+                continue
             if "getitem" in target or target in VIEW_OPS:
                 describe(n.name, val, "view", of=args[0] if args else None, op=target, attrs=attrs)
                 continue
@@ -154,7 +243,7 @@ def convert(ep, name: str = "graph") -> Dict[str, Any]:
                 b["kind"] = "external"
             else:
                 b["live"] = [born.get(bid, 0), last.get(bid, len(ops))]
-    return {"name": name, "symbols": [], "inputs": inputs, "outputs": outputs, "buffers": list(buffers.values()),
+    return {"name": name, "symbols": sorted(symbols), "inputs": inputs, "outputs": outputs, "buffers": list(buffers.values()),
             "ops": ops, "fusion_groups": [], "barriers": []}
 
 
@@ -169,12 +258,50 @@ class Graph:
     notes: List[str] = field(default_factory=list)      # what the rewrites did, for inspection
 
     @classmethod
-    def load(cls, src) -> "Graph":
+    def load(cls, src, dims: Optional[Dict[str, int]] = None) -> "Graph":
+        """Parse the schema.  A graph with symbolic extents is bound here: ``dims`` gives every name in its
+        ``symbols`` an integer, and each shape, ``host`` scalar and view / op argument written as an expression
+        (or as ``"$name"`` of a host scalar) becomes the integer it evaluates to -- what the reference does per
+        call (``call(model, name, ...; dims)``, ``evalshape``, graph.jl:150-167) happens once per binding, since
+        the executor sizes its buffers when it is built.  One graph file serves any number of bindings."""
         d = json.load(open(src)) if isinstance(src, str) else src
-        if d.get("symbols"):
-            raise UnsupportedOp(f"graph {d.get('name')}: symbolic extents {d['symbols']} (this executor is static-shape)")
-        return cls(d["name"], list(d["inputs"]), list(d["outputs"]), {b["id"]: dict(b) for b in d["buffers"]},
-                   [dict(o, attrs=dict(o.get("attrs", {}))) for o in d["ops"]])
+        syms = list(d.get("symbols") or [])
+        dims = dict(dims or {})
+        missing = [x for x in syms if x not in dims]
+        if missing:
+            raise ValueError(f"graph {d.get('name')}: symbolic extents {missing} need values (dims={{...}})")
+        buffers = {b["id"]: dict(b) for b in d["buffers"]}
+        ops = [dict(o, attrs=dict(o.get("attrs", {}))) for o in d["ops"]]
+        if syms:
+            host = {b["id"]: evalexpr(b["expr"], dims) for b in buffers.values() if b["kind"] == "host" and b.get("expr") is not None}
+            names = set(syms)
+
+            def bind(v):
+                if isinstance(v, list):
+                    return [bind(x) for x in v]
+                if isinstance(v, str):
+                    if v.startswith("$") and v[1:] in host:
+                        return host[v[1:]]
+                    if _mentions(v, names):
+                        return evalexpr(v, dims)
+                return v
+
+            for b in buffers.values():
+                if "shape" in b:
+                    b["shape"] = [evalexpr(x, dims) for x in b["shape"]]
+                if "shapes" in b:
+                    b["shapes"] = [None if sh is None else [evalexpr(x, dims) for x in sh] for sh in b["shapes"]]
+                if b["kind"] == "view" and b.get("attrs"):
+                    b["attrs"] = {k: bind(v) for k, v in b["attrs"].items()}
+                if b["kind"] == "host":
+                    b["value"] = host.get(b["id"])
+            for o in ops:
+                o["attrs"] = {k: bind(v) for k, v in o["attrs"].items()}
+                o["in"] = [i for i in o["in"] if i not in host]
+            for b in buffers.values():
+                if b["kind"] == "view" and b.get("of") in host:
+                    raise UnsupportedOp(f"{b['id']}: a view of the host scalar {b['of']}")
+        return cls(d["name"], list(d["inputs"]), list(d["outputs"]), buffers, ops)
 
     # -- queries the rewrites share
     def root(self, bid: str) -> str:
@@ -593,7 +720,7 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
     ``permute(0, 2, 1, 3)``): the kernel writes token-major, the swap becomes the view it already is, and
     the ``reshape`` that follows is a free view instead of a copy."""
     for o in g.ops:
-        if o["aten"] not in SDPA_OPS:
+        if o["aten"] not in SDPA_OPS and o["aten"] != "sdpa_append":
             continue
         rd = g.readers(o["id"])
         if len(rd) == 1 and "getitem" in g.buffers[rd[0]].get("op", "") and g.buffers[rd[0]]["attrs"].get("arg1", 0) == 0:
@@ -619,7 +746,250 @@ def fold_sdpa_transpose(g: Graph) -> Graph:
     return g
 
 
+GATHER_OPS = ("embedding.default", "index.Tensor")
+
+
+def _row_gather(g: Graph, o) -> Optional[tuple]:
+    """``(table, ids)`` if ``o`` gathers whole rows of a constant 2-D table by an int64 tensor: ``embedding(table, ids)``
+    or ``index.Tensor(table, [ids])`` (advanced indexing along the first axis only)."""
+    if o is None or o["aten"] not in GATHER_OPS or len(o["in"]) != 2:
+        return None
+    table, ids = o["in"]
+    if o["aten"] == "index.Tensor" and o["attrs"].get("arg1") != [f"${ids}"]:
+        return None
+    tb, ib = g.buffers[g.root(table)], g.buffers[ids]
+    if tb["kind"] != "weight" or len(g.buffers[table].get("shape", [])) != 2 or ib.get("dtype") != "int64":
+        return None
+    return table, ids
+
+
+def fold_embedding_sum(g: Graph) -> Graph:
+    """``embedding(tokens, ids) + positions[cache_position]`` -- the first two lines of the decoder step
+    (export_whisper_decoder.py:150-152) -- is one gather that adds the two rows on the way: one launch for three,
+    and no broadcast add of a ``(1, D)`` row over ``B`` rows left in the graph."""
+    for add in [o for o in g.ops if o["aten"] == "add.Tensor" and len(o["in"]) == 2 and o["attrs"].get("alpha", 1) == 1]:
+        a, b = (g.op(i) for i in add["in"])
+        ga, gb = _row_gather(g, a), _row_gather(g, b)
+        if ga is None or gb is None:
+            continue
+        na, nb = (math.prod(g.buffers[x[1]]["shape"]) for x in (ga, gb))
+        if nb != 1 and nb != na:
+            if na != 1:
+                continue
+            (a, ga, na), (b, gb, nb) = (b, gb, nb), (a, ga, na)
+        if g.buffers[ga[0]]["shape"][1] != g.buffers[gb[0]]["shape"][1]:
+            continue
+        if _consumers(g, a["out"]) != {add["id"]} or _consumers(g, b["out"]) != {add["id"]}:
+            continue
+        at = g.ops.index(add)
+        g.ops[at] = {"id": add["id"], "aten": "embedding.default", "in": [ga[0], ga[1], gb[0], gb[1]], "out": add["out"], "attrs": {}}
+        g.ops = [o for o in g.ops if o["id"] not in (a["id"], b["id"])]
+        g.notes.append(f"fold {a['id']} + {b['id']} into one gather ({add['id']})")
+    return g
+
+
+CACHE_WRITES = ("index_copy.default", "index_put.default")
+MASK_VIEWS = RESHAPES + ("expand.default", "unsqueeze.default")
+
+
+def _cache_write(g: Graph, o) -> Optional[Dict[str, Any]]:
+    """``dst.index_copy(2, position, rows)`` / ``index_put(dst, [None, None, position], rows)`` with ``dst`` an input of the
+    graph (or a ``select`` of one: the layer's plane of a stacked cache) of shape (B, H, T, E), ``position`` a one-element
+    int64 input and ``rows`` (B, H, 1, E): the decoder step's cache update (export_whisper_decoder.py:170-177)."""
+    if o is None or o["aten"] not in CACHE_WRITES or len(o["in"]) != 3:
+        return None
+    dst, pos, rows = o["in"]
+    a = o["attrs"]
+    if o["aten"] == "index_copy.default":
+        if a.get("arg1") not in (2, -2):
+            return None
+    elif a.get("arg1") != [None, None, f"${pos}"] or a.get("arg3") or a.get("accumulate"):
+        return None
+    db, pb, rb = g.buffers[dst], g.buffers[pos], g.buffers[rows]
+    sh = db.get("shape") or []
+    if len(sh) != 4 or pb["kind"] != "external" or pos not in g.inputs or pb.get("dtype") != "int64" or list(pb.get("shape", [])) != [1]:
+        return None
+    if list(rb.get("shape", [])) != [sh[0], sh[1], 1, sh[3]] or db.get("dtype") != "float16" or rb.get("dtype") != "float16":
+        return None
+    plane, x = None, dst
+    while g.buffers[x]["kind"] == "view":                # the input itself, or select(input, 0, layer) through aliases
+        v = g.buffers[x]
+        if v["op"] == "select.int" and plane is None and v["attrs"].get("arg1") == 0 and len(g.buffers[v["of"]].get("shape", [])) == 5:
+            plane = v["attrs"].get("arg2")
+        elif v["op"] not in ("alias.default", "detach.default"):
+            return None
+        x = v["of"]
+    if x not in g.inputs:
+        return None
+    if plane is not None and plane < 0:
+        plane += g.buffers[x]["shape"][0]
+    return {"cache": x, "plane": plane, "dst": dst, "pos": pos, "rows": rows}
+
+
+def _position_mask(g: Graph, bid: str, pos: str, T: int) -> Optional[List[str]]:
+    """The ops behind ``bid`` if it is ``where(arange(T) <= position, 0, lowest)`` shown through reshapes and broadcasts
+    along every axis but the keys': slots up to and including ``position`` take part, the rest are masked out
+    (export_whisper_decoder.py:158-166).  ``lowest`` is -inf or the dtype's most negative value: next to any real
+    score its exponential is exactly 0 in fp32, so the masked softmax equals the softmax over the first
+    ``position + 1`` keys."""
+    x = bid
+    while g.buffers[x]["kind"] == "view":
+        v = g.buffers[x]
+        sh = v.get("shape") or []
+        if v["op"] not in MASK_VIEWS or not sh or sh[-1] != T:
+            return None
+        x = v["of"]
+    wh = g.op(x)
+    if wh is None or wh["aten"] != "where.self" or len(wh["in"]) != 3 or list(g.buffers[x].get("shape", [])) != [T]:
+        return None
+    cond, keep, drop = (g.op(i) for i in wh["in"])
+
+    def filled(o):
+        if o is None or o["in"]:
+            return None
+        if o["aten"] == "zeros.default":
+            return 0.0
+        if o["aten"] == "full.default":
+            v = o["attrs"].get("arg1")
+            return float(v) if isinstance(v, (int, float, str)) and not isinstance(v, bool) else None
+        return None
+
+    lo = filled(drop)
+    if cond is None or cond["aten"] != "le.Tensor" or cond["in"] != [cond["in"][0], pos] or filled(keep) != 0.0 or lo is None or lo > -6.0e4:
+        return None
+    ar = g.op(cond["in"][0])
+    a = ar["attrs"] if ar is not None else {}
+    steps = ar is not None and not ar["in"] and (
+        (ar["aten"] == "arange.default" and a.get("arg0") == T) or
+        (ar["aten"] == "arange.start_step" and a.get("arg0") == 0 and a.get("arg1") == T and a.get("arg2", 1) == 1) or
+        (ar["aten"] == "arange.start" and a.get("arg0") == 0 and a.get("arg1") == T))
+    return [wh["id"], cond["id"], keep["id"], drop["id"], ar["id"]] if steps else None
+
+
+def fold_cache_step(g: Graph) -> Graph:
+    """The functional cache update of an exported decoder step becomes an in-place one.
+
+    Matched, per attention: ``K = cache_k[layer].index_copy(2, position, k_new)``, the same for ``V``, and
+    ``scaled_dot_product_attention(q, K, V, mask)`` with one query row, where the only other reader of ``K`` / ``V`` is
+    the ``stack`` (``cat`` + ``view`` once decomposed) that returns every layer's plane as the new cache, in layer order
+    and in the input's shape.  The three ops become ``sdpa_append``: the new rows go into slot ``position`` of the
+    *input* cache, and attention runs over it -- in one launch where the single-workgroup kernel covers the shape.
+    If the mask is the position mask (``_position_mask``) it goes away: the kernel takes ``position + 1`` as the number
+    of valid keys, which a ``kv_len_from_position`` op computes on the device once per step; any other mask stays
+    an operand.  The returned cache becomes an alias of the input (the caller's tensor is updated, and is what the
+    call returns), which removes the 2 x 18 MB of copies per token the reference pays for a functional graph
+    (ops.jl:1018-1023, decode.jl:186-203).  Requires that nothing else reads the cache plane, so no op can observe the
+    difference between "a new tensor" and "the same tensor, updated"."""
+    writes = {o["id"]: w for o in g.ops if (w := _cache_write(g, o)) is not None}
+    if not writes:
+        return g
+    # which attention reads which pair of writes
+    plans = []
+    for att in [o for o in g.ops if o["aten"] in SDPA_OPS]:
+        if len(att["in"]) < 3 or att["in"][1] not in writes or att["in"][2] not in writes:
+            continue
+        wk, wv = writes[att["in"][1]], writes[att["in"][2]]
+        qsh = g.buffers[att["in"][0]].get("shape") or []
+        a = att["attrs"]
+        pd, pc = SDPA_OPS[att["aten"]]
+        if wk["pos"] != wv["pos"] or wk["plane"] != wv["plane"] or wk["cache"] == wv["cache"] or len(qsh) != 4 or qsh[2] != 1:
+            continue
+        if a.get("is_causal", a.get(f"arg{pc}", False)) or a.get("dropout_p", a.get(f"arg{pd}", 0.0)) not in (0, 0.0):
+            continue
+        plans.append((att, att["in"][1], att["in"][2]))
+    # per cache input: every plane written once, each write read by its attention and by the op that returns the planes
+    by_cache: Dict[str, Dict[Any, str]] = {}
+    for att, ik, iv in plans:
+        for wid in (ik, iv):
+            by_cache.setdefault(writes[wid]["cache"], {})[writes[wid]["plane"]] = wid
+    returned: Dict[str, tuple] = {}
+    for cache, planes in by_cache.items():
+        shape = g.buffers[cache]["shape"]
+        order = [planes.get(i) for i in range(shape[0])] if len(shape) == 5 else [planes.get(None)]
+        if any(w is None for w in order):
+            continue
+        joins = [o for o in g.ops if o["aten"] in ("stack.default", "cat.default") and o["in"] == order and o["attrs"].get("arg1", 0) == 0]
+        if len(shape) == 4:                              # a single-layer cache returned as it is
+            if order[0] in g.outputs:
+                returned[cache] = (None, order[0])
+            continue
+        for j in joins:
+            outs = [x for x in ([j["out"]] + [v for v in g.readers(j["out"]) if g.buffers.get(v, {}).get("kind") == "view"])
+                    if x in g.outputs and g.buffers[x].get("shape") == shape]
+            if outs and _consumers(g, j["out"]) == {"<output>"}:
+                returned[cache] = (j, outs[0])
+                break
+    done = []
+    for att, ik, iv in plans:
+        wk, wv = writes[ik], writes[iv]
+        if wk["cache"] not in returned or wv["cache"] not in returned:
+            continue
+        jk, jv = returned[wk["cache"]][0], returned[wv["cache"]][0]
+        allowed_k = {att["id"]} | ({jk["id"]} if jk else {"<output>"})
+        allowed_v = {att["id"]} | ({jv["id"]} if jv else {"<output>"})
+        if _consumers(g, ik) != allowed_k or _consumers(g, iv) != allowed_v:
+            continue
+        if any(_consumers(g, c) != set(by_cache[c].values()) for c in (wk["cache"], wv["cache"])):
+            continue                                    # someone else reads the cache, through whatever view: it would see the new rows
+        done.append((att, ik, iv))
+    if not done:
+        return g
+    # all or nothing per cache: a returned tensor that aliases the input must have had every plane written in place
+    covered: Dict[str, set] = {}
+    for att, ik, iv in done:
+        for wid in (ik, iv):
+            covered.setdefault(writes[wid]["cache"], set()).add(wid)
+    ok_cache = {c for c, ws in covered.items() if ws == set(by_cache[c].values())}
+    done = [d for d in done if writes[d[1]]["cache"] in ok_cache and writes[d[2]]["cache"] in ok_cache]
+    lens: Dict[tuple, str] = {}
+    for att, ik, iv in done:
+        wk, wv = writes[ik], writes[iv]
+        B, H, T, E = g.buffers[wk["dst"]]["shape"]
+        key = (wk["pos"], B, T)
+        if key not in lens:                             # position + 1 as the per-row key count, once per step
+            lid = f"kv_len_{wk['pos']}_{T}"
+            g.buffers[lid] = {"id": lid, "kind": "transient", "shape": [B], "dtype": "int32"}
+            g.ops.insert(0, {"id": lid, "aten": "kv_len_from_position", "in": [wk["pos"]], "out": lid, "attrs": {"cap": T + 1}})
+            lens[key] = lid
+        ins = [att["in"][0], wk["dst"], wv["dst"], wk["rows"], wv["rows"], lens[key]]
+        attrs = {k: v for k, v in att["attrs"].items() if k in ("scale", "token_major")}
+        mask = att["in"][3] if len(att["in"]) > 3 else None
+        if mask is not None:
+            if _position_mask(g, mask, wk["pos"], T) is None:
+                ins.append(mask)
+                attrs["masked"] = True
+        else:
+            attrs["all_slots"] = True                   # no mask in the export: every slot takes part, written or not
+        at = g.ops.index(att)
+        g.ops[at] = {"id": att["id"], "aten": "sdpa_append", "in": ins, "out": att["out"], "attrs": attrs}
+        g.ops = [o for o in g.ops if o["id"] not in (ik, iv)]
+        for wid in (ik, iv):                            # the "new" plane is the input's plane
+            g.buffers[wid].update(kind="view", of=writes[wid]["dst"], op="alias.default", attrs={})
+        g.notes.append(f"fold {ik} / {iv} / {att['id']} into an in-place sdpa_append on {wk['cache']} / {wv['cache']}")
+    for cache in ok_cache:
+        j, out = returned[cache]
+        if j is not None:
+            g.ops.remove(j)
+            for x in [j["out"]] + [v for v in g.readers(j["out"]) if g.buffers.get(v, {}).get("kind") == "view"]:
+                g.buffers[x].update(kind="view", of=cache, op="alias.default", attrs={})
+        g.notes.append(f"output {out} is the input {cache}, updated in place")
+    return prune(g)
+
+
+def prune(g: Graph) -> Graph:
+    """Drop ops whose result nothing reads any more (the mask arithmetic once the mask became a length)."""
+    while True:
+        dead = [o for o in g.ops if not _consumers(g, o["out"]) and o["aten"] != "sdpa_append" and
+                not any(_consumers(g, m["out"]) for m in o["attrs"].get("members", []))]
+        if not dead:
+            return g
+        for o in dead:
+            g.ops.remove(o)
+            g.notes.append(f"drop {o['id']} (unused)")
+
+
 def optimize(g: Graph) -> Graph:
+    g = fold_cache_step(fold_embedding_sum(g))
     return group_linears(fold_sdpa_transpose(fold_attention(fold_layernorms(fold_layernorm_prologues(
         fold_clamps(fold_residuals(fold_layerscale(fold_activations(g)))))))))
 
@@ -666,7 +1036,7 @@ class Executor:
             b = graph.buffers[o["out"]]
             if "shape" in b:
                 shape, dtype = list(b["shape"]), b["dtype"]
-            elif o["aten"] in SDPA_OPS:                   # a tuple result: only the attention output is materialised
+            elif o["aten"] in SDPA_OPS or o["aten"] == "sdpa_append":   # a tuple result: only the attention output is materialised
                 shape, dtype = list(b["shapes"][0]), b["dtypes"][0]
             else:
                 continue
@@ -941,13 +1311,46 @@ class Executor:
         else:
             K.convolution_(self.ctx, out, x, w, bias, xy(stride), xy(padding), xy(dilation), a.get("arg8", 1))
 
+    def _embedding(self, o):
+        """embedding(table, ids) / index.Tensor(table, [ids]) along the first axis (ops.jl:1754-1783, 1524-1640); with
+        four operands the sum of two gathers ``fold_embedding_sum`` made."""
+        ins = o["in"]
+        if o["aten"] == "index.Tensor" and o["attrs"].get("arg1") != [f"${ins[1]}"]:
+            raise UnsupportedOp(f"{o['id']}: index.Tensor other than a gather of rows along the first axis")
+        t2, i2 = (self.get(ins[2]), self.get(ins[3])) if len(ins) == 4 else (None, None)
+        K.embedding_(self.ctx, self.t[o["out"]], self.get(ins[0]), self.get(ins[1]), t2, i2)
+
+    def _kv_len(self, o):
+        K.kv_len_from_position_(self.ctx, self.t[o["out"]], self.get(o["in"][0]), o["attrs"]["cap"])
+
+    def _sdpa_append(self, o):
+        """The folded cache step: write the new rows into the input cache and attend over it.  One launch where the
+        single-workgroup kernel covers the shape and the mask became a length; two (append, attention) otherwise."""
+        a = o["attrs"]
+        q, ck, cv, kn, vn, kv_len = (self.get(i) for i in o["in"][:6])
+        out = self.t[o["out"]]
+        self.ctx.ws.reset()
+        if not a.get("masked") and not a.get("all_slots"):
+            try:
+                K.sdpa_append(self.ctx, q, ck, cv, kn, vn, kv_len, a.get("scale"), out=out)
+                return
+            except K.DeclineError as e:
+                if e.status != K.L.DECLINE_UNSUPPORTED:
+                    raise
+        K.kv_append_(self.ctx, ck, cv, kn, vn, kv_len)
+        if a.get("masked"):
+            K.sdpa(self.ctx, q, ck, cv, self.get(o["in"][6]), a.get("scale"), out=out)
+        else:
+            K.sdpa(self.ctx, q, ck, cv, None, a.get("scale"), out=out, kv_len=None if a.get("all_slots") else kv_len)
+
     HANDLERS = {"linear.default": _linear, "addmm.default": _linear, "mm.default": _linear,
                 **dict.fromkeys(SDPA_OPS, _sdpa), "layer_norm.default": _layer_norm,
                 "native_layer_norm.default": _native_layer_norm, "add.Tensor": _add,
                 "gelu.default": _activation, "relu.default": _activation, "convolution.default": _convolution,
                 "bmm.default": _bmm, "cat.default": _cat, **dict.fromkeys(SOFTMAX_OPS, _softmax),
                 "mul.Tensor": _scale, "div.Tensor": _scale, "clone.default": _clone, "clamp.default": _clamp,
-                "linear_group": _linear_group}
+                "linear_group": _linear_group, "embedding.default": _embedding, "index.Tensor": _embedding,
+                "kv_len_from_position": _kv_len, "sdpa_append": _sdpa_append}
 
     def replayable(self, *inputs: torch.Tensor):
         """Run once eagerly (binds inputs, sizes the workspace, stacks folded constants), then capture the whole graph as

@@ -744,3 +744,58 @@ def add_(ctx: Ctx, out, a, b):
     if rc != L.OK:
         raise DeclineError("mi_add_f16", rc)
     return out
+
+
+# ----------------------------------------------------------------------------- the decoder step's gathers
+
+def embedding_(ctx: Ctx, out, table, ids, table2=None, ids2=None):
+    """``out[i] = table[ids[i]]`` (+ ``table2[ids2[i]]``, ``ids2`` one id for every row or one per row): aten::embedding
+    (ops.jl:1754-1783) and the first-axis gather of aten::index.Tensor; with both tables the decoder step's token +
+    position embedding.  ``ids``: int64, any shape; ``out``: fp16 ``ids.shape + (D,)`` (leading singleton axes free)."""
+    lib = L.init()
+    if not _is_f16_cuda(out, table) or table.dim() != 2 or not table.is_contiguous() or not out.is_contiguous():
+        raise DeclineError("embedding_: fp16 cuda operands, a contiguous (V, D) table", L.DECLINE_OPERANDS)
+    V, D = table.shape
+    n = ids.numel()
+    if ids.dtype != torch.int64 or not ids.is_cuda or not ids.is_contiguous() or n < 1 or out.numel() != n * D or out.shape[-1] != D:
+        raise DeclineError(f"embedding_: ids must be contiguous cuda int64 and out hold ids.numel() rows of {D}", L.DECLINE_OPERANDS)
+    n2 = V2 = 0
+    if table2 is not None:
+        if not _is_f16_cuda(table2) or table2.dim() != 2 or not table2.is_contiguous() or table2.shape[1] != D:
+            raise DeclineError("embedding_: the second table must be a contiguous fp16 (V2, D) matrix", L.DECLINE_OPERANDS)
+        if ids2 is None or ids2.dtype != torch.int64 or not ids2.is_cuda or not ids2.is_contiguous() or ids2.numel() not in (1, n):
+            raise DeclineError("embedding_: ids2 must be cuda int64 with one id, or one per row", L.DECLINE_OPERANDS)
+        n2, V2 = ids2.numel(), table2.shape[0]
+    rc = lib.mi_embedding_f16(out.data_ptr(), table.data_ptr(), ids.data_ptr(), n, D, V, _ptr(table2), _ptr(ids2), n2, V2, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_embedding_f16", rc)
+    return out
+
+
+def kv_len_from_position_(ctx: Ctx, kv_len, position, cap: int):
+    """``kv_len[b] = clamp(position + 1, 0, cap)``: the exported step's ``cache_position`` (int64, one for all rows or one
+    per row) as the count of valid keys the attention kernels take (decode.jl:186-203)."""
+    if kv_len.dtype != torch.int32 or not kv_len.is_cuda or not kv_len.is_contiguous() or \
+            position.dtype != torch.int64 or not position.is_cuda or not position.is_contiguous() or position.numel() not in (1, kv_len.numel()):
+        raise DeclineError("kv_len_from_position_: int32 (B,) lengths and int64 positions (1 or B of them) on the GPU", L.DECLINE_OPERANDS)
+    rc = L.init().mi_kv_len_from_position(kv_len.data_ptr(), position.data_ptr(), position.numel(), kv_len.numel(), int(cap), ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_kv_len_from_position", rc)
+    return kv_len
+
+
+def kv_append_(ctx: Ctx, cache_k, cache_v, k_new, v_new, kv_len):
+    """Write the new token's rows ``(B,H,1,E)`` into slot ``kv_len[b] - 1`` of ``cache_k`` / ``cache_v`` ``(B,H,Lmax,E)``,
+    in place: the exported step's ``index_put`` on the cache (ops.jl:1003-1025) without the copy of the whole tensor."""
+    if not _is_f16_cuda(cache_k, cache_v, k_new, v_new) or cache_k.dim() != 4 or k_new.dim() != 4:
+        raise DeclineError("kv_append_: operands", L.DECLINE_OPERANDS)
+    B, H, Lmax, E = cache_k.shape
+    if tuple(cache_v.shape) != (B, H, Lmax, E) or cache_v.stride() != cache_k.stride() or tuple(k_new.shape) != (B, H, 1, E) or \
+            tuple(v_new.shape) != (B, H, 1, E) or k_new.stride() != v_new.stride():
+        raise DeclineError("kv_append_: caches (B,H,Lmax,E) with equal strides, new rows (B,H,1,E) with equal strides", L.DECLINE_OPERANDS)
+    if kv_len.dtype != torch.int32 or not kv_len.is_cuda or kv_len.numel() != B:
+        raise DeclineError("kv_append_: kv_len must be a cuda int32 (B,) tensor", L.DECLINE_OPERANDS)
+    rc = L.init().mi_kv_append_f16(cache_k.data_ptr(), cache_v.data_ptr(), _strides_elbh(cache_k), Lmax, k_new.data_ptr(), v_new.data_ptr(),
+                                   _strides_elbh(k_new), kv_len.data_ptr(), E, H, B, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_kv_append_f16", rc)

@@ -31,7 +31,8 @@ def _weights(d, ffn, seed, layout):
 
 def _oracle_layer_step(Wh, x, self_k, self_v, cross_k, cross_v, length, H, E):
     """The same layer step from the oracle's CPU kernels; self_k/self_v (B,H,Lmax,E) are updated in place,
-    ``length`` (B,) counts the live slots including the new one."""
+    ``length`` (B,) counts the live slots including the new one; Lmax + 1 marks a row stepped while full, whose
+    new K/V is not stored and which attends over the Lmax stored keys."""
     B, d = x.shape
     h, _, _ = oracle.layernorm_f16(x, Wh["ln1_g"], Wh["ln1_b"])
     qkv = oracle.gemm_f16(h, Wh["wqkv"], Wh["bqkv"])
@@ -40,7 +41,7 @@ def _oracle_layer_step(Wh, x, self_k, self_v, cross_k, cross_v, length, H, E):
         if 1 <= length[b] <= self_k.shape[2]:
             self_k[b, :, length[b] - 1, :] = k[b, :, 0, :]
             self_v[b, :, length[b] - 1, :] = v[b, :, 0, :]
-    att = oracle.sdpa_threepass_f16(np.ascontiguousarray(q), self_k, self_v, kv_len=length.astype(np.int32))
+    att = oracle.sdpa_threepass_f16(np.ascontiguousarray(q), self_k, self_v, kv_len=np.minimum(length, self_k.shape[2]).astype(np.int32))
     x1 = oracle.gemm_f16(att.reshape(B, d), Wh["wo"], Wh["bo"], residual=x)
     h, _, _ = oracle.layernorm_f16(x1, Wh["ln2_g"], Wh["ln2_b"])
     qc = oracle.gemm_f16(h, Wh["wq_c"], Wh["bq_c"]).reshape(B, H, 1, E)
@@ -84,9 +85,13 @@ def test_kv_advance_clamps(ctx):
     cache = KVCache(1, 5, 1, 8, max_target=4, src_len=1)
     cache.length.copy_(torch.tensor([0, 1, 3, 4, 2], dtype=torch.int32))
     cache.advance(ctx)
-    assert to_host(cache.length).tolist() == [1, 2, 4, 4, 3]
-    cache.advance(ctx, -3)
+    assert to_host(cache.length).tolist() == [1, 2, 4, 5, 3]      # capacity + 1: "this row was stepped while full"
+    assert cache.overflowed()
+    cache.advance(ctx)
+    assert to_host(cache.length).tolist() == [2, 3, 5, 5, 4]      # and there it stops
+    cache.advance(ctx, -4)
     assert to_host(cache.length).tolist() == [0, 0, 1, 1, 0]
+    assert not cache.overflowed()
 
 
 @pytest.mark.parametrize("layout", ["kf", "fk"])
@@ -118,7 +123,7 @@ def test_decoder_layer_steps_match_oracle(ctx, B, layout):
         cache.advance(ctx)
         out.fill_(float("nan"))
         decoder_layer_step(ctx, Wd, cache, 0, to_dev(x), out, buf)
-        length = np.minimum(length + 1, Lmax)
+        length = np.minimum(length + 1, Lmax + 1)
         want = _oracle_layer_step(Wh, x, hk, hv, ck[0], cv[0], length, H, E)
         assert_parity(to_host(out), want, what=f"decoder layer B{B} {layout} step {step}")
         assert to_host(cache.length).tolist() == length.tolist()
