@@ -366,7 +366,10 @@ int mi_kv_append_f16(void *cache_k, void *cache_v, const int64_t cache_strides[4
  * the newest token (k_new, v_new: 1 x E per head and batch, element strides new_strides as (E, L, H, B)) is taken
  * as key kv_len[b] - 1 and written into that slot of the cache on the way; out = attention of q over the first
  * kv_len[b] keys.  cache_k / cache_v are written to.  Only what the single-launch kernel covers (E <= 64, at most
- * 640 cache slots, 16-byte addressable rows); MI_DECLINE_UNSUPPORTED otherwise, and the caller makes the two calls.
+ * 4096 (head, batch) rows, 16-byte addressable rows); MI_DECLINE_UNSUPPORTED otherwise, and the caller makes the two
+ * calls.  The key range may be cut over several workgroups per row that merge inside the launch through counters and
+ * partials in a static device array (16 banks taken in turn: more than 16 such launches -- this call or mi_sdpa_f16
+ * with Lq = 1 -- in flight together on one GPU would share a bank and race).
  * Replaces index_put + cat + scaled_dot_product_attention of the exported decoder step
  * (WhisperRunner/src/decode.jl:186-203, tools/export_whisper_decoder.py). */
 int mi_sdpa_append_f16(void *out, int out_dtype, const int64_t out_strides[4],

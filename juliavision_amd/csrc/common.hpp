@@ -159,6 +159,9 @@ struct NhwcGather {
 // True once mi_init has run successfully on this process (defined in gemm.hip).
 bool mi_ready();
 int mi_num_cus();
+// True if the current device deals workgroups to its XCDs round robin by workgroup id (ids that differ by a multiple
+// of 8 share an L2), as a probe launch at mi_init showed; kernels whose workgroups exchange data through one L2 ask.
+bool mi_xcd_round_robin();
 int mi_sdpa_init();
 // Y[M x N] = A[M x K] . B (+bias) with B either [K][NB-padded N] (b_kn) or [N][K]; defined in gemm.hip.
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,

@@ -1022,10 +1022,9 @@ __global__ void gemm_scalar_kernel(GemmArgs p, int b_kn) {
 // Layer-norm statistics of up to MT rows of A, one wave per row, in the summation order of
 // layernorm_vec_kernel (a lane takes the 16-byte chunks lane, lane + 64, ...; butterfly over the wave):
 // the fused result is bit-identical to running that kernel first.  stats[m] = (mean, rstd).
-template <int MT>
+template <int MT, int NCH = 8>                              // rows up to NCH * 512 halves stay in registers between the passes
 __device__ __forceinline__ void ln_row_stats(const GemmArgs &p, float (*stats)[2], int tid) {
     const int lane = tid & 63, wave = tid >> 6;
-    constexpr int NCH = 8;                                   // rows up to 4096 halves stay in registers between the passes
     for (int m = wave; m < MT && m < p.M; m += 4) {
         const half_t *row = p.A + (long)m * p.ldA;
         float s = 0.0f, s2 = 0.0f;
@@ -1198,20 +1197,71 @@ __global__ void skinny_epilogue_kernel(GemmArgs p, const float *part, int nsplit
 // [F][K] weights (K-contiguous): one wave per output column, lanes stride K in 16-byte chunks,
 // wave reduction, and the epilogue in the same launch: no workspace, no second kernel.  The
 // activations are staged in LDS once per workgroup (dynamic: MT rows of K halves).
-template <int MT>
-__global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p, int rows_per_wave) {
+//
+// A decode-sized call moves a few MB, so its duration is a chain of trips to memory, not bandwidth.  Everything whose
+// address does not depend on loaded data is therefore requested at the top, before anything is waited for: the wave's
+// weight row (FK_PF chunks of 16 bytes per lane: K <= 6144 whole), its bias and residual elements, the thread's
+// share of the activations and of gamma / beta.  The statistics of the layer-norm prologue, the staging and the dot
+// products then run on data that arrives together: one trip instead of three or four in a row.
+// FK_PF = 3 (K <= 1536) or 12: the registers of the up-front requests decide how many waves a SIMD holds, and a
+// wide output (1280 -> 5120 is five waves per SIMD, a vocabulary projection many more) needs them all resident.
+template <int MT, int FK_PF>
+__global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p) {
+    // activation chunks per thread requested up front: the whole MT x K panel up to four per thread
+    constexpr int FK_XCAP = MT == 8 ? 1 : 4;              // eight rows of accumulators and operands leave room for one
+    constexpr int FK_XPF = (MT * FK_PF * 64 + 255) / 256 < FK_XCAP ? (MT * FK_PF * 64 + 255) / 256 : FK_XCAP;
     extern __shared__ __align__(16) char smem[];
     half_t *xs = reinterpret_cast<half_t *>(smem);       // [MT][K]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     __shared__ float lnst[MT][2];
     const int kch = p.K >> 3;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    const int n = blockIdx.x * 4 + wave;
+    const bool live = n < p.N;                            // uniform over the wave
+    const half_t *bp = p.B + (long)(live ? n : 0) * p.ldB;
+    u32x4 w[FK_PF];
+#pragma unroll
+    for (int i = 0; i < FK_PF; i++) w[i] = live && lane * 8 + 512 * i < p.K ? ldg16(bp + lane * 8 + 512 * i) : z;
+    float bv = 0.0f, rv = 0.0f;
+    if (live && lane < p.M) {
+        if (p.bias_mode == MI_BIAS_COL) bv = (float)p.bias[n];
+        else if (p.bias_mode == MI_BIAS_ROW) bv = (float)p.bias[lane];
+        if (p.residual && !p.out_f32) rv = (float)p.residual[(long)lane * p.ldY + n];
+    }
+    u32x4 xr[FK_XPF], gr[FK_XPF], br[FK_XPF];
+#pragma unroll
+    for (int i = 0; i < FK_XPF; i++) {
+        const int c = tid + 256 * i, m = c / kch, ch = c % kch;
+        xr[i] = gr[i] = br[i] = z;
+        if (c < MT * kch && m < p.M) {
+            xr[i] = ldg16(p.A + (long)m * p.ldA + ch * 8);
+            if (p.ln_on && p.ln_gamma) gr[i] = ldg16(p.ln_gamma + ch * 8);
+            if (p.ln_on && p.ln_beta) br[i] = ldg16(p.ln_beta + ch * 8);
+        }
+    }
     if (p.ln_on) {                                      // uniform
-        ln_row_stats<MT>(p, lnst, tid);
+        ln_row_stats<MT, (FK_PF < 8 ? FK_PF : 8)>(p, lnst, tid);
         __syncthreads();
     }
-    for (int c = tid; c < MT * kch; c += 256) {
+#pragma unroll
+    for (int i = 0; i < FK_XPF; i++) {
+        const int c = tid + 256 * i, m = c / kch, ch = c % kch;
+        if (c < MT * kch) {
+            u32x4 v = xr[i];
+            if (p.ln_on && m < p.M) {
+                const half8v x = as_half8(v), gv = as_half8(gr[i]), bb = as_half8(br[i]);
+                half8v o;
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    o[j] = ln_norm1((float)x[j], lnst[m][0], lnst[m][1], p.ln_gamma != nullptr, (float)gv[j], p.ln_beta != nullptr, (float)bb[j]);
+                v = __builtin_bit_cast(u32x4, o);
+            }
+            *reinterpret_cast<u32x4 *>(xs + (long)m * p.K + ch * 8) = v;
+        }
+    }
+    for (int c = tid + 256 * FK_XPF; c < MT * kch; c += 256) {
         const int m = c / kch, ch = c % kch;
-        u32x4 v = {0u, 0u, 0u, 0u};
+        u32x4 v = z;
         if (m < p.M) {
             v = ldg16(p.A + (long)m * p.ldA + ch * 8);
             if (p.ln_on) v = ln_apply8(p, v, lnst[m][0], lnst[m][1], ch * 8);
@@ -1219,50 +1269,47 @@ __global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p, int rows_per
         *reinterpret_cast<u32x4 *>(xs + (long)m * p.K + ch * 8) = v;
     }
     __syncthreads();
-    for (int r = 0; r < rows_per_wave; r++) {
-        const int n = (blockIdx.x * 4 + wave) * rows_per_wave + r;
-        if (n >= p.N) break;                              // uniform over the wave
-        const half_t *bp = p.B + (long)n * p.ldB;
-        float acc[MT];
+    if (!live) return;
+    float acc[MT];
 #pragma unroll
-        for (int m = 0; m < MT; m++) acc[m] = 0.0f;
-        for (int kb = lane * 8; kb < p.K; kb += 4 * 512) {
-            u32x4 w[4];
-            const u32x4 z = {0u, 0u, 0u, 0u};
-#pragma unroll
-            for (int i = 0; i < 4; i++) w[i] = kb + 512 * i < p.K ? ldg16(bp + kb + 512 * i) : z;
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                if (kb + 512 * i < p.K) {
-#pragma unroll
-                    for (int m = 0; m < MT; m++) {
-                        const u32x4 x = *reinterpret_cast<const u32x4 *>(xs + (long)m * p.K + kb + 512 * i);
-#pragma unroll
-                        for (int q = 0; q < 4; q++) {
-                            const uint32_t wq = w[i][q], xq = x[q];     // bit_cast wants an addressable scalar, not a vector element
-                            acc[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, wq), __builtin_bit_cast(half2v, xq), acc[m], false);
-                        }
-                    }
-                }
-            }
-        }
-        float mine = 0.0f;                                // lane m keeps row m's sum
+    for (int m = 0; m < MT; m++) acc[m] = 0.0f;
+    auto dot = [&](const u32x4 &wv, int k) {
 #pragma unroll
         for (int m = 0; m < MT; m++) {
-            float sres = acc[m];
-            sres = wave_sum(sres);
-            if (lane == m) mine = sres;
-        }
-        if (lane < p.M) {
-            const int m = lane;
-            float v = mine + (p.bias_mode == MI_BIAS_COL ? (float)p.bias[n] : p.bias_mode == MI_BIAS_ROW ? (float)p.bias[m] : 0.0f);
-            const long off = (long)m * p.ldY + n;
-            if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(v, p.epi);
-            else {
-                half_t o = (half_t)apply_epi((float)(half_t)v, p.epi);
-                if (p.residual) o = (half_t)((float)o + (float)p.residual[off]);
-                reinterpret_cast<half_t *>(p.Y)[off] = o;
+            const u32x4 x = *reinterpret_cast<const u32x4 *>(xs + (long)m * p.K + k);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t wq = wv[q], xq = x[q];     // bit_cast wants an addressable scalar, not a vector element
+                acc[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, wq), __builtin_bit_cast(half2v, xq), acc[m], false);
             }
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < FK_PF; i++)
+        if (lane * 8 + 512 * i < p.K) dot(w[i], lane * 8 + 512 * i);
+    for (int kb = lane * 8 + 512 * FK_PF; kb < p.K; kb += 4 * 512) {
+        u32x4 t[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) t[i] = kb + 512 * i < p.K ? ldg16(bp + kb + 512 * i) : z;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (kb + 512 * i < p.K) dot(t[i], kb + 512 * i);
+    }
+    float mine = 0.0f;                                    // lane m keeps row m's sum
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+        float sres = acc[m];
+        sres = wave_sum(sres);
+        if (lane == m) mine = sres;
+    }
+    if (lane < p.M) {
+        const float v = mine + bv;
+        const long off = (long)lane * p.ldY + n;
+        if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(v, p.epi);
+        else {
+            half_t o = (half_t)apply_epi((float)(half_t)v, p.epi);
+            if (p.residual) o = (half_t)((float)o + rv);
+            reinterpret_cast<half_t *>(p.Y)[off] = o;
         }
     }
 }
@@ -1738,12 +1785,18 @@ int run_skinny(GemmArgs a, bool b_kn, void *ws, size_t ws_bytes, hipStream_t st)
         // One weight row per wave.  More rows per wave would amortise the staging of the activations, but the
         // rows of a wave run one after the other, each a chain of dependent memory trips: measured slower at
         // every batch size (1280 -> 5120, batch 8: 9.1 us with one row, 13.7 us with four).
-        int rpw = 1;
-        dim3 grid((unsigned)ceil_div(a.N, 4 * rpw));
-        if (mt == 1)      hipLaunchKernelGGL(skinny_fk_kernel<1>, grid, dim3(256), lds, st, a, rpw);
-        else if (mt == 2) hipLaunchKernelGGL(skinny_fk_kernel<2>, grid, dim3(256), lds, st, a, rpw);
-        else if (mt == 4) hipLaunchKernelGGL(skinny_fk_kernel<4>, grid, dim3(256), lds, st, a, rpw);
-        else              hipLaunchKernelGGL(skinny_fk_kernel<8>, grid, dim3(256), lds, st, a, rpw);
+        dim3 grid((unsigned)ceil_div(a.N, 4));
+        if (a.K <= 1536) {
+            if (mt == 1)      hipLaunchKernelGGL((skinny_fk_kernel<1, 3>), grid, dim3(256), lds, st, a);
+            else if (mt == 2) hipLaunchKernelGGL((skinny_fk_kernel<2, 3>), grid, dim3(256), lds, st, a);
+            else if (mt == 4) hipLaunchKernelGGL((skinny_fk_kernel<4, 3>), grid, dim3(256), lds, st, a);
+            else              hipLaunchKernelGGL((skinny_fk_kernel<8, 3>), grid, dim3(256), lds, st, a);
+        } else {
+            if (mt == 1)      hipLaunchKernelGGL((skinny_fk_kernel<1, 12>), grid, dim3(256), lds, st, a);
+            else if (mt == 2) hipLaunchKernelGGL((skinny_fk_kernel<2, 12>), grid, dim3(256), lds, st, a);
+            else if (mt == 4) hipLaunchKernelGGL((skinny_fk_kernel<4, 12>), grid, dim3(256), lds, st, a);
+            else              hipLaunchKernelGGL((skinny_fk_kernel<8, 12>), grid, dim3(256), lds, st, a);
+        }
     }
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
@@ -1863,6 +1916,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
 
 bool mi_ready() { return g_ready; }
 int mi_num_cus() { return g_cus; }
+bool mi_xcd_round_robin() { return sk_usable(); }
 
 // Split-K planes of a GEMM issued through mi_internal_gemm.
 size_t mi_internal_gemm_workspace(int64_t T, int64_t K, int64_t F, int64_t nbatch) {
@@ -1950,10 +2004,14 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 0, 2>, lna_lds_bytes<128, 2, 4>(LNA_KMAX));
     bad |= raise_lds(gemm_pipe_kernel<64, 64, 2, 2, 1, 2>, lna_lds_bytes<64, 2, 2>(LNA_KMAX));
     bad |= raise_lds(gemm_pipe_kernel<64, 64, 2, 2, 0, 2>, lna_lds_bytes<64, 2, 2>(LNA_KMAX));
-    bad |= raise_lds(skinny_fk_kernel<1>, (int)SKINNY_FK_LDS_MAX);
-    bad |= raise_lds(skinny_fk_kernel<2>, (int)SKINNY_FK_LDS_MAX);
-    bad |= raise_lds(skinny_fk_kernel<4>, (int)SKINNY_FK_LDS_MAX);
-    bad |= raise_lds(skinny_fk_kernel<8>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<1, 3>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<2, 3>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<4, 3>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<8, 3>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<1, 12>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<2, 12>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<4, 12>, (int)SKINNY_FK_LDS_MAX);
+    bad |= raise_lds(skinny_fk_kernel<8, 12>, (int)SKINNY_FK_LDS_MAX);
     bad |= mi_sdpa_init();
     bad |= scratch_of_current_device() == nullptr;
     sk_probe_current_device();      // a device that fails the probe only loses that path

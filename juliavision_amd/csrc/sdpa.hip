@@ -14,6 +14,8 @@
 // Operands are (E, L, H, B) with element strides (the reference's layout,
 // DNNKernels/src/kernels/extern/attention.jl:1-22); out is dense (E, Lq, H, B).
 #include "common.hpp"
+#include <atomic>
+#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -25,7 +27,8 @@ struct SdpaArgs {
     const void *bias;
     long bs[4];                    // (Lk, Lq, H, B) element strides, 0 = broadcast
     const int *kv_len;
-    float *part_o, *part_ml;       // split partials: [split][row][E], [split][row][2]
+    float *part_o, *part_ml;       // split partials: [split][row][E], [split][row][2] (sdpa_decode_kernel: [row][split])
+    unsigned *tickets;             // sdpa_decode_kernel with nsplit > 1: one arrival counter per (head, batch), zero between launches
     // sdpa_decode_kernel only: the newest key/value row (1 x E per head and batch); when set, key kv_len - 1 is
     // taken from here instead of the cache and written into the cache on the way (k, v are then written to)
     const half_t *k_new, *v_new;
@@ -779,63 +782,91 @@ __global__ __launch_bounds__(256) void sdpa_rows_kernel(SdpaArgs p) {
     }
 }
 
-// Single query row per (head, batch), whole key range in one workgroup of 8 waves: nothing to merge in a second
-// launch.  A wave takes keys 8 at a time (8 lanes per key, one 16-byte chunk of the head dim each) with a stride
-// of 64 keys, in rounds of SD_U passes whose K and V loads are all issued before the first is used, the next
-// round's before the current round is consumed: about 190 KB in flight per workgroup.
+// Single query row per (head, batch): 8-wave workgroups, `nsplit` of them per row, each over its share of the key
+// range.  A wave takes keys 8 at a time (8 lanes per key, one 16-byte chunk of the head dim each) with a stride of
+// 64 keys, in rounds of SD_U passes whose K and V loads are all issued before the first is used, the next round's
+// before the current round is consumed: about 190 KB in flight per workgroup.
+//
+// Such a launch moves a few MB, so its duration is a chain of trips to memory.  Every address is therefore made
+// independent of loaded data: the key range is cut by the cache's capacity (p.Lk), not by kv_len, and keys are
+// requested up to the capacity -- valid memory whatever the length -- together with the length itself, the query
+// and the new row; the length only masks scores afterwards.  One trip, then arithmetic.
+//
+// nsplit > 1: the workgroups of one row run on one XCD (workgroup ids are dealt to XCDs round robin, so ids that
+// differ by multiples of 8 share an L2), write their partial (max, sum, o[E]) to part_o / part_ml, and take a ticket;
+// whoever draws the last ticket merges the partials in split order -- so the result does not depend on who that
+// is -- writes the row and puts the ticket counter back to zero.  Nobody waits for anybody: every workgroup exits
+// after its own work.  The exchange stays inside that one L2: a partial is written with plain stores, waited for
+// (vmcnt) and followed by the ticket, an atomic the L2 performs; the merging workgroup reads with loads that go to
+// the L2.  A device-scope release per workgroup instead (__threadfence) writes the whole L2 back each time: measured
+// 63 us for 320 workgroups against 6 us unsplit.  The host only splits on a device whose probe showed the round-robin
+// placement this relies on.
 constexpr int SD_U = 6;
 __global__ __launch_bounds__(512) void sdpa_decode_kernel(SdpaArgs p) {
     __shared__ float red_ml[8][2];
     __shared__ float red_o[8][64];
+    __shared__ int is_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int grp = lane >> 3, cl = lane & 7;
-    const int h = blockIdx.x, b = blockIdx.z;
-    int Lk = p.Lk;
-    bool room = true;                          // a length past the capacity: the cache is full, the new row is not stored
-    if (p.kv_len) { const int n = p.kv_len[b]; room = n <= Lk; Lk = max(0, min(Lk, n)); }
+    const int S = p.nsplit;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int split = slot % S, unit = (slot / S) * 8 + xcd;
+    if (unit >= p.H * p.B) return;                       // the grid is padded to whole groups of 8 rows
+    const int h = unit % p.H, b = unit / p.H;
+    const int cap = p.Lk;
+    const int npass = (cap + 63) / 64, per = (npass + S - 1) / S;
+    const int t_lo = split * per, t_hi = min(npass, t_lo + per);
     const half_t *qp = p.q + h * p.qs[2] + b * p.qs[3];
-    const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
-    const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
+    half_t *kb = const_cast<half_t *>(p.k) + h * p.ks[2] + b * p.ks[3];
+    half_t *vb = const_cast<half_t *>(p.v) + h * p.vs[2] + b * p.vs[3];
     const int e0 = cl * 8;
     const bool eok = e0 < p.E;
     const u32x4 z = {0u, 0u, 0u, 0u};
+    const int n_raw = p.kv_len ? p.kv_len[b] : cap;
     u32x4 kc[2][SD_U], vc[2][SD_U];
     // pass t of this wave covers keys 64 t + 8 wave + grp
     auto fetch = [&](int set, int t0) {
 #pragma unroll
         for (int u = 0; u < SD_U; u++) {
-            const int key = 64 * (t0 + u) + 8 * wave + grp;
-            const int kk = min(key, Lk - 1);
-            const bool on = eok && 64 * (t0 + u) < Lk;           // uniform over the workgroup in its second half
-            const bool fresh = p.k_new && room && kk == Lk - 1;  // the row that this step appends
-            const half_t *kp = fresh ? p.k_new + h * p.ns[2] + b * p.ns[3] : kb + (long)kk * p.ks[1];
-            const half_t *vp = fresh ? p.v_new + h * p.ns[2] + b * p.ns[3] : vb + (long)kk * p.vs[1];
-            kc[set][u] = on ? ldg16(kp + e0) : z;
-            vc[set][u] = on ? ldg16(vp + e0) : z;
-            if (fresh && on && key == Lk - 1) {                  // exactly eight lanes of the workgroup own it
-                *reinterpret_cast<u32x4 *>(const_cast<half_t *>(kb) + (long)kk * p.ks[1] + e0) = kc[set][u];
-                *reinterpret_cast<u32x4 *>(const_cast<half_t *>(vb) + (long)kk * p.vs[1] + e0) = vc[set][u];
-            }
+            const int kk = min(64 * (t0 + u) + 8 * wave + grp, cap - 1);
+            const bool on = eok && t0 + u < t_hi;
+            kc[set][u] = on ? ldg16(kb + (long)kk * p.ks[1] + e0) : z;
+            vc[set][u] = on ? ldg16(vb + (long)kk * p.vs[1] + e0) : z;
         }
     };
-    const int npass = (Lk + 63) / 64;
-    if (npass > 0) fetch(0, 0);
-    if (npass > SD_U) fetch(1, SD_U);
+    if (t_lo < t_hi) fetch(0, t_lo);
+    if (t_lo + SD_U < t_hi) fetch(1, t_lo + SD_U);
+    u32x4 kn = z, vn = z;                                // the row that this step appends
+    if (p.k_new && eok) {
+        kn = ldg16(p.k_new + h * p.ns[2] + b * p.ns[3] + e0);
+        vn = ldg16(p.v_new + h * p.ns[2] + b * p.ns[3] + e0);
+    }
     float qv[8];
     {
         const half8v t = as_half8(eok ? ldg16(qp + e0) : z);
 #pragma unroll
         for (int j = 0; j < 8; j++) qv[j] = (float)t[j] * p.scale;
     }
+    // a length past the capacity: the cache is full, the new row is neither stored nor attended
+    const int Lk = max(0, min(cap, n_raw));
+    const int fresh = p.k_new && n_raw <= cap ? Lk - 1 : -1;
     float m = -INFINITY, l = 0.0f, acc[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) acc[j] = 0.0f;
     auto consume = [&](int set, int t0) {
 #pragma unroll
         for (int u = 0; u < SD_U; u++) {
-            if (64 * (t0 + u) < Lk) {                            // uniform: the shuffles below need the whole wave
+            if (t0 + u < t_hi && 64 * (t0 + u) < Lk) {           // uniform: the shuffles below need the whole wave
                 const int key = 64 * (t0 + u) + 8 * wave + grp;
-                const half8v kt = as_half8(kc[set][u]), vt = as_half8(vc[set][u]);
+                u32x4 kr = kc[set][u], vr = vc[set][u];
+                if (key == fresh) {                              // exactly eight lanes of one workgroup own it
+                    kr = kn; vr = vn;
+                    if (eok) {
+                        *reinterpret_cast<u32x4 *>(kb + (long)key * p.ks[1] + e0) = kn;
+                        *reinterpret_cast<u32x4 *>(vb + (long)key * p.vs[1] + e0) = vn;
+                    }
+                }
+                const half8v kt = as_half8(kr), vt = as_half8(vr);
                 float d = 0.0f;
 #pragma unroll
                 for (int j = 0; j < 8; j++) d = fmaf(qv[j], (float)kt[j], d);
@@ -853,11 +884,11 @@ __global__ __launch_bounds__(512) void sdpa_decode_kernel(SdpaArgs p) {
             }
         }
     };
-    for (int t0 = 0; t0 < npass; t0 += 2 * SD_U) {
+    for (int t0 = t_lo; t0 < t_hi; t0 += 2 * SD_U) {
         consume(0, t0);
-        if (t0 + 2 * SD_U < npass) fetch(0, t0 + 2 * SD_U);
-        if (t0 + SD_U < npass) consume(1, t0 + SD_U);
-        if (t0 + 3 * SD_U < npass) fetch(1, t0 + 3 * SD_U);
+        if (t0 + 2 * SD_U < t_hi) fetch(0, t0 + 2 * SD_U);
+        if (t0 + SD_U < t_hi) consume(1, t0 + SD_U);
+        if (t0 + 3 * SD_U < t_hi) fetch(1, t0 + 3 * SD_U);
     }
     // merge the 8 groups of the wave, then the 8 waves through LDS (flash.jl:1385-1391)
 #pragma unroll
@@ -877,18 +908,61 @@ __global__ __launch_bounds__(512) void sdpa_decode_kernel(SdpaArgs p) {
         if (lane == 0) { red_ml[wave][0] = m; red_ml[wave][1] = l; }
     }
     __syncthreads();
-    if (tid < p.E) {
-        float mm = -INFINITY;
+    float mm = -INFINITY, L = 0.0f, O = 0.0f;
+    if (tid < 64) {
 #pragma unroll
         for (int w = 0; w < 8; w++) mm = fmaxf(mm, red_ml[w][0]);
         const float mu = mm == -INFINITY ? 0.0f : mm;
-        float L = 0.0f, O = 0.0f;
 #pragma unroll
         for (int w = 0; w < 8; w++) {
             const float a = __expf(red_ml[w][0] - mu);
             L += a * red_ml[w][1];
             O += a * red_o[w][tid];
         }
+    }
+    if (S > 1) {                                         // uniform
+        const long row = (long)unit * S + split;
+        if (tid < p.E) p.part_o[row * p.E + tid] = O;
+        if (tid == 0) { p.part_ml[row * 2] = mm; p.part_ml[row * 2 + 1] = L; }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's part of the partial has reached the L2 ...
+        __syncthreads();                                  // ... and so has everybody's, before the ticket is drawn
+        if (tid == 0) {
+            const unsigned t = __hip_atomic_fetch_add(p.tickets + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = t == (unsigned)(S - 1);
+            if (is_last) __hip_atomic_store(p.tickets + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+        }
+        __syncthreads();
+        if (!is_last) return;
+        mm = -INFINITY; L = 0.0f; O = 0.0f;
+        if (tid < p.E) {
+            const long r0 = (long)unit * S;
+            for (int s0 = 0; s0 < S; s0 += 8) {
+                float ms[8], ls[8], os_[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const long r = r0 + min(s0 + j, S - 1);
+                    // read at the L2, past this compute unit's own cache
+                    ms[j] = s0 + j < S ? __hip_atomic_load(p.part_ml + r * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+                    ls[j] = __hip_atomic_load(p.part_ml + r * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    os_[j] = __hip_atomic_load(p.part_o + r * p.E + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                float mb = mm;
+#pragma unroll
+                for (int j = 0; j < 8; j++) mb = fmaxf(mb, ms[j]);
+                const float mu = mb == -INFINITY ? 0.0f : mb;
+                const float a0 = __expf(mm - mu);
+                L *= a0; O *= a0;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float a = __expf(ms[j] - mu);  // a split past the end has m = -inf: weight 0
+                    L += a * ls[j];
+                    O += a * os_[j];
+                }
+                mm = mb;
+            }
+        }
+    }
+    if (tid < p.E) {
         const float r = L > 0.0f ? O / L : 0.0f;
         const long oo = (long)b * p.os[3] + (long)h * p.os[2] + (long)tid * p.os[0];
         if (p.out_f32) reinterpret_cast<float *>(p.out)[oo] = r;
@@ -977,13 +1051,61 @@ int flash_splits(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     return (int)want;
 }
 
-// A single query row over a short key range (the decoder's self-attention over its cache) runs in one launch, one
-// workgroup per (head, batch): back to back 7.1 us against 8.2 us for splits + merge at 448 keys, 3.9 us against
-// 6.9 us at 4 (inside a dependent chain at 448 keys the two forms tie, the single launch at about 10 us of its own);
-// the work follows the device-side kv_len and the cache write can ride along (mi_sdpa_append_f16).  Longer ranges need more workgroups than heads to pull on HBM: 1500 keys
-// take 14.7 us this way at batch 1, 10.1 us split 24 ways.
+// A single query row (a decode step) runs in one launch of sdpa_decode_kernel: the work follows the device-side kv_len
+// and the cache write can ride along (mi_sdpa_append_f16).  Twenty heads alone leave most of the chip idle and give each
+// workgroup a long chain of keys, so a long key range is cut over several workgroups per row -- at most one workgroup
+// per compute unit, a round of six 64-key passes each -- which merge inside the launch.  Head dim <= 64, 16-byte addressable
+// operands, no additive mask; the rest goes to sdpa_rows_kernel (+ sdpa_merge_kernel).
+constexpr int SD_BANKS = 16, SD_TICKETS = 4096, SD_PART_FLOATS = 1 << 16;
+// Arrival counters and partials of the split form: a launch takes the next of SD_BANKS banks, so launches in flight
+// together on one GPU (up to SD_BANKS of them) do not touch each other's.  Zero when the module loads; every launch
+// leaves its counters at zero.
+static __device__ unsigned sd_ticket_words[SD_BANKS * SD_TICKETS];
+static __device__ __align__(256) float sd_part_words[SD_BANKS * SD_PART_FLOATS];
+constexpr int SD_MAX_DEVICES = 64;
+unsigned *g_sd_tickets[SD_MAX_DEVICES] = {};
+float *g_sd_parts[SD_MAX_DEVICES] = {};
+std::atomic<unsigned> g_sd_launch{0};
+
 bool one_pass_decode(const SdpaArgs &a, bool vec) {
-    return a.Lq == 1 && vec && !a.bias && a.E <= 64 && a.Lk >= 1 && a.Lk <= 640;
+    return a.Lq == 1 && vec && !a.bias && a.E <= 64 && a.Lk >= 1 && (int64_t)a.H * a.B <= SD_TICKETS;
+}
+
+int decode_splits(int64_t E, int64_t Lk, int64_t H, int64_t B) {
+    const int64_t units = H * B, passes = ceil_div(Lk, 64);
+    // The exchange adds about 3 us of its own (partial out, ticket, partials in: three trips in a row), a workgroup
+    // walks six passes in about one trip: 448 keys stay whole (5.9 us either way at batch 1), 1500 keys are cut
+    // four ways at batch 1 (11.1 us whole, 7.2 us cut in 4, 10.2 us cut in 12) and three ways at batch 4.
+    int64_t want = mi_num_cus() / units;                 // at most one workgroup per compute unit
+    if (want > ceil_div(passes, SD_U)) want = ceil_div(passes, SD_U);      // one round of passes each
+    if (passes <= 8) want = 1;
+    if (want > 32) want = 32;
+    while (want > 1 && units * want * (E + 2) > SD_PART_FLOATS) want--;
+    if (want < 1) want = 1;
+#ifdef MI_LAB
+    if (const char *f = getenv("MI_FORCE_DSPLIT")) { want = atoi(f); if (want > passes) want = passes; if (want < 1) want = 1; }
+#endif
+    // no empty split: with `per` passes each, the last one must still start inside the range
+    while (want > 1 && ceil_div(passes, want) * (want - 1) >= passes) want--;
+    return (int)want;
+}
+
+// Fills in the split count and, for a split launch, this launch's bank of counters and partials, and launches.
+int launch_decode(SdpaArgs &a, hipStream_t st) {
+    a.nsplit = decode_splits(a.E, a.Lk, a.H, a.B);
+    if (a.nsplit > 1) {
+        int dev = -1;
+        if (!mi_xcd_round_robin() || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SD_MAX_DEVICES || !g_sd_tickets[dev]) a.nsplit = 1;
+        else {
+            const unsigned bank = g_sd_launch++ % SD_BANKS;
+            a.tickets = g_sd_tickets[dev] + (size_t)bank * SD_TICKETS;
+            a.part_o = g_sd_parts[dev] + (size_t)bank * SD_PART_FLOATS;
+            a.part_ml = a.part_o + (size_t)a.H * a.B * a.nsplit * a.E;
+        }
+    }
+    const unsigned units8 = (unsigned)ceil_div((int64_t)a.H * a.B, 8);
+    hipLaunchKernelGGL(sdpa_decode_kernel, dim3(units8 * 8 * a.nsplit), dim3(512), 0, st, a);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
 // A mask the fused kernel can carry: keys contiguous (a lane reads runs of four), the other axes any stride including
@@ -1016,6 +1138,7 @@ int fill(SdpaArgs &a, void *out, int out_dtype, const int64_t *os, const void *q
     else { a.os[0] = 1; a.os[1] = E; a.os[2] = E * Lq; a.os[3] = E * Lq * H; }
     a.bias = bias; a.bias_f32 = bias_dtype == MI_F32; a.kv_len = kv_len;
     a.part_o = a.part_ml = nullptr;
+    a.tickets = nullptr;
     a.k_new = a.v_new = nullptr;
     for (int i = 0; i < 4; i++) a.ns[i] = 0;
     a.E = (int)E; a.Lq = (int)Lq; a.Lk = (int)Lk; a.H = (int)H; a.B = (int)B;
@@ -1035,6 +1158,15 @@ void launch_rows(const SdpaArgs &a, bool vec, dim3 grid, hipStream_t st) {
 // default 64 KiB of dynamic LDS.
 int mi_sdpa_init() {
     int bad = 0;
+    {   // this device's copies of the decode kernel's counters and partials (zeroed at load; never named in host code again)
+        int dev = -1;
+        void *t = nullptr, *pw = nullptr;
+        if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < SD_MAX_DEVICES &&
+            hipGetSymbolAddress(&t, HIP_SYMBOL(sd_ticket_words)) == hipSuccess && hipGetSymbolAddress(&pw, HIP_SYMBOL(sd_part_words)) == hipSuccess) {
+            g_sd_tickets[dev] = reinterpret_cast<unsigned *>(t);
+            g_sd_parts[dev] = reinterpret_cast<float *>(pw);
+        }
+    }
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
@@ -1073,7 +1205,7 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
     if (rc != MI_OK) return MI_SDPA_DECLINE;
     int path = sdpa_path(a);
     const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
-    if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? (one_pass_decode(a, vec) ? 1 : rows_splits(Lq, Lk, H, B))
+    if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? (one_pass_decode(a, vec) ? decode_splits(E, Lk, H, B) : rows_splits(Lq, Lk, H, B))
                                   : (path == MI_SDPA_FLASH && !has_bias) ? flash_splits(E, Lq, Lk, H, B) : 1;
     return path;
 }
@@ -1140,11 +1272,7 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
     }
     // rows path
     bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
-    if (one_pass_decode(a, vec)) {
-        a.nsplit = 1;
-        hipLaunchKernelGGL(sdpa_decode_kernel, dim3((unsigned)H, 1, (unsigned)B), dim3(512), 0, st, a);
-        return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
-    }
+    if (one_pass_decode(a, vec)) return launch_decode(a, st);
     a.nsplit = Lq < 64 ? rows_splits(Lq, Lk, H, B) : 1;
     if (a.nsplit > 1) {
         size_t rows = (size_t)Lq * H * B;
@@ -1184,8 +1312,7 @@ int mi_sdpa_append_f16(void *out, int out_dtype, const int64_t out_strides[4],
     const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E) &&
                      vec_addressable(a.k_new, a.ns, a.E) && vec_addressable(a.v_new, a.ns, a.E);
     if (!one_pass_decode(a, vec)) return MI_DECLINE_UNSUPPORTED;      // the caller appends and attends in two calls
-    hipLaunchKernelGGL(sdpa_decode_kernel, dim3((unsigned)H, 1, (unsigned)B), dim3(512), 0, (hipStream_t)stream, a);
-    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+    return launch_decode(a, (hipStream_t)stream);
 }
 
 }  // extern "C"

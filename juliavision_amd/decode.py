@@ -138,7 +138,7 @@ def decoder_layer_step(ctx: Ctx, W: DecoderLayerWeights, cache: KVCache, layer: 
 
     normed_linear(buf.qkv, W.wqkv, x, W.ln1_g, W.ln1_b, W.bqkv)
     q, k_new, v_new = (buf.qkv[:, i * d:(i + 1) * d].unflatten(1, (H, 1, E)) for i in range(3))
-    if FUSE_APPEND and E <= 64 and E % 8 == 0 and cache.max_target <= 640:
+    if FUSE_APPEND and E <= 64 and E % 8 == 0:
         # one launch: the new row is key length - 1 and goes into its cache slot on the way
         sdpa_append(ctx, q, cache.self_k[layer], cache.self_v[layer], k_new, v_new, cache.length, out=heads(buf.att))
     else:

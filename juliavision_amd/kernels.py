@@ -495,7 +495,7 @@ def sdpa_append(ctx: Ctx, q, cache_k, cache_v, k_new, v_new, kv_len, scale=None,
     become key ``kv_len[b] - 1`` and are stored into that slot of ``cache_k``/``cache_v`` (B,H,Lmax,E); ``out``
     (B,H,1,E) = attention of ``q`` (B,H,1,E) over the first ``kv_len[b]`` keys.  One launch in place of the exported
     step's ``index_put`` + ``cat`` + attention (WhisperRunner/src/decode.jl:186-203).  Raises ``DeclineError`` with
-    ``L.DECLINE_UNSUPPORTED`` for shapes the single-launch kernel does not cover (head dim > 64, more than 640 slots):
+    ``L.DECLINE_UNSUPPORTED`` for shapes the single-launch kernel does not cover (head dim > 64, rows not 16-byte addressable):
     the caller then appends and attends in two calls."""
     if not _is_f16_cuda(q, cache_k, cache_v, k_new, v_new) or q.dim() != 4 or cache_k.dim() != 4:
         raise DeclineError("sdpa_append: operands", L.DECLINE_OPERANDS)

@@ -172,10 +172,11 @@ def test_step_graph_replays_match_eager(ctx):
         assert to_host(cg.length).tolist() == [t + 1] * B
 
 
-@pytest.mark.parametrize("E,Lmax", [(64, 448), (32, 70), (64, 16)])
+@pytest.mark.parametrize("E,Lmax", [(64, 448), (32, 70), (64, 16), (64, 1500), (48, 2049), (64, 8000)])
 def test_fused_append_and_attend_equals_the_two_calls(ctx, E, Lmax):
     """mi_sdpa_append_f16 against mi_kv_append_f16 followed by mi_sdpa_f16 on a twin cache: the same cache bits, the
-    same output bits (both attend with the one-launch kernel), and the oracle's attention over the updated cache."""
+    same output bits (both attend with the one-launch kernel, its key range cut over the same number of workgroups),
+    and the oracle's attention over the updated cache."""
     import torch
     import juliavision_amd as jv
     B, H = 4, 3
@@ -207,7 +208,7 @@ def test_fused_append_declines_what_the_one_launch_kernel_does_not_cover(ctx):
     import torch
     import juliavision_amd as jv
     from juliavision_amd import _lib as L
-    B, H, E, Lmax = 1, 2, 64, 700                                       # more than 640 slots
+    B, H, E, Lmax = 1, 2, 128, 64                                       # head dim over 64
     z = lambda *s: torch.zeros(s, dtype=torch.float16, device="cuda")
     with pytest.raises(jv.DeclineError) as e:
         jv.sdpa_append(ctx, z(B, H, 1, E), z(B, H, Lmax, E), z(B, H, Lmax, E), z(B, H, 1, E), z(B, H, 1, E),

@@ -337,15 +337,20 @@ def test_reference_point_follows_scores_that_grow_along_the_keys(ctx, B, H, Lq, 
     assert np.all(np.isfinite(got))
 
 
-@pytest.mark.parametrize("Lk", [1, 7, 8, 63, 64, 65, 383, 384, 385, 448, 640])
+@pytest.mark.parametrize("Lk", [1, 7, 8, 63, 64, 65, 383, 384, 385, 448, 640, 1500, 4097])
 @pytest.mark.parametrize("E", [64, 40, 16])
 def test_single_query_over_a_short_key_range_runs_in_one_launch(ctx, Lk, E):
-    """Lq = 1 and at most 640 keys (the decoder's self-attention over its cache): one workgroup per (head, batch),
-    eight waves striding the keys in rounds of six passes.  Key counts around the pass (64) and round (384) sizes."""
+    """Lq = 1 (a decode step): one launch, eight-wave workgroups striding the keys in rounds of six passes, the key
+    range beyond 512 keys cut over several workgroups (a round of six passes each) that merge inside the launch.
+    Key counts around the pass (64) and round (384) sizes, and ranges that split 2, 4 and 11 ways."""
     import juliavision_amd as jv
     q, k, v = _qkv(3, 5, 1, Lk, E, 401 + Lk)
     plan = jv.sdpaplan(ctx, to_dev(q), to_dev(k), to_dev(v))
-    assert type(plan).__name__ == "RowsSDPAPlan" and plan.nsplit == 1, plan
+    passes = (Lk + 63) // 64
+    want = 1 if passes <= 8 else max(1, min(ctx.dev.cores // 15, -(-passes // 6)))
+    while want > 1 and -(-((Lk + 63) // 64) // want) * (want - 1) >= (Lk + 63) // 64:
+        want -= 1
+    assert type(plan).__name__ == "RowsSDPAPlan" and plan.nsplit == want, plan
     _check(ctx, q, k, v, expect="RowsSDPAPlan", what=f"one-launch decode attention Lk{Lk} E{E}")
     lens = [Lk, 0, max(1, Lk // 2)]
     got = _check(ctx, q, k, v, kv_len=lens, out_dtype="f32", expect="RowsSDPAPlan", what=f"one-launch decode attention Lk{Lk} E{E} kv_len")
