@@ -1314,6 +1314,120 @@ __global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p) {
     }
 }
 
+// The same product with the activations in registers instead of LDS, for the few rows of a decode step: a lane's
+// weight chunks sit at k = 8 lane + 512 i, so it needs exactly those chunks of every activation row and asks for
+// them itself (the rows come from the L2: every wave of the launch reads the same few KB).  No staging, no barrier:
+// a wave is a chain of one trip to memory, the norm statistics (its own copy, same summation order as
+// ln_row_stats, so the same bits), the dot products, one wave reduction and a store.  R output columns per wave,
+// all their weight rows requested up front.  (MT + R + 2) * PF chunks of registers: built for one and two rows of
+// K <= 1536 (78 to 119 registers, four to six waves per SIMD); four rows, or K = 5120, would leave a SIMD one or
+// two waves and stay with the staged kernel.
+template <int MT, int PF, int R>
+__global__ __launch_bounds__(256) void skinny_fk_reg_kernel(GemmArgs p) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    const int n0 = (blockIdx.x * 4 + wave) * R;
+    if (n0 >= p.N) return;                                // uniform over the wave; no barrier below
+    u32x4 w[R][PF];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const half_t *bp = p.B + (long)min(n0 + r, p.N - 1) * p.ldB;
+#pragma unroll
+        for (int i = 0; i < PF; i++) w[r][i] = lane * 8 + 512 * i < p.K ? ldg16(bp + lane * 8 + 512 * i) : z;
+    }
+    u32x4 x[MT][PF], gr[PF], br[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        const int k = lane * 8 + 512 * i;
+        gr[i] = br[i] = z;
+#pragma unroll
+        for (int m = 0; m < MT; m++) x[m][i] = m < p.M && k < p.K ? ldg16(p.A + (long)m * p.ldA + k) : z;
+        if (p.ln_on && k < p.K) {
+            if (p.ln_gamma) gr[i] = ldg16(p.ln_gamma + k);
+            if (p.ln_beta) br[i] = ldg16(p.ln_beta + k);
+        }
+    }
+    float bv[R], rv[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        bv[r] = rv[r] = 0.0f;
+        if (lane < p.M && n0 + r < p.N) {
+            if (p.bias_mode == MI_BIAS_COL) bv[r] = (float)p.bias[n0 + r];
+            else if (p.bias_mode == MI_BIAS_ROW) bv[r] = (float)p.bias[lane];
+            if (p.residual && !p.out_f32) rv[r] = (float)p.residual[(long)lane * p.ldY + n0 + r];
+        }
+    }
+    if (p.ln_on) {                                        // uniform
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < PF; i++) {
+                if (lane * 8 + 512 * i < p.K) {
+                    const half8v t = as_half8(x[m][i]);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) s1 += (float)t[j];
+                }
+            }
+            s1 = wave_sum(s1);
+            const float mu = s1 / (float)p.K;
+#pragma unroll
+            for (int i = 0; i < PF; i++) {
+                if (lane * 8 + 512 * i < p.K) {
+                    const half8v t = as_half8(x[m][i]);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) { const float d = (float)t[j] - mu; s2 = fmaf(d, d, s2); }
+                }
+            }
+            s2 = wave_sum(s2);
+            const float rs = 1.0f / sqrtf(s2 / (float)p.K + p.ln_eps);
+#pragma unroll
+            for (int i = 0; i < PF; i++) {
+                const half8v t = as_half8(x[m][i]), gv = as_half8(gr[i]), bb = as_half8(br[i]);
+                half8v o;
+#pragma unroll
+                for (int j = 0; j < 8; j++) o[j] = ln_norm1((float)t[j], mu, rs, p.ln_gamma != nullptr, (float)gv[j], p.ln_beta != nullptr, (float)bb[j]);
+                x[m][i] = lane * 8 + 512 * i < p.K ? __builtin_bit_cast(u32x4, o) : z;
+            }
+        }
+    }
+    float acc[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int m = 0; m < MT; m++) acc[r][m] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int m = 0; m < MT; m++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const uint32_t wq = w[r][i][q], xq = x[m][i][q];
+                    acc[r][m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, wq), __builtin_bit_cast(half2v, xq), acc[r][m], false);
+                }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float mine = 0.0f;                                // lane m keeps row m's sum
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const float sres = wave_sum(acc[r][m]);
+            if (lane == m) mine = sres;
+        }
+        if (lane < p.M && n0 + r < p.N) {
+            const float v = mine + bv[r];
+            const long off = (long)lane * p.ldY + n0 + r;
+            if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(v, p.epi);
+            else {
+                half_t o = (half_t)apply_epi((float)(half_t)v, p.epi);
+                if (p.residual) o = (half_t)((float)o + rv[r]);
+                reinterpret_cast<half_t *>(p.Y)[off] = o;
+            }
+        }
+    }
+}
+
 // Split-K epilogue: out = epi(round(sum_s part[s] + bias)) (+ residual), four columns per thread.
 // The counterpart of mm_epilogue_kernel! (matmul.jl:192-217): the planes are fp32 M x N.
 __global__ void splitk_epilogue_kernel(GemmArgs p, const float *part, int nsplit) {
@@ -1785,6 +1899,27 @@ int run_skinny(GemmArgs a, bool b_kn, void *ws, size_t ws_bytes, hipStream_t st)
         // One weight row per wave.  More rows per wave would amortise the staging of the activations, but the
         // rows of a wave run one after the other, each a chain of dependent memory trips: measured slower at
         // every batch size (1280 -> 5120, batch 8: 9.1 us with one row, 13.7 us with four).
+        // One or two rows without a norm in front: activations in registers, no staging (hot in a replayed graph at
+        // batch 1: 2.88 / 3.13 / 3.34 us for 1280 -> 1280 / 3840 / 5120 against 3.01 / 3.33 / 3.57 us staged).  With
+        // the layer-norm prologue every wave would normalise its own copy of the row -- 4.5 / 6.1 / 6.9 us against
+        // 3.9 / 4.3 / 4.7 us -- so that stays staged, and so does a very wide output (51866 columns: 24.5 against 23.0 us).
+        int R = 1;
+#ifdef MI_LAB
+        if (const char *f = getenv("MI_FORCE_GEMV_R")) R = atoi(f);
+        if (R >= 1 && a.K <= 1536 && mt <= 2) {
+#else
+        if (!a.ln_on && a.N <= 8192 && a.K <= 1536 && mt <= 2) {
+#endif
+            dim3 rg((unsigned)ceil_div(a.N, 4 * R));
+            if (R == 2) {
+                if (mt == 1)      hipLaunchKernelGGL((skinny_fk_reg_kernel<1, 3, 2>), rg, dim3(256), 0, st, a);
+                else              hipLaunchKernelGGL((skinny_fk_reg_kernel<2, 3, 2>), rg, dim3(256), 0, st, a);
+            } else {
+                if (mt == 1)      hipLaunchKernelGGL((skinny_fk_reg_kernel<1, 3, 1>), rg, dim3(256), 0, st, a);
+                else              hipLaunchKernelGGL((skinny_fk_reg_kernel<2, 3, 1>), rg, dim3(256), 0, st, a);
+            }
+            return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+        }
         dim3 grid((unsigned)ceil_div(a.N, 4));
         if (a.K <= 1536) {
             if (mt == 1)      hipLaunchKernelGGL((skinny_fk_kernel<1, 3>), grid, dim3(256), lds, st, a);
