@@ -69,13 +69,14 @@ __device__ __forceinline__ void static_for(F &&f) {
 //     first product is already in the base-2 exponent domain;
 //   * the reference point M of the running softmax is subtracted by the MFMA itself:
 //     the first product carries one extra k-step whose operands contribute
-//     1.0 * (-M[query]) to every score, so it delivers t = s - M and p = exp2(t)
+//     1.0 * (-M[query]) to every score -- or, in the ping-pong form, starts its chain from
+//     -M[query] instead of zero -- so it delivers t = s - M and p = exp2(t)
 //     needs no further arithmetic (M is kept fp16-representable so that what is
 //     subtracted is exactly what the bookkeeping assumes);
 //   * M is a *stale* reference, not the running maximum: it moves on the first
-//     block and when a probability would leave fp16 range (the block's largest t
-//     reaches 16; one v_max3_f32 per two scores keeps track of it), and then to the
-//     block maximum.  The result is the same softmax -- every term of a row carries the
+//     block and when a probability would leave fp16 range (some t reaches 16: the
+//     fp32 row sum then grows by 2^16 in one block, which is what is tested), and then
+//     to the block maximum.  The result is the same softmax -- every term of a row carries the
 //     same factor 2^-M -- with the rescaling of flash.jl:25-38 applied lazily (the
 //     reference's `lazyrescale`, flash.jl:1041-1096, skips it when no maximum grew;
 //     this skips it until fp16 would overflow);
@@ -86,7 +87,9 @@ __device__ __forceinline__ void static_for(F &&f) {
 // half a key block apart by two workgroup barriers per block, so that while one of them is in its
 // exponentials the other is in its matrix half (the block's second product and the next block's first):
 // the matrix pipe and the vector ALU of a SIMD are then busy with different waves instead of both
-// waves wanting the same unit at the same time.  Waves 0-3 do all the global -> LDS staging.
+// waves wanting the same unit at the same time.  All eight waves stage: a wave writes its sixteenth of block j + 2
+// in its own matrix half of block j, into the stage whose last readers finished before the barrier it just passed,
+// and two barriers lie between the later group's write and the first read of that stage.
 //
 // KH = 2 (grids that leave every CU at most one workgroup): eight waves on 128 queries.  Waves w and w+4 own the
 // same 32 queries and share a SIMD; a stage holds 128 keys, of which waves 0-3 take the first 64 and waves 4-7 the
@@ -104,11 +107,11 @@ constexpr int flash_vld(int EP) { return EP == 96 ? EP : EP + 32; }
 // log2(e), ahead of the exponentials -- the reference's bias term of attention.jl:55-59, which its own fused kernel
 // declines (flash.jl:1327).
 template <int EP, bool PP, int KH = 1, int BIAS = 0>      // BIAS: 0 none, 1 fp16, 2 fp32
-__global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH == 1) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
+__global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH == 1 && (BIAS == 0 || EP == 64)) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
     static_assert(BIAS == 0 || (!PP && KH == 1), "the mask rides in the four-wave form");
     // PP with KH = 2: the two key-half groups of the eight-wave form (same 128 queries) take turns at the vector
     // and matrix units like the two query groups of the 256-query form do; every thread stages.
-    constexpr int BC = 64, BR = (PP && KH == 1) ? 256 : 128, NT = KH == 2 ? 512 : 256;     // NT: threads that stage K and V
+    constexpr int BC = 64, BR = (PP && KH == 1) ? 256 : 128, NT = (KH == 2 || PP) ? 512 : 256;     // NT: threads that stage K and V
     constexpr int BCS = BC * KH;                                                // keys per LDS stage
     constexpr int KLD = EP + 8, VLD = flash_vld(EP);
     constexpr int KS = EP / 16;       // k16 steps over the head dim
@@ -125,7 +128,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     const int grp = wave >> 2;                               // PP, KH = 2: 0 = waves 0-3, 1 = waves 4-7
     const int qw = KH == 2 ? (wave & 3) : wave;              // which 32 queries of the block
     const int gk = KH == 2 ? grp * BC : 0;                   // this wave's first key within a stage
-    const bool loader = !PP || KH == 2 || grp == 0;
+    constexpr bool loader = true;                            // every wave stages its share of a key block
     const int hl = lane >> 5, l32 = lane & 31;
     // Workgroups are dealt to the 8 XCDs round-robin in launch order; renumbering them so that each XCD
     // owns a contiguous run keeps all query blocks of a head on one XCD, whose L2 then holds that head's
@@ -234,9 +237,17 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     for (int t = 0; t < ET; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o_acc[t][r] = 0.0f;
-    // The reference point M rides along as one more k-step of the first product:
-    // an operand pair that contributes 1.0 * (-M[query]) to every score.
+    // The reference point M rides along in the first product.  SEED (the 256-query ping-pong form, whose matrix half
+    // is the longer one): every score of a lane belongs to its one query, so the chain starts from -M[query] in all
+    // sixteen accumulator registers instead of from zero (config 4: 87 -> 79 us).  Otherwise: one more k-step with the
+    // operand pair 1.0 and -M, two MFMAs more per block but sixteen registers fewer -- the forms that run two
+    // workgroups per CU or are 96 wide sit at the register limit, and measured the same or slower with the seed
+    // (config 3 19.0 -> 19.5 us, the 72-wide windows 13.4 -> 15.2 us).
+    constexpr bool SEED = PP && KH == 1;
+    float16v negm;
     half8v kext, qext;
+#pragma unroll
+    for (int r = 0; r < 16; r++) negm[r] = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) { kext[j] = (half_t)0.0f; qext[j] = (half_t)0.0f; }
     if (hl == 0) kext[0] = (half_t)1.0f;
@@ -265,7 +276,6 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
     const int vtoff = (gk + 4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
     const int ktoff = (gk + l32) * KLD + 8 * hl;
-    const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // t = s*scale*log2(e) - M, straight out of the MFMA chain
     auto qk = [&](float16v (&s)[2], int st) {
@@ -273,11 +283,11 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
 #pragma unroll
         for (int kt = 0; kt < 2; kt++) {
             const half_t *kp_ = kbase + 32 * kt * KLD;
-            s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], zero16, 0, 0, 0);
+            s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], negm, 0, 0, 0);
 #pragma unroll
             for (int ks = 1; ks < KS; ks++)
                 s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_ + 16 * ks), qf[ks], s[kt], 0, 0, 0);
-            s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, s[kt], 0, 0, 0);
+            if constexpr (!SEED) s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, s[kt], 0, 0, 0);
         }
     };
     // p = 2^t as fp16 MFMA operands; the row sum is kept in fp32 with plain adds (v_dot2_f32_f16 on the
@@ -396,10 +406,6 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         half8v pf[2][2];
         float l_new = l_run;
         probs(sc, pf, l_new);
-        // the largest exponent of the block, three at a time: what tells that a probability left fp16 range
-        float tmax = fmaxf(sc[0][0], sc[1][0]);
-#pragma unroll
-        for (int r = 1; r < 16; r++) tmax = fmaxf(fmaxf(tmax, sc[0][r]), sc[1][r]);
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * KS, 0);
 #pragma unroll
         for (int g = 0; g < 2 * KS + 2; g++) {
@@ -407,11 +413,16 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
             __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + 2), 0);     // the remaining vector work trails the last MFMA
         }
         __builtin_amdgcn_sched_barrier(0);
-        // A probability leaves fp16 range at t >= 16 (2^16 rounds to infinity; the row sum, kept in fp32 from the
-        // unrounded values, would not show it).  Then, and on the first block, settle a new reference point: the
-        // block maximum, for the rows that outgrew the old one by 2^TH; rescale what was accumulated; redo the
-        // exponentials.
-        if (__any(first || tmax >= 15.9f)) {
+        // A probability leaves fp16 range at t >= 16 (2^16 rounds to infinity).  The row sum, kept in fp32 from the
+        // unrounded values, tells: it cannot have grown by less than 2^16 - 16 if one of the block's terms did
+        // (and if it grew that much through many smaller terms, settling a new reference point is still right, only
+        // not needed).  Then, and on the first block, settle a new reference point: the block maximum, for the rows
+        // that outgrew the old one by 2^TH; rescale what was accumulated; redo the exponentials.  The maximum is only
+        // looked for here: the fast path spends no instruction on it.
+        if (__any(first || !(l_new - l_run < 65504.0f))) {
+            float tmax = fmaxf(sc[0][0], sc[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; r++) tmax = fmaxf(fmaxf(tmax, sc[0][r]), sc[1][r]);
             float mx = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
             const bool grow = (mx > TH || first) && mx != -INFINITY;
             const half_t m16 = (half_t)(m_ref + (grow ? mx : 0.0f));
@@ -419,7 +430,10 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
             const float alpha = __builtin_amdgcn_exp2f(-d);
             m_ref += d;
             l_run *= alpha;
-            if (hl == 0) qext[0] = -m16;
+            if constexpr (SEED) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) negm[r] = -(float)m16;
+            } else if (hl == 0) qext[0] = -m16;
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
