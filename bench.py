@@ -727,6 +727,9 @@ def detail_benchmarks(lib, L, stream, only=None):
     # config 1: the linear, both weight layouts
     gemm_case("c1_linear_1500x1280x5120_W[K][F]_bias", 1500, 1280, 5120, L.W_KF)
     gemm_case("c1_linear_1500x1280x5120_W[F][K]_bias", 1500, 1280, 5120, L.W_FK)
+    # not a BASELINE config: the same kernel family where the grid fills the chip for many rounds (256 x 256 tiles)
+    gemm_case("square_4096x4096x4096_W[K][F]_bias", 4096, 4096, 4096, L.W_KF, sets=2, reps=10)
+    gemm_case("square_8192x8192x8192_W[K][F]_bias", 8192, 8192, 8192, L.W_KF, sets=1, reps=5)
     gemm_case("c2_proj_1500x1280x1280", 1500, 1280, 1280, L.W_KF)
     gemm_case("c2_fc2_1500x5120x1280", 1500, 5120, 1280, L.W_KF)
     # config 3: ViT-S/14 shapes

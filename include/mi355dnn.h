@@ -227,10 +227,13 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4],
 /* ---------------------------------------------------------------- convolution
  * Reference layout: x (W,H,Cin,N) = row-major [N][Cin][H][W]; w (KW,KH,Cin,Cout) =
  * [Cout][Cin][KH][KW]; out (OW,OH,Cout,N); bias[Cout] or NULL; stride / padding /
- * dilation as (x, y) pairs; act MI_EPI_NONE or MI_EPI_RELU; groups must be 1
- * (anything else declines, as the reference routes grouped convolutions to its
- * direct kernel).  fp32 accumulation seeded with the bias, one rounding, relu
- * on the rounded value.
+ * dilation as (x, y) pairs; act MI_EPI_NONE or MI_EPI_RELU (anything else returns
+ * MI_DECLINE_UNSUPPORTED).  groups = 1 runs as a GEMM (1x1, implicit, or im2col: see
+ * mi_conv2d_f16_plan); groups > 1 -- w then holds Cin / groups input channels per filter --
+ * runs a direct kernel, one thread per output element, as the reference routes
+ * grouped convolutions to its direct kernel (conv.jl:100-145); Cin or Cout not
+ * divisible by groups declines.  fp32 accumulation seeded with the bias, one rounding,
+ * relu on the rounded value.
  * Replaces convolution!(ctx, out, x, w, bias, stride, padding, dilation, groups; act)
  * -- conv.jl:100-145 -- and convolution_coopmat! / im2col_kernel! /
  * conv_epilogue_kernel! -- conv_coopmat.jl:246-392; the implicit-GEMM path (stride_x 1,

@@ -717,8 +717,13 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         sk_s = idx % p.sk_S;
         sk_tile = xcd * p.sk_tpx + idx / p.sk_S;
         if (sk_tile >= p.tiles_m * p.tiles_n) return;          // the whole workgroup: the last XCD's run may be short
-        tm_ = sk_tile % p.tiles_m;
-        tn_ = sk_tile / p.tiles_m;
+        // an XCD's run of the tile order covers about as many row tiles as column tiles (group_m rows per column
+        // step), so its L2 pulls few panels of either operand: 1500 x 5120 -> 1280 fetched 156 MB with runs that
+        // walked whole columns of 12 row tiles
+        const int width = p.group_m * p.tiles_n, g = sk_tile / width, in = sk_tile - g * width;
+        const int first = g * p.group_m, gsz = min(p.tiles_m - first, p.group_m);
+        tm_ = first + in % gsz;
+        tn_ = in / gsz;
     } else {
         tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
     }
@@ -1720,6 +1725,7 @@ int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
     a.tiles_m = (int)ceil_div(a.M, BM);
     a.tiles_n = (int)ceil_div(a.N, BN);
     a.group_m = 1;
+    while (a.group_m * a.group_m < (int)ceil_div((int64_t)a.tiles_m * a.tiles_n, 8) && a.group_m < a.tiles_m) a.group_m++;
     a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
                             : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
     if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? 64 : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;

@@ -326,9 +326,10 @@ RESHAPES = ("view.default", "_unsafe_view.default", "reshape.default", "alias.de
 
 def fold_activations(g: Graph) -> Graph:
     """gelu / relu whose only producer is a linear op -- directly or through a chain of views, as the
-    decomposed ``addmm`` + ``view`` form of ``linear`` has it -- read by nothing else becomes that op's
-    epilogue (foldrelu.jl:60-125); the activation's buffer then aliases what it used to read.  An
-    elementwise function commutes with any view, so the chain may reshape or permute freely."""
+    decomposed ``addmm`` + ``view`` form of ``linear`` has it -- or an ordinary convolution, read by nothing
+    else, becomes that op's epilogue (foldrelu.jl:60-125; the convolution kernels take it as ``act``); the
+    activation's buffer then aliases what it used to read.  An elementwise function commutes with any view,
+    so the chain may reshape or permute freely."""
     for act in [o for o in g.ops if o["aten"] in ACTIVATIONS]:
         if act["aten"] == "gelu.default" and act["attrs"].get("approximate", "none") != "none":
             continue                                    # only the erf form is the folded epilogue's arithmetic
@@ -338,7 +339,9 @@ def fold_activations(g: Graph) -> Graph:
             chain.append(g.buffers[chain[-1]]["of"])
         prod = g.op(chain[-1])
         single = g.readers(src) == [act["id"]] and all(len(g.readers(c)) == 1 for c in chain[1:]) and not any(c in g.outputs for c in chain)
-        if prod is None or prod["aten"] not in LINEAR_OPS or not single or "epilogue" in prod["attrs"] or "residual" in prod["attrs"]:
+        # an ordinary (not transposed) convolution takes relu, the reference's ``act`` (conv.jl:100-145); gelu after one stays an op
+        conv = prod is not None and prod["aten"] == "convolution.default" and not prod["attrs"].get("arg6") and act["aten"] == "relu.default"
+        if prod is None or not (prod["aten"] in LINEAR_OPS or conv) or not single or "epilogue" in prod["attrs"] or "residual" in prod["attrs"]:
             continue
         prod["attrs"]["epilogue"] = ACTIVATIONS[act["aten"]]
         g.ops.remove(act)
@@ -1309,7 +1312,7 @@ class Executor:
         if a.get("arg6"):
             K.convolutiontranspose_(self.ctx, out, x, w, bias, xy(stride), xy(padding), xy(dilation), xy(outpad), a.get("arg8", 1))
         else:
-            K.convolution_(self.ctx, out, x, w, bias, xy(stride), xy(padding), xy(dilation), a.get("arg8", 1))
+            K.convolution_(self.ctx, out, x, w, bias, xy(stride), xy(padding), xy(dilation), a.get("arg8", 1), act=a.get("epilogue", "none"))
 
     def _embedding(self, o):
         """embedding(table, ids) / index.Tensor(table, [ids]) along the first axis (ops.jl:1754-1783, 1524-1640); with

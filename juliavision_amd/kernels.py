@@ -80,7 +80,14 @@ def caps() -> DeviceCaps:
 class Workspace:
     """Per-op bump scratch (workspace.jl:19-106): ``reset()`` before every op,
     ``scratch(nbytes)`` hands out 256-byte aligned device memory valid until the
-    next reset.  Grows by reallocation between ops, never inside one."""
+    next reset.  Grows by reallocation between ops, never inside one.
+
+    A captured graph (``StepGraph``, ``Executor.replayable``) holds the addresses it was captured with -- split-K
+    planes, split-KV partials, convolution scratch -- for as long as it may be replayed.  So a buffer that was
+    ever handed out is never given back: growing retires the old buffer into ``_retired``, where it stays until
+    the workspace itself goes, and a replay after later growth still writes memory that nothing else owns.
+    Growing *during* a capture cannot work (the allocation would be captured too) and raises: run the step
+    eagerly once first, as both graph wrappers do, so that the workspace has reached its size."""
 
     ALIGN = 256
 
@@ -88,11 +95,10 @@ class Workspace:
         self.device = torch.device(device)
         self.buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=self.device)
         self.off = 0
-        self._pending = []
+        self._retired = []
 
     def reset(self):
         self.off = 0
-        self._pending.clear()
 
     def scratch(self, nbytes: int) -> int:
         if nbytes <= 0:
@@ -100,8 +106,9 @@ class Workspace:
         base = self.buf.data_ptr()
         start = (-(base + self.off)) % self.ALIGN + self.off
         if start + nbytes > self.buf.numel():
-            # Stream order keeps the old buffer alive for kernels already enqueued.
-            self._pending.append(self.buf)
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError(f"Workspace would have to grow to {nbytes} bytes inside a graph capture: run the step eagerly once before capturing it")
+            self._retired.append(self.buf)              # kernels already enqueued, and graphs already captured, keep using it
             self.buf = torch.empty(max(2 * self.buf.numel(), nbytes + self.ALIGN), dtype=torch.uint8, device=self.device)
             self.off = 0
             base = self.buf.data_ptr()

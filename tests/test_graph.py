@@ -673,3 +673,46 @@ def test_executor_replays_as_one_captured_graph(ctx):
         with torch.no_grad():
             ref = m.float()(x.float().cpu()).numpy()
         assert_parity(got.float().cpu().numpy(), ref, what=f"replay {seed}")
+
+
+def _conv_relu_stack(seed=0):
+    import torch
+    import torch.nn as nn
+
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.c1, self.c2, self.c3 = nn.Conv2d(16, 32, 3, padding=1), nn.Conv2d(32, 32, 1), nn.ConvTranspose2d(32, 8, 2, stride=2)
+
+        def forward(self, x):
+            y = torch.relu(self.c1(x))                      # folds: the convolution's own act
+            y = torch.nn.functional.gelu(self.c2(y))        # gelu after a convolution has no such slot: stays an op
+            return torch.relu(self.c3(y))                   # nor has the transposed convolution
+
+    torch.manual_seed(seed)
+    return M().eval().half()
+
+
+def test_relu_after_a_convolution_becomes_its_act():
+    import torch
+    from juliavision_amd import graph as G
+    m = _conv_relu_stack()
+    g = G.optimize(G.Graph.load(G.convert(torch.export.export(m, (torch.randn(1, 16, 24, 24).half(),)).run_decompositions(), "convs")))
+    left = [o["aten"] for o in g.ops]
+    assert left.count("relu.default") == 1 and left.count("gelu.default") == 1 and left.count("convolution.default") == 3, (left, g.notes)
+    convs = [o for o in g.ops if o["aten"] == "convolution.default"]
+    assert [o["attrs"].get("epilogue") for o in convs] == ["relu", None, None]
+
+
+@pytest.mark.gpu
+def test_convolution_with_folded_relu_runs_on_the_kernels(ctx):
+    import torch
+    from juliavision_amd import graph as G
+    m = _conv_relu_stack(seed=3)
+    x = torch.randn(1, 16, 24, 24).half()
+    run = G.Executor(G.optimize(G.Graph.load(G.convert(torch.export.export(m, (x,)).run_decompositions(), "convs"))), m.state_dict(), ctx)
+    with torch.no_grad():
+        want = m.float()(x.float()).numpy()
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    assert_parity(got.float().cpu().numpy(), want, what="conv + relu folded, conv + gelu, transposed conv + relu")
