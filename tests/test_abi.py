@@ -98,13 +98,16 @@ def test_sdpa_planner():
     assert _sdpa_plan(64, 128, 128, 2, 1, ptr=0x10002)[0] == "rows"
     assert _sdpa_plan(64, 128, 128, 2, 1, scale=-1.0)[0] == "rows"
     assert _sdpa_plan(512, 128, 128, 2, 1)[0] == "decline"
-    # key splits for decode-sized Lq aim at two workgroups per CU (flash.jl:1288-1303): 20 rows -> many splits,
-    # 160 rows -> fewer, never more than one split per 64 keys
+    # a single query row runs in one launch whose key range is cut over workgroups that merge inside it: at most one
+    # workgroup per CU, a round of six 64-key passes each (24 passes over 20 rows -> 4 ways; 160 rows fill the chip whole);
+    # anything the one-launch kernel does not take (here a mask) gets the rows kernel's splits, two workgroups per CU,
+    # never more than one per 64 keys (flash.jl:1288-1303)
     p1, n1 = _sdpa_plan(64, 1, 1500, 20, 1)
     p8, n8 = _sdpa_plan(64, 1, 1500, 20, 8)
-    assert p1 == p8 == "rows" and n1 == 24 and 1 <= n8 < n1
-    assert _sdpa_plan(64, 1, 448, 20, 1) == ("rows", 1)                      # a short key range: one launch, one workgroup per head
-    assert _sdpa_plan(64, 1, 700, 20, 1)[1] == 11
+    assert p1 == p8 == "rows" and n1 == 4 and n8 == 1
+    assert _sdpa_plan(64, 1, 448, 20, 1) == ("rows", 1)                      # a short key range: one workgroup per head
+    assert _sdpa_plan(64, 1, 700, 20, 1)[1] == 2                             # 11 passes: two rounds
+    assert _sdpa_plan(64, 1, 1500, 20, 1, bias=1)[1] == 24                   # masked: the rows kernel, split 24 ways
     assert _sdpa_plan(64, 23, 17, 4, 1)[1] == 1
 
 

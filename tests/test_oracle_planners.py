@@ -40,29 +40,38 @@ def test_key_split_rule():
 
 
 def test_decode_attention_keeps_the_two_workgroups_per_core_rule():
-    """mi_sdpa_f16_plan's split count for single-query attention aims, like splitcount (flash.jl:1288-1303), at two
-    workgroups per core (256 CUs, 64-key blocks, one query row per workgroup): min(ceil(2 CUs / rows), blocks, 64).
-    Equal to the reference's count at config 5's cross-attention at batch 1; elsewhere never fewer splits than the
-    reference's rule, which rounds the wanted count down and re-derives it from equal whole-block chunks.  A single
-    query over at most 640 keys is not split at all."""
+    """mi_sdpa_f16_plan's split count for the rows kernel (a few query rows, or one row with a mask) aims, like
+    splitcount (flash.jl:1288-1303), at two workgroups per core (256 CUs, 64-key blocks, one query row per workgroup):
+    min(ceil(2 CUs / rows), blocks, 64).  Equal to the reference's count at config 5's cross-attention at batch 1;
+    elsewhere never fewer splits than the reference's rule, which rounds the wanted count down and re-derives it from
+    equal whole-block chunks.  A single unmasked query row takes the one-launch kernel, whose own rule is different
+    (its workgroups merge inside the launch, which costs three trips to memory, so it cuts far less): at most one
+    workgroup per core and a round of six 64-key passes each, nothing below nine passes."""
     import ctypes as C
     from juliavision_amd import _lib as L
     lib = L.load()
 
-    def nsplit(E, Lq, Lk, H, B):
+    def nsplit(E, Lq, Lk, H, B, bias=0):
         ns = C.c_int(0)
         st = L.strides4(1, E, E * Lq, E * Lq * H)
         sk = L.strides4(1, E, E * Lk, E * Lk * H)
-        path = lib.mi_sdpa_f16_plan(0x10000, st, 0x20000, sk, 0x30000, sk, 0, 1, E, Lq, Lk, H, B, 0.125, C.byref(ns))
+        path = lib.mi_sdpa_f16_plan(0x10000, st, 0x20000, sk, 0x30000, sk, bias, 1, E, Lq, Lk, H, B, 0.125, C.byref(ns))
         assert L.SDPA_PATHS[path] == "rows"
         return ns.value
 
-    assert nsplit(64, 1, 1500, 20, 1) == P.splitcount(256, 1, 1500, 1, 64, 20) == 24
-    assert nsplit(64, 1, 700, 20, 1) == P.splitcount(256, 1, 700, 1, 64, 20) == 11
-    assert nsplit(64, 1, 448, 20, 1) == nsplit(64, 1, 448, 20, 8) == 1         # up to 640 keys: a single launch, no splits
-    for (Lq, Lk, H, B) in [(1, 1500, 20, 4), (1, 1500, 20, 8), (1, 700, 20, 4), (1, 1000, 20, 8), (1, 4096, 8, 1), (3, 100, 2, 1),
-                           (23, 4096, 8, 1), (5, 100, 2, 1), (2, 17, 4, 1), (7, 64, 1, 1), (1, 100000, 1, 1)]:
+    assert nsplit(64, 1, 1500, 20, 1, bias=1) == P.splitcount(256, 1, 1500, 1, 64, 20) == 24
+    assert nsplit(64, 1, 700, 20, 1, bias=1) == P.splitcount(256, 1, 700, 1, 64, 20) == 11
+    for (Lq, Lk, H, B, bias) in [(1, 1500, 20, 4, 1), (1, 1500, 20, 8, 1), (1, 700, 20, 4, 1), (1, 1000, 20, 8, 1), (1, 4096, 8, 1, 1),
+                                 (3, 100, 2, 1, 0), (23, 4096, 8, 1, 0), (5, 100, 2, 1, 0), (2, 17, 4, 1, 0), (7, 64, 1, 1, 0), (1, 100000, 1, 1, 1)]:
         rows = Lq * H * B
-        mine = nsplit(64, Lq, Lk, H, B)
+        mine = nsplit(64, Lq, Lk, H, B, bias)
         assert mine == max(1, min(P.cld(2 * 256, rows), P.cld(Lk, 64), 64)), (Lq, Lk, H, B)
         assert mine >= min(64, P.splitcount(256, Lq, Lk, 1, 64, H * B)), (Lq, Lk, H, B)
+    # the one-launch kernel's own count
+    for (Lk, H, B, want) in [(448, 20, 1, 1), (448, 20, 8, 1), (512, 20, 1, 1), (700, 20, 1, 2), (1500, 20, 1, 4), (1500, 20, 4, 3),
+                             (1500, 20, 8, 1), (4096, 8, 1, 11), (100000, 1, 1, 32)]:
+        passes = P.cld(Lk, 64)
+        rule = 1 if passes <= 8 else max(1, min(256 // (H * B), P.cld(passes, 6), 32))
+        while rule > 1 and P.cld(passes, rule) * (rule - 1) >= passes:
+            rule -= 1
+        assert nsplit(64, 1, Lk, H, B) == rule == want, (Lk, H, B)
