@@ -185,9 +185,9 @@ def test_rows_sum_to_one(ctx):
     assert np.max(np.abs(got.astype(np.float32) - 1.0)) < 2e-3
 
 
-def test_config4_attention_band(ctx):
-    """BASELINE config 4 attention at full size (L=4096, 16 heads x 64); the oracle checks a band of
-    query rows of two heads (the full three-pass form takes minutes on the CPU)."""
+def test_config4_attention_full(ctx):
+    """BASELINE config 4 attention at full size (L=4096, 16 heads x 64) against the oracle's composed fp32 form on every
+    query row of every head (0.4 s of CPU per head), head by head so that one bad head cannot hide in the average."""
     import torch
     import juliavision_amd as jv
     B, H, L, E = 1, 16, 4096, 64
@@ -197,10 +197,9 @@ def test_config4_attention_band(ctx):
     torch.cuda.synchronize()
     got = to_host(out)
     assert np.all(np.isfinite(got))
-    for h in (0, 15):
-        rows = np.r_[0:16, 2040:2056, 4080:4096]
-        want = oracle.sdpa_ref_f32(q[:, h:h + 1, rows], k[:, h:h + 1], v[:, h:h + 1])
-        assert_parity(got[:, h:h + 1, rows], want, what=f"config4 head {h}")
+    for h in range(H):
+        want = oracle.sdpa_ref_f32(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1])
+        assert_parity(got[:, h:h + 1], want, what=f"config4 head {h}")
 
 
 def test_token_major_output(ctx):
