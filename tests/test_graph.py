@@ -716,3 +716,34 @@ def test_convolution_with_folded_relu_runs_on_the_kernels(ctx):
     got = run(x.cuda())
     torch.cuda.synchronize()
     assert_parity(got.float().cpu().numpy(), want, what="conv + relu folded, conv + gelu, transposed conv + relu")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["composite", "decomposed"])
+def test_exported_block_matches_the_oracle_composition(ctx, mode):
+    """The exported block against the composition of the oracle's CPU kernels that the hand-composed encoder layer is held
+    to (layer norm, one rounding per GEMM, activation on the rounded value, residual with one more rounding, three-pass
+    attention), fed the module's own weights: the graph route and the oracle agree, not only the graph route and torch."""
+    import numpy as np
+    import torch
+    import oracle
+    from juliavision_amd import graph as G
+    from test_configs_gpu import _oracle_layer
+    d, heads, ffn, T = 128, 2, 256, 70
+    m = _block(d, heads, ffn, seed=5)
+    with torch.no_grad():
+        m.k.bias = torch.nn.Parameter(torch.zeros(d).half())          # the oracle's packed q/k/v bias needs all three
+    ep, x = _export(m, T, d) if mode == "composite" else _decomposed(m)
+    run = G.Executor(G.optimize(G.Graph.load(G.convert(ep, "block"))), m.state_dict(), ctx)
+    got = run(x.cuda())
+    torch.cuda.synchronize()
+    np16 = lambda t: t.detach().cpu().numpy().astype(np.float16)
+    kf = lambda lin: np.ascontiguousarray(np16(lin.weight).T)           # torch [F][K] -> the oracle's [K][F]
+    h = {"wqkv": np.concatenate([kf(m.q), kf(m.k), kf(m.v)], axis=1), "bqkv": np.concatenate([np16(m.q.bias), np16(m.k.bias), np16(m.v.bias)]),
+         "wo": kf(m.o), "bo": np16(m.o.bias), "w1": kf(m.fc1), "b1": np16(m.fc1.bias), "w2": kf(m.fc2), "b2": np16(m.fc2.bias),
+         "ln1_g": np16(m.ln1.weight), "ln1_b": np16(m.ln1.bias), "ln2_g": np16(m.ln2.weight), "ln2_b": np16(m.ln2.bias)}
+    x16 = np16(x)[0]
+    want = _oracle_layer(h, x16, heads, 1e-5)
+    assert_parity(got.float().cpu().numpy()[0], want, what=f"exported block ({mode}) against the oracle's composition")
+    assert_parity(got.float().cpu().numpy()[0] - x16.astype(np.float32), want.astype(np.float32) - x16.astype(np.float32),
+                  what="the block's update alone")
