@@ -556,6 +556,110 @@ def whisper_graph_case(nl=32, steps=10):
             "frac_mfma_peak_graph": round(flop / replay / 1e12 / PEAK_F16_TFLOPS, 4)}
 
 
+def decoder_graph_case(steps=100):
+    """Config 5's model as a whole, from its exported graph: a decoder step written the way the reference's export wrapper
+    writes Whisper-large-v3-turbo's (tools/export_whisper_decoder.py:90-240: token + position embedding, the
+    arange <= cache_position mask, 4 pre-LN layers of d_model 1280 with 20 x 64 heads whose new K/V rows go into a
+    448-slot cache by index_copy, cross-attention over 1500 precomputed states, FFN 5120, final norm, logits through the
+    tied 51866 x 1280 embedding, caches returned through stack), exported on the meta device, converted, rewritten --
+    the functional cache update becomes the in-place one, the mask a key count -- and replayed as one captured graph."""
+    import time
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+    import juliavision_amd as jv
+    from juliavision_amd import graph as G
+    from juliavision_amd.decode import StepGraph
+    d, H, ffn, NL, V, T, S = 1280, 20, 5120, 4, 51866, 448, 1500
+    hd = d // H
+
+    class Layer(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.ln1, self.ln2, self.ln3 = nn.LayerNorm(d), nn.LayerNorm(d), nn.LayerNorm(d)
+            self.q, self.k, self.v, self.o = nn.Linear(d, d), nn.Linear(d, d, bias=False), nn.Linear(d, d), nn.Linear(d, d)
+            self.cq, self.co = nn.Linear(d, d), nn.Linear(d, d)
+            self.fc1, self.fc2 = nn.Linear(d, ffn), nn.Linear(ffn, d)
+
+    class Step(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.embed_tokens, self.embed_positions = nn.Embedding(V, d), nn.Embedding(T, d)
+            self.layers = nn.ModuleList([Layer() for _ in range(NL)])
+            self.layer_norm = nn.LayerNorm(d)
+
+        def forward(self, ids, self_k, self_v, cross_k, cross_v, cache_position):
+            B = self_k.shape[1]
+            h = self.embed_tokens(ids) + self.embed_positions.weight[cache_position]
+            idx = torch.arange(T, device=h.device)
+            lowest = torch.full((), torch.finfo(h.dtype).min, dtype=h.dtype, device=h.device)
+            mask = torch.where(idx <= cache_position, torch.zeros((), dtype=h.dtype, device=h.device), lowest).view(1, 1, 1, T).expand(B, H, 1, T)
+            heads = lambda t: t.view(B, 1, H, hd).transpose(1, 2)
+            newk, newv = [], []
+            for i, l in enumerate(self.layers):
+                r, h = h, l.ln1(h)
+                q = heads(l.q(h) * hd ** -0.5)
+                K_ = self_k[i].index_copy(2, cache_position, heads(l.k(h)))
+                V_ = self_v[i].index_copy(2, cache_position, heads(l.v(h)))
+                newk.append(K_)
+                newv.append(V_)
+                h = r + l.o(F.scaled_dot_product_attention(q, K_, V_, attn_mask=mask, scale=1.0).transpose(1, 2).reshape(B, 1, d))
+                r, h = h, l.ln2(h)
+                o = F.scaled_dot_product_attention(heads(l.cq(h) * hd ** -0.5), cross_k[i], cross_v[i], scale=1.0)
+                h = r + l.co(o.transpose(1, 2).reshape(B, 1, d))
+                r, h = h, l.ln3(h)
+                h = r + l.fc2(F.gelu(l.fc1(h)))
+            return F.linear(self.layer_norm(h), self.embed_tokens.weight), torch.stack(newk), torch.stack(newv)
+
+    t0 = time.perf_counter()
+    with torch.device("meta"):
+        m = Step().eval().half()
+        z = lambda *sh: torch.empty(*sh, dtype=torch.float16)
+        args = (torch.empty(1, 1, dtype=torch.long), z(NL, 1, H, T, hd), z(NL, 1, H, T, hd), z(NL, 1, H, S, hd), z(NL, 1, H, S, hd),
+                torch.empty(1, dtype=torch.long))
+    table = torch.export.default_decompositions()
+    table.pop(torch.ops.aten.scaled_dot_product_attention.default, None)     # an accelerator export keeps the fused op
+    spec = G.convert(torch.export.export(m, args).run_decompositions(table), "whisper_decoder_step")
+    g = G.optimize(G.Graph.load(spec))
+    host_s = time.perf_counter() - t0
+    if sum(o["aten"] == "sdpa_append" for o in g.ops) != NL:
+        raise RuntimeError("the exported step's cache update did not fold: " + "; ".join(g.notes[-5:]))
+    torch.manual_seed(0)
+    weights = {}
+    for k, v in m.state_dict().items():
+        norm_scale = k.endswith("weight") and v.dim() == 1
+        weights[k] = torch.ones(v.shape, dtype=torch.float16, device="cuda") if norm_scale else \
+            torch.randn(v.shape, dtype=torch.float16, device="cuda") * 0.02
+    ctx = jv.Ctx("cuda")
+    run = G.Executor(g, weights, ctx)
+    f16 = torch.float16
+    ids = torch.randint(0, V, (1, 1), device="cuda")
+    sk, sv = (torch.randn(NL, 1, H, T, hd, dtype=f16, device="cuda") for _ in range(2))
+    ck, cv = (torch.randn(NL, 1, H, S, hd, dtype=f16, device="cuda") for _ in range(2))
+    pos = torch.tensor([T - 1], device="cuda")                       # the last slot: every step attends the full cache
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / steps
+
+    step = lambda: run(ids, sk, sv, ck, cv, pos)
+    eager = timed(step)
+    replay = timed(StepGraph(step).replay)
+    logits, nk, _ = run(ids, sk, sv, ck, cv, pos)
+    if not bool(torch.isfinite(logits).all()) or nk.data_ptr() != sk.data_ptr():
+        raise RuntimeError("exported decoder step: non-finite logits, or the returned cache is not the caller's")
+    mb = 2.0 * (NL * (3 * d * d + 3 * d * d + 2 * d * ffn) + V * d) + 2.0 * 2 * H * hd * (T + S) * NL
+    return {"layers": NL, "ops_exported": len(spec["ops"]), "launches_after_rewrites": len(g.ops), "export_and_rewrite_host_s": round(host_s, 2),
+            "eager_us": round(eager * 1e6, 1), "graph_us": round(replay * 1e6, 1), "MB_per_token": round(mb / 1e6, 1),
+            "GB/s_graph": round(mb / replay / 1e9, 1), "frac_hbm_peak_graph": round(mb / replay / 1e9 / PEAK_HBM_GBS, 4)}
+
+
 def encoder_stack_case(nl=4, steps=50):
     """BASELINE config 2's block as it occurs in a stack: `nl` Whisper-shaped blocks in sequence (1500 x 1280, 20 x 64
     heads, FFN 5120, [K][F] weights), each block's first norm written by the previous block's last GEMM.  Reported per
@@ -846,6 +950,10 @@ def detail_benchmarks(lib, L, stream, only=None):
     name = "c5_decode_step_4layers_vocab51866_b1"
     if only is None or only in name:
         out[name] = decode_step_case()
+
+    name = "c5_decode_step_from_exported_graph_b1"
+    if only is None or only in name:
+        out[name] = decoder_graph_case()
 
     # config 4: global attention at 4096 and the 3x3 conv
     attn_case("c4_attn_L4096_16x64", 1, 16, 4096, 4096, 64)

@@ -397,13 +397,17 @@ def group_linears(g: Graph) -> Graph:
     """Linear ops that read the same activations with the same extents -- the q, k and v projections of an attention
     written with three ``Linear`` modules -- become one op, ``linear_group``, run as a single batched GEMM launch over
     weights the executor stacks plane after plane when it binds them (three 1500 x 1280 x 1280 projections: 23 us
-    as one launch of 180 tiles, 3 x 16 us apart).  The members keep their result buffers: planes of one allocation."""
+    as one launch of 180 tiles, 3 x 16 us apart).  The members keep their result buffers: planes of one allocation.
+    Decode-sized members that all carry the same layer norm as their prologue (``fold_layernorm_prologues``) become one
+    GEMV instead: the weights laid end to end along the output axis, the norm computed once, the results column bands
+    of one buffer -- the fused q/k/v projection of the hand-composed decoder layer."""
     def key(o):
         pos = {"linear.default": (0, 1, 2), "addmm.default": (1, 2, 0), "mm.default": (0, 1, None)}[o["aten"]]
         x, w = o["in"][pos[0]], o["in"][pos[1]]
         b = o["in"][pos[2]] if pos[2] is not None and len(o["in"]) > pos[2] else None
         return x, w, b
-    plain = lambda o: o["aten"] in LINEAR_OPS and not any(k in o["attrs"] for k in ("epilogue", "residual", "ln_out", "ln_in", "clamp"))
+    plain = lambda o: o["aten"] in LINEAR_OPS and not any(k in o["attrs"] for k in ("epilogue", "residual", "ln_out", "clamp"))
+    norm_of = lambda o: tuple(o["attrs"].get(k) for k in ("ln_in", "ln_in_gamma", "ln_in_beta", "ln_in_eps"))
     done = set()
     for first in [o for o in g.ops if plain(o)]:
         if first["id"] in done or first not in g.ops:
@@ -425,7 +429,7 @@ def group_linears(g: Graph) -> Graph:
             same_x = x == x0 or (reshaped_root(x) is not None and reshaped_root(x) == reshaped_root(x0) and
                                  g.buffers[x].get("shape") == xs.get("shape"))
             same_w = g.buffers[w].get("shape") == g.buffers[w0].get("shape") and g.buffers[g.root(w)]["kind"] == "weight"
-            if same_x and same_w and (b is None or g.buffers[g.root(b)]["kind"] == "weight") and \
+            if same_x and same_w and (b is None or g.buffers[g.root(b)]["kind"] == "weight") and norm_of(o) == norm_of(first) and \
                     g.buffers[o["out"]].get("shape") == g.buffers[first["out"]].get("shape") and o["out"] not in g.outputs:
                 members.append(o)
         # (buffers are written once, so a later member can run where the first one stands: its operands exist there)
@@ -438,9 +442,16 @@ def group_linears(g: Graph) -> Graph:
             spec.append({"out": o["out"], "w": w, "b": b, "aten": o["aten"], "colscale": o["attrs"].get("colscale")})
             done.add(o["id"])
         g.ops = [o for o in g.ops if o not in members[1:]]
-        g.ops[at] = {"id": first["id"] + "_group", "aten": "linear_group", "in": [x0] + [m["w"] for m in spec] + [m["b"] for m in spec if m["b"]],
-                     "out": first["out"], "attrs": {"members": spec}}
-        g.notes.append("one launch for " + ", ".join(m["out"] for m in spec))
+        attrs = {"members": spec}
+        extra = []
+        if first["attrs"].get("ln_in"):
+            # decode-sized members that each carry the same norm as their prologue: one GEMV over the members' weights
+            # laid end to end along the output axis, the norm computed once, the results column bands of one buffer
+            attrs.update({k: first["attrs"].get(k) for k in ("ln_in", "ln_in_gamma", "ln_in_beta", "ln_in_eps")})
+            extra = [first["attrs"][k] for k in ("ln_in_gamma", "ln_in_beta") if first["attrs"].get(k)]
+        g.ops[at] = {"id": first["id"] + "_group", "aten": "linear_group", "in": [x0] + [m["w"] for m in spec] + [m["b"] for m in spec if m["b"]] + extra,
+                     "out": first["out"], "attrs": attrs}
+        g.notes.append("one launch for " + ", ".join(m["out"] for m in spec) + (" (norm prologue shared)" if extra or attrs.get("ln_in") else ""))
     return g
 
 
@@ -503,7 +514,7 @@ def fold_clamps(g: Graph) -> Graph:
 
 
 def fold_layernorm_prologues(g: Graph) -> Graph:
-    """A layer norm over the last axis that only one linear op reads (through reshapes at most) becomes that GEMM's
+    """A layer norm over the last axis that only linear ops read (through reshapes at most) becomes their GEMMs'
     prologue (``ln_matmul_``) where the kernels can take it and it is the faster choice (``kernels.ln_matmul_folds``,
     ``ln_matmul_pays``): the rows are normalised on their way into LDS, so the normalised activations never exist in
     memory and the norm costs no launch.  Today that is the decode-sized case (at most 8 rows: a decoder step's norms);
@@ -516,41 +527,50 @@ def fold_layernorm_prologues(g: Graph) -> Graph:
         if feat is None or list(a.get("arg1", [])) != [feat] or xb.get("dtype") != "float16":
             continue
         readers = _consumers(g, ln["out"])
-        if len(readers) != 1 or "<output>" in readers:
-            continue
-        lin = g.op(next(iter(readers)))
-        if lin is None or lin["aten"] not in LINEAR_OPS or any(k in lin["attrs"] for k in ("ln_in", "ln_out", "clamp")):
-            continue
-        xpos = {"linear.default": 0, "addmm.default": 1, "mm.default": 0}[lin["aten"]]
-        wpos = {"linear.default": 1, "addmm.default": 2, "mm.default": 1}[lin["aten"]]
-        chain = [lin["in"][xpos]]
-        ok = True
-        while chain[-1] != ln["out"]:
-            b = g.buffers[chain[-1]]
-            if b["kind"] != "view" or not (b.get("op") in RESHAPES or "getitem" in b.get("op", "")) or \
-                    ("getitem" not in b.get("op", "") and (b.get("shape") or [None])[-1] != feat):
-                ok = False
-                break
-            chain.append(b["of"])
-        if not ok or sum(1 for i in lin["in"] if i == lin["in"][xpos]) != 1:
-            continue
-        wshape = g.buffers[lin["in"][wpos]].get("shape") or []
-        if len(wshape) != 2 or g.buffers[g.root(lin["in"][wpos])]["kind"] != "weight":
-            continue
-        F = wshape[0] if lin["aten"] == "linear.default" else wshape[1]
-        T = 1
-        for d in (xb.get("shape") or [])[:-1]:
-            T *= d
-        if not (K.ln_matmul_folds(T, feat, F) and K.ln_matmul_pays(T, feat, F)):
+        if not readers or "<output>" in readers:
             continue
         if any(g.op(g.root(i)) is not None for i in ln["in"][1:]):
             continue                                    # gamma / beta must be constants
-        lin["attrs"].update(ln_in=True, ln_in_gamma=ln["in"][1] if len(ln["in"]) > 1 else None,
-                            ln_in_beta=ln["in"][2] if len(ln["in"]) > 2 else None, ln_in_eps=a.get("arg4", a.get("eps", 1e-5)))
+        T = 1
+        for d in (xb.get("shape") or [])[:-1]:
+            T *= d
+        # several readers are fine when each of them can take the norm (the q, k and v projections of a decoder layer:
+        # group_linears then runs them as one GEMV with one norm); one that cannot keeps the norm as an op for all
+        lins = []
+        for rid in sorted(readers, key=lambda r: g.ops.index(g.op(r))):
+            lin = g.op(rid)
+            if lin is None or lin["aten"] not in LINEAR_OPS or any(k in lin["attrs"] for k in ("ln_in", "ln_out", "clamp")):
+                break
+            xpos = {"linear.default": 0, "addmm.default": 1, "mm.default": 0}[lin["aten"]]
+            wpos = {"linear.default": 1, "addmm.default": 2, "mm.default": 1}[lin["aten"]]
+            chain = [lin["in"][xpos]]
+            ok = True
+            while chain[-1] != ln["out"]:
+                b = g.buffers[chain[-1]]
+                if b["kind"] != "view" or not (b.get("op") in RESHAPES or "getitem" in b.get("op", "")) or \
+                        ("getitem" not in b.get("op", "") and (b.get("shape") or [None])[-1] != feat):
+                    ok = False
+                    break
+                chain.append(b["of"])
+            if not ok or sum(1 for i in lin["in"] if i == lin["in"][xpos]) != 1:
+                break
+            wshape = g.buffers[lin["in"][wpos]].get("shape") or []
+            if len(wshape) != 2 or g.buffers[g.root(lin["in"][wpos])]["kind"] != "weight":
+                break
+            F = wshape[0] if lin["aten"] == "linear.default" else wshape[1]
+            if not (K.ln_matmul_folds(T, feat, F) and K.ln_matmul_pays(T, feat, F)):
+                break
+            lins.append(lin)
+        if len(lins) != len(readers):
+            continue
+        for lin in lins:
+            lin["attrs"].update(ln_in=True, ln_in_gamma=ln["in"][1] if len(ln["in"]) > 1 else None,
+                                ln_in_beta=ln["in"][2] if len(ln["in"]) > 2 else None, ln_in_eps=a.get("arg4", a.get("eps", 1e-5)))
+        lin = lins[0]
         g.ops.remove(ln)
         ob = g.buffers[ln["out"]]
         ob.update(kind="view", of=ln["in"][0], op="alias.default", attrs={})
-        g.notes.append(f"fold {ln['id']} into the prologue of {lin['id']}")
+        g.notes.append(f"fold {ln['id']} into the prologue of " + ", ".join(l["id"] for l in lins))
     return g
 
 
@@ -1031,6 +1051,13 @@ class Executor:
             if o["aten"] == "linear_group":               # the members' results are planes of one allocation
                 mem = o["attrs"]["members"]
                 b0 = graph.buffers[mem[0]["out"]]
+                if o["attrs"].get("ln_in"):               # ... or column bands of one (rows, n F) matrix
+                    F, rows = b0["shape"][-1], math.prod(b0["shape"][:-1])
+                    bands = torch.empty((rows, len(mem) * F), dtype=_DTYPES[b0["dtype"]], device=self.device)
+                    for i, m in enumerate(mem):
+                        self.t[m["out"]] = bands[:, i * F:(i + 1) * F].view(list(b0["shape"]))
+                    self.t[o["id"]] = bands
+                    continue
                 planes = torch.empty([len(mem)] + list(b0["shape"]), dtype=_DTYPES[b0["dtype"]], device=self.device)
                 for i, m in enumerate(mem):
                     self.t[m["out"]] = planes[i]
@@ -1164,12 +1191,23 @@ class Executor:
                 ws.append(w)
                 bs.append(b)
             fk = all(w.stride(0) == 1 and w.stride(1) == w.shape[0] for w in ws)       # every member a transposed [F][K] matrix
-            W = torch.stack([w.t() for w in ws]).transpose(1, 2) if fk else torch.stack([w.contiguous() for w in ws])
-            B = None if all(b is None for b in bs) else torch.stack([torch.zeros_like(next(x for x in bs if x is not None)) if b is None else b for b in bs])
+            filled = [torch.zeros_like(next(x for x in bs if x is not None)) if b is None else b for b in bs] if any(b is not None for b in bs) else None
+            if o["attrs"].get("ln_in"):                   # end to end along the output axis, in the members' own memory layout
+                W = torch.cat([w.t() for w in ws]).t() if fk else torch.cat([w.contiguous() for w in ws], dim=1)
+                B = None if filled is None else torch.cat(filled)
+            else:
+                W = torch.stack([w.t() for w in ws]).transpose(1, 2) if fk else torch.stack([w.contiguous() for w in ws])
+                B = None if filled is None else torch.stack(filled)
             self.scaled[o["id"]] = (W, B)
         W, B = self.scaled[o["id"]]
         x = self._rows(self.get(o["in"][0]))
         planes = self.t[o["id"]]
+        if o["attrs"].get("ln_in"):
+            a = o["attrs"]
+            self.ctx.ws.reset()
+            K.ln_matmul_(self.ctx, planes, W, x, self.get(a["ln_in_gamma"]) if a.get("ln_in_gamma") else None,
+                         self.get(a["ln_in_beta"]) if a.get("ln_in_beta") else None, a.get("ln_in_eps", 1e-5), B)
+            return
         K.batchedmatmul_(self.ctx, planes.view(len(mem), -1, planes.shape[-1]), W, x.unsqueeze(0), B)
 
     def _sdpa(self, o):

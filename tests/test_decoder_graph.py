@@ -117,6 +117,12 @@ def test_cache_step_folds_into_in_place_appends(mode):
     assert sum(a in G.SDPA_OPS for a in left) == 2
     emb = next(o for o in g.ops if o["aten"] == "embedding.default")
     assert len(emb["in"]) == 4 and emb["in"][1] == "x" and emb["in"][3] == "cache_position"
+    # q, k and v read one norm: a single product over their weights end to end, the norm as its prologue; every other
+    # norm sits in front of one linear and becomes that linear's prologue -- no norm launch is left, 8 launches a layer
+    groups = [o for o in g.ops if o["aten"] == "linear_group"]
+    assert len(groups) == 2 and all(len(o["attrs"]["members"]) == 3 and o["attrs"]["ln_in"] for o in groups), g.notes
+    assert groups[0]["attrs"]["ln_in_gamma"].endswith("layers_0_ln1_weight")
+    assert not any("layer_norm" in a for a in left) and len(left) == 3 + 2 * 8
 
 
 def test_cache_write_that_someone_else_reads_is_left_functional():
