@@ -276,6 +276,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
     const int vtoff = (gk + 4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
     const int ktoff = (gk + l32) * KLD + 8 * hl;
+    const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // t = s*scale*log2(e) - M, straight out of the MFMA chain
     auto qk = [&](float16v (&s)[2], int st) {
@@ -283,7 +284,10 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
 #pragma unroll
         for (int kt = 0; kt < 2; kt++) {
             const half_t *kp_ = kbase + 32 * kt * KLD;
-            s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], negm, 0, 0, 0);
+            if constexpr (SEED)
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], negm, 0, 0, 0);
+            else
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], zero16, 0, 0, 0);
 #pragma unroll
             for (int ks = 1; ks < KS; ks++)
                 s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_ + 16 * ks), qf[ks], s[kt], 0, 0, 0);
@@ -406,6 +410,15 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         half8v pf[2][2];
         float l_new = l_run;
         probs(sc, pf, l_new);
+        // Four-wave forms: the block's largest exponent, three at a time, found under the next block's first product
+        // (these forms sit at the register limit, and the maximum taken here is what lets the scores' registers go
+        // early: with the test below on the row sum alone the 96-wide instance spills twice as much).
+        float tmax = 0.0f;
+        if constexpr (!PP) {
+            tmax = fmaxf(sc[0][0], sc[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; r++) tmax = fmaxf(fmaxf(tmax, sc[0][r]), sc[1][r]);
+        }
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * KS, 0);
 #pragma unroll
         for (int g = 0; g < 2 * KS + 2; g++) {
@@ -417,12 +430,15 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         // unrounded values, tells: it cannot have grown by less than 2^16 - 16 if one of the block's terms did
         // (and if it grew that much through many smaller terms, settling a new reference point is still right, only
         // not needed).  Then, and on the first block, settle a new reference point: the block maximum, for the rows
-        // that outgrew the old one by 2^TH; rescale what was accumulated; redo the exponentials.  The maximum is only
-        // looked for here: the fast path spends no instruction on it.
-        if (__any(first || !(l_new - l_run < 65504.0f))) {
-            float tmax = fmaxf(sc[0][0], sc[1][0]);
+        // that outgrew the old one by 2^TH; rescale what was accumulated; redo the exponentials.  In the eight-wave
+        // forms the maximum is only looked for here: their fast path spends no instruction on it.
+        const bool outgrown = PP ? !(l_new - l_run < 65504.0f) : tmax >= 15.9f;
+        if (__any(first || outgrown)) {
+            if constexpr (PP) {
+                tmax = fmaxf(sc[0][0], sc[1][0]);
 #pragma unroll
-            for (int r = 1; r < 16; r++) tmax = fmaxf(fmaxf(tmax, sc[0][r]), sc[1][r]);
+                for (int r = 1; r < 16; r++) tmax = fmaxf(fmaxf(tmax, sc[0][r]), sc[1][r]);
+            }
             float mx = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
             const bool grow = (mx > TH || first) && mx != -INFINITY;
             const half_t m16 = (half_t)(m_ref + (grow ? mx : 0.0f));
