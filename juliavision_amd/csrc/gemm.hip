@@ -11,11 +11,13 @@
 #include <cstdlib>
 #include <atomic>
 
-// Arrival flags of the split-K peer reduction (gemm_pp_kernel, SK): SK_BANKS banks of SK_FLAGS words; a launch uses
-// the bank its epoch selects and writes the epoch itself, so flags are never cleared and launches that overlap on one
-// GPU (up to SK_BANKS of them) do not see each other's.  Zero when the module loads; epochs start at 1.
-constexpr int SK_BANKS = 16, SK_FLAGS = 4096;
-static __device__ unsigned sk_flag_words[SK_BANKS * SK_FLAGS];
+// Arrival flags of the split-K peer reduction (gemm_pp_kernel, SK): SK_BANKS banks of SK_FLAGS words, and as many
+// counters behind them (word i's counter is word i + SK_WORDS).  A launch uses the bank its epoch selects, so launches
+// that overlap on one GPU (up to SK_BANKS of them) do not see each other's.  Every word is zero when the module loads
+// and zero again when a launch ends: the last consumer of a flag clears it (and its counter), so a captured launch --
+// whose epoch and bank are fixed at capture -- starts every replay from clean flags.
+constexpr int SK_BANKS = 16, SK_FLAGS = 4096, SK_WORDS = SK_BANKS * SK_FLAGS;
+static __device__ unsigned sk_flag_words[2 * SK_WORDS];
 
 // Static device scratch of the allocation-free entry point (see mi_gemm_f16_noalloc).
 static __device__ __align__(256) unsigned char scratch[MI_NOALLOC_SCRATCH_BYTES];
@@ -52,7 +54,7 @@ struct GemmArgs {
     unsigned long long *clk;
     // Split-K with the partial tiles exchanged between the workgroups of a tile instead of written as planes
     // (ping-pong kernel, SK instances): sk_S workgroups per tile, tiles dealt sk_tpx per XCD; partials in sk_part,
-    // per-wave arrival flags in sk_flags (they carry sk_epoch, unique per launch: nothing is ever cleared).
+    // per-wave arrival flags in sk_flags (they carry sk_epoch; the last reader of a flag clears it).
     int sk_S, sk_tpx;
     float *sk_part;
     unsigned *sk_flags;
@@ -959,6 +961,24 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
             for (int r = 0; r < 16; r++) {
                 tot[0][r] = sk_s == 0 ? own[0][r] + blk[0][r >> 2][r & 3] : blk[0][r >> 2][r & 3] + own[0][r];
                 if (NQ == 4) tot[1][r] = sk_s == 0 ? own[1][r] + blk[1][r >> 2][r & 3] : blk[1][r >> 2][r & 3] + own[1][r];
+            }
+        }
+        // What the partners sent has arrived (the sums above used it).  The last wave to have consumed a partner's
+        // partials clears that partner's flag -- with two slices that is this wave, with four the third to count itself
+        // in -- so the next launch on this bank, which for a replayed graph carries this same epoch, starts from zero.
+        if (lane == 0) {
+#pragma unroll
+            for (int bi = 0; bi < 3; bi++) {
+                if (S == 4 || bi == 0) {
+                    const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;
+                    unsigned *f = p.sk_flags + ((long)sk_tile * S + src) * 8 + wave;
+                    bool last = true;
+                    if (S == 4) {
+                        last = __hip_atomic_fetch_add(f + SK_WORDS, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 2u;
+                        if (last) __hip_atomic_store(f + SK_WORDS, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    if (last) __hip_atomic_store(f, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
         }
 #ifdef MI_LAB_TS

@@ -309,10 +309,12 @@ def test_output_larger_than_2g_elements_is_indexed_in_64_bits(ctx, layout):
 
 
 @pytest.mark.parametrize("layout", ["kf", "fk"])
-@pytest.mark.parametrize("T,K,F", [(1370, 1536, 384), (200, 2048, 256), (1500, 5120, 1280), (200, 256, 328), (4, 1280, 1280), (77, 2048, 264)])
+@pytest.mark.parametrize("T,K,F", [(1370, 1536, 384), (200, 2048, 256), (1500, 5120, 1280), (200, 256, 328), (4, 1280, 1280), (77, 2048, 264),
+                                   (1370, 384, 384), (64, 128, 64), (130, 512, 1024), (1000, 256, 520), (2500, 128, 192), (65, 1536, 384)])
 def test_layer_norm_of_the_output_rides_in_the_gemm(ctx, T, K, F, layout):
     """matmul_ln_ against the oracle's gemm -> layernorm, and bit for bit (both outputs) against matmul_ followed by
-    layernorm_: split-K shapes (the norm is in the plane-summing pass), unsplit and decode-sized ones (two kernels)."""
+    layernorm_: split-K shapes (the norm is in the plane-summing pass), unsplit and decode-sized ones (two kernels; one
+    to sixteen column tiles a row panel, one and two chunks a lane in the norm, ragged last panels)."""
     import torch
     import juliavision_amd as jv
     X = oracle.randn_f16((T, K), 91, 0, 1.0 / np.sqrt(K))
@@ -335,6 +337,39 @@ def test_layer_norm_of_the_output_rides_in_the_gemm(ctx, T, K, F, layout):
         assert_parity(to_host(out), y, what=f"matmul_ln_ output T{T} K{K} F{F} {layout}")
         assert_parity(to_host(normed), h, what=f"matmul_ln_ norm T{T} K{K} F{F} {layout}")
         assert np.array_equal(to_host(out), to_host(out2)) and np.array_equal(to_host(normed), to_host(normed2))
+
+
+@pytest.mark.parametrize("T,K,F", [(1500, 5120, 1280), (1370, 1536, 384)])
+def test_in_launch_exchange_starts_clean_on_every_replay(ctx, T, K, F):
+    """A captured launch carries the flag bank and epoch it was given at capture.  The split-K exchange
+    (1500 x 5120 -> 1280) leaves its flags at zero, so a replay waits for this replay's partners and not for what the
+    last replay left behind: three replays over changing inputs each equal the eager result on the same inputs, bit
+    for bit (the second shape runs without an exchange)."""
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd.decode import StepGraph
+    w = to_dev(oracle.randn_f16((K, F), 61, 0, 1.0))
+    b, r = to_dev(oracle.randn_f16((F,), 62, 0, 0.1)), to_dev(oracle.randn_f16((T, F), 63, 0.2, 1.0))
+    g, be = to_dev(oracle.randn_f16((F,), 64, 1.0, 0.2)), to_dev(oracle.randn_f16((F,), 65, 0, 0.2))
+    x = to_dev(oracle.randn_f16((T, K), 66, 0, 1.0 / np.sqrt(K)))
+    y, h = (poison(torch.empty((T, F), dtype=torch.float16, device="cuda")) for _ in range(2))
+
+    def step():
+        ctx.ws.reset()
+        jv.matmul_ln_(ctx, y, h, w, x, g, be, 1e-6, b, residual=r)
+
+    graph = StepGraph(step)
+    for it in range(3):
+        x.copy_(to_dev(oracle.randn_f16((T, K), 70 + it, 0, 1.0 / np.sqrt(K))))
+        poison(y), poison(h)
+        graph.replay()
+        torch.cuda.synchronize()
+        y2, h2 = (poison(torch.empty_like(y)) for _ in range(2))
+        ctx.ws.reset()
+        jv.matmul_(ctx, y2, w, x, b, residual=r)
+        jv.layernorm_(ctx, h2, None, None, y2, g, be, F, 1e-6)
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), y2.view(torch.int16)) and torch.equal(h.view(torch.int16), h2.view(torch.int16)), it
 
 
 @pytest.mark.parametrize("T,K,F,with_norm", [(300, 256, 384, True), (200, 2048, 256, True), (130, 128, 520, False), (4, 256, 384, True)])
