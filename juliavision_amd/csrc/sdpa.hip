@@ -636,6 +636,242 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
 }
 
 // ------------------------------------------------------------------------------------------
+// Fused attention for grids that leave most of the chip idle (head size 64, no mask): a workgroup owns 32 queries,
+// and its NW waves (8, or 4 so that two workgroups share a CU) each walk their own run of whole 64-key blocks, so the
+// chain a wave walks is Lk / NW keys long instead of Lk / 2.  Nothing is shared between the waves until the end, so
+// nothing is staged for anyone else and the loop has no workgroup barrier: a wave takes its K fragments straight from
+// memory in the layout the first product wants (lane = key, 16 bytes of one row per k-step: every row is read whole over
+// the four k-steps), and passes its V block through a private stretch of LDS only for the transposing read of the second
+// product (the wave's LDS operations complete in order: the write of block j + 1 follows the reads of block j without a
+// wait).  Both are requested a block ahead.  The softmax is flash_fwd_kernel's (lazy reference point).  The waves'
+// (O, M, l) meet in LDS and are merged with the rescaling identity of flash.jl:1385-1391, each thread finishing four
+// consecutive head-dim values of one query.
+template <int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void flash_short_kernel(SdpaArgs p) {
+    constexpr int EP = 64, KS = 4, ET = 2, BC = 64, VLD = flash_vld(64);
+    constexpr int WREG = BC * VLD * 2;                        // bytes of a wave's V stretch; holds its (O, m, l) afterwards
+    static_assert((ET * 16 + 2) * 64 * 4 <= WREG, "a wave's partial fits its own stretch");
+    extern __shared__ __align__(16) char smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int hl = lane >> 5, l32 = lane & 31;
+    half_t *Vw = reinterpret_cast<half_t *>(smem + wave * WREG);
+    int qblk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    {
+        // all query blocks of a head on one XCD (workgroups are dealt to the XCDs round robin)
+        const int nqb = gridDim.x, total = nqb * gridDim.y * gridDim.z;
+        if ((total & 7) == 0) {
+            int id = blockIdx.x + nqb * (blockIdx.y + gridDim.y * blockIdx.z);
+            id = (id & 7) * (total >> 3) + (id >> 3);
+            qblk = id % nqb;
+            h = (id / nqb) % gridDim.y;
+            b = id / (nqb * gridDim.y);
+        }
+    }
+    const int q0 = qblk * 32;
+    const half_t *qb = p.q + h * p.qs[2] + b * p.qs[3];
+    const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
+    const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
+    int Lk = p.Lk;
+    if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
+    // this wave's keys: whole 64-key blocks, [kbeg, kend)
+    const int per = (((Lk + BC - 1) / BC + NW - 1) / NW) * BC;
+    const int kbeg = wave * per, kend = min(Lk, kbeg + per);
+    const int nblk = kend > kbeg ? (kend - kbeg + BC - 1) / BC : 0;
+    const int last = p.Lk - 1;                                // rows past the end re-read the last key that exists
+    const float c = p.scale * LOG2E;
+
+    u32x4 qraw[KS];
+    {
+        const int qr = min(q0 + l32, p.Lq - 1);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) qraw[ks] = ldg16(qb + (long)qr * p.qs[1] + 16 * ks + 8 * hl);
+    }
+    // K fragments of a block: tile kt (32 keys), k-step ks: key = key0 + 32 kt + l32, head dim 16 ks + 8 hl .. +7
+    auto load_k = [&](u32x4 (&kf)[2][KS], int key0) {
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+            const half_t *row = kb + (long)min(key0 + 32 * kt + l32, last) * p.ks[1] + 8 * hl;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) kf[kt][ks] = ldg16(row + 16 * ks);
+        }
+    };
+    // the wave's V block, 8 chunks of 16 bytes per lane: chunk lane + 64 i = (key, 8 head-dim values)
+    u32x4 vr[8];
+    auto load_v = [&](int key0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int cidx = lane + 64 * i;
+            vr[i] = ldg16(vb + (long)min(key0 + (cidx >> 3), last) * p.vs[1] + (cidx & 7) * 8);
+        }
+    };
+    auto store_v = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int cidx = lane + 64 * i;
+            *reinterpret_cast<u32x4 *>(Vw + (cidx >> 3) * VLD + (cidx & 7) * 8) = vr[i];
+        }
+    };
+    u32x4 ka[2][KS], kc[2][KS];
+    if (nblk > 0) { load_k(ka, kbeg); load_v(kbeg); }
+    half8v qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        const half8v t = as_half8(qraw[ks]);
+#pragma unroll
+        for (int j = 0; j < 8; j++) qf[ks][j] = (half_t)((float)t[j] * c);
+    }
+    float16v o_acc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o_acc[t][r] = 0.0f;
+    float m_run = 0.0f, l_run = 0.0f;                        // m_run: the reference point, always exactly representable in fp16
+    const int vtoff = (4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    // The reference point of the running softmax is subtracted by the first product itself -- one more k-step with the
+    // operand pair 1.0 and -M[query] -- and moves lazily, as in flash_fwd_kernel: on a wave's first block, and when a
+    // probability would leave fp16 range (seen in the fp32 row sum growing by 2^16 within a block).
+    constexpr float TH = 8.0f;
+    half8v kext, qext;
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) { kext[jj] = (half_t)0.0f; qext[jj] = (half_t)0.0f; }
+    if (hl == 0) kext[0] = (half_t)1.0f;
+    bool first = true;
+    auto probs = [&](const float16v (&sx)[2], half8v (&pf)[2][2], float &l) {
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(sx[kt][r]), p1 = __builtin_amdgcn_exp2f(sx[kt][r + 1]);
+                pf[kt][r >> 3][r & 7] = (half_t)p0;
+                pf[kt][r >> 3][(r & 7) + 1] = (half_t)p1;
+                l += p0 + p1;
+            }
+    };
+    auto iter = [&](u32x4 (&kcur)[2][KS], u32x4 (&knext)[2][KS], int j) {
+        const int key0 = kbeg + j * BC;
+        store_v();                                           // block j's V (requested one block ago) into the stretch
+        if (j + 1 < nblk) { load_k(knext, key0 + BC); load_v(key0 + BC); }
+        float16v sc[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+            sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(kcur[kt][0]), qf[0], zero16, 0, 0, 0);
+#pragma unroll
+            for (int ks = 1; ks < KS; ks++) sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(kcur[kt][ks]), qf[ks], sc[kt], 0, 0, 0);
+            sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, sc[kt], 0, 0, 0);
+        }
+        if (key0 + BC > kend) {                              // the ragged last block: excluded keys get -inf
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (key0 + 32 * kt + 8 * (r >> 2) + 4 * hl + (r & 3) >= kend) sc[kt][r] = -INFINITY;
+        }
+        half8v pf[2][2];
+        float l_new = l_run;
+        probs(sc, pf, l_new);
+        if (__any(first || !(l_new - l_run < 65504.0f))) {
+            float tmax = fmaxf(sc[0][0], sc[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; r++) tmax = fmaxf(fmaxf(tmax, sc[0][r]), sc[1][r]);
+            const float mx = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const bool grow = (mx > TH || first) && mx != -INFINITY;
+            const half_t m16 = (half_t)(m_run + (grow ? mx : 0.0f));
+            const float d = (float)m16 - m_run;
+            const float alpha = __builtin_amdgcn_exp2f(-d);
+            m_run += d;
+            l_run *= alpha;
+            if (hl == 0) qext[0] = -m16;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) sc[kt][r] -= d;
+#pragma unroll
+            for (int t = 0; t < ET; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o_acc[t][r] *= alpha;
+            l_new = l_run;
+            probs(sc, pf, l_new);
+        }
+        l_run = l_new;
+        first = false;
+        // O^T += V^T . P^T
+#pragma unroll
+        for (int t = 0; t < ET; t++) {
+            const half_t *vp = Vw + vtoff + 32 * t;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int bb = 0; bb < 2; bb++) {
+                    const half_t *vq = vp + (32 * kt + 16 * bb) * VLD;
+                    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(vq));
+                    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(vq + 8 * VLD));
+                    short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    o_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, both), pf[kt][bb], o_acc[t], 0, 0, 0);
+                }
+        }
+    };
+    int j = 0;
+    for (; j + 2 <= nblk; j += 2) {
+        iter(ka, kc, j);
+        iter(kc, ka, j + 1);
+    }
+    if (j < nblk) iter(ka, kc, j);
+
+    // both lanes of a query hold half of its row sum
+    l_run += __shfl_xor(l_run, 32, 64);
+    // the wave's partial, lane-major, into its own stretch (its reads of V are behind it)
+    float *xo = reinterpret_cast<float *>(smem + wave * WREG);
+#pragma unroll
+    for (int t = 0; t < ET; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) xo[(t * 16 + r) * 64 + lane] = o_acc[t][r];
+    xo[(ET * 16) * 64 + lane] = m_run;
+    xo[(ET * 16 + 1) * 64 + lane] = l_run;
+    __syncthreads();
+    // Thread (src lane, group) finishes query q0 + l32 at head dims 32 t + 8 g + 4 hl .. +3 for its (t, g).
+    float aw[NW], mm = -INFINITY, den = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+        // a wave that saw no valid key has l = 0 and a meaningless reference point
+        const float *xw = reinterpret_cast<const float *>(smem + w * WREG);
+        aw[w] = xw[(ET * 16 + 1) * 64 + lane] > 0.0f ? xw[(ET * 16) * 64 + lane] : -INFINITY;
+        mm = fmaxf(mm, aw[w]);
+    }
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+        const float *xw = reinterpret_cast<const float *>(smem + w * WREG);
+        aw[w] = aw[w] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(aw[w] - mm);
+        den += aw[w] * xw[(ET * 16 + 1) * 64 + lane];
+    }
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    const int qi = q0 + l32;
+    constexpr int COMBOS = 8 / NW;                            // (t, g) pairs per thread: 8 pairs over NW waves
+#pragma unroll
+    for (int cidx = 0; cidx < COMBOS; cidx++) {
+        const int tg = wave * COMBOS + cidx, t = tg >> 2, g = tg & 3;
+        float o4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            const float *xw = reinterpret_cast<const float *>(smem + w * WREG);
+#pragma unroll
+            for (int i = 0; i < 4; i++) o4[i] += aw[w] * xw[(t * 16 + 4 * g + i) * 64 + lane];
+        }
+        if (qi < p.Lq) {
+            const long off = (long)b * p.os[3] + (long)h * p.os[2] + (long)qi * p.os[1] + 32 * t + 8 * g + 4 * hl;
+            if (p.out_f32) {
+                const float4v o = {o4[0] * inv, o4[1] * inv, o4[2] * inv, o4[3] * inv};
+                *reinterpret_cast<float4v *>(reinterpret_cast<float *>(p.out) + off) = o;
+            } else {
+                const half4v o = {(half_t)(o4[0] * inv), (half_t)(o4[1] * inv), (half_t)(o4[2] * inv), (half_t)(o4[3] * inv)};
+                *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(p.out) + off) = o;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // One workgroup (4 waves) per (query row, key split).  A wave walks keys 8 at a
 // time: 8 lanes share a key, each owning 8-element head-dim chunks c, c+8, ...
 // (NCH chunks, E <= 64 NCH).  Every 8-lane group keeps its own running
@@ -1043,6 +1279,7 @@ __global__ void sdpa_merge_kernel(SdpaArgs p) {
 
 // ------------------------------------------------------------------------------------------
 constexpr int flash_lds_bytes(int EP) { return 3 * 64 * (EP + 8) * 2 + 3 * 64 * flash_vld(EP) * 2; }
+constexpr int flash_short_lds_bytes(int NW) { return NW * 64 * flash_vld(64) * 2; }
 
 bool vec_addressable(const half_t *ptr, const long st[4], int E) {
     return st[0] == 1 && E % 8 == 0 && st[1] % 8 == 0 && st[2] % 8 == 0 && st[3] % 8 == 0 && aligned_to(ptr, 16);
@@ -1079,6 +1316,24 @@ int flash_splits(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     // no empty split: with `per` blocks each, the last one must still start inside the keys
     while (want > 1 && ceil_div(blocks, want) * (want - 1) >= blocks) want--;
     return (int)want;
+}
+
+// Head size 64, no mask, and at most about one 32-query workgroup per compute unit: flash_short_kernel, unless key
+// splits over workgroups are estimated faster still (a handful of tiles over thousands of keys).  A SIMD finishes a 32 x 64 block of it in
+// about 1.3 us whether it holds one of its waves or two, so what counts is that every SIMD gets one wave: 6 heads x 1344
+// (252 workgroups) 18.5 -> 11.8 us, 12 heads x 577 12.3 -> 7.6 us, 4 heads x 640 over 300 keys 10.6 -> 6.3 us; at 6
+// heads x 1370 two CUs of 256 hold two workgroups, which then take twice as long (17.6 us against 18.5 us), and
+// beyond that the 128-query forms are as fast or faster.
+bool flash_short(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    const int64_t tiles = ceil_div(Lq, 32) * H * B, cus = mi_num_cus();
+#ifdef MI_LAB
+    if (const char *f = getenv("MI_FORCE_SHORT")) return E == 64 && atoi(f) > 0;
+#endif
+    if (E != 64 || Lk < 128 || tiles > cus + cus / 16) return false;
+    // against key splits over workgroups (few tiles, many keys): 4.5 us + 1.3 us per block of a wave's quarter here,
+    // 3 us + 1 us per block of a split + the 6 us merge launch there
+    const int64_t blocks = ceil_div(Lk, 64), ns = flash_splits(E, Lq, Lk, H, B);
+    return ns == 1 || 4.5 + 1.3 * (double)ceil_div(blocks, 4) <= 9.0 + 1.0 * (double)ceil_div(blocks, ns);
 }
 
 // A single query row (a decode step) runs in one launch of sdpa_decode_kernel: the work follows the device-side kv_len
@@ -1200,6 +1455,7 @@ int mi_sdpa_init() {
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_short_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_short_lds_bytes(4)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
@@ -1216,7 +1472,7 @@ extern "C" {
 size_t mi_sdpa_f16_workspace(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, int has_bias) {
     // sized for the path the call will most likely take: the fused kernel's key splits for Lq >= 64 without
     // an additive mask (unused if the operands turn out not to be 16-byte addressable), the rows kernel's below
-    int ns = Lq >= 64 ? (has_bias ? 1 : flash_splits(E, Lq, Lk, H, B)) : rows_splits(Lq, Lk, H, B);
+    int ns = Lq >= 64 ? ((has_bias || flash_short(E, Lq, Lk, H, B)) ? 1 : flash_splits(E, Lq, Lk, H, B)) : rows_splits(Lq, Lk, H, B);
     if (ns <= 1) return 0;
     size_t rows = (size_t)Lq * H * B;
     return round_up((size_t)ns * rows * E * sizeof(float), 256) + round_up((size_t)ns * rows * 2 * sizeof(float), 256);
@@ -1236,7 +1492,7 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
     int path = sdpa_path(a);
     const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
     if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? (one_pass_decode(a, vec) ? decode_splits(E, Lk, H, B) : rows_splits(Lq, Lk, H, B))
-                                  : (path == MI_SDPA_FLASH && !has_bias) ? flash_splits(E, Lq, Lk, H, B) : 1;
+                                  : (path == MI_SDPA_FLASH && !has_bias && !flash_short(E, Lq, Lk, H, B)) ? flash_splits(E, Lq, Lk, H, B) : 1;
     return path;
 }
 
@@ -1272,6 +1528,10 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
         } else if (pp) {
             dim3 grid((unsigned)ceil_div(Lq, 256), (unsigned)H, (unsigned)B);
             hipLaunchKernelGGL((flash_fwd_kernel<64, true>), grid, dim3(512), flash_lds_bytes(64), st, a);
+        } else if (flash_short(E, Lq, Lk, H, B)) {
+            a.nsplit = 1;
+            dim3 grid((unsigned)ceil_div(Lq, 32), (unsigned)H, (unsigned)B);
+            hipLaunchKernelGGL(flash_short_kernel<4>, grid, dim3(256), flash_short_lds_bytes(4), st, a);
         } else {
             // few query blocks: split the keys over workgroups too, if the caller brought the workspace for it
             a.nsplit = flash_splits(E, Lq, Lk, H, B);

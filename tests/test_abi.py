@@ -90,7 +90,11 @@ def test_sdpa_planner():
     # an additive mask (planned as a dense fp16 (Lk, Lq, H, B) array) stays in the fused kernel where its rows start on
     # 4-byte boundaries -- the reference's fused plan declines every mask, Decline(:bias), flash.jl:1327 -- keys unsplit
     assert _sdpa_plan(64, 1500, 1500, 20, 1, bias=1) == ("flash", 1)
-    assert _sdpa_plan(64, 128, 2048, 1, 1, bias=1) == ("flash", 1) and _sdpa_plan(64, 128, 2048, 1, 1)[1] > 1
+    assert _sdpa_plan(64, 128, 8192, 1, 1, bias=1) == ("flash", 1) and _sdpa_plan(64, 128, 8192, 1, 1)[1] > 1
+    # head size 64 on few tiles: four waves a 32-query tile, each with a quarter of the keys, unless the keys are so many
+    # that splits over workgroups win (above); a wider head keeps the splits
+    assert _sdpa_plan(64, 128, 2048, 1, 1) == ("flash", 1) and _sdpa_plan(64, 1370, 1370, 6, 1) == ("flash", 1)
+    assert _sdpa_plan(72, 128, 2048, 1, 1)[1] > 1
     assert _sdpa_plan(64, 1500, 1371, 20, 1, bias=1)[0] == "rows"          # odd row length: fp16 rows at 2-byte offsets
     assert _sdpa_plan(64, 1, 448, 20, 1)[0] == "rows"
     assert _sdpa_plan(20, 128, 128, 2, 1)[0] == "rows"                     # E not a multiple of 8

@@ -249,21 +249,22 @@ def test_eight_wave_kernel_odd_key_counts_and_random_lengths(ctx, B, H, Lq, Lk, 
 def test_fused_kernel_splits_keys_on_small_grids(ctx):
     """Few query blocks and very many keys: the fused kernel also splits the keys over workgroups and a merge joins
     the partials.  Ragged last split, per-batch kv_len that leaves the later split without a key (one row of the
-    batch with none at all), fp32 and token-major outputs; config 3's shape stays in one pass."""
+    batch with none at all), fp32 and token-major outputs; config 3's shape stays in one pass.  Head size 48 here: at
+    64 these extents run the short-chain form, which splits the keys inside the workgroup."""
     import torch
     import juliavision_amd as jv
     q, k, v = _qkv(1, 6, 1370, 1370, 64, 131)
     plan = jv.sdpaplan(ctx, to_dev(q), to_dev(k), to_dev(v))
     assert type(plan).__name__ == "FlashPlan" and plan.nsplit == 1, plan
     _check(ctx, q, k, v, expect="FlashPlan", what="config 3 attention")
-    q, k, v = _qkv(1, 2, 300, 2000, 64, 135)
+    q, k, v = _qkv(1, 2, 300, 2000, 48, 135)
     assert jv.sdpaplan(ctx, to_dev(q), to_dev(k), to_dev(v)).nsplit == 2
     _check(ctx, q, k, v, expect="FlashPlan", what="two key splits, ragged second")
-    q, k, v = _qkv(3, 2, 200, 1700, 64, 141)
+    q, k, v = _qkv(3, 2, 200, 1700, 48, 141)
     assert jv.sdpaplan(ctx, to_dev(q), to_dev(k), to_dev(v)).nsplit == 2
     got = _check(ctx, q, k, v, kv_len=[1700, 0, 70], out_dtype="f32", expect="FlashPlan", what="key splits with kv_len")
     assert np.all(got[1] == 0)
-    buf = poison(torch.empty((3, 200, 2, 64), dtype=torch.float16, device="cuda"))
+    buf = poison(torch.empty((3, 200, 2, 48), dtype=torch.float16, device="cuda"))
     ctx.ws.reset()
     jv.sdpa(ctx, to_dev(q), to_dev(k), to_dev(v), None, None, out=buf.permute(0, 2, 1, 3))
     torch.cuda.synchronize()
@@ -272,29 +273,43 @@ def test_fused_kernel_splits_keys_on_small_grids(ctx):
     from juliavision_amd import _lib as L
     lib = L.init()
     dq, dk, dv = to_dev(q), to_dev(k), to_dev(v)
-    out = poison(torch.empty((3, 2, 200, 64), dtype=torch.float16, device="cuda"))
+    out = poison(torch.empty((3, 2, 200, 48), dtype=torch.float16, device="cuda"))
     st = lambda t: L.strides4(t.stride(3), t.stride(2), t.stride(1), t.stride(0))
     rc = lib.mi_sdpa_f16(out.data_ptr(), L.F16, None, dq.data_ptr(), st(dq), dk.data_ptr(), st(dk), dv.data_ptr(), st(dv),
-                         None, L.F16, None, None, 64, 200, 1700, 2, 3, 0.125, None, 0, torch.cuda.current_stream().cuda_stream)
+                         None, L.F16, None, None, 48, 200, 1700, 2, 3, 48 ** -0.5, None, 0, torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
     assert_parity(to_host(out), oracle.sdpa_ref_f32(q, k, v), what="no workspace: one pass")
 
 
 @pytest.mark.parametrize("Lk", [256, 257, 319, 320, 321, 383, 384, 385, 447, 448, 449, 1000])
-@pytest.mark.parametrize("Lq,E", [(64, 64), (130, 64), (200, 32)])
-def test_fused_kernel_key_halves_on_one_workgroup_per_cu_grids(ctx, Lq, Lk, E):
-    """Grids of at most one workgroup per CU with 256 keys or more run eight waves, each pair of waves sharing its
-    queries and taking alternate 64-key halves of a 128-key stage; the halves merge in LDS.  Key counts around the
-    64- and 128-key boundaries: the second half's last block empty, ragged, exactly full."""
-    q, k, v = _qkv(2, 3, Lq, Lk, E, 211 + Lk)
-    _check(ctx, q, k, v, expect="FlashPlan", what=f"key halves Lq{Lq} Lk{Lk} E{E}")
+@pytest.mark.parametrize("B,H,Lq,E", [(12, 12, 64, 64), (5, 12, 130, 64), (2, 3, 200, 32)])
+def test_fused_kernel_key_halves_on_one_workgroup_per_cu_grids(ctx, B, H, Lq, Lk, E):
+    """Grids of at most one 128-query workgroup per CU with 256 keys or more (and, at head size 64, more 32-query tiles
+    than the short-chain form takes: 288 and 300 here) run eight waves, each pair of waves sharing its queries and taking
+    alternate 64-key halves of a 128-key stage; the halves merge in LDS.  Key counts around the 64- and 128-key
+    boundaries: the second half's last block empty, ragged, exactly full."""
+    q, k, v = _qkv(B, H, Lq, Lk, E, 211 + Lk)
+    _check(ctx, q, k, v, expect="FlashPlan", what=f"key halves B{B} H{H} Lq{Lq} Lk{Lk} E{E}")
 
 
-def test_fused_kernel_key_halves_masks_and_layouts(ctx):
+@pytest.mark.parametrize("Lk", [128, 129, 255, 256, 257, 300, 511, 512, 513, 767, 768, 769, 1000, 1370])
+@pytest.mark.parametrize("B,H,Lq", [(2, 3, 64), (1, 6, 130), (1, 2, 1370)])
+def test_short_chain_form_on_small_grids(ctx, B, H, Lq, Lk):
+    """Head size 64 and at most about one 32-query tile per CU: four waves per tile, each walking its own quarter of the
+    keys (whole 64-key blocks), K fragments straight from memory, partials merged in LDS.  Key counts around the
+    boundaries of a wave's share: waves without a key, with a ragged block, with exactly full ones; a ragged last tile
+    of queries."""
+    q, k, v = _qkv(B, H, Lq, Lk, 64, 411 + Lk)
+    _check(ctx, q, k, v, expect="FlashPlan", what=f"short chain B{B} H{H} Lq{Lq} Lk{Lk}")
+
+
+@pytest.mark.parametrize("H,HP", [(2, 6), (10, 32)])
+def test_fused_kernel_key_halves_masks_and_layouts(ctx, H, HP):
+    """H = 2, HP = 6: the short-chain form (60 and 54 tiles); H = 10, HP = 32: the key-halves form (300 and 288)."""
     import torch
     import juliavision_amd as jv
-    q, k, v = _qkv(6, 2, 150, 300, 64, 251)
+    q, k, v = _qkv(6, H, 150, 300, 64, 251)
     # kv_len leaves the second half of the keys without a valid one (10, 64), with exactly one (65), a ragged
     # second stage (129, 200), and a row of the batch with none at all (0)
     got = _check(ctx, q, k, v, kv_len=[10, 64, 65, 129, 0, 200], out_dtype="f32", expect="FlashPlan", what="key halves with kv_len")
@@ -306,7 +321,7 @@ def test_fused_kernel_key_halves_masks_and_layouts(ctx):
     k2[:, :, 64:128] *= np.float16(3.0)
     _check(ctx, q2, k2, v, expect="FlashPlan", what="key halves, one half with far larger scores")
     # token-major output and packed strided q/k/v, as the encoder block calls it
-    B, H, L, E = 1, 6, 260, 64
+    B, H, L, E = 1, HP, 260, 64
     qkv = oracle.randn_f16((L, 3 * H * E), 261)
     dqkv = to_dev(qkv)
     views = [dqkv[:, i * H * E:(i + 1) * H * E].unflatten(1, (H, E)).permute(1, 0, 2).unsqueeze(0) for i in range(3)]
@@ -320,7 +335,7 @@ def test_fused_kernel_key_halves_masks_and_layouts(ctx):
 
 
 @pytest.mark.parametrize("B,H,Lq,Lk,which", [(1, 2, 128, 200, "four waves"), (4, 16, 300, 200, "eight waves, 256 queries"),
-                                             (1, 3, 128, 400, "key halves"), (1, 2, 200, 2000, "key splits")])
+                                             (1, 3, 128, 400, "short chain"), (8, 12, 128, 400, "key halves"), (1, 2, 200, 8000, "key splits")])
 def test_reference_point_follows_scores_that_grow_along_the_keys(ctx, B, H, Lq, Lk, which):
     """The fused kernel exponentiates against a reference point that it moves only when it must.  Keys whose scores
     exceed everything before them by far more than fp16's exponent range (here by up to ~2^60 from one 64-key block
