@@ -108,7 +108,7 @@ constexpr int flash_vld(int EP) { return EP == 96 ? EP : EP + 32; }
 // declines (flash.jl:1327).
 template <int EP, bool PP, int KH = 1, int BIAS = 0>      // BIAS: 0 none, 1 fp16, 2 fp32
 __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH == 1 && (BIAS == 0 || EP == 64)) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
-    static_assert(BIAS == 0 || (!PP && KH == 1), "the mask rides in the four-wave form");
+    static_assert(BIAS == 0 || (!PP && KH == 1) || (PP && KH == 2 && BIAS == 1 && EP == 64), "the mask rides in the four-wave form, and as fp16 in the key-halves form");
     // PP with KH = 2: the two key-half groups of the eight-wave form (same 128 queries) take turns at the vector
     // and matrix units like the two query groups of the 256-query form do; every thread stages.
     constexpr int BC = 64, BR = (PP && KH == 1) ? 256 : 128, NT = (KH == 2 || PP) ? 512 : 256;     // NT: threads that stage K and V
@@ -1455,6 +1455,7 @@ int mi_sdpa_init() {
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_short_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_short_lds_bytes(4)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
@@ -1519,7 +1520,10 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
             a.nsplit = 1;
             dim3 grid((unsigned)ceil_div(Lq, 128), (unsigned)H, (unsigned)B);
             const bool f32 = a.bias_f32 != 0;
-            if (E <= 64)      { if (f32) hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 2>), grid, dim3(256), flash_lds_bytes(64), st, a);
+            // an fp16 mask on a grid of at most one workgroup per CU: the key-halves form carries it too
+            if (E <= 64 && !f32 && ceil_div(Lq, 128) * H * B <= (int64_t)mi_num_cus() && Lk >= 256)
+                hipLaunchKernelGGL((flash_fwd_kernel<64, true, 2, 1>), grid, dim3(512), 2 * flash_lds_bytes(64), st, a);
+            else if (E <= 64) { if (f32) hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 2>), grid, dim3(256), flash_lds_bytes(64), st, a);
                                 else     hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 1>), grid, dim3(256), flash_lds_bytes(64), st, a); }
             else if (E <= 96) { if (f32) hipLaunchKernelGGL((flash_fwd_kernel<96, false, 1, 2>), grid, dim3(256), flash_lds_bytes(96), st, a);
                                 else     hipLaunchKernelGGL((flash_fwd_kernel<96, false, 1, 1>), grid, dim3(256), flash_lds_bytes(96), st, a); }

@@ -128,7 +128,9 @@ def test_full_bias_f32(ctx):
     (1, 2, 300, 333, 64, "full32"),       # dense fp32, an odd row length (fp32 rows are always dword aligned)
     (2, 2, 128, 130, 72, "causal16"),     # 0 / -inf lower-triangular mask (Lq, Lk) broadcast over batch and heads, head size 72
     (1, 1, 192, 320, 128, "full32"),      # the 128-wide instance
-    (1, 20, 1500, 1500, 64, "pad16"),     # config 2's attention with a padding mask
+    (1, 20, 1500, 1500, 64, "pad16"),     # config 2's attention with a padding mask: an fp16 mask on a grid of at most one workgroup
+    (2, 4, 300, 700, 64, "causal16"),     # per CU over 256 keys or more rides in the eight-wave key-halves form (so does full16 above)
+    (3, 2, 150, 450, 64, "full16"),       # ... second half of the last stage with two keys
 ])
 def test_additive_mask_rides_in_the_fused_kernel(ctx, B, H, Lq, Lk, E, kind):
     """Encoder-sized attention with an additive mask: the mask tile joins the scores inside the fused kernel (the
