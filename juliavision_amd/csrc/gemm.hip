@@ -1295,46 +1295,73 @@ __global__ __launch_bounds__(256) void skinny_fk_kernel(GemmArgs p) {
     }
     __syncthreads();
     if (!live) return;
-    float acc[MT];
+    // A wave walks columns n, n + 4 gridDim.x, ...: one for the widths of a decoder layer (the launcher gives every
+    // column its wave), several for a vocabulary-sized output, where the staged activations and their norm are then
+    // paid once per workgroup instead of once per four columns and the next column's row is requested under the
+    // current one's dot products.
+    const int stride = (int)gridDim.x * 4;
+    for (int nc = n; nc < p.N; nc += stride) {
+        const int nn = nc + stride;
+        const bool more = nn < p.N;                       // uniform over the wave
+        const half_t *bn = p.B + (long)(more ? nn : nc) * p.ldB;
+        u32x4 wn[FK_PF];
+        float bvn = 0.0f, rvn = 0.0f;
+        if (more) {
 #pragma unroll
-    for (int m = 0; m < MT; m++) acc[m] = 0.0f;
-    auto dot = [&](const u32x4 &wv, int k) {
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const u32x4 x = *reinterpret_cast<const u32x4 *>(xs + (long)m * p.K + k);
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const uint32_t wq = wv[q], xq = x[q];     // bit_cast wants an addressable scalar, not a vector element
-                acc[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, wq), __builtin_bit_cast(half2v, xq), acc[m], false);
+            for (int i = 0; i < FK_PF; i++) wn[i] = lane * 8 + 512 * i < p.K ? ldg16(bn + lane * 8 + 512 * i) : z;
+            if (lane < p.M) {
+                if (p.bias_mode == MI_BIAS_COL) bvn = (float)p.bias[nn];
+                else if (p.bias_mode == MI_BIAS_ROW) bvn = (float)p.bias[lane];
+                if (p.residual && !p.out_f32) rvn = (float)p.residual[(long)lane * p.ldY + nn];
             }
         }
-    };
+        float acc[MT];
 #pragma unroll
-    for (int i = 0; i < FK_PF; i++)
-        if (lane * 8 + 512 * i < p.K) dot(w[i], lane * 8 + 512 * i);
-    for (int kb = lane * 8 + 512 * FK_PF; kb < p.K; kb += 4 * 512) {
-        u32x4 t[4];
+        for (int m = 0; m < MT; m++) acc[m] = 0.0f;
+        auto dot = [&](const u32x4 &wv, int k) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) t[i] = kb + 512 * i < p.K ? ldg16(bp + kb + 512 * i) : z;
+            for (int m = 0; m < MT; m++) {
+                const u32x4 x = *reinterpret_cast<const u32x4 *>(xs + (long)m * p.K + k);
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (kb + 512 * i < p.K) dot(t[i], kb + 512 * i);
-    }
-    float mine = 0.0f;                                    // lane m keeps row m's sum
+                for (int q = 0; q < 4; q++) {
+                    const uint32_t wq = wv[q], xq = x[q];     // bit_cast wants an addressable scalar, not a vector element
+                    acc[m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, wq), __builtin_bit_cast(half2v, xq), acc[m], false);
+                }
+            }
+        };
 #pragma unroll
-    for (int m = 0; m < MT; m++) {
-        float sres = acc[m];
-        sres = wave_sum(sres);
-        if (lane == m) mine = sres;
-    }
-    if (lane < p.M) {
-        const float v = mine + bv;
-        const long off = (long)lane * p.ldY + n;
-        if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(v, p.epi);
-        else {
-            half_t o = (half_t)apply_epi((float)(half_t)v, p.epi);
-            if (p.residual) o = (half_t)((float)o + rv);
-            reinterpret_cast<half_t *>(p.Y)[off] = o;
+        for (int i = 0; i < FK_PF; i++)
+            if (lane * 8 + 512 * i < p.K) dot(w[i], lane * 8 + 512 * i);
+        const half_t *bc = p.B + (long)nc * p.ldB;
+        for (int kb = lane * 8 + 512 * FK_PF; kb < p.K; kb += 4 * 512) {
+            u32x4 t[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) t[i] = kb + 512 * i < p.K ? ldg16(bc + kb + 512 * i) : z;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (kb + 512 * i < p.K) dot(t[i], kb + 512 * i);
+        }
+        float mine = 0.0f;                                    // lane m keeps row m's sum
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            float sres = acc[m];
+            sres = wave_sum(sres);
+            if (lane == m) mine = sres;
+        }
+        if (lane < p.M) {
+            const float v = mine + bv;
+            const long off = (long)lane * p.ldY + nc;
+            if (p.out_f32) reinterpret_cast<float *>(p.Y)[off] = apply_epi(v, p.epi);
+            else {
+                half_t o = (half_t)apply_epi((float)(half_t)v, p.epi);
+                if (p.residual) o = (half_t)((float)o + rv);
+                reinterpret_cast<half_t *>(p.Y)[off] = o;
+            }
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < FK_PF; i++) w[i] = wn[i];
+            bv = bvn; rv = rvn;
         }
     }
 }
@@ -1946,7 +1973,10 @@ int run_skinny(GemmArgs a, bool b_kn, void *ws, size_t ws_bytes, hipStream_t st)
             }
             return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
         }
-        dim3 grid((unsigned)ceil_div(a.N, 4));
+        // every column its own wave up to eight workgroups per CU; beyond that (a vocabulary projection) a wave walks
+        // several columns behind one staging of the activations
+        const int64_t wgs = ceil_div(a.N, 4), cap = (int64_t)g_cus * 8;
+        dim3 grid((unsigned)(wgs < cap ? wgs : cap));
         if (a.K <= 1536) {
             if (mt == 1)      hipLaunchKernelGGL((skinny_fk_kernel<1, 3>), grid, dim3(256), lds, st, a);
             else if (mt == 2) hipLaunchKernelGGL((skinny_fk_kernel<2, 3>), grid, dim3(256), lds, st, a);

@@ -53,10 +53,12 @@ def test_gemm_no_bias_row_bias_residual(ctx):
 @pytest.mark.parametrize("layout", ["kf", "fk"])
 @pytest.mark.parametrize("T,K,F", [
     (1, 8, 8), (2, 72, 136), (3, 264, 200), (5, 1288, 392), (6, 4104, 128), (7, 640, 1032), (8, 2048, 136),
+    (2, 264, 12344), (8, 1544, 9000),
 ])
 def test_decode_sized_rows_ragged_extents(ctx, T, K, F, layout):
     """T <= 8 takes the bandwidth kernels: K not a multiple of their 32- and 512-deep strides, F not a multiple of
-    their 128-column blocks, every row count their templates round up from."""
+    their 128-column blocks, every row count their templates round up from; outputs so wide that a wave of the
+    [F][K] kernel walks several columns (more than 8 workgroups of four columns per CU), some waves one more than others."""
     import juliavision_amd as jv
     import torch
     W = torch.zeros((K, F), dtype=torch.float16, device="cuda")
@@ -208,7 +210,7 @@ def test_split_k_partials_exchanged_inside_the_launch(ctx):
 
 
 @pytest.mark.parametrize("layout", ["kf", "fk"])
-@pytest.mark.parametrize("T,K,F", [(1, 1280, 1280), (4, 1280, 3840), (8, 264, 136), (3, 2048, 520)])
+@pytest.mark.parametrize("T,K,F", [(1, 1280, 1280), (4, 1280, 3840), (8, 264, 136), (3, 2048, 520), (1, 1280, 10008)])
 def test_layer_norm_folded_into_decode_sized_gemv(ctx, T, K, F, layout):
     """ln_matmul_ against the oracle's layernorm -> gemm, and bit for bit against the two device calls in sequence."""
     import torch
