@@ -234,6 +234,16 @@ def test_eight_wave_kernel_on_large_grids(ctx):
     _check(ctx, q, k[:, :, :129], v[:, :, :129], out_dtype="f32", expect="FlashPlan", what="8-wave three blocks f32")
 
 
+@pytest.mark.parametrize("Lk", [256, 257, 319, 320, 321, 383, 384, 385, 449, 1000])
+def test_eight_wave_kernel_key_counts_around_block_boundaries(ctx, Lk):
+    """256-query workgroups that cover the chip: key counts around the 64- and 128-key boundaries, a ragged last query
+    block, per-batch lengths (0, below one block, a block short of the end), fp32 output."""
+    q, k, v = _qkv(4, 16, 700, Lk, 64, 9000 + Lk, std=1.3)
+    _check(ctx, q, k, v, expect="FlashPlan", what=f"8-wave Lk{Lk}")
+    got = _check(ctx, q, k, v, kv_len=[Lk, 0, 37, Lk - 60], out_dtype="f32", expect="FlashPlan", what=f"8-wave kv_len Lk{Lk}")
+    assert np.all(got[1] == 0)
+
+
 @pytest.mark.parametrize("B,H,Lq,Lk,E", [(4, 16, 768, 65, 64), (4, 12, 1024, 257, 32), (2, 48, 520, 129, 64),
                                          (4, 16, 768, 1, 64), (3, 22, 770, 300, 48)])
 def test_eight_wave_kernel_odd_key_counts_and_random_lengths(ctx, B, H, Lq, Lk, E):
@@ -337,7 +347,8 @@ def test_fused_kernel_key_halves_masks_and_layouts(ctx, H, HP):
 
 
 @pytest.mark.parametrize("B,H,Lq,Lk,which", [(1, 2, 128, 200, "four waves"), (4, 16, 300, 200, "eight waves, 256 queries"),
-                                             (1, 3, 128, 400, "short chain"), (8, 12, 128, 400, "key halves"), (1, 2, 200, 8000, "key splits")])
+                                             (1, 3, 128, 400, "short chain"), (8, 12, 128, 400, "key halves"), (1, 2, 200, 8000, "key splits"),
+                                             (4, 24, 300, 400, "eight waves, 256 queries, 400 keys")])
 def test_reference_point_follows_scores_that_grow_along_the_keys(ctx, B, H, Lq, Lk, which):
     """The fused kernel exponentiates against a reference point that it moves only when it must.  Keys whose scores
     exceed everything before them by far more than fp16's exponent range (here by up to ~2^60 from one 64-key block
