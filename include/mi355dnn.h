@@ -89,7 +89,11 @@ int mi_set_clock_probe(void *dev_u64x4);
  *   to out_dtype, the activation applied to the ROUNDED value (matmul.jl:210-214).
  *   residual (fp16, same layout as Y, or NULL; fp16 output only) is added after the
  *   activation with one more rounding: the graph's own add.Tensor (ops.jl:186-197).
- * Replaces matmul!(ctx, out, A, B, bias; epi) -- matmul.jl:78-79,99-100,133-137,235-273. */
+ * Replaces matmul!(ctx, out, A, B, bias; epi) -- matmul.jl:78-79,99-100,133-137,235-273.
+ * Concurrency: a launch that splits K inside the kernel (the workgroups of a tile exchange partial tiles through
+ * arrival flags) takes the next of 16 banks of flag words held in static device memory, and leaves its bank zeroed.
+ * Up to 16 such launches may overlap on one GPU (different streams); a captured launch keeps the bank it was given at
+ * capture, so two captured graphs that hold the same bank must not be replayed at the same time. */
 int mi_gemm_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,
                 int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
                 int w_layout, int bias_mode, int epi, int out_dtype,
