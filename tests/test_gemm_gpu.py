@@ -177,8 +177,9 @@ def test_split_k_narrow_outputs(ctx, layout):
 def test_split_k_partials_exchanged_inside_the_launch(ctx):
     """Config 2's second MLP linear (1500 x 5120 -> 1280) splits K over two workgroups per 128 x 128 tile that exchange
     their partial tiles through L2 and per-wave arrival flags instead of writing fp32 planes.  The flags carry a
-    per-launch epoch and are never cleared: forty launches back to back on one stream, alternating two problems in one
-    workspace, must each give the bits of the first launch of that problem; and the result meets the oracle."""
+    per-launch epoch and are cleared by their last reader: forty launches back to back on one stream, alternating two
+    problems in one workspace, must each give the bits of the first launch of that problem; and the result meets the
+    oracle."""
     import torch
     from juliavision_amd import _lib as L
     lib = L.init()
