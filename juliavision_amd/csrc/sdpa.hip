@@ -1303,7 +1303,24 @@ int rows_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
 // and the merge is a second launch of about 6 us, so splitting pays only when the query blocks leave most
 // of the chip idle and every split still walks a dozen blocks (config 3's 66 workgroups x 22 blocks do
 // not: 21.9 us unsplit, 21.1 us at best split three ways).
+int flash_splits_over_workgroups(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B);
+
+// Head sizes 65 .. 96 over 1024 keys or more, at most one 128-query workgroup per CU: the eight-wave key-halves form at
+// 96 wide (two waves per SIMD in ping-pong, no second launch) where the grid covers more than half of the chip or the
+// keys would not be split over workgroups anyway -- 8 heads x 4096 x 72 (the reference's SAM 2.1 global attention):
+// 87.8 us as two key splits + merge launch, 76.0 us so; 12 heads x 1024 x 80: 28.8 -> 25.1 us.  Shorter key ranges stay
+// with four waves (16 windows x 8 heads x 256 x 72: 13.4 us against 16.0 us).
+bool flash_halves96(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    const int64_t wgs = ceil_div(Lq, 128) * H * B, cus = mi_num_cus();
+    if (E <= 64 || E > 96 || Lk < 1024 || wgs > cus) return false;
+    return wgs * 2 > cus || flash_splits_over_workgroups(E, Lq, Lk, H, B) == 1;
+}
+
 int flash_splits(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    return flash_halves96(E, Lq, Lk, H, B) ? 1 : flash_splits_over_workgroups(E, Lq, Lk, H, B);
+}
+
+int flash_splits_over_workgroups(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     const int64_t wgs = ceil_div(Lq, 128) * H * B, cus = mi_num_cus();
     // At head size 64 a grid of up to one workgroup per CU runs the eight-wave key-halves variant instead; wider
     // heads have no such variant, and two workgroups per CU is what gives their SIMDs a second wave.
@@ -1456,6 +1473,7 @@ int mi_sdpa_init() {
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, true, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_short_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_short_lds_bytes(4)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
@@ -1554,6 +1572,8 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
             const bool halves = E <= 64 && a.nsplit == 1 && ceil_div(Lq, 128) * H * B <= (int64_t)mi_num_cus() && Lk >= 256;
             // (its two key-half groups in ping-pong: 25.1 -> 23.8 us on 20 heads x 1500, 20.1 -> 19.4 us on 6 heads x 1370)
             if (halves)       hipLaunchKernelGGL((flash_fwd_kernel<64, true, 2>), grid, dim3(512), 2 * flash_lds_bytes(64), st, a);
+            else if (a.nsplit == 1 && flash_halves96(E, Lq, Lk, H, B))
+                hipLaunchKernelGGL((flash_fwd_kernel<96, true, 2>), grid, dim3(512), 2 * flash_lds_bytes(96), st, a);
             else if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false>), grid, dim3(256), flash_lds_bytes(64), st, a);
             else if (E <= 96) hipLaunchKernelGGL((flash_fwd_kernel<96, false>), grid, dim3(256), flash_lds_bytes(96), st, a);
             else         hipLaunchKernelGGL((flash_fwd_kernel<128, false>), grid, dim3(256), flash_lds_bytes(128), st, a);

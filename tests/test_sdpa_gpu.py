@@ -59,12 +59,28 @@ def test_flash_shapes(ctx, B, H, Lq, Lk, E):
     (1, 2, 130, 129, 88, {"out_dtype": "f32"}),            # one key in the last block; fp32 rows out
     (1, 1, 192, 320, 96, {}),                              # the variant's full width
     (1, 1, 128, 2048, 72, {}),                             # one query block over 32 key blocks: the keys are split over workgroups
+    (1, 8, 520, 1030, 72, {}),                             # 1024 keys or more, keys not split over workgroups: eight waves on the two
+    (3, 4, 300, 1153, 96, {"kv_len": [1153, 0, 1025], "out_dtype": "f32"}),   # halves of a 128-key stage, 96 wide; ragged last stage,
+    (1, 16, 2048, 1100, 80, {}),                           # per-batch lengths; a grid over more than half of the chip
 ])
 def test_flash_head_sizes_65_to_96(ctx, B, H, Lq, Lk, E, kw):
     """Head sizes in (64, 96] run the 96-wide instance of the fused kernel (six k-steps in the first product, three
     32-wide output tiles), not the 128-wide one."""
     q, k, v = _qkv(B, H, Lq, Lk, E, 61)
     _check(ctx, q, k, v, expect="FlashPlan", what=f"flash {B},{H},{Lq},{Lk},{E}", **kw)
+
+
+def test_wide_heads_key_halves_follow_growing_scores(ctx):
+    """The 96-wide key-halves form moves its reference point like the others: keys far above everything before them, in
+    the first and in the second half of a stage."""
+    q, k, v = _qkv(1, 8, 300, 1200, 72, 303)
+    q = (q.astype(np.float32) * 3.0).astype(np.float16)
+    k = k.copy()
+    k[:, :, 70:75] *= np.float16(4.0)
+    k[:, :, 150:152] *= np.float16(8.0)
+    k[:, :, 1100] *= np.float16(10.0)
+    got = _check(ctx, q, k, v, expect="FlashPlan", what="growing scores, 96-wide key halves")
+    assert np.all(np.isfinite(got))
 
 
 def test_flash_small_inputs_and_f32_out(ctx):
