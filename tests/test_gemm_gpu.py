@@ -342,6 +342,41 @@ def test_layer_norm_of_the_output_rides_in_the_gemm(ctx, T, K, F, layout):
         assert np.array_equal(to_host(out), to_host(out2)) and np.array_equal(to_host(normed), to_host(normed2))
 
 
+def test_in_launch_exchanges_on_two_streams_do_not_meet(ctx):
+    """Launches that overlap on one GPU take different banks of flag words: the same split-K problem issued alternately
+    on two streams, twelve times each without a synchronisation in between, gives the bits of a launch that ran alone."""
+    import torch
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    T, K, F = 1500, 5120, 1280
+    x = to_dev(oracle.randn_f16((T, K), 51, 0, 1.0 / np.sqrt(K)))
+    w = to_dev(oracle.randn_f16((K, F), 52))
+    b, r = to_dev(oracle.randn_f16((F,), 53, 0, 0.02)), to_dev(oracle.randn_f16((T, F), 54))
+    need = lib.mi_gemm_f16_workspace(T, K, F, L.W_KF, 1)
+    assert need > 0
+
+    def launch(y, ws, stream):
+        rc = lib.mi_gemm_f16(y.data_ptr(), x.data_ptr(), w.data_ptr(), b.data_ptr(), r.data_ptr(), T, K, F, F, K, F,
+                             L.W_KF, L.BIAS_COL, L.EPI["none"], L.F16, ws.data_ptr(), need, stream.cuda_stream)
+        assert rc == L.OK
+
+    alone = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+    ws0 = torch.empty(need, dtype=torch.uint8, device="cuda")
+    launch(alone, ws0, torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    wss = [torch.empty(need, dtype=torch.uint8, device="cuda") for _ in streams]      # a workspace belongs to one stream at a time
+    outs = [[poison(torch.empty((T, F), dtype=torch.float16, device="cuda")) for _ in range(12)] for _ in streams]
+    torch.cuda.synchronize()
+    for i in range(12):
+        for s, stream in enumerate(streams):
+            launch(outs[s][i], wss[s], stream)
+    torch.cuda.synchronize()
+    for s in range(2):
+        for y in outs[s]:
+            assert torch.equal(y.view(torch.int16), alone.view(torch.int16))
+
+
 @pytest.mark.parametrize("T,K,F", [(1500, 5120, 1280), (1370, 1536, 384)])
 def test_in_launch_exchange_starts_clean_on_every_replay(ctx, T, K, F):
     """A captured launch carries the flag bank and epoch it was given at capture.  The split-K exchange
