@@ -136,9 +136,12 @@ def test_conv_planner_and_extents():
     ws = lib.mi_conv2d_f16_workspace(64, 64, 1024, 1, 3, 3, 256, 1, 1, 1, 1, 1, 1)
     planes = ws - (2 * 1024 * 66 * 72 * 2 + 256 * 9216 * 2)
     assert planes >= 2 * 256 * 4096 * 4 and planes % (256 * 4096 * 4) == 0
-    # im2col scratch: col[CRS->8][PQ->8] fp16 (+ padded weights when CRS % 8 != 0)
+    # im2col scratch: col[CRS->64][PQ->8] fp16 + the weights padded likewise (588 taps: 640; under 256 taps the depth
+    # is rounded up to 8 only)
     ws3 = lib.mi_conv2d_f16_workspace(518, 518, 3, 1, 14, 14, 384, 14, 14, 0, 0, 1, 1)
-    assert ws3 == -(-(592 * 1376 * 2) // 256) * 256 + 384 * 592 * 2
+    assert ws3 == -(-(640 * 1376 * 2) // 256) * 256 + 384 * 640 * 2
+    ws4 = lib.mi_conv2d_f16_workspace(64, 64, 5, 1, 3, 3, 32, 1, 1, 1, 1, 1, 1)                # 45 taps -> 48
+    assert ws4 >= 48 * 4096 * 2 + 32 * 48 * 2 and ws4 < 56 * 4096 * 2 + 32 * 56 * 2 + (1 << 20)
     assert lib.mi_conv2d_f16_workspace(256, 256, 144, 1, 1, 1, 256, 1, 1, 0, 0, 1, 1) == 0
 
 
