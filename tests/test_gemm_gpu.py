@@ -313,11 +313,13 @@ def test_output_larger_than_2g_elements_is_indexed_in_64_bits(ctx, layout):
 
 @pytest.mark.parametrize("layout", ["kf", "fk"])
 @pytest.mark.parametrize("T,K,F", [(1370, 1536, 384), (200, 2048, 256), (1500, 5120, 1280), (200, 256, 328), (4, 1280, 1280), (77, 2048, 264),
-                                   (1370, 384, 384), (64, 128, 64), (130, 512, 1024), (1000, 256, 520), (2500, 128, 192), (65, 1536, 384)])
+                                   (1370, 384, 384), (64, 128, 64), (130, 512, 1024), (1000, 256, 520), (2500, 128, 192), (65, 1536, 384),
+                                   (9, 192, 8), (40, 2048, 376), (8190, 128, 384), (8200, 128, 384), (33, 2112, 384)])
 def test_layer_norm_of_the_output_rides_in_the_gemm(ctx, T, K, F, layout):
     """matmul_ln_ against the oracle's gemm -> layernorm, and bit for bit (both outputs) against matmul_ followed by
     layernorm_: split-K shapes (the norm is in the plane-summing pass), unsplit and decode-sized ones (two kernels; one
-    to sixteen column tiles a row panel, one and two chunks a lane in the norm, ragged last panels)."""
+    to sixteen column tiles a row panel, one and two chunks a lane in the norm, ragged last panels, rows of eight
+    columns, eight thousand rows of 384)."""
     import torch
     import juliavision_amd as jv
     X = oracle.randn_f16((T, K), 91, 0, 1.0 / np.sqrt(K))
