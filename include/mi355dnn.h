@@ -276,6 +276,27 @@ size_t mi_conv2d_nhwc_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t
                                     int64_t KW, int64_t KH, int64_t Cout,
                                     int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
                                     int64_t dil_x, int64_t dil_y);
+/* The convolution of mi_conv2d_f16 (groups = 1) with its output token-major: out[n][m][co], m = oh * OW + ow, one row
+ * of Cout values per output pixel at pitch ld_out, images out_image_stride elements apart -- what a ViT's
+ * flatten(2).transpose(1, 2) makes of the channel-major result -- plus, if given, residual[n][m][co] (fp16, the same
+ * pitch, images res_image_stride apart; 0 = one residual for every image, the position embedding), added to the
+ * rounded result with one more rounding, as an add after the convolution would.  ld_out and the strides are
+ * multiples of 8, out and residual 16-byte aligned.  The im2col matrix is written token-major and is the GEMM's
+ * row-major operand, the weights are its K-contiguous operand as they lie, the bias is per column: patch embedding
+ * + position embedding in three launches instead of convolution (three), transpose and add.
+ * The reference runs these as separate ops: convolution! (conv.jl:100-145), its permute, add (ops.jl); its fold
+ * passes merge neighbours of this kind into one kernel's epilogue (foldrelu.jl:60-125). */
+int mi_conv2d_tokens_f16(void *out, int64_t ld_out, int64_t out_image_stride,
+                         const void *x, const void *w, const void *bias, const void *residual, int64_t res_image_stride,
+                         int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                         int64_t KW, int64_t KH, int64_t Cout,
+                         int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                         int64_t dil_x, int64_t dil_y, int act,
+                         void *ws, size_t ws_bytes, void *stream);
+size_t mi_conv2d_tokens_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N,
+                                      int64_t KW, int64_t KH, int64_t Cout,
+                                      int64_t stride_x, int64_t stride_y, int64_t pad_x, int64_t pad_y,
+                                      int64_t dil_x, int64_t dil_y);
 /* ATen's output extent -- convsize, conv.jl:309. */
 int64_t mi_convsize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t d);
 

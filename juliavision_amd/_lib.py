@@ -52,6 +52,8 @@ SIGNATURES = {
     "mi_conv2d_f16_plan": (_int, [_i64] * 14),
     "mi_conv2d_nhwc_f16": (_int, [_vp] * 4 + [_i64] * 13 + [_int, _vp, _sz, _vp]),
     "mi_conv2d_nhwc_f16_workspace": (_sz, [_i64] * 13),
+    "mi_conv2d_tokens_f16": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i64] + [_i64] * 13 + [_int, _vp, _sz, _vp]),
+    "mi_conv2d_tokens_f16_workspace": (_sz, [_i64] * 13),
     "mi_convsize": (_i64, [_i64] * 5),
     "mi_convtranspose2d_f16": (_int, [_vp] * 4 + [_i64] * 16 + [_vp, _sz, _vp]),
     "mi_convtranspose2d_f16_workspace": (_sz, [_i64] * 16),

@@ -163,10 +163,10 @@ int mi_num_cus();
 // of 8 share an L2), as a probe launch at mi_init showed; kernels whose workgroups exchange data through one L2 ask.
 bool mi_xcd_round_robin();
 int mi_sdpa_init();
-// Y[M x N] = A[M x K] . B (+bias) with B either [K][NB-padded N] (b_kn) or [N][K]; defined in gemm.hip.
+// Y[M x N] = A[M x K] . B (+bias) (+ residual, fp16, addressed like Y) with B either [K][NB-padded N] (b_kn) or [N][K]; defined in gemm.hip.
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
                      long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st,
-                     const ConvGather *gather = nullptr, const NhwcGather *agather = nullptr);
+                     const ConvGather *gather = nullptr, const NhwcGather *agather = nullptr, const void *residual = nullptr);
 // Workspace bytes such a call needs (fp32 planes when it splits K); T > 8 rows.
 size_t mi_internal_gemm_workspace(int64_t T, int64_t K, int64_t F, int64_t nbatch);

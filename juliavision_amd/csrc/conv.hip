@@ -50,6 +50,32 @@ __global__ void im2col_kernel(half_t *col, ConvArgs a, int PQP, int CRSP) {
     *reinterpret_cast<half8v *>(col + (long)n * PQP * CRSP + (long)c * PQP + m0) = val;
 }
 
+// The same matrix token-major: col[n][m][c], c = (ci, kh, kw) fastest and zero from CRS to CRSP -- the row-major A
+// operand of a GEMM whose output rows are pixels.  A thread gathers eight consecutive c of one pixel (one 16-byte store).
+__global__ void im2col_rows_kernel(half_t *col, ConvArgs a, int CRSP) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int groups = CRSP >> 3;
+    const int PQ = a.OW * a.OH, CRS = a.Cin * a.KH * a.KW;
+    if (idx >= groups * PQ) return;
+    const int n = blockIdx.y;
+    const int c0 = (idx % groups) * 8, m = idx / groups;
+    const int ow = m % a.OW, oh = m / a.OW;
+    const int ix0 = ow * a.sx - a.px, iy0 = oh * a.sy - a.py;
+    int kw = c0 % a.KW, t = c0 / a.KW, kh = t % a.KH, ci = t / a.KH;
+    const half_t *xp = a.x + (long)n * a.Cin * a.Hi * a.Wi;
+    half8v val;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        val[j] = (half_t)0.0f;
+        if (c0 + j < CRS) {
+            const int ix = ix0 + kw * a.dx, iy = iy0 + kh * a.dy;
+            if (ix >= 0 && ix < a.Wi && iy >= 0 && iy < a.Hi) val[j] = xp[((long)ci * a.Hi + iy) * a.Wi + ix];
+        }
+        if (++kw == a.KW) { kw = 0; if (++kh == a.KH) { kh = 0; ci++; } }
+    }
+    *reinterpret_cast<half8v *>(col + ((long)n * PQ + m) * CRSP + c0) = val;
+}
+
 // xp[n][ci][Hp][Wp]: x with py rows of zeros above and below and px (and the round-up to a multiple
 // of 8) columns left and right; one 16-byte store per thread.  What the implicit-GEMM path reads.
 // The same launch re-lays the weights as w2[co][kh][kw][ci] (blocks past the padding work, image 0
@@ -282,6 +308,71 @@ int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
     if (hipGetLastError() != hipSuccess) return MI_ERROR_LAUNCH;
     return mi_internal_gemm(out, wuse, col, bias, a.Cout, PQ, (int)PQP, (int)CRSP, PQ, CRSP, PQP, 1, MI_BIAS_ROW, epi, 0,
                             a.N, (long)a.Cout * PQ, 0, PQP * CRSP, reinterpret_cast<char *>(ws) + col_bytes + wp_bytes, gemm_bytes, st);
+}
+
+// The convolution with its output token-major: out[n][m][co], m = (oh, ow), a row of Cout values per pixel at pitch
+// ld_out, images out_image_stride apart -- what a patch embedding's flatten + transpose makes of the channel-major
+// result -- and optionally + residual[n][m][co] (same pitch, images res_image_stride apart, 0 = one for all: the
+// position embedding).  out[m][co] = col[m][c] . w[co][c]^T: the im2col matrix written token-major is the row-major
+// operand, the weights are the K-contiguous one as they lie (padded to the matrix's depth), the bias is per column
+// and the residual joins in the GEMM's store with one more rounding, like an add after the convolution.
+size_t mi_conv2d_tokens_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, int64_t KW, int64_t KH, int64_t Cout,
+                                      int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy) {
+    ConvArgs a;
+    if (fill(a, nullptr, nullptr, nullptr, nullptr, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, 1, MI_EPI_NONE) != MI_OK) return 0;
+    int64_t PQP, CRSP;
+    im2col_extents(a, PQP, CRSP);
+    const int64_t PQ = (int64_t)a.OW * a.OH;
+    const size_t col = round_up((size_t)N * PQ * CRSP * 2, 256);
+    const size_t wp = CRSP != (int64_t)Cin * KH * KW ? round_up((size_t)Cout * CRSP * 2, 256) : 0;
+    return col + wp + mi_internal_gemm_workspace(PQ, CRSP, Cout, 1);
+}
+
+int mi_conv2d_tokens_f16(void *out, int64_t ld_out, int64_t out_image_stride,
+                         const void *x, const void *w, const void *bias, const void *residual, int64_t res_image_stride,
+                         int64_t Wi, int64_t Hi, int64_t Cin, int64_t N, int64_t KW, int64_t KH, int64_t Cout,
+                         int64_t sx, int64_t sy, int64_t px, int64_t py, int64_t dx, int64_t dy, int act,
+                         void *ws, size_t ws_bytes, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !x || !w) return MI_DECLINE_OPERANDS;
+    ConvArgs a;
+    int rc = fill(a, out, x, w, bias, Wi, Hi, Cin, N, KW, KH, Cout, sx, sy, px, py, dx, dy, 1, act);
+    if (rc != MI_OK) return rc;
+    if (N == 0) return MI_OK;
+    const int64_t PQ = (int64_t)a.OW * a.OH;
+    if (ld_out < Cout || (N > 1 && out_image_stride < PQ * ld_out) || res_image_stride < 0) return MI_DECLINE_EXTENT;
+    if (ld_out % 8 || out_image_stride % 8 || res_image_stride % 8 || !aligned_to(out, 16) || (residual && !aligned_to(residual, 16)))
+        return MI_DECLINE_OPERANDS;
+    hipStream_t st = (hipStream_t)stream;
+    int64_t PQP, CRSP;
+    im2col_extents(a, PQP, CRSP);
+    const int CRS = a.Cin * a.KH * a.KW;
+    const size_t col_bytes = round_up((size_t)N * PQ * CRSP * 2, 256);
+    const size_t wp_bytes = CRSP != CRS ? round_up((size_t)Cout * CRSP * 2, 256) : 0;
+    const size_t gemm_bytes = mi_internal_gemm_workspace(PQ, CRSP, Cout, 1);
+    if (!ws || ws_bytes < col_bytes + wp_bytes + gemm_bytes || !aligned_to(ws, 256)) return MI_DECLINE_WORKSPACE;
+    if (PQ * CRSP > INT32_MAX) return MI_DECLINE_EXTENT;
+    half_t *col = reinterpret_cast<half_t *>(ws);
+    const half_t *wuse = a.w;
+    hipLaunchKernelGGL(im2col_rows_kernel, dim3((unsigned)ceil_div(PQ * (CRSP / 8), 256), (unsigned)a.N), dim3(256), 0, st, col, a, (int)CRSP);
+    if (wp_bytes) {
+        half_t *wp = reinterpret_cast<half_t *>(reinterpret_cast<char *>(ws) + col_bytes);
+        hipLaunchKernelGGL(padweight_kernel, dim3((unsigned)ceil_div((int64_t)Cout * CRSP, 256)), dim3(256), 0, st, wp, a.w, a.Cout, CRS, (int)CRSP);
+        wuse = wp;
+    }
+    if (hipGetLastError() != hipSuccess) return MI_ERROR_LAUNCH;
+    const int epi = a.relu ? MI_EPI_RELU : MI_EPI_NONE;
+    void *gws = reinterpret_cast<char *>(ws) + col_bytes + wp_bytes;
+    // the residual is addressed like the output; images whose residuals lie at another distance go one launch each
+    const bool together = !residual || N == 1 || res_image_stride == out_image_stride;
+    for (int64_t n = 0; n < (together ? 1 : N); n++) {
+        half_t *yo = reinterpret_cast<half_t *>(out) + n * out_image_stride;
+        const half_t *ro = residual ? reinterpret_cast<const half_t *>(residual) + n * res_image_stride : nullptr;
+        rc = mi_internal_gemm(yo, col + n * PQ * CRSP, wuse, bias, (int)PQ, a.Cout, a.Cout, (int)CRSP, ld_out, CRSP, CRSP, 0, MI_BIAS_COL, epi, 0,
+                              together ? N : 1, out_image_stride, PQ * CRSP, 0, gws, gemm_bytes, st, nullptr, nullptr, ro);
+        if (rc != MI_OK) return rc;
+    }
+    return MI_OK;
 }
 
 // Channels-last convolution as an implicit GEMM with nothing staged: out[(n,oh,ow)][Cout] = patch[(n,oh,ow)][(kh,kw,ci)] .

@@ -2121,7 +2121,7 @@ size_t mi_internal_gemm_workspace(int64_t T, int64_t K, int64_t F, int64_t nbatc
 int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, int M, int N, int NB, int K,
                      long ldY, long ldA, long ldB, int b_kn, int bias_mode, int epi, int out_f32,
                      long nbatch, long sY, long sA, long sB, void *ws, size_t ws_bytes, hipStream_t st,
-                     const ConvGather *gather, const NhwcGather *agather) {
+                     const ConvGather *gather, const NhwcGather *agather, const void *residual) {
     GemmArgs a;
     a.cv = ConvGather{};
     a.ag = NhwcGather{};
@@ -2129,7 +2129,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
     a.clk = nullptr;
     a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
-    a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = nullptr;
+    a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = out_f32 ? nullptr : (const half_t *)residual;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
     a.tiles_m = a.tiles_n = a.group_m = 1; a.vec_store = 0;

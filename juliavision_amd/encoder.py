@@ -18,7 +18,7 @@ from typing import List, Optional
 
 import torch
 
-from .kernels import Ctx, add_, convolution_, convsize, layernorm_, ln_matmul_, ln_matmul_folds, ln_matmul_pays, matmul_, matmul_ln_, sdpa, transposeLE_
+from .kernels import Ctx, add_, convolution_tokens_, convsize, layernorm_, ln_matmul_, ln_matmul_folds, ln_matmul_pays, matmul_, matmul_ln_, sdpa
 
 
 @dataclass
@@ -112,7 +112,6 @@ class ViTEncoder:
         if tuple(W.pos.shape) != (self.T, d) or tuple(W.cls.shape) != (1, d):
             raise ValueError(f"pos must be ({self.T}, {d}) and cls (1, {d})")
         f16 = torch.float16
-        self.patches = torch.empty((1, d, self.gh, self.gw), dtype=f16, device=device)      # channel-major, as the convolution writes
         self.tokens = [torch.empty((self.T, d), dtype=f16, device=device) for _ in range(2)]
         self.out = torch.empty((self.T, d), dtype=f16, device=device)
         self.buf = EncoderBuffers(self.T, d, ffn, device)
@@ -121,10 +120,8 @@ class ViTEncoder:
         """``image``: (1, 3, H, W) fp16.  Fills and returns ``tokens[0]``."""
         W, tok = self.W, self.tokens[0]
         ctx.ws.reset()
-        convolution_(ctx, self.patches, image, W.patch_w, W.patch_b, (self.P, self.P), (0, 0), (1, 1), 1)
-        # channel-major (d, patches) -> token-major rows 1.. of the token matrix
-        transposeLE_(ctx, tok[1:], self.patches.view(W.patch_w.shape[0], self.T - 1))
-        add_(ctx, tok[1:], tok[1:], W.pos[1:])
+        # the convolution's GEMM writes token rows 1.. itself, position embedding joined in its store
+        convolution_tokens_(ctx, tok[1:].unsqueeze(0), image, W.patch_w, W.patch_b, (self.P, self.P), (0, 0), (1, 1), residual=W.pos[1:])
         add_(ctx, tok[:1], W.cls, W.pos[:1])
         return tok
 

@@ -580,6 +580,37 @@ def convolution_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, groups, *
     return out
 
 
+def convolution_tokens_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, *, residual=None, act="none"):
+    """The convolution with its output as tokens: ``x`` (N,Cin,H,W), ``w`` (Cout,Cin,KH,KW) contiguous fp16, ``out``
+    (N, OH*OW, Cout) with the last axis contiguous (a view into a token matrix will do) = ``convolution_``'s result
+    after ``flatten(2).transpose(1, 2)``, plus ``residual`` -- (OH*OW, Cout) for every image or (N, OH*OW, Cout), with
+    ``out``'s row pitch -- added with one more rounding (a position embedding).  ``mi_conv2d_tokens_f16``."""
+    if not _is_f16_cuda(x, w, out) or x.dim() != 4 or w.dim() != 4 or out.dim() != 3 or not (x.is_contiguous() and w.is_contiguous()):
+        raise DeclineError("convolution_tokens_: operands", L.DECLINE_OPERANDS)
+    lib = L.init()
+    N, Cin, Hi, Wi = x.shape
+    Cout, cin_w, KH, KW = w.shape
+    OW = convsize(Wi, KW, stride[0], padding[0], dilation[0])
+    OH = convsize(Hi, KH, stride[1], padding[1], dilation[1])
+    if cin_w != Cin or tuple(out.shape) != (N, OH * OW, Cout) or out.stride(2) != 1:
+        raise DeclineError("convolution_tokens_: out must be (N, OH*OW, Cout) with contiguous rows and w (Cout,Cin,KH,KW)", L.DECLINE_OPERANDS)
+    _check_vecs("convolution_tokens_", L.DECLINE_OPERANDS, ("bias", bias, Cout))
+    rs = 0
+    if residual is not None:
+        if not _is_f16_cuda(residual) or residual.dim() not in (2, 3) or tuple(residual.shape[-2:]) != (OH * OW, Cout) or \
+                residual.stride(-1) != 1 or residual.stride(-2) != out.stride(1) or (residual.dim() == 3 and residual.shape[0] != N):
+            raise DeclineError("convolution_tokens_: residual must be ([N,] OH*OW, Cout) fp16 with out's row pitch", L.DECLINE_OPERANDS)
+        rs = residual.stride(0) if residual.dim() == 3 and N > 1 else 0
+    args = (Wi, Hi, Cin, N, KW, KH, Cout, stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1])
+    need = lib.mi_conv2d_tokens_f16_workspace(*args)
+    ws = ctx.ws.scratch(need)
+    rc = lib.mi_conv2d_tokens_f16(out.data_ptr(), out.stride(1), out.stride(0) if N > 1 else 0, x.data_ptr(), w.data_ptr(), _ptr(bias),
+                                  _ptr(residual), rs, *args, L.EPI[act], ws, need, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_conv2d_tokens_f16", rc)
+    return out
+
+
 def convolution_nhwc_(ctx: Ctx, out, x, w, bias, stride, padding, dilation, *, act="none"):
     """The convolution over channels-last tensors: ``x`` (N,H,W,Cin), ``w`` (Cout,KH,KW,Cin), ``out`` (N,OH,OW,Cout), all
     contiguous fp16; pairs are ``(x, y)``.  An implicit GEMM with no staging pass (``mi_conv2d_nhwc_f16``); needs

@@ -64,6 +64,62 @@ def test_conv_1x1_and_relu_and_nobias(ctx):
     _conv(ctx, 1, 8, 20, 20, 16, 3, 3, 2, 2, d=2)
 
 
+@pytest.mark.parametrize("N,Cin,H,W,Cout,K,s,p,res,relu", [
+    (1, 3, 70, 70, 384, 14, 14, 0, "shared", False),      # a ViT-S/14 patch embedding on a 5 x 5 grid: 588 taps -> 640
+    (1, 3, 518, 518, 384, 14, 14, 0, "shared", False),    # config 3's, full size
+    (2, 3, 56, 56, 64, 8, 8, 0, "shared", False),         # one position embedding for two images
+    (2, 3, 56, 56, 64, 8, 8, 0, "each", True),            # a residual per image, relu before it
+    (3, 5, 20, 24, 40, 3, 1, 1, None, False),             # overlapping taps with padding, 45 -> 48 taps
+    (1, 16, 9, 9, 24, 4, 4, 0, "shared", False),          # a 2 x 2 grid: four tokens (the decode-sized GEMM inside)
+])
+def test_conv_writes_tokens_with_the_position_embedding(ctx, N, Cin, H, W, Cout, K, s, p, res, relu):
+    """mi_conv2d_tokens_f16 into rows 1.. of a token matrix (row 0 stays as it was), against the oracle's direct
+    convolution transposed to tokens and the residual added with a rounding of its own, and bit for bit against
+    convolution_ -> transposeLE_ -> add_."""
+    import torch
+    import juliavision_amd as jv
+    x = oracle.randn_f16((N, Cin, H, W), 41)
+    w = oracle.randn_f16((Cout, Cin, K, K), 42, 0, 0.05)
+    b = oracle.randn_f16((Cout,), 43, 0, 0.5)
+    conv = oracle.conv2d_f16(x, w, b, (s, s), (p, p), (1, 1), 1, relu)                 # (N, Cout, OH, OW)
+    PQ = conv.shape[2] * conv.shape[3]
+    want = np.ascontiguousarray(conv.reshape(N, Cout, PQ).transpose(0, 2, 1))
+    r = None
+    if res is not None:
+        r = oracle.randn_f16((N if res == "each" else 1, PQ, Cout), 44)
+        want = (want.astype(np.float32) + r.astype(np.float32)).astype(np.float16)
+    dx, dw, db = to_dev(x), to_dev(w), to_dev(b)
+    dr = None if r is None else (to_dev(r) if res == "each" else to_dev(r[0]))
+    tok = poison(torch.empty((N, 1 + PQ, Cout), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.convolution_tokens_(ctx, tok[:, 1:], dx, dw, db, (s, s), (p, p), (1, 1), residual=dr, act="relu" if relu else "none")
+    # the three separate ops
+    chan = poison(torch.empty((N, Cout, conv.shape[2], conv.shape[3]), dtype=torch.float16, device="cuda"))
+    tok2 = poison(torch.empty((N, PQ, Cout), dtype=torch.float16, device="cuda"))
+    ctx.ws.reset()
+    jv.convolution_(ctx, chan, dx, dw, db, (s, s), (p, p), (1, 1), 1, act="relu" if relu else "none")
+    jv.transposeLE_(ctx, tok2.unsqueeze(1), chan.view(N, 1, Cout, PQ))
+    if dr is not None:
+        for n in range(N):
+            jv.add_(ctx, tok2[n], tok2[n], dr[n] if res == "each" else dr)
+    torch.cuda.synchronize()
+    got = to_host(tok[:, 1:])
+    assert_parity(got, want, what=f"conv -> tokens {N},{Cin},{H},{W}->{Cout} k{K} s{s} p{p} res={res}")
+    if PQ > 8:            # four tokens run the decode-sized kernel, whose dot products sum in another order than the MFMA tiles
+        assert np.array_equal(got, to_host(tok2))
+    assert bool(torch.isnan(tok[:, 0]).all())                                         # row 0 of each image untouched
+
+
+def test_conv_tokens_declines_misaligned_rows(ctx):
+    import torch
+    import juliavision_amd as jv
+    from juliavision_amd import _lib as L
+    z = lambda *sh: torch.zeros(sh, dtype=torch.float16, device="cuda")
+    with pytest.raises(jv.DeclineError) as e:                                         # a row pitch of 36 halves
+        jv.convolution_tokens_(ctx, z(1, 16, 36)[:, :, :32], z(1, 3, 16, 16), z(32, 3, 4, 4), None, (4, 4), (0, 0), (1, 1))
+    assert e.value.status == L.DECLINE_OPERANDS
+
+
 def test_conv_grouped_direct(ctx):
     _conv(ctx, 1, 8, 10, 10, 16, 3, 3, 1, 1, groups=4, expect="direct", relu=True)
 
