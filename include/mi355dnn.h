@@ -283,7 +283,8 @@ size_t mi_conv2d_nhwc_f16_workspace(int64_t Wi, int64_t Hi, int64_t Cin, int64_t
  * rounded result with one more rounding, as an add after the convolution would.  ld_out and the strides are
  * multiples of 8, out and residual 16-byte aligned.  The im2col matrix is written token-major and is the GEMM's
  * row-major operand, the weights are its K-contiguous operand as they lie, the bias is per column: patch embedding
- * + position embedding in three launches instead of convolution (three), transpose and add.
+ * + position embedding in two launches (im2col with the weight padding in its last blocks, GEMM) instead of
+ * convolution, transpose and add.
  * The reference runs these as separate ops: convolution! (conv.jl:100-145), its permute, add (ops.jl); its fold
  * passes merge neighbours of this kind into one kernel's epilogue (foldrelu.jl:60-125). */
 int mi_conv2d_tokens_f16(void *out, int64_t ld_out, int64_t out_image_stride,

@@ -19,12 +19,25 @@ struct ConvArgs {
     int sx, sy, px, py, dx, dy, groups, relu;
 };
 
+// wp[co][CRSP] = w[co][CRS] zero-padded: the blocks of an im2col launch past its own work do this (image 0 only), so
+// that padding the weights to the matrix's depth is not a launch of its own.
+__device__ __forceinline__ void padweight_block(half_t *wp, const half_t *w, int Cout, int CRS, int CRSP, int block) {
+    const int idx = block * blockDim.x + threadIdx.x;
+    if (idx >= Cout * CRSP) return;
+    const int c = idx % CRSP, co = idx / CRSP;
+    wp[idx] = c < CRS ? w[(long)co * CRS + c] : (half_t)0.0f;
+}
+
 // col[c][m], m fastest: c = (ci, kh, kw) with kw fastest, m = (oh, ow) with ow
 // fastest (the order of im2col_kernel!, conv_coopmat.jl:259-286).  Rows c >= CRS
 // and columns m >= PQ are zero, as are taps that fall in the padding.  A thread
 // produces eight consecutive pixels of one row c (one 16-byte store), so the
 // index decomposition is paid once per eight elements; 32-bit arithmetic throughout.
-__global__ void im2col_kernel(half_t *col, ConvArgs a, int PQP, int CRSP) {
+__global__ void im2col_kernel(half_t *col, ConvArgs a, int PQP, int CRSP, half_t *wp, int col_blocks) {
+    if ((int)blockIdx.x >= col_blocks) {
+        if (blockIdx.y == 0) padweight_block(wp, a.w, a.Cout, a.Cin * a.KH * a.KW, CRSP, blockIdx.x - col_blocks);
+        return;
+    }
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     const int groups = PQP >> 3;
     if (idx >= groups * CRSP) return;
@@ -52,7 +65,11 @@ __global__ void im2col_kernel(half_t *col, ConvArgs a, int PQP, int CRSP) {
 
 // The same matrix token-major: col[n][m][c], c = (ci, kh, kw) fastest and zero from CRS to CRSP -- the row-major A
 // operand of a GEMM whose output rows are pixels.  A thread gathers eight consecutive c of one pixel (one 16-byte store).
-__global__ void im2col_rows_kernel(half_t *col, ConvArgs a, int CRSP) {
+__global__ void im2col_rows_kernel(half_t *col, ConvArgs a, int CRSP, half_t *wp, int col_blocks) {
+    if ((int)blockIdx.x >= col_blocks) {
+        if (blockIdx.y == 0) padweight_block(wp, a.w, a.Cout, a.Cin * a.KH * a.KW, CRSP, blockIdx.x - col_blocks);
+        return;
+    }
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     const int groups = CRSP >> 3;
     const int PQ = a.OW * a.OH, CRS = a.Cin * a.KH * a.KW;
@@ -121,14 +138,6 @@ __global__ void conv_pad_kernel(half_t *xp, half_t *w2, ConvArgs a, int Hp, int 
     const long at = (((long)n * a.Cin + ci) * Hp + yp) * Wp + c8;
     *reinterpret_cast<half8v *>(xp + at) = v0;
     *reinterpret_cast<half8v *>(xp + shifted + at) = v1;
-}
-
-// wp[co][CRSP] = w[co][CRS] zero-padded
-__global__ void padweight_kernel(half_t *wp, const half_t *w, int Cout, int CRS, int CRSP) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= Cout * CRSP) return;
-    const int c = idx % CRSP, co = idx / CRSP;
-    wp[idx] = c < CRS ? w[(long)co * CRS + c] : (half_t)0.0f;
 }
 
 // One thread per output; fp32 accumulator seeded with the bias; the loop order
@@ -299,12 +308,10 @@ int mi_conv2d_f16(void *out, const void *x, const void *w, const void *bias,
     if (PQP * CRSP > INT32_MAX) return MI_DECLINE_EXTENT;
     half_t *col = reinterpret_cast<half_t *>(ws);
     const half_t *wuse = a.w;
-    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)ceil_div(PQP / 8 * CRSP, 256), (unsigned)a.N), dim3(256), 0, st, col, a, (int)PQP, (int)CRSP);
-    if (wp_bytes) {
-        half_t *wp = reinterpret_cast<half_t *>(reinterpret_cast<char *>(ws) + col_bytes);
-        hipLaunchKernelGGL(padweight_kernel, dim3((unsigned)ceil_div((int64_t)Cout * CRSP, 256)), dim3(256), 0, st, wp, a.w, a.Cout, CRS, (int)CRSP);
-        wuse = wp;
-    }
+    half_t *wp = wp_bytes ? reinterpret_cast<half_t *>(reinterpret_cast<char *>(ws) + col_bytes) : nullptr;
+    const int col_blocks = (int)ceil_div(PQP / 8 * CRSP, 256), w_blocks = wp ? (int)ceil_div((int64_t)Cout * CRSP, 256) : 0;
+    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)(col_blocks + w_blocks), (unsigned)a.N), dim3(256), 0, st, col, a, (int)PQP, (int)CRSP, wp, col_blocks);
+    if (wp) wuse = wp;
     if (hipGetLastError() != hipSuccess) return MI_ERROR_LAUNCH;
     return mi_internal_gemm(out, wuse, col, bias, a.Cout, PQ, (int)PQP, (int)CRSP, PQ, CRSP, PQP, 1, MI_BIAS_ROW, epi, 0,
                             a.N, (long)a.Cout * PQ, 0, PQP * CRSP, reinterpret_cast<char *>(ws) + col_bytes + wp_bytes, gemm_bytes, st);
@@ -354,12 +361,10 @@ int mi_conv2d_tokens_f16(void *out, int64_t ld_out, int64_t out_image_stride,
     if (PQ * CRSP > INT32_MAX) return MI_DECLINE_EXTENT;
     half_t *col = reinterpret_cast<half_t *>(ws);
     const half_t *wuse = a.w;
-    hipLaunchKernelGGL(im2col_rows_kernel, dim3((unsigned)ceil_div(PQ * (CRSP / 8), 256), (unsigned)a.N), dim3(256), 0, st, col, a, (int)CRSP);
-    if (wp_bytes) {
-        half_t *wp = reinterpret_cast<half_t *>(reinterpret_cast<char *>(ws) + col_bytes);
-        hipLaunchKernelGGL(padweight_kernel, dim3((unsigned)ceil_div((int64_t)Cout * CRSP, 256)), dim3(256), 0, st, wp, a.w, a.Cout, CRS, (int)CRSP);
-        wuse = wp;
-    }
+    half_t *wp = wp_bytes ? reinterpret_cast<half_t *>(reinterpret_cast<char *>(ws) + col_bytes) : nullptr;
+    const int col_blocks = (int)ceil_div(PQ * (CRSP / 8), 256), w_blocks = wp ? (int)ceil_div((int64_t)Cout * CRSP, 256) : 0;
+    hipLaunchKernelGGL(im2col_rows_kernel, dim3((unsigned)(col_blocks + w_blocks), (unsigned)a.N), dim3(256), 0, st, col, a, (int)CRSP, wp, col_blocks);
+    if (wp) wuse = wp;
     if (hipGetLastError() != hipSuccess) return MI_ERROR_LAUNCH;
     const int epi = a.relu ? MI_EPI_RELU : MI_EPI_NONE;
     void *gws = reinterpret_cast<char *>(ws) + col_bytes + wp_bytes;
