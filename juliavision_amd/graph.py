@@ -811,6 +811,66 @@ def fold_embedding_sum(g: Graph) -> Graph:
     return g
 
 
+def fold_patch_tokens(g: Graph) -> Graph:
+    """``cat(cls.expand(B, -1, -1), conv(img).flatten(2).transpose(1, 2), dim=1) + pos`` -- a ViT's patch embedding -- is
+    one op: the convolution's GEMM writes token rows 1.. itself with the position embedding as its residual
+    (``mi_conv2d_tokens_f16``), row 0 is ``cls + pos[0]``.  No channel-major result, no transposing copy, no add."""
+    for cat in [o for o in g.ops if o["aten"] == "cat.default" and len(o["in"]) == 2]:
+        sh = g.buffers[cat["out"]].get("shape") or []
+        if len(sh) != 3 or cat["attrs"].get("arg1", 0) % 3 != 1 or sh[1] < 2:
+            continue
+        B, T, C = sh
+        first, second = cat["in"]
+        # the class token: a weight of C values shown as (B, 1, C) through reshapes and an expand
+        cls, x, plain = g.root(first), first, True
+        while g.buffers[x]["kind"] == "view":
+            plain = plain and g.buffers[x]["op"] in RESHAPES + ("expand.default",)
+            x = g.buffers[x]["of"]
+        cb = g.buffers[cls]
+        if not plain or cb["kind"] != "weight" or math.prod(cb["shape"]) != C or list(g.buffers[first].get("shape", [])) != [B, 1, C]:
+            continue
+        # the patches: the last two axes of a (B, C, P) reshape of an ordinary convolution's (B, C, gh, gw) result, swapped
+        v = g.buffers[second]
+        if v["kind"] != "view" or list(v.get("shape", [])) != [B, T - 1, C]:
+            continue
+        va = v.get("attrs", {})
+        if v["op"] == "permute.default":
+            swapped = list(va.get("arg1", [])) == [0, 2, 1]
+        else:
+            swapped = v["op"] == "transpose.int" and {va.get("arg1", 0) % 3, va.get("arg2", 0) % 3} == {1, 2}
+        x = v["of"]
+        while swapped and g.buffers[x]["kind"] == "view":
+            w = g.buffers[x]
+            if w["op"] not in RESHAPES + ("flatten.using_ints",) or list(w.get("shape", [])) != [B, C, T - 1]:
+                swapped = False
+            x = w["of"]
+        conv = g.op(x) if swapped else None
+        if conv is None or conv["aten"] != "convolution.default" or conv["attrs"].get("arg6") or conv["attrs"].get("arg8", 1) != 1 \
+                or len(conv["attrs"].get("arg3", [])) != 2 or len(conv["in"]) not in (2, 3):
+            continue
+        csh = g.buffers[conv["out"]].get("shape") or []
+        if len(csh) != 4 or csh[0] != B or csh[1] != C or csh[2] * csh[3] != T - 1:
+            continue
+        users = _consumers(g, cat["out"])
+        if _consumers(g, conv["out"]) != {cat["id"]} or len(users) != 1:
+            continue
+        add = g.op(next(iter(users)))
+        if add is None or add["aten"] != "add.Tensor" or len(add["in"]) != 2 or add["attrs"].get("alpha", 1) != 1 or cat["out"] not in add["in"]:
+            continue
+        other = add["in"][1] if add["in"][0] == cat["out"] else add["in"][0]
+        pos = g.root(other)
+        pb = g.buffers[pos]
+        if pb["kind"] != "weight" or math.prod(pb["shape"]) != T * C or list(pb["shape"][-2:]) != [T, C] or \
+                list(g.buffers[other].get("shape", [])[-2:]) != [T, C]:
+            continue
+        at = g.ops.index(add)
+        g.ops[at] = {"id": add["id"], "aten": "patch_tokens", "in": list(conv["in"]) + [cls, pos], "out": add["out"],
+                     "attrs": dict(conv["attrs"], has_bias=len(conv["in"]) == 3)}
+        g.ops = [o for o in g.ops if o["id"] not in (conv["id"], cat["id"])]
+        g.notes.append(f"fold {conv['id']} -> tokens, {cat['id']} and {add['id']} into one patch embedding")
+    return g
+
+
 CACHE_WRITES = ("index_copy.default", "index_put.default")
 MASK_VIEWS = RESHAPES + ("expand.default", "unsqueeze.default")
 
@@ -1012,7 +1072,7 @@ def prune(g: Graph) -> Graph:
 
 
 def optimize(g: Graph) -> Graph:
-    g = fold_cache_step(fold_embedding_sum(g))
+    g = fold_patch_tokens(fold_cache_step(fold_embedding_sum(g)))
     return group_linears(fold_sdpa_transpose(fold_attention(fold_layernorms(fold_layernorm_prologues(
         fold_clamps(fold_residuals(fold_layerscale(fold_activations(g)))))))))
 
@@ -1352,6 +1412,23 @@ class Executor:
         else:
             K.convolution_(self.ctx, out, x, w, bias, xy(stride), xy(padding), xy(dilation), a.get("arg8", 1), act=a.get("epilogue", "none"))
 
+    def _patch_tokens(self, o):
+        """The folded patch embedding: convolution -> token rows 1.. with the position embedding joined in the GEMM's
+        store, and the class row ``cls + pos[0]`` of every image."""
+        a, ins = o["attrs"], o["in"]
+        nb = 3 if a["has_bias"] else 2
+        x, w = self.get(ins[0]), self.get(ins[1])
+        bias = self.get(ins[2]) if a["has_bias"] else None
+        out = self.t[o["out"]]
+        B, T, C = out.shape
+        cls, pos = self.get(ins[nb]).view(1, C), self.get(ins[nb + 1]).view(T, C)
+        xy = lambda p: tuple(list(p)[::-1])
+        self.ctx.ws.reset()
+        K.convolution_tokens_(self.ctx, out[:, 1:], x, w, bias, xy(a["arg3"]), xy(a["arg4"]), xy(a["arg5"]), residual=pos[1:],
+                              act=a.get("epilogue", "none"))
+        for b in range(B):
+            K.add_(self.ctx, out[b, :1], cls, pos[:1])
+
     def _embedding(self, o):
         """embedding(table, ids) / index.Tensor(table, [ids]) along the first axis (ops.jl:1754-1783, 1524-1640); with
         four operands the sum of two gathers ``fold_embedding_sum`` made."""
@@ -1391,7 +1468,7 @@ class Executor:
                 "bmm.default": _bmm, "cat.default": _cat, **dict.fromkeys(SOFTMAX_OPS, _softmax),
                 "mul.Tensor": _scale, "div.Tensor": _scale, "clone.default": _clone, "clamp.default": _clamp,
                 "linear_group": _linear_group, "embedding.default": _embedding, "index.Tensor": _embedding,
-                "kv_len_from_position": _kv_len, "sdpa_append": _sdpa_append}
+                "kv_len_from_position": _kv_len, "sdpa_append": _sdpa_append, "patch_tokens": _patch_tokens}
 
     def replayable(self, *inputs: torch.Tensor):
         """Run once eagerly (binds inputs, sizes the workspace, stacks folded constants), then capture the whole graph as

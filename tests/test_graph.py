@@ -475,9 +475,10 @@ def test_dinov2_like_encoder_folds_to_five_calls_per_block():
     assert aten.count("bmm.default") == 4 and aten.count("_softmax.default") == 2 and aten.count("cat.default") == 1
     g = G.optimize(G.Graph.load(d))
     left = [o["aten"] for o in g.ops]
-    # convolution, cat, + position embedding, first norm; per block: qkv, attention, projection, fc1, fc2 -- the
-    # other norms ride in the GEMM that writes their input, LayerScale in the weights, residuals in the stores
-    assert left == ["convolution.default", "cat.default", "add.Tensor", "native_layer_norm.default"] + \
+    # the patch embedding (convolution written as tokens, class row, position embedding: one op), first norm; per
+    # block: qkv, attention, projection, fc1, fc2 -- the other norms ride in the GEMM that writes their input,
+    # LayerScale in the weights, residuals in the stores
+    assert left == ["patch_tokens", "native_layer_norm.default"] + \
         ["addmm.default", "scaled_dot_product_attention.default", "addmm.default", "addmm.default", "addmm.default"] * 2, (left, g.notes)
     assert sum("colscale" in o["attrs"] for o in g.ops) == 4 and sum("residual" in o["attrs"] for o in g.ops) == 4
     assert sum("ln_out" in o["attrs"] for o in g.ops) == 4
@@ -510,19 +511,43 @@ def test_division_by_a_weight_vector_is_not_folded_as_layerscale():
             assert not folded and "div.Tensor" in left, (mode, left, g.notes)
 
 
+def test_patch_embedding_whose_feature_map_is_also_a_result_is_not_folded():
+    """The fold drops the channel-major convolution result; a graph that returns it keeps the three ops."""
+    import torch
+    import torch.nn as nn
+    from juliavision_amd import graph as G
+
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.pe, self.cls, self.pos = nn.Conv2d(3, 32, 8, 8), nn.Parameter(torch.zeros(1, 1, 32)), nn.Parameter(torch.zeros(1, 10, 32))
+
+        def forward(self, img):
+            f = self.pe(img)
+            x = f.flatten(2).transpose(1, 2)
+            return torch.cat((self.cls.expand(x.shape[0], -1, -1), x), dim=1) + self.pos, f
+
+    ep = torch.export.export(M().eval().half(), (torch.randn(1, 3, 24, 24).half(),)).run_decompositions()
+    g = G.optimize(G.Graph.load(G.convert(ep, "pe")))
+    assert [o["aten"] for o in g.ops] == ["convolution.default", "cat.default", "add.Tensor"], g.notes
+
+
 @pytest.mark.gpu
-def test_dinov2_like_encoder_runs_on_the_kernels(ctx):
+@pytest.mark.parametrize("B", [1, 2])
+def test_dinov2_like_encoder_runs_on_the_kernels(ctx, B):
     import torch
     from juliavision_amd import graph as G
     m = _dinov2_like(seed=5)
-    x = torch.rand(1, 3, 70, 70).half()
+    x = torch.rand(B, 3, 70, 70).half()
     ep = torch.export.export(m, (x,)).run_decompositions()
-    run = G.Executor(G.optimize(G.Graph.load(G.convert(ep, "vit"))), m.state_dict(), ctx)
+    g = G.optimize(G.Graph.load(G.convert(ep, "vit")))
+    assert g.ops[0]["aten"] == "patch_tokens"
+    run = G.Executor(g, m.state_dict(), ctx)
     with torch.no_grad():
         want = m.float()(x.float()).numpy()
     got = run(x.cuda())
     torch.cuda.synchronize()
-    assert got.shape == (1, 26, 128)
+    assert got.shape == (B, 26, 128)
     assert_parity(got.float().cpu().numpy(), want, what="DINOv2-like encoder from its exported graph")
 
 
