@@ -13,13 +13,13 @@ Shapes follow torch order as in the reference's ``KVCache`` (decode.jl:52-58):
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import Callable, List, Optional
 
 import torch
 
 from . import _lib as L
-from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, matmul_heads_, sdpa, sdpa_append
+from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, matmul_heads_, sdpa, sdpa_append, transposeLE_
 
 
 # Fold the cache write into the self-attention launch where the one-launch kernel covers the shape.
@@ -105,6 +105,23 @@ class DecoderLayerWeights:
     b1: torch.Tensor
     w2: torch.Tensor
     b2: torch.Tensor
+
+    LINEARS = ("wqkv", "wo", "wq_c", "wo_c", "w1", "w2")
+
+    def k_contiguous(self, ctx: Ctx) -> "DecoderLayerWeights":
+        """The same layer with every linear weight held as ``[F][K]`` memory (a transposed ``(K, F)`` view): what the
+        decode-sized kernels stream fastest -- one launch per linear instead of K-slices plus a sum.  Done once at load
+        with the layout kernel; weights that already lie that way are kept as they are."""
+        out = {}
+        for name in self.LINEARS:
+            w = getattr(self, name)
+            if w.stride(0) == 1:                           # already [F][K]
+                out[name] = w
+                continue
+            fk = torch.empty((w.shape[1], w.shape[0]), dtype=w.dtype, device=w.device)
+            transposeLE_(ctx, fk, w)
+            out[name] = fk.t()
+        return replace(self, **out)
 
 
 class DecodeBuffers:

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import oracle
-from util import assert_parity, to_dev, to_host
+from util import assert_parity, poison, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
 
@@ -129,6 +129,33 @@ def test_decoder_layer_steps_match_oracle(ctx, B, layout):
         assert to_host(cache.length).tolist() == length.tolist()
         # the cache rows written on the device are the oracle's rows (fp16 outputs of the same GEMV, within rounding)
         assert_parity(to_host(cache.self_k[0]), hk, what=f"self_k after step {step}")
+
+
+def test_weights_relaid_at_load_run_the_one_launch_linears(ctx):
+    """DecoderLayerWeights.k_contiguous: [K][F] weights re-laid once to [F][K] hold the same values, and a layer step
+    over them gives the bits of a step over weights that were [F][K] from the start."""
+    import torch
+    from juliavision_amd.decode import DecodeBuffers, KVCache, decoder_layer_step
+    B, d, H, E, ffn = 2, 256, 4, 64, 512
+    _, Wkf = _weights(d, ffn, 100, "kf")
+    _, Wfk = _weights(d, ffn, 100, "fk")
+    Wre = Wkf.k_contiguous(ctx)
+    torch.cuda.synchronize()
+    for name in Wkf.LINEARS:
+        a, b = getattr(Wre, name), getattr(Wkf, name)
+        assert a.stride(0) == 1 and a.shape == b.shape and bool((a == b).all()), name
+        assert getattr(Wfk.k_contiguous(ctx), name) is getattr(Wfk, name)          # nothing to do: kept
+    outs = []
+    for W in (Wre, Wfk):
+        cache = KVCache(1, B, H, E, max_target=16, src_len=40)
+        cache.cross_k.copy_(to_dev(oracle.randn_f16((1, B, H, 40, E), 31)))
+        cache.cross_v.copy_(to_dev(oracle.randn_f16((1, B, H, 40, E), 32)))
+        buf, out = DecodeBuffers(B, d, ffn), poison(torch.empty((B, d), dtype=torch.float16, device="cuda"))
+        cache.advance(ctx)
+        decoder_layer_step(ctx, W, cache, 0, to_dev(oracle.randn_f16((B, d), 60)), out, buf)
+        torch.cuda.synchronize()
+        outs.append(to_host(out))
+    assert np.isfinite(outs[0]).all() and np.array_equal(outs[0], outs[1])
 
 
 def test_step_graph_replays_match_eager(ctx):
