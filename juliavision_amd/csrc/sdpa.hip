@@ -871,6 +871,227 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void flash_short_kernel(S
     }
 }
 
+// The short-chain form on 64-query tiles, for grids whose 32-query tiles would be a few more than the CUs (6 heads x
+// 1370: 258) and for the traffic: in flash_short_kernel every 32-query tile reads all of its head's K and V from the L2,
+// and with 43 tiles a head that read is what the loop waits for.  Here eight waves share a tile: wave w takes key
+// quarter w % 4 for query half w / 4, and the two waves of a quarter share its K and V through LDS -- one of them fetches
+// the K block, the other the V block, a block ahead, 8 chunks of 16 bytes a lane -- so a tile of twice the queries reads
+// the same bytes.  K lies in LDS row-major with 16 bytes of padding (conflict-free 16-byte fragment reads), V as in
+// flash_short_kernel.  One buffer per quarter: a workgroup barrier after the writes of block j, another before the
+// writes of block j + 1; every wave takes part in every barrier (quarters with fewer blocks idle through the rest).
+__global__ __launch_bounds__(512, 1) void flash_pair_kernel(SdpaArgs p) {
+    constexpr int EP = 64, KS = 4, ET = 2, BC = 64, NQ = 4, VLD = flash_vld(64), KLD = EP + 8;
+    constexpr int KBYTES = BC * KLD * 2, VBYTES = BC * VLD * 2, QREG = KBYTES + VBYTES;      // a quarter's K and V
+    constexpr int WPART = (ET * 16 + 2) * 64 * 4;                                            // a wave's (O, m, l)
+    static_assert(8 * WPART <= NQ * QREG, "the partials fit where the stages were");
+    extern __shared__ __align__(16) char smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int kq = wave & 3, qh = wave >> 2;
+    const int hl = lane >> 5, l32 = lane & 31;
+    half_t *Kw = reinterpret_cast<half_t *>(smem + kq * QREG);
+    half_t *Vw = reinterpret_cast<half_t *>(smem + kq * QREG + KBYTES);
+    int qblk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    {
+        const int nqb = gridDim.x, total = nqb * gridDim.y * gridDim.z;
+        if ((total & 7) == 0) {
+            int id = blockIdx.x + nqb * (blockIdx.y + gridDim.y * blockIdx.z);
+            id = (id & 7) * (total >> 3) + (id >> 3);
+            qblk = id % nqb;
+            h = (id / nqb) % gridDim.y;
+            b = id / (nqb * gridDim.y);
+        }
+    }
+    const int q0 = qblk * 64 + 32 * qh;
+    const half_t *qb = p.q + h * p.qs[2] + b * p.qs[3];
+    const half_t *kb = p.k + h * p.ks[2] + b * p.ks[3];
+    const half_t *vb = p.v + h * p.vs[2] + b * p.vs[3];
+    int Lk = p.Lk;
+    if (p.kv_len) Lk = max(0, min(Lk, p.kv_len[b]));
+    const int per = (((Lk + BC - 1) / BC + NQ - 1) / NQ) * BC;
+    const int nmax = per / BC;                                // barriers are counted over this, by every wave
+    const int kbeg = kq * per, kend = min(Lk, kbeg + per);
+    const int nblk = kend > kbeg ? (kend - kbeg + BC - 1) / BC : 0;
+    const int last = p.Lk - 1;
+    const float c = p.scale * LOG2E;
+
+    u32x4 qraw[KS];
+    {
+        const int qr = min(q0 + l32, p.Lq - 1);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) qraw[ks] = ldg16(qb + (long)qr * p.qs[1] + 16 * ks + 8 * hl);
+    }
+    // this wave's share of a block: the K rows (query half 0) or the V rows (query half 1), chunk lane + 64 i = (key, 8 head dims)
+    const half_t *src = qh == 0 ? kb : vb;
+    const long srow = qh == 0 ? p.ks[1] : p.vs[1];
+    half_t *dst = qh == 0 ? Kw : Vw;
+    const int dld = qh == 0 ? KLD : VLD;
+    u32x4 pre[8];
+    auto fetch = [&](int key0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int cidx = lane + 64 * i;
+            pre[i] = ldg16(src + (long)min(key0 + (cidx >> 3), last) * srow + (cidx & 7) * 8);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int cidx = lane + 64 * i;
+            *reinterpret_cast<u32x4 *>(dst + (cidx >> 3) * dld + (cidx & 7) * 8) = pre[i];
+        }
+    };
+    if (nblk > 0) fetch(kbeg);
+    half8v qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        const half8v t = as_half8(qraw[ks]);
+#pragma unroll
+        for (int j = 0; j < 8; j++) qf[ks][j] = (half_t)((float)t[j] * c);
+    }
+    float16v o_acc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o_acc[t][r] = 0.0f;
+    float m_run = 0.0f, l_run = 0.0f;
+    const int ktoff = l32 * KLD + 8 * hl;
+    const int vtoff = (4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    constexpr float TH = 8.0f;
+    half8v kext, qext;
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) { kext[jj] = (half_t)0.0f; qext[jj] = (half_t)0.0f; }
+    if (hl == 0) kext[0] = (half_t)1.0f;
+    bool first = true;
+    auto probs = [&](const float16v (&sx)[2], half8v (&pf)[2][2], float &l) {
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(sx[kt][r]), p1 = __builtin_amdgcn_exp2f(sx[kt][r + 1]);
+                pf[kt][r >> 3][r & 7] = (half_t)p0;
+                pf[kt][r >> 3][(r & 7) + 1] = (half_t)p1;
+                l += p0 + p1;
+            }
+    };
+    for (int j = 0; j < nmax; j++) {
+        const bool live = j < nblk;                          // uniform over the wave, and the same for both waves of a quarter
+        const int key0 = kbeg + j * BC;
+        if (j > 0) __syncthreads();                          // block j - 1 has been read by everyone
+        if (live) stage();
+        if (j + 1 < nblk) fetch(key0 + BC);
+        __syncthreads();                                     // block j is in place
+        if (!live) continue;
+        float16v sc[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+            const half_t *kp_ = Kw + ktoff + 32 * kt * KLD;
+            sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], zero16, 0, 0, 0);
+#pragma unroll
+            for (int ks = 1; ks < KS; ks++)
+                sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_ + 16 * ks), qf[ks], sc[kt], 0, 0, 0);
+            sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, sc[kt], 0, 0, 0);
+        }
+        if (key0 + BC > kend) {
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (key0 + 32 * kt + 8 * (r >> 2) + 4 * hl + (r & 3) >= kend) sc[kt][r] = -INFINITY;
+        }
+        half8v pf[2][2];
+        float l_new = l_run;
+        probs(sc, pf, l_new);
+        if (__any(first || !(l_new - l_run < 65504.0f))) {
+            float tmax = fmaxf(sc[0][0], sc[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; r++) tmax = fmaxf(fmaxf(tmax, sc[0][r]), sc[1][r]);
+            const float mx = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const bool grow = (mx > TH || first) && mx != -INFINITY;
+            const half_t m16 = (half_t)(m_run + (grow ? mx : 0.0f));
+            const float d = (float)m16 - m_run;
+            const float alpha = __builtin_amdgcn_exp2f(-d);
+            m_run += d;
+            l_run *= alpha;
+            if (hl == 0) qext[0] = -m16;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) sc[kt][r] -= d;
+#pragma unroll
+            for (int t = 0; t < ET; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o_acc[t][r] *= alpha;
+            l_new = l_run;
+            probs(sc, pf, l_new);
+        }
+        l_run = l_new;
+        first = false;
+#pragma unroll
+        for (int t = 0; t < ET; t++) {
+            const half_t *vp = Vw + vtoff + 32 * t;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int bb = 0; bb < 2; bb++) {
+                    const half_t *vq = vp + (32 * kt + 16 * bb) * VLD;
+                    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(vq));
+                    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(vq + 8 * VLD));
+                    short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    o_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, both), pf[kt][bb], o_acc[t], 0, 0, 0);
+                }
+        }
+    }
+    l_run += __shfl_xor(l_run, 32, 64);
+    __syncthreads();                                         // the last blocks have been read: the stages become the partials
+    float *xo = reinterpret_cast<float *>(smem + wave * WPART);
+#pragma unroll
+    for (int t = 0; t < ET; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) xo[(t * 16 + r) * 64 + lane] = o_acc[t][r];
+    xo[(ET * 16) * 64 + lane] = m_run;
+    xo[(ET * 16 + 1) * 64 + lane] = l_run;
+    __syncthreads();
+    // the four quarters of this wave's query half meet; wave kq finishes (t, g) pairs 2 kq and 2 kq + 1 of its 32 queries
+    float aw[NQ], mm = -INFINITY, den = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NQ; w++) {
+        const float *xw = reinterpret_cast<const float *>(smem + (qh * NQ + w) * WPART);
+        aw[w] = xw[(ET * 16 + 1) * 64 + lane] > 0.0f ? xw[(ET * 16) * 64 + lane] : -INFINITY;
+        mm = fmaxf(mm, aw[w]);
+    }
+#pragma unroll
+    for (int w = 0; w < NQ; w++) {
+        const float *xw = reinterpret_cast<const float *>(smem + (qh * NQ + w) * WPART);
+        aw[w] = aw[w] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(aw[w] - mm);
+        den += aw[w] * xw[(ET * 16 + 1) * 64 + lane];
+    }
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    const int qi = q0 + l32;
+#pragma unroll
+    for (int cidx = 0; cidx < 2; cidx++) {
+        const int tg = kq * 2 + cidx, t = tg >> 2, g = tg & 3;
+        float o4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int w = 0; w < NQ; w++) {
+            const float *xw = reinterpret_cast<const float *>(smem + (qh * NQ + w) * WPART);
+#pragma unroll
+            for (int i = 0; i < 4; i++) o4[i] += aw[w] * xw[(t * 16 + 4 * g + i) * 64 + lane];
+        }
+        if (qi < p.Lq) {
+            const long off = (long)b * p.os[3] + (long)h * p.os[2] + (long)qi * p.os[1] + 32 * t + 8 * g + 4 * hl;
+            if (p.out_f32) {
+                const float4v o = {o4[0] * inv, o4[1] * inv, o4[2] * inv, o4[3] * inv};
+                *reinterpret_cast<float4v *>(reinterpret_cast<float *>(p.out) + off) = o;
+            } else {
+                const half4v o = {(half_t)(o4[0] * inv), (half_t)(o4[1] * inv), (half_t)(o4[2] * inv), (half_t)(o4[3] * inv)};
+                *reinterpret_cast<half4v *>(reinterpret_cast<half_t *>(p.out) + off) = o;
+            }
+        }
+    }
+}
+
+
 // ------------------------------------------------------------------------------------------
 // One workgroup (4 waves) per (query row, key split).  A wave walks keys 8 at a
 // time: 8 lanes share a key, each owning 8-element head-dim chunks c, c+8, ...
@@ -1280,6 +1501,7 @@ __global__ void sdpa_merge_kernel(SdpaArgs p) {
 // ------------------------------------------------------------------------------------------
 constexpr int flash_lds_bytes(int EP) { return 3 * 64 * (EP + 8) * 2 + 3 * 64 * flash_vld(EP) * 2; }
 constexpr int flash_short_lds_bytes(int NW) { return NW * 64 * flash_vld(64) * 2; }
+constexpr int flash_pair_lds_bytes() { return 4 * (64 * (64 + 8) * 2 + 64 * flash_vld(64) * 2); }
 
 bool vec_addressable(const half_t *ptr, const long st[4], int E) {
     return st[0] == 1 && E % 8 == 0 && st[1] % 8 == 0 && st[2] % 8 == 0 && st[3] % 8 == 0 && aligned_to(ptr, 16);
@@ -1352,6 +1574,21 @@ bool flash_short(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     const int64_t blocks = ceil_div(Lk, 64), ns = flash_splits(E, Lq, Lk, H, B);
     return ns == 1 || 4.5 + 1.3 * (double)ceil_div(blocks, 4) <= 9.0 + 1.0 * (double)ceil_div(blocks, ns);
 }
+
+// The same on 64-query tiles (flash_pair_kernel) where the 32-query tiles would not all find a CU of their own but the
+// 64-query tiles do.  Replayed, against what ran there before (key halves on 128-query tiles, or 32-query tiles two to a
+// CU): 6 heads x 1370 17.8 -> 14.3 us, 16 x 1024 15.8 -> 11.3, 10 x 1500 26.5 -> 14.8, 8 x 2048 31.1 -> 19.6, 6 x 2500
+// 34.5 -> 21.1, 4 x 4096 44.1 -> 30.0; where the 32-query tiles fit they are faster (6 x 1344 11.7 against 13.4 us), and
+// at 12 x 1370 (264 tiles of 64) the key-halves form is (19.4 against 26.5 us).
+bool flash_pair(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    const int64_t tiles32 = ceil_div(Lq, 32) * H * B, tiles64 = ceil_div(Lq, 64) * H * B, cus = mi_num_cus();
+#ifdef MI_LAB
+    if (const char *f = getenv("MI_FORCE_PAIR")) return E == 64 && atoi(f) > 0;
+#endif
+    return E == 64 && Lk >= 128 && tiles32 > cus && tiles64 <= cus;
+}
+// either of the two: one launch, keys not split over workgroups
+bool flash_unsplit(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) { return flash_pair(E, Lq, Lk, H, B) || flash_short(E, Lq, Lk, H, B); }
 
 // A single query row (a decode step) runs in one launch of sdpa_decode_kernel: the work follows the device-side kv_len
 // and the cache write can ride along (mi_sdpa_append_f16).  Twenty heads alone leave most of the chip idle and give each
@@ -1475,6 +1712,7 @@ int mi_sdpa_init() {
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, true, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_short_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_short_lds_bytes(4)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, flash_pair_lds_bytes()) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64)) != hipSuccess;
@@ -1491,7 +1729,7 @@ extern "C" {
 size_t mi_sdpa_f16_workspace(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, int has_bias) {
     // sized for the path the call will most likely take: the fused kernel's key splits for Lq >= 64 without
     // an additive mask (unused if the operands turn out not to be 16-byte addressable), the rows kernel's below
-    int ns = Lq >= 64 ? ((has_bias || flash_short(E, Lq, Lk, H, B)) ? 1 : flash_splits(E, Lq, Lk, H, B)) : rows_splits(Lq, Lk, H, B);
+    int ns = Lq >= 64 ? ((has_bias || flash_unsplit(E, Lq, Lk, H, B)) ? 1 : flash_splits(E, Lq, Lk, H, B)) : rows_splits(Lq, Lk, H, B);
     if (ns <= 1) return 0;
     size_t rows = (size_t)Lq * H * B;
     return round_up((size_t)ns * rows * E * sizeof(float), 256) + round_up((size_t)ns * rows * 2 * sizeof(float), 256);
@@ -1511,7 +1749,7 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
     int path = sdpa_path(a);
     const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
     if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? (one_pass_decode(a, vec) ? decode_splits(E, Lk, H, B) : rows_splits(Lq, Lk, H, B))
-                                  : (path == MI_SDPA_FLASH && !has_bias && !flash_short(E, Lq, Lk, H, B)) ? flash_splits(E, Lq, Lk, H, B) : 1;
+                                  : (path == MI_SDPA_FLASH && !has_bias && !flash_unsplit(E, Lq, Lk, H, B)) ? flash_splits(E, Lq, Lk, H, B) : 1;
     return path;
 }
 
@@ -1550,6 +1788,10 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
         } else if (pp) {
             dim3 grid((unsigned)ceil_div(Lq, 256), (unsigned)H, (unsigned)B);
             hipLaunchKernelGGL((flash_fwd_kernel<64, true>), grid, dim3(512), flash_lds_bytes(64), st, a);
+        } else if (flash_pair(E, Lq, Lk, H, B)) {
+            a.nsplit = 1;
+            dim3 grid((unsigned)ceil_div(Lq, 64), (unsigned)H, (unsigned)B);
+            hipLaunchKernelGGL(flash_pair_kernel, grid, dim3(512), flash_pair_lds_bytes(), st, a);
         } else if (flash_short(E, Lq, Lk, H, B)) {
             a.nsplit = 1;
             dim3 grid((unsigned)ceil_div(Lq, 32), (unsigned)H, (unsigned)B);

@@ -311,12 +311,12 @@ def test_fused_kernel_splits_keys_on_small_grids(ctx):
 
 
 @pytest.mark.parametrize("Lk", [256, 257, 319, 320, 321, 383, 384, 385, 447, 448, 449, 1000])
-@pytest.mark.parametrize("B,H,Lq,E", [(12, 12, 64, 64), (5, 12, 130, 64), (2, 3, 200, 32)])
+@pytest.mark.parametrize("B,H,Lq,E", [(5, 20, 256, 64), (4, 20, 300, 64), (2, 3, 200, 32)])
 def test_fused_kernel_key_halves_on_one_workgroup_per_cu_grids(ctx, B, H, Lq, Lk, E):
-    """Grids of at most one 128-query workgroup per CU with 256 keys or more (and, at head size 64, more 32-query tiles
-    than the short-chain form takes: 288 and 300 here) run eight waves, each pair of waves sharing its queries and taking
-    alternate 64-key halves of a 128-key stage; the halves merge in LDS.  Key counts around the 64- and 128-key
-    boundaries: the second half's last block empty, ragged, exactly full."""
+    """Grids of at most one 128-query workgroup per CU with 256 keys or more (and, at head size 64, more 64-query tiles
+    than CUs: 400 and 400 here) run eight waves, each pair of waves sharing its queries and taking alternate 64-key
+    halves of a 128-key stage; the halves merge in LDS.  Key counts around the 64- and 128-key boundaries: the second
+    half's last block empty, ragged, exactly full."""
     q, k, v = _qkv(B, H, Lq, Lk, E, 211 + Lk)
     _check(ctx, q, k, v, expect="FlashPlan", what=f"key halves B{B} H{H} Lq{Lq} Lk{Lk} E{E}")
 
@@ -332,9 +332,21 @@ def test_short_chain_form_on_small_grids(ctx, B, H, Lq, Lk):
     _check(ctx, q, k, v, expect="FlashPlan", what=f"short chain B{B} H{H} Lq{Lq} Lk{Lk}")
 
 
-@pytest.mark.parametrize("H,HP", [(2, 6), (10, 32)])
+@pytest.mark.parametrize("Lk", [128, 129, 191, 192, 193, 255, 256, 257, 300, 511, 512, 513, 769, 1000, 1370])
+@pytest.mark.parametrize("B,H,Lq", [(12, 12, 64), (5, 12, 130), (1, 6, 1370), (3, 40, 65)])
+def test_pair_form_where_64_query_tiles_fit_the_cus(ctx, B, H, Lq, Lk):
+    """Head size 64, more 32-query tiles than CUs, at most one 64-query tile per CU: eight waves per tile, wave w on key
+    quarter w % 4 for query half w / 4, the two waves of a quarter sharing its K and V through LDS.  Key counts around
+    the boundaries of a quarter's share (quarters without a key, with a ragged block, with exactly full ones); tiles
+    whose second query half is ragged (130, 1370) or a single query (65)."""
+    q, k, v = _qkv(B, H, Lq, Lk, 64, 511 + Lk)
+    _check(ctx, q, k, v, expect="FlashPlan", what=f"pair form B{B} H{H} Lq{Lq} Lk{Lk}")
+
+
+@pytest.mark.parametrize("H,HP", [(2, 6), (10, 32), (20, 64)])
 def test_fused_kernel_key_halves_masks_and_layouts(ctx, H, HP):
-    """H = 2, HP = 6: the short-chain form (60 and 54 tiles); H = 10, HP = 32: the key-halves form (300 and 288)."""
+    """H = 2, HP = 6: the short-chain form (60 and 54 tiles of 32 queries); H = 10, HP = 32: the pair form (300 and 288
+    tiles of 32, 180 and 160 of 64); H = 20, HP = 64: the key-halves form (360 and 320 tiles of 64, 240 and 192 of 128)."""
     import torch
     import juliavision_amd as jv
     q, k, v = _qkv(6, H, 150, 300, 64, 251)
