@@ -958,10 +958,8 @@ __global__ __launch_bounds__(512, 1) void flash_pair_kernel(SdpaArgs p) {
     const int vtoff = (4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
     const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     constexpr float TH = 8.0f;
-    half8v kext, qext;
-#pragma unroll
-    for (int jj = 0; jj < 8; jj++) { kext[jj] = (half_t)0.0f; qext[jj] = (half_t)0.0f; }
-    if (hl == 0) kext[0] = (half_t)1.0f;
+    // the reference point is the first product's accumulator input: every score of a lane belongs to its one query
+    float16v negm = zero16;
     bool first = true;
     auto probs = [&](const float16v (&sx)[2], half8v (&pf)[2][2], float &l) {
 #pragma unroll
@@ -986,11 +984,10 @@ __global__ __launch_bounds__(512, 1) void flash_pair_kernel(SdpaArgs p) {
 #pragma unroll
         for (int kt = 0; kt < 2; kt++) {
             const half_t *kp_ = Kw + ktoff + 32 * kt * KLD;
-            sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], zero16, 0, 0, 0);
+            sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_), qf[0], negm, 0, 0, 0);
 #pragma unroll
             for (int ks = 1; ks < KS; ks++)
                 sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_ + 16 * ks), qf[ks], sc[kt], 0, 0, 0);
-            sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, sc[kt], 0, 0, 0);
         }
         if (key0 + BC > kend) {
 #pragma unroll
@@ -1013,7 +1010,8 @@ __global__ __launch_bounds__(512, 1) void flash_pair_kernel(SdpaArgs p) {
             const float alpha = __builtin_amdgcn_exp2f(-d);
             m_run += d;
             l_run *= alpha;
-            if (hl == 0) qext[0] = -m16;
+#pragma unroll
+            for (int r = 0; r < 16; r++) negm[r] = -(float)m16;
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
