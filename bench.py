@@ -842,6 +842,10 @@ def detail_benchmarks(lib, L, stream, only=None):
     gemm_case("c3_fc1_1370x384x1536", 1370, 384, 1536, L.W_KF, epi="gelu")
     gemm_case("c3_fc2_1370x1536x384", 1370, 1536, 384, L.W_KF)
     attn_case("c3_attn_L1370_6x64", 1, 6, 1370, 1370, 64)
+    # other grids of more 32-query tiles than CUs and at most one 64-query tile per CU (ViT-B/16 at 1024 tokens, a half-width
+    # Whisper encoder): the 64-query form whose key quarters share K and V through LDS, like config 3's
+    attn_case("vit_attn_L1024_16x64", 1, 16, 1024, 1024, 64)
+    attn_case("attn_L1500_10x64", 1, 10, 1500, 1500, 64)
     attn_case("c2_attn_L1500_20x64", 1, 20, 1500, 1500, 64)
     # the same attention with an additive mask: it stays in the fused kernel (the reference's fused plan declines masks)
     attn_case("c2_attn_L1500_20x64_padding_mask", 1, 20, 1500, 1500, 64, mask="pad")
