@@ -78,6 +78,31 @@ int mi_device_caps(int64_t out[6]);
  * launch ran at.  The caller keeps the buffer alive while it is registered.  Process-wide, not thread safe. */
 int mi_set_clock_probe(void *dev_u64x4);
 
+/* Device-side failures (no counterpart in the reference, whose kernels never wait for one another).  A few kernels
+ * here exchange data between workgroups inside one launch and wait for each other a bounded time; a wait that gives
+ * up cannot be reported by the call that enqueued the launch, so it is recorded in a sticky word in device memory.
+ * mi_device_status SYNCHRONISES the current device (the one exception to "calls never synchronise") and returns the
+ * OR of enum mi_device_status_bits raised since the last reset, or -1 if the device cannot be read.  With reset != 0
+ * it also clears the word and zeroes the exchange's flag banks (a workgroup that gave up has not released them): do
+ * that before reusing the device after a nonzero status, and re-run the affected work -- its outputs hold NaN where
+ * a workgroup gave up. */
+enum mi_device_status_bits {
+    MI_DEVSTAT_EXCHANGE_TIMEOUT = 1,  /* split-K exchange of mi_gemm_f16: a partner workgroup did not arrive in time   */
+    MI_DEVSTAT_EXCHANGE_XCD = 2,      /* split-K exchange: partner workgroups did not share an XCD (one L2)            */
+    MI_DEVSTAT_STEP_BARRIER = 4       /* mi_decoder_layer_step_f16: a workgroup gave up at a barrier between phases    */
+};
+int mi_device_status(int reset);
+/* Process-wide switch for the in-launch split-K exchange of mi_gemm_f16 and its variants (on by default where the
+ * device passed the XCD probe at mi_init).  Off: split K goes through fp32 planes in ws and a summing launch; plans
+ * and workspace sizes follow the switch, so query workspaces after setting it. */
+int mi_set_in_launch_exchange(int enabled);
+/* Test aid: makes the exchange's bounded waits fail from the host side, so that the failure path can be exercised
+ * with every kernel still exiting normally.  spin_limit: polls before a wave gives up (<= 0 restores the default);
+ * publish_xor: XORed into the epoch a wave publishes (nonzero: no partner ever sees the epoch it waits for);
+ * xcc_xor: XORed into the XCD id a wave expects of its partners (nonzero: every partner looks misplaced).
+ * (0, 0, 0) restores ordinary operation.  Process-wide, not thread safe. */
+int mi_test_exchange_faults(int spin_limit, unsigned publish_xor, unsigned xcc_xor);
+
 /* ---------------------------------------------------------------- GEMM
  * Y[T x F] = epi(round(X[T x K] . W + bias)) (+ residual)
  *   X   fp16 [T][K], ldX.
@@ -92,8 +117,15 @@ int mi_set_clock_probe(void *dev_u64x4);
  * Replaces matmul!(ctx, out, A, B, bias; epi) -- matmul.jl:78-79,99-100,133-137,235-273.
  * Concurrency: a launch that splits K inside the kernel (the workgroups of a tile exchange partial tiles through
  * arrival flags) takes the next of 16 banks of flag words held in static device memory, and leaves its bank zeroed.
- * Up to 16 such launches may overlap on one GPU (different streams); a captured launch keeps the bank it was given at
- * capture, so two captured graphs that hold the same bank must not be replayed at the same time. */
+ * Such a launch assumes that all its workgroups become resident together, which holds on an otherwise idle GPU (the
+ * grid is at most one workgroup per compute unit) and is NOT guaranteed while kernels of other streams occupy
+ * compute units: a workgroup waits for its partners a bounded time only, and if the bound is reached -- or a partner
+ * turns out to run on another XCD -- it stores NaN over its part of Y and raises the sticky status word that
+ * mi_device_status reads; the call itself has long returned MI_OK.  A caller that overlaps streams should either
+ * check mi_device_status at its synchronisation points or switch the exchange off (mi_set_in_launch_exchange(0):
+ * K-slices then go through fp32 planes in ws and a second launch, as on a device that fails the XCD probe).
+ * Up to 16 such launches may be in flight on one GPU; a captured launch keeps the bank it was given at capture, so
+ * two captured graphs that hold the same bank must not be replayed at the same time. */
 int mi_gemm_f16(void *Y, const void *X, const void *W, const void *bias, const void *residual,
                 int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
                 int w_layout, int bias_mode, int epi, int out_dtype,
@@ -190,6 +222,15 @@ int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,
                      int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
                      int w_layout, int out_dtype, int64_t nbatch, int64_t sY, int64_t sX, int64_t sW);
 
+/* mi_gemm_f16_plan for a device the caller describes: caps are the six values of mi_device_caps (NULL: the current
+ * device), of which the planner reads [0] (matrix unit present; without it the tiled MFMA path is not offered) and
+ * [5] (compute units, which decide tiles and K-splits).  ksplit_out (optional) receives the number of K-slices the
+ * plan would use.  The reference's planners take a DeviceCaps value for the same purpose: tests ask about hardware
+ * they do not have (DNNKernels/test/test_flash.jl:328,363,373-377; context.jl:68).  Never launches, needs no GPU. */
+int mi_gemm_f16_plan_caps(const int64_t caps[6], const void *Y, const void *X, const void *W,
+                          int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                          int w_layout, int out_dtype, int64_t nbatch, int64_t sY, int64_t sX, int64_t sW, int *ksplit_out);
+
 /* ---------------------------------------------------------------- attention
  * out(E,Lq,H,B) = softmax_over_keys(scale * q.k + bias) . v
  *   q (E,Lq,H,B), k (E,Lk,H,B), v (E,Lk,H,B): fp16, each given as a base pointer
@@ -227,6 +268,15 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4],
                      int has_bias, int has_kv_len,
                      int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale,
                      int *nsplit_out);
+
+/* mi_sdpa_f16_plan for a device the caller describes (see mi_gemm_f16_plan_caps): without a matrix unit the fused
+ * kernel is not offered, and the compute-unit count decides the key splits (splitcount(dev, ...), flash.jl:1288-1303). */
+int mi_sdpa_f16_plan_caps(const int64_t caps[6], const void *q, const int64_t q_strides[4],
+                          const void *k, const int64_t k_strides[4],
+                          const void *v, const int64_t v_strides[4],
+                          int has_bias, int has_kv_len,
+                          int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale,
+                          int *nsplit_out);
 
 /* ---------------------------------------------------------------- convolution
  * Reference layout: x (W,H,Cin,N) = row-major [N][Cin][H][W]; w (KW,KH,Cin,Cout) =
@@ -341,6 +391,14 @@ int64_t mi_convtransposesize(int64_t n, int64_t k, int64_t s, int64_t p, int64_t
  * mi_gemm_f16 takes ragged T, K, F as they are. */
 int mi_transpose_le_f16(void *out, const int64_t out_strides[4], const void *in, const int64_t in_strides[4],
                         int64_t E, int64_t L, int64_t H, int64_t B, void *stream);
+
+/* w_fk[F][K] (pitch ld_fk) = transpose of w_kf[K][F] (pitch ld_kf): a weight in the reference's hoisted layout
+ * (hoistpermutes, DNNKernels/src/hoistcasts.jl:47-112) re-laid K-contiguous, to be done ONCE where the model uploads
+ * its weights (Model, DNNKernels/src/driver.jl:165-168) and passed from then on with w_layout = MI_W_FK.  Values
+ * are unchanged, so every product is bit-identical to the one over the original; what changes is the route: decode-
+ * sized linears (T <= 8) run as one launch without a workspace instead of K-slices plus a summing launch, and the
+ * tiled GEMM reads both operands K-contiguous.  One launch of the transpose kernel of mi_transpose_le_f16. */
+int mi_relayout_weight_f16(void *w_fk, int64_t ld_fk, const void *w_kf, int64_t ld_kf, int64_t K, int64_t F, void *stream);
 
 /* ---------------------------------------------------------------- layer norm + glue
  * `groups` rows of C contiguous fp16 elements; mean in fp32, variance about that

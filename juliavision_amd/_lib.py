@@ -34,6 +34,9 @@ SIGNATURES = {
     "mi_init": (_int, []),
     "mi_device_caps": (_int, [_i64p]),
     "mi_set_clock_probe": (_int, [_vp]),
+    "mi_device_status": (_int, [_int]),
+    "mi_set_in_launch_exchange": (_int, [_int]),
+    "mi_test_exchange_faults": (_int, [_int, C.c_uint, C.c_uint]),
     "mi_gemm_f16": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
     "mi_gemm_f16_batched": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_i64] * 5 + [_vp, _sz, _vp]),
     "mi_gemv_f16": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp, _sz, _vp]),
@@ -44,6 +47,8 @@ SIGNATURES = {
     "mi_gemm_f16_workspace": (_sz, [_i64, _i64, _i64, _int, _i64]),
     "mi_gemm_f16_noalloc": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp]),
     "mi_gemm_f16_plan": (_int, [_vp] * 3 + [_i64] * 6 + [_int] * 2 + [_i64] * 4),
+    "mi_gemm_f16_plan_caps": (_int, [_i64p] + [_vp] * 3 + [_i64] * 6 + [_int] * 2 + [_i64] * 4 + [C.POINTER(C.c_int)]),
+    "mi_sdpa_f16_plan_caps": (_int, [_i64p, _vp, _i64p, _vp, _i64p, _vp, _i64p, _int, _int] + [_i64] * 5 + [_f32, C.POINTER(C.c_int)]),
     "mi_sdpa_f16": (_int, [_vp, _int, _i64p, _vp, _i64p, _vp, _i64p, _vp, _i64p, _vp, _int, _i64p, _vp] + [_i64] * 5 + [_f32, _vp, _sz, _vp]),
     "mi_sdpa_f16_workspace": (_sz, [_i64] * 5 + [_int]),
     "mi_sdpa_f16_plan": (_int, [_vp, _i64p, _vp, _i64p, _vp, _i64p, _int, _int] + [_i64] * 5 + [_f32, C.POINTER(C.c_int)]),
@@ -60,6 +65,7 @@ SIGNATURES = {
     "mi_convtranspose2d_f16_plan": (_int, [_i64] * 16),
     "mi_convtransposesize": (_i64, [_i64] * 6),
     "mi_transpose_le_f16": (_int, [_vp, _i64p, _vp, _i64p, _i64, _i64, _i64, _i64, _vp]),
+    "mi_relayout_weight_f16": (_int, [_vp, _i64, _vp, _i64, _i64, _i64, _vp]),
     "mi_layernorm_f16": (_int, [_vp] * 6 + [_i64, _i64, _f32, _vp]),
     "mi_softmax_f16": (_int, [_vp, _vp, _int, _i64, _i64, _f32, _vp]),
     "mi_scale_f16": (_int, [_vp, _vp, _f32, _i64, _vp]),

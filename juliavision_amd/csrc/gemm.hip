@@ -7,8 +7,8 @@
 //   A is K-contiguous.  B is either N-contiguous [K][N] (B_KN) or K-contiguous
 //   [N][K].  For a linear layer M = tokens, N = features, A = X, B = W.
 #include "common.hpp"
+#include "sk_exchange.hpp"
 #include <type_traits>
-#include <cstdlib>
 #include <atomic>
 
 // Arrival flags of the split-K peer reduction (gemm_pp_kernel, SK): SK_BANKS banks of SK_FLAGS words, and as many
@@ -18,6 +18,10 @@
 // whose epoch and bank are fixed at capture -- starts every replay from clean flags.
 constexpr int SK_BANKS = 16, SK_FLAGS = 4096, SK_WORDS = SK_BANKS * SK_FLAGS;
 static __device__ unsigned sk_flag_words[2 * SK_WORDS];
+
+// Sticky device status word (mi_device_status): kernels OR a bit of enum mi_device_status_bits into word 0 when a
+// bounded wait inside a launch gave up; nothing on the device ever clears it.
+static __device__ unsigned device_status_words[4];
 
 // Static device scratch of the allocation-free entry point (see mi_gemm_f16_noalloc).
 static __device__ __align__(256) unsigned char scratch[MI_NOALLOC_SCRATCH_BYTES];
@@ -59,6 +63,9 @@ struct GemmArgs {
     float *sk_part;
     unsigned *sk_flags;
     unsigned sk_epoch;
+    int sk_spin;                      // polls before a wave gives up on its partners
+    unsigned sk_pub_xor, sk_xcc_xor;  // zero in ordinary use: mi_test_exchange_faults makes the waits fail from the host side
+    unsigned *status;                 // the device's sticky status word
 };
 
 // ------------------------------------------------------------------------------------------
@@ -694,8 +701,33 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
 // others into its partners' slots of sk_part (plain stores: they stay in the shared L2), waits for them to be
 // acknowledged, and raises its flag; it then waits (bounded) for the same wave of every partner, adds what they sent
 // in slice order (the result does not depend on which workgroup sums), and stores its share through the usual
-// epilogue.  Every workgroup publishes before it waits, and the grid fits the device in one round (the launcher
-// checks), so the waits cannot be circular.
+// epilogue.  Every workgroup publishes before it waits, so the waits are not circular among resident workgroups; the
+// launcher only checks that the grid fits an IDLE device in one round.  Under overlap (another stream's kernel holding
+// CUs) a partner may not be resident yet: the wait is bounded, and a wave that runs into the bound -- or finds its
+// partner on another XCD -- raises the device's sticky status word (mi_device_status), stores NaN over its share of Y
+// and releases nothing (sk_exchange.hpp has the protocol; tests/sk_exchange_host_test.cpp runs it on CPU threads).
+struct SkDeviceMem {
+    __device__ static unsigned load(const unsigned *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    __device__ static void store(unsigned *p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    __device__ static unsigned fetch_add(unsigned *p, unsigned v) { return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    __device__ static void pause() { __builtin_amdgcn_s_sleep(1); }
+};
+using SkExchange = sk::Exchange<SkDeviceMem>;
+
+// A wave whose exchange failed marks its share of the output instead of storing a plausible sum: NaN in the output
+// type over rows [r0, r0 + 32) x columns [c0, c0 + ncols) of the tile.
+// (Scalars by value: a reference to the kernel's argument block would force the block into private memory.)
+__device__ __noinline__ void sk_poison_region(void *Y, long ldY, int M, int N, int out_f32, int r0, int c0, int ncols, int lane) {
+    for (int e = lane; e < 32 * ncols; e += 64) {
+        const int m = r0 + e / ncols, n = c0 + e % ncols;
+        if (m < M && n < N) {
+            const long off = (long)m * ldY + n;
+            if (out_f32) reinterpret_cast<unsigned *>(Y)[off] = 0x7fc00000u;
+            else reinterpret_cast<unsigned short *>(Y)[off] = (unsigned short)0x7e00u;
+        }
+    }
+}
+
 template <int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool B_KN, bool PINGPONG, bool SK = false>
 __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
     static_assert(WAVES_M * WAVES_N == 8, "two groups of four waves");
@@ -853,21 +885,13 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         if (t < nk) issue(t, t);
     wait_next(-1);                // tile 0
     barrier();
-#ifdef MI_LAB_TS
-    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[0] = clock64(); }
-#endif
     if (grp == 1) barrier();
     half4v cb[TN][4];
     int stage = 0;
     for (int kt = 0; kt < nk; kt++) {
         // memory phase
-#ifdef ABL_NOREAD
-        if (kt == 0)
-#endif
         fread(stage);
-#ifndef ABL_NOLOAD
         if (kt + STAGES - 1 < nk) issue(kt + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
-#endif
         if (kt + 1 == nk) load_col_bias<TN, WTN>(p, cb, n0, wn, lane, bz);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (grp == 1) wait_next(kt);
@@ -882,9 +906,6 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         if (!(PINGPONG && grp == 1 && kt + 1 == nk)) barrier();
         stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
-#ifdef MI_LAB_TS
-    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[1] = clock64(); }
-#endif
     if constexpr (SK) {
         // A wave's accumulators are NQ = TM * TN sub-tiles of 32 x 32, q = i * TM + j; sub-tile q goes to slice q % S.
         constexpr int NQ = TM * TN;
@@ -905,11 +926,9 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         });
         // the partials must have reached L2 before the flag can be seen
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const unsigned my_xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u;      // HW_REG_XCC_ID, bits 3:0
         unsigned *myflag = p.sk_flags + ((long)sk_tile * S + sk_s) * 8 + wave;
-        if (lane == 0) __hip_atomic_store(myflag, p.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#ifdef MI_LAB_TS
-        if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[4] = clock64(); }
-#endif
+        if (lane == 0) SkExchange::publish(myflag, p.sk_epoch ^ p.sk_pub_xor, my_xcc);
         // the sub-tiles this wave keeps (slot 0, and slot 1 when it keeps two)
         float16v own[2];
         static_for<NQ>([&](auto Q) {
@@ -920,29 +939,34 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         });
         // Wait (bounded) for the same wave of every partner, then fetch everything they sent in one trip: at most three
         // blocks of sixteen registers (three partners' one sub-tile, or one partner's one or two).  The three polls of a
-        // round are in flight together: a poll is a trip past the L1.
-        {
-            const unsigned *f[3];
-#pragma unroll
-            for (int bi = 0; bi < 3; bi++) {
-                const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;
-                f[bi] = p.sk_flags + ((long)sk_tile * S + src) * 8 + wave;
-            }
-            for (int spins = 0; spins < (1 << 18); spins++) {
-                const unsigned u0 = __hip_atomic_load(f[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const unsigned u1 = __hip_atomic_load(f[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const unsigned u2 = __hip_atomic_load(f[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (u0 == p.sk_epoch && u1 == p.sk_epoch && u2 == p.sk_epoch) break;
-                __builtin_amdgcn_s_sleep(1);
-            }
-        }
-        asm volatile("" ::: "memory");
-        // Ordinary loads: this CU has not touched these lines since the kernel began (its L1 was invalidated then), so
-        // they come from the L2 the partners' acknowledged stores are in.
-        float4v blk[3][4];
+        // round are in flight together: a poll is a trip past the L1.  Co-residency of the partners is NOT guaranteed
+        // (another stream's kernel can hold an XCD's CUs): the bound is the guard, and a wave that runs into it says so.
+        unsigned *fl[3];
 #pragma unroll
         for (int bi = 0; bi < 3; bi++) {
             const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;      // S = 4: the bi-th partner in slice order
+            fl[bi] = p.sk_flags + ((long)sk_tile * S + src) * 8 + wave;
+        }
+        const unsigned *const cfl[3] = {fl[0], fl[1], fl[2]};
+        const sk::WaitResult wr = SkExchange::wait(cfl, S == 4 ? 3 : 1, p.sk_epoch, my_xcc ^ p.sk_xcc_xor, p.sk_spin);
+        asm volatile("" ::: "memory");
+        if (wr != sk::ARRIVED) {
+            // Loud failure: the sticky status word, NaN over this wave's share of Y, flags left as they are (the host
+            // zeroes the banks when it reads the status).  The wave still leaves the kernel normally.
+            if (lane == 0) __hip_atomic_fetch_or(p.status, wr == sk::TIMED_OUT ? (unsigned)MI_DEVSTAT_EXCHANGE_TIMEOUT : (unsigned)MI_DEVSTAT_EXCHANGE_XCD,
+                                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // (the exchange runs unbatched launches only: bz = 0)
+            if (NSL == 1) sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * (sk_s % TM), n0 + wn * WTN + 32 * (sk_s / TM), 32, lane);
+            else sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * sk_s, n0 + wn * WTN, WTN, lane);
+            if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
+            return;
+        }
+        // Ordinary loads: this CU has not touched these lines since the kernel began (its L1 was invalidated then), so
+        // they come from the L2 the partners' acknowledged stores are in (the wait has checked that it is this XCD's).
+        float4v blk[3][4];
+#pragma unroll
+        for (int bi = 0; bi < 3; bi++) {
+            const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;
             if (S == 4 || bi < NSL) {
                 const float *from = part_of(sk_s, src) + (S == 4 ? 0 : bi * 1024);
 #pragma unroll
@@ -968,22 +992,9 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
         // in -- so the next launch on this bank, which for a replayed graph carries this same epoch, starts from zero.
         if (lane == 0) {
 #pragma unroll
-            for (int bi = 0; bi < 3; bi++) {
-                if (S == 4 || bi == 0) {
-                    const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;
-                    unsigned *f = p.sk_flags + ((long)sk_tile * S + src) * 8 + wave;
-                    bool last = true;
-                    if (S == 4) {
-                        last = __hip_atomic_fetch_add(f + SK_WORDS, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 2u;
-                        if (last) __hip_atomic_store(f + SK_WORDS, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-                    if (last) __hip_atomic_store(f, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-            }
+            for (int bi = 0; bi < 3; bi++)
+                if (S == 4 || bi == 0) SkExchange::release(fl[bi], fl[bi] + SK_WORDS, S == 4 ? 3 : 1);
         }
-#ifdef MI_LAB_TS
-        if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[5] = clock64(); }
-#endif
         // One kept sub-tile (S = NQ): q = s.  Two (S = 2 of four): q = s and s + 2, the 32-row half j = s at both
         // 32-column halves.
         if (NSL == 1) {
@@ -998,16 +1009,10 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
             float16v two[2][1] = {{tot[0]}, {tot[1]}};
             store_tile<1, 2, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, two, cb, smem, m0 + 32 * sk_s, n0, wm, wn, wave, lane, bz);
         }
-#ifdef MI_LAB_TS
-        if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[2] = clock64(); t[3] = wall_clock64(); }
-#endif
         if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
         return;
     }
     store_tile<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz);
-#ifdef MI_LAB_TS
-    if (p.clk && lane == 0) { unsigned long long *t = p.clk + 8 + (blockIdx.x * 8 + wave) * 8; t[2] = clock64(); t[3] = wall_clock64(); }
-#endif
     if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
 }
 
@@ -1604,6 +1609,9 @@ __global__ __launch_bounds__(256) void splitk_epilogue_ln_kernel(GemmArgs p, con
 // ------------------------------------------------------------------------------------------
 bool g_ready = false;
 int g_cus = 256;
+// Inside mi_*_plan_caps the planners answer for the device the caller describes instead of the one they run on.
+thread_local int tl_plan_cus = 0;          // > 0: compute units to plan for
+thread_local bool tl_plan_mfma = true;     // false: the described device has no matrix unit
 unsigned long long *g_clock_probe = nullptr;      // mi_set_clock_probe
 
 // Scratch of mi_gemm_f16_noalloc: every GPU the library runs on holds its own copy of this array, at its own
@@ -1613,8 +1621,13 @@ constexpr int MAX_DEVICES = 64;
 void *g_scratch_ptr[MAX_DEVICES] = {};
 
 unsigned *g_sk_flags_ptr[MAX_DEVICES] = {};
+unsigned *g_status_ptr[MAX_DEVICES] = {};    // the device's copy of device_status_words
 int g_sk_state[MAX_DEVICES] = {};            // 0: not probed, 1: usable, -1: this device does not deal workgroups round robin
 std::atomic<unsigned> g_sk_epoch{0};
+std::atomic<bool> g_sk_enabled{true};        // mi_set_in_launch_exchange
+constexpr int SK_SPIN_DEFAULT = 1 << 18;     // polls of a few hundred ns each: a partner that has not shown up after ~0.1 s will not
+int g_sk_spin = SK_SPIN_DEFAULT;             // mi_test_exchange_faults
+unsigned g_sk_pub_xor = 0, g_sk_xcc_xor = 0;
 
 // Workgroup -> XCD: every workgroup of a 1024-workgroup probe writes the id of the XCD it runs on (HW_REG_XCC_ID).
 __global__ void xcc_probe_kernel(unsigned *out) {
@@ -1628,7 +1641,9 @@ int sk_probe_current_device() {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return -1;
     if (g_sk_state[dev]) return g_sk_state[dev];
-    void *ptr = nullptr;
+    void *ptr = nullptr, *sptr = nullptr;
+    if (hipGetSymbolAddress(&sptr, HIP_SYMBOL(device_status_words)) != hipSuccess || !sptr) return g_sk_state[dev] = -1;
+    g_status_ptr[dev] = reinterpret_cast<unsigned *>(sptr);
     if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(sk_flag_words)) != hipSuccess || !ptr) return g_sk_state[dev] = -1;
     g_sk_flags_ptr[dev] = reinterpret_cast<unsigned *>(ptr);
     constexpr int NP = 1024;
@@ -1642,7 +1657,7 @@ int sk_probe_current_device() {
 }
 bool sk_usable() {
     int dev = -1;
-    return hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MAX_DEVICES && g_sk_state[dev] == 1;
+    return g_sk_enabled.load() && hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MAX_DEVICES && g_sk_state[dev] == 1;
 }
 
 // The current device's copy of `scratch`; resolved once per device, with that device current.  Null on failure.
@@ -1682,7 +1697,7 @@ constexpr int gemm_lds_bytes() {
 // multiple of 32 within [64, SKN_KMAX].
 int skinny_kper(int64_t K, int64_t F) {
     const int64_t colblocks = ceil_div(F, SKN_COLS);
-    const int64_t want = ceil_div(2 * (int64_t)g_cus, colblocks);
+    const int64_t want = ceil_div(2 * (int64_t)mi_num_cus(), colblocks);
     int64_t kper = (int64_t)round_up((size_t)ceil_div(K, want), 32);
     if (kper < 64) kper = 64;
     if (kper > SKN_KMAX) kper = SKN_KMAX;
@@ -1780,10 +1795,11 @@ int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
     a.sk_S = split;
     a.sk_tpx = (int)ceil_div(tiles, 8);
     a.sk_part = reinterpret_cast<float *>(ws);
-    unsigned epoch = ++g_sk_epoch;
-    if (epoch == 0) epoch = ++g_sk_epoch;               // zero is what untouched flags hold
-    a.sk_epoch = epoch;
-    a.sk_flags = g_sk_flags_ptr[dev] + (size_t)(epoch % SK_BANKS) * SK_FLAGS;
+    const unsigned launch = ++g_sk_epoch;
+    a.sk_epoch = sk::epoch_of(launch);
+    a.sk_flags = g_sk_flags_ptr[dev] + (size_t)(launch % SK_BANKS) * SK_FLAGS;
+    a.sk_spin = g_sk_spin; a.sk_pub_xor = g_sk_pub_xor; a.sk_xcc_xor = g_sk_xcc_xor;
+    a.status = g_status_ptr[dev];
     a.clk = g_clock_probe;
     dim3 grid((unsigned)(8 * a.sk_tpx * split), 1);
     constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
@@ -1797,11 +1813,6 @@ int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
 // output, same bits, and the plan (hence the workspace) stays a function of the extents alone.
 int launch_tile(int tile, const GemmArgs &a, bool b_kn, int64_t nbatch, hipStream_t st) {
     const bool plain = !a.cv.xp && !a.ag.x;
-#ifdef MI_LAB
-    if (tile == 6) return launch_pp<128, 256, 64, 3, 2, 4, false>(a, b_kn, nbatch, st);
-    if (tile == 7) return launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
-    if (tile == 8) return launch_pp<128, 128, 64, 3, 2, 4, true>(a, b_kn, nbatch, st);
-#endif
     switch (tile) {
         case 0: return plain ? launch_pp<128, 256, 64, 3, 2, 4, true>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
         case 1: return launch_pipe<192, 128, 2, 4>(a, b_kn, nbatch, st);
@@ -1849,11 +1860,11 @@ struct TilePlan { int tile, split; bool peer; };      // peer: the K-slices exch
 
 double tile_cost_us(int64_t M, int64_t N, int64_t K, int64_t nbatch, int tile, int split) {
     const TileModel &t = TILE_MODELS[tile];
-    const double cus = (double)g_cus;
+    const double cus = (double)mi_num_cus();
     const int64_t wg = ceil_div(M, t.bm) * ceil_div(N, t.bn) * nbatch * split;
-    const int64_t rounds = ceil_div(wg, (int64_t)g_cus);
-    const double load = wg < g_cus ? (double)wg / cus : 1.0;
-    const double step = wg <= g_cus ? t.step_lo + (t.step_full - t.step_lo) * load : t.step_full * t.round * (double)rounds;
+    const int64_t rounds = ceil_div(wg, (int64_t)mi_num_cus());
+    const double load = wg < mi_num_cus() ? (double)wg / cus : 1.0;
+    const double step = wg <= mi_num_cus() ? t.step_lo + (t.step_full - t.step_lo) * load : t.step_full * t.round * (double)rounds;
     double us = 2.0 + (t.fixed - 2.0) * (1.0 + 0.8 * (double)(rounds - 1)) + (t.fixed - 2.0) * 0.4 * load + (double)(K / (64 * split)) * step;
     if (split > 1) us += 4.0 + 0.25 * (double)split * (double)M * (double)N * 4.0 / 1e6;
     return us;
@@ -1873,20 +1884,21 @@ double sk_exchange_us(int64_t wg, int bm, int bn, int split) {
 size_t sk_workspace_bytes(int64_t M, int64_t N, int bm, int bn, int split) { return (size_t)(ceil_div(M, bm) * ceil_div(N, bn)) * split * bm * bn * 4; }
 bool sk_fits(int64_t M, int64_t N, int64_t K, int bm, int bn, int split) {
     const int64_t tiles = ceil_div(M, bm) * ceil_div(N, bn), tpx = ceil_div(tiles, 8);
-    return (split == 2 || (split == 4 && bn == 256)) && K % (64 * split) == 0 && K / split >= 128 && 8 * tpx * split <= g_cus &&
+    return (split == 2 || (split == 4 && bn == 256)) && K % (64 * split) == 0 && K / split >= 128 && 8 * tpx * split <= mi_num_cus() &&
            8 * tpx * split * 8 <= SK_FLAGS;
 }
 // Before mi_init (planner queries without a device) the path is assumed: a workspace sized for it also holds the planes
 // the same split falls back to.
 bool sk_planned() {
     int dev = -1;
+    if (!g_sk_enabled.load()) return false;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return true;
     return g_sk_state[dev] != -1;
 }
 double sk_cost_us(int64_t M, int64_t N, int64_t K, int tile, int split) {
     const TileModel &t = TILE_MODELS[tile];
     const int64_t wg = ceil_div(M, t.bm) * ceil_div(N, t.bn) * split;
-    const double load = (double)wg / (double)g_cus;
+    const double load = (double)wg / (double)mi_num_cus();
     const double step = t.step_lo + (t.step_full - t.step_lo) * load;
     return 2.0 + (t.fixed - 2.0) * (0.4 + 0.6 / (double)split) + (t.fixed - 2.0) * 0.4 * load + (double)(K / (64 * split)) * step +
            sk_exchange_us(wg, t.bm, t.bn, split);
@@ -1925,7 +1937,7 @@ int gemm_path(const GemmArgs &a, bool b_kn, int64_t nbatch) {
     if (a.M < 1 || a.N < 1 || a.K < 1) return MI_GEMM_DECLINE;
     bool addr = mfma_addressable(a, b_kn);
     if (a.M <= 8 && nbatch == 1 && addr && (b_kn || (size_t)8 * a.K * sizeof(half_t) <= SKINNY_FK_LDS_MAX)) return MI_GEMM_SKINNY;
-    if (addr) return MI_GEMM_MFMA;
+    if (addr && tl_plan_mfma) return MI_GEMM_MFMA;
     return MI_GEMM_SCALAR;
 }
 
@@ -1957,12 +1969,7 @@ int run_skinny(GemmArgs a, bool b_kn, void *ws, size_t ws_bytes, hipStream_t st)
         // the layer-norm prologue every wave would normalise its own copy of the row -- 4.5 / 6.1 / 6.9 us against
         // 3.9 / 4.3 / 4.7 us -- so that stays staged, and so does a very wide output (51866 columns: 24.5 against 23.0 us).
         int R = 1;
-#ifdef MI_LAB
-        if (const char *f = getenv("MI_FORCE_GEMV_R")) R = atoi(f);
-        if (R >= 1 && a.K <= 1536 && mt <= 2) {
-#else
         if (!a.ln_on && a.N <= 8192 && a.K <= 1536 && mt <= 2) {
-#endif
             dim3 rg((unsigned)ceil_div(a.N, 4 * R));
             if (R == 2) {
                 if (mt == 1)      hipLaunchKernelGGL((skinny_fk_reg_kernel<1, 3, 2>), rg, dim3(256), 0, st, a);
@@ -1975,7 +1982,7 @@ int run_skinny(GemmArgs a, bool b_kn, void *ws, size_t ws_bytes, hipStream_t st)
         }
         // every column its own wave up to eight workgroups per CU; beyond that (a vocabulary projection) a wave walks
         // several columns behind one staging of the activations
-        const int64_t wgs = ceil_div(a.N, 4), cap = (int64_t)g_cus * 8;
+        const int64_t wgs = ceil_div(a.N, 4), cap = (int64_t)mi_num_cus() * 8;
         dim3 grid((unsigned)(wgs < cap ? wgs : cap));
         if (a.K <= 1536) {
             if (mt == 1)      hipLaunchKernelGGL((skinny_fk_kernel<1, 3>), grid, dim3(256), lds, st, a);
@@ -2017,6 +2024,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
     a.clk = nullptr;
     a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
+    a.sk_spin = 0; a.sk_pub_xor = a.sk_xcc_xor = 0; a.status = nullptr;
     return MI_OK;
 }
 
@@ -2043,18 +2051,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
         if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
         TilePlan tp = {4, 1, false};
-#ifdef MI_LAB
-        // timing builds only: MI_FORCE_TILE = 1 + tile index (7: ping-pong 128 x 256 with both wave groups in phase,
-        // 8: the pipelined kernel's 128 x 256), MI_FORCE_SPLIT = K-slices
-        const char *ft = getenv("MI_FORCE_TILE"), *fs = getenv("MI_FORCE_SPLIT");
-        const bool forced = pipe && ft && atoi(ft) > 0;
-        if (forced) tp = {atoi(ft) - 1, fs ? atoi(fs) : 1, false};
-        if (forced && atoi(ft) == 20) tp = {0, fs ? atoi(fs) : 2, true};      // 20, 21: the peer reduction on 128 x 256, 128 x 128
-        if (forced && atoi(ft) == 21) tp = {2, 2, true};
-        if (pipe && !forced) {
-#else
         if (pipe) {
-#endif
             tp = plan_tiles(a.M, a.N, a.K, nbatch, true);
             if (tp.split > 1 && !(ws && aligned_to(ws, 256) && ws_bytes >= plan_workspace_bytes(tp, a.M, a.N)))
                 tp = plan_tiles(a.M, a.N, a.K, nbatch, false);
@@ -2094,8 +2091,8 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         // K not a multiple of 64 (or a single tile deep): the unpipelined kernel, big tiles as soon as they cover half the CUs
         const int64_t big = ceil_div(a.M, 128) * ceil_div(a.N, 256) * nbatch;
         const int64_t mid = ceil_div(a.M, 128) * ceil_div(a.N, 128) * nbatch;
-        if (big * 2 > g_cus) return launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
-        if (mid >= (g_cus * 3) / 8) return launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
+        if (big * 2 > mi_num_cus()) return launch_mfma<GEMM_BIG>(a, b_kn, nbatch, st);
+        if (mid >= (mi_num_cus() * 3) / 8) return launch_mfma<GEMM_MID>(a, b_kn, nbatch, st);
         return launch_mfma<GEMM_SMALL>(a, b_kn, nbatch, st);
     }
     long total = (long)a.M * a.N;
@@ -2106,7 +2103,14 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
 }  // namespace
 
 bool mi_ready() { return g_ready; }
-int mi_num_cus() { return g_cus; }
+int mi_num_cus() { return tl_plan_cus > 0 ? tl_plan_cus : g_cus; }
+bool mi_plan_mfma() { return tl_plan_mfma; }
+void mi_plan_caps_begin(const int64_t *caps) {
+    if (!caps) return;
+    tl_plan_mfma = caps[0] != 0;
+    tl_plan_cus = caps[5] > 0 ? (int)(caps[5] > 65536 ? 65536 : caps[5]) : 1;
+}
+void mi_plan_caps_end() { tl_plan_cus = 0; tl_plan_mfma = true; }
 bool mi_xcd_round_robin() { return sk_usable(); }
 
 // Split-K planes of a GEMM issued through mi_internal_gemm.
@@ -2129,6 +2133,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
     a.clk = nullptr;
     a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
+    a.sk_spin = 0; a.sk_pub_xor = a.sk_xcc_xor = 0; a.status = nullptr;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = out_f32 ? nullptr : (const half_t *)residual;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
@@ -2179,12 +2184,6 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 2>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true>, pp_lds_bytes<128, 256, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, true>, pp_lds_bytes<128, 256, 64, 3>());
-#ifdef MI_LAB
-    bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, true, true>, pp_lds_bytes<128, 128, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, false, true>, pp_lds_bytes<128, 128, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, false>, pp_lds_bytes<128, 256, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, false>, pp_lds_bytes<128, 256, 64, 3>());
-#endif
     bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, false, true, true>, pp_lds_bytes<128, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 256, 64, 3>());
@@ -2214,6 +2213,33 @@ int mi_init(void) {
 int mi_set_clock_probe(void *dev_u64x4) {
     if (dev_u64x4 && !aligned_to(dev_u64x4, 8)) return MI_DECLINE_OPERANDS;
     g_clock_probe = reinterpret_cast<unsigned long long *>(dev_u64x4);
+    return MI_OK;
+}
+
+int mi_device_status(int reset) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES || !g_status_ptr[dev]) return -1;
+    if (hipDeviceSynchronize() != hipSuccess) return -1;
+    unsigned word = 0;
+    if (hipMemcpy(&word, g_status_ptr[dev], sizeof(word), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+    if (reset) {
+        // a wave that gave up released nothing: zero every bank of flags and counters along with the word
+        bool ok = hipMemset(g_status_ptr[dev], 0, sizeof(unsigned)) == hipSuccess;
+        if (g_sk_flags_ptr[dev]) ok = ok && hipMemset(g_sk_flags_ptr[dev], 0, sizeof(unsigned) * 2 * SK_WORDS) == hipSuccess;
+        if (!ok || hipDeviceSynchronize() != hipSuccess) return -1;
+    }
+    return (int)(word & 0x7fffffffu);
+}
+
+int mi_set_in_launch_exchange(int enabled) {
+    g_sk_enabled.store(enabled != 0);
+    return MI_OK;
+}
+
+int mi_test_exchange_faults(int spin_limit, unsigned publish_xor, unsigned xcc_xor) {
+    g_sk_spin = spin_limit > 0 ? spin_limit : SK_SPIN_DEFAULT;
+    g_sk_pub_xor = publish_xor & sk::EPOCH_MASK;
+    g_sk_xcc_xor = xcc_xor & 15u;
     return MI_OK;
 }
 
@@ -2249,6 +2275,20 @@ int mi_gemm_f16_plan(const void *Y, const void *X, const void *W,
                        MI_EPI_NONE, out_dtype, sY, sX, sW);
     if (rc != MI_OK) return MI_GEMM_DECLINE;
     return gemm_path(a, w_layout == MI_W_KF, nbatch < 1 ? 1 : nbatch);
+}
+
+int mi_gemm_f16_plan_caps(const int64_t caps[6], const void *Y, const void *X, const void *W,
+                          int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                          int w_layout, int out_dtype, int64_t nbatch, int64_t sY, int64_t sX, int64_t sW, int *ksplit_out) {
+    mi_plan_caps_begin(caps);
+    const int path = mi_gemm_f16_plan(Y, X, W, T, K, F, ldY, ldX, ldW, w_layout, out_dtype, nbatch, sY, sX, sW);
+    if (ksplit_out) {
+        *ksplit_out = 1;
+        if (path == MI_GEMM_MFMA && K % 64 == 0 && K >= 128) *ksplit_out = plan_tiles(T, F, K, nbatch < 1 ? 1 : nbatch, true).split;
+        if (path == MI_GEMM_SKINNY && w_layout == MI_W_KF) *ksplit_out = skinny_splits(K, F);
+    }
+    mi_plan_caps_end();
+    return path;
 }
 
 int mi_gemm_f16_batched(void *Y, const void *X, const void *W, const void *bias, const void *residual,

@@ -377,6 +377,59 @@ def test_in_launch_exchanges_on_two_streams_do_not_meet(ctx):
     for s in range(2):
         for y in outs[s]:
             assert torch.equal(y.view(torch.int16), alone.view(torch.int16))
+    assert lib.mi_device_status(0) == 0, "a workgroup gave up waiting for its partner"
+
+
+def test_a_missed_exchange_is_loud(ctx):
+    """A workgroup of the in-launch split-K exchange waits for its partners a bounded time.  The waits are made to fail
+    from the host (mi_test_exchange_faults: a handful of polls, and partners that publish an epoch nobody waits for, or
+    that seem to sit on another XCD), so every kernel still runs to its end: the call returns MI_OK as always, the
+    device's sticky status word names the reason, Y holds NaN instead of a plausible sum, and after the reset that
+    mi_device_status(1) performs the same launch is right again.  With the exchange switched off the K-slices go
+    through planes."""
+    import torch
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    st = torch.cuda.current_stream().cuda_stream
+    T, K, F = 1500, 5120, 1280
+    X, W = oracle.randn_f16((T, K), 81, 0, 1.0 / np.sqrt(K)), oracle.randn_f16((K, F), 82)
+    b, R = oracle.randn_f16((F,), 83, 0, 0.02), oracle.randn_f16((T, F), 84)
+    dX, dW, db, dR = to_dev(X), to_dev(W), to_dev(b), to_dev(R)
+
+    def launch():
+        need = lib.mi_gemm_f16_workspace(T, K, F, L.W_KF, 1)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        y = torch.zeros((T, F), dtype=torch.float16, device="cuda")
+        rc = lib.mi_gemm_f16(y.data_ptr(), dX.data_ptr(), dW.data_ptr(), db.data_ptr(), dR.data_ptr(), T, K, F, F, K, F,
+                             L.W_KF, L.BIAS_COL, L.EPI["none"], L.F16, ws.data_ptr(), need, st)
+        assert rc == L.OK
+        torch.cuda.synchronize()
+        return y
+
+    assert lib.mi_device_status(1) == 0
+    try:
+        lib.mi_test_exchange_faults(16, 0x5A5A5, 0)
+        y = launch()
+        assert lib.mi_device_status(0) == 1, "a wait that gave up must raise MI_DEVSTAT_EXCHANGE_TIMEOUT"
+        assert lib.mi_device_status(1) == 1 and lib.mi_device_status(0) == 0      # sticky until reset
+        assert bool(torch.isnan(y).all()), "no workgroup may store a sum it could not complete"
+        lib.mi_test_exchange_faults(0, 0, 1)
+        y = launch()
+        assert lib.mi_device_status(1) == 2, "partners on another XCD must raise MI_DEVSTAT_EXCHANGE_XCD"
+        assert bool(torch.isnan(y).all())
+    finally:
+        lib.mi_test_exchange_faults(0, 0, 0)
+        lib.mi_device_status(1)
+    peer = launch()
+    assert lib.mi_device_status(0) == 0
+    assert_parity(to_host(peer), oracle.gemm_f16(X, W, b, residual=R), what="exchange after a reset")
+    try:
+        lib.mi_set_in_launch_exchange(0)
+        planes = launch()
+    finally:
+        lib.mi_set_in_launch_exchange(1)
+    assert lib.mi_device_status(0) == 0
+    assert_parity(to_host(planes), oracle.gemm_f16(X, W, b, residual=R), what="K-slices through planes")
 
 
 @pytest.mark.parametrize("T,K,F", [(1500, 5120, 1280), (1370, 1536, 384)])
