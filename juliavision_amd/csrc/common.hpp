@@ -85,8 +85,11 @@ MI_DEVICE float erf_as(float x) {
 //   v >= 0:  0.5 v (2 - P e) = v - v q        v < 0:  0.5 v (P e) = v q        both:  max(v, 0) - u q.
 // Same polynomial, same coefficients; the difference from the textbook order is rounding in the last fp32 place
 // (and, for v < -3, none of the cancellation in 1 - (1 - P e)), far below the fp16 result's resolution.
+// u is capped at 64: beyond |v| = 14 the exponential is exactly 0 in fp32 and the result max(v, 0) either way, and
+// with the cap v = +inf gives +inf as the reference's expression does (uncapped, -inf * 0 + inf would be NaN).  At
+// v = -inf the reference's 0.5 v (1 + erf) is -inf * 0 = NaN; this form gives -0.
 MI_DEVICE float gelu_erf(float v) {
-    const float u = fabsf(v);
+    const float u = fminf(fabsf(v), 64.0f);
     const float t = __builtin_amdgcn_rcpf(fmaf(u, 0.3275911f * 0.70710678118654752440f, 1.0f));
     float pl = fmaf(0.5f * 1.061405429f, t, -0.5f * 1.453152027f);
     pl = fmaf(pl, t, 0.5f * 1.421413741f);
@@ -159,6 +162,11 @@ struct NhwcGather {
 // True once mi_init has run successfully on this process (defined in gemm.hip).
 bool mi_ready();
 int mi_num_cus();
+// Planning for a device other than the current one (mi_*_plan_caps): between begin and end, on this thread,
+// mi_num_cus() and mi_plan_mfma() answer for caps (the six values of mi_device_caps); caps == nullptr changes nothing.
+bool mi_plan_mfma();
+void mi_plan_caps_begin(const int64_t *caps);
+void mi_plan_caps_end();
 // True if the current device deals workgroups to its XCDs round robin by workgroup id (ids that differ by a multiple
 // of 8 share an L2), as a probe launch at mi_init showed; kernels whose workgroups exchange data through one L2 ask.
 bool mi_xcd_round_robin();

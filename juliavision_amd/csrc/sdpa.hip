@@ -1519,6 +1519,25 @@ int rows_splits(int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     return (int)want;
 }
 
+// Between 8 and 63 queries over a long key range -- the reference's flash-decoding case, 23 queries over 4096 keys
+// (SAM 2.1's mask decoder attending the image; flash.jl:1288-1303, kernelplans.jl:300-312): one 128-query tile per
+// (head, batch) of the fused kernel with the keys cut over workgroups, two workgroups per compute unit as the
+// reference's splitcount aims for, every split at least four 64-key blocks; sdpa_merge_kernel joins the partials.
+// (One workgroup per query row -- sdpa_rows_kernel -- re-reads K and V once per row.)
+// Only while the (head, batch) tiles alone leave the chip mostly idle: beyond that a workgroup per query row fills it.
+bool flash_few_queries(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    return Lq >= 8 && Lq < 64 && Lk >= 512 && E <= 128 && H * B * 2 <= (int64_t)mi_num_cus();
+}
+int few_query_splits(int64_t Lk, int64_t H, int64_t B) {
+    const int64_t tiles = H * B, blocks = ceil_div(Lk, 64);
+    int64_t want = ceil_div(2 * (int64_t)mi_num_cus(), tiles);
+    if (want > blocks / 4) want = blocks / 4;
+    if (want > 32) want = 32;
+    if (want < 1) want = 1;
+    while (want > 1 && ceil_div(blocks, want) * (want - 1) >= blocks) want--;      // no empty split
+    return (int)want;
+}
+
 // Key splits for the fused kernel.  A workgroup spends about 1 us per 64-key block plus 3 us of start-up,
 // and the merge is a second launch of about 6 us, so splitting pays only when the query blocks leave most
 // of the chip idle and every split still walks a dozen blocks (config 3's 66 workgroups x 22 blocks do
@@ -1537,6 +1556,7 @@ bool flash_halves96(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
 }
 
 int flash_splits(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    if (flash_few_queries(E, Lq, Lk, H, B)) return few_query_splits(Lk, H, B);
     return flash_halves96(E, Lq, Lk, H, B) ? 1 : flash_splits_over_workgroups(E, Lq, Lk, H, B);
 }
 
@@ -1563,9 +1583,6 @@ int flash_splits_over_workgroups(int64_t E, int64_t Lq, int64_t Lk, int64_t H, i
 // beyond that the 128-query forms are as fast or faster.
 bool flash_short(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     const int64_t tiles = ceil_div(Lq, 32) * H * B, cus = mi_num_cus();
-#ifdef MI_LAB
-    if (const char *f = getenv("MI_FORCE_SHORT")) return E == 64 && atoi(f) > 0;
-#endif
     if (E != 64 || Lk < 128 || tiles > cus + cus / 16) return false;
     // against key splits over workgroups (few tiles, many keys): 4.5 us + 1.3 us per block of a wave's quarter here,
     // 3 us + 1 us per block of a split + the 6 us merge launch there
@@ -1580,13 +1597,12 @@ bool flash_short(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
 // at 12 x 1370 (264 tiles of 64) the key-halves form is (19.4 against 26.5 us).
 bool flash_pair(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
     const int64_t tiles32 = ceil_div(Lq, 32) * H * B, tiles64 = ceil_div(Lq, 64) * H * B, cus = mi_num_cus();
-#ifdef MI_LAB
-    if (const char *f = getenv("MI_FORCE_PAIR")) return E == 64 && atoi(f) > 0;
-#endif
     return E == 64 && Lk >= 128 && tiles32 > cus && tiles64 <= cus;
 }
 // either of the two: one launch, keys not split over workgroups
-bool flash_unsplit(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) { return flash_pair(E, Lq, Lk, H, B) || flash_short(E, Lq, Lk, H, B); }
+bool flash_unsplit(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B) {
+    return !flash_few_queries(E, Lq, Lk, H, B) && (flash_pair(E, Lq, Lk, H, B) || flash_short(E, Lq, Lk, H, B));
+}
 
 // A single query row (a decode step) runs in one launch of sdpa_decode_kernel: the work follows the device-side kv_len
 // and the cache write can ride along (mi_sdpa_append_f16).  Twenty heads alone leave most of the chip idle and give each
@@ -1619,9 +1635,6 @@ int decode_splits(int64_t E, int64_t Lk, int64_t H, int64_t B) {
     if (want > 32) want = 32;
     while (want > 1 && units * want * (E + 2) > SD_PART_FLOATS) want--;
     if (want < 1) want = 1;
-#ifdef MI_LAB
-    if (const char *f = getenv("MI_FORCE_DSPLIT")) { want = atoi(f); if (want > passes) want = passes; if (want < 1) want = 1; }
-#endif
     // no empty split: with `per` passes each, the last one must still start inside the range
     while (want > 1 && ceil_div(passes, want) * (want - 1) >= passes) want--;
     return (int)want;
@@ -1658,7 +1671,8 @@ int sdpa_path(const SdpaArgs &a) {
     if (a.H > 65535 || a.B > 65535 || (int64_t)a.Lq * a.H * 64 > INT32_MAX) return MI_SDPA_DECLINE;
     bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
     bool out_ok = (aligned_to(a.out, 16) || a.out == nullptr) && a.os[0] == 1 && a.os[1] % 8 == 0 && a.os[2] % 8 == 0 && a.os[3] % 8 == 0;
-    if (vec && out_ok && (!a.bias || flash_bias_ok(a)) && a.scale > 0.0f && a.E <= 128 && a.Lq >= 64 && a.Lk >= 1) return MI_SDPA_FLASH;
+    const bool enough_queries = a.Lq >= 64 || (!a.bias && flash_few_queries(a.E, a.Lq, a.Lk, a.H, a.B));
+    if (mi_plan_mfma() && vec && out_ok && (!a.bias || flash_bias_ok(a)) && a.scale > 0.0f && a.E <= 128 && enough_queries && a.Lk >= 1) return MI_SDPA_FLASH;
     return MI_SDPA_ROWS;
 }
 
@@ -1728,6 +1742,8 @@ size_t mi_sdpa_f16_workspace(int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64
     // sized for the path the call will most likely take: the fused kernel's key splits for Lq >= 64 without
     // an additive mask (unused if the operands turn out not to be 16-byte addressable), the rows kernel's below
     int ns = Lq >= 64 ? ((has_bias || flash_unsplit(E, Lq, Lk, H, B)) ? 1 : flash_splits(E, Lq, Lk, H, B)) : rows_splits(Lq, Lk, H, B);
+    // few queries over many keys: whichever of the two routes the operands allow must find its partials' room
+    if (!has_bias && flash_few_queries(E, Lq, Lk, H, B) && few_query_splits(Lk, H, B) > ns) ns = few_query_splits(Lk, H, B);
     if (ns <= 1) return 0;
     size_t rows = (size_t)Lq * H * B;
     return round_up((size_t)ns * rows * E * sizeof(float), 256) + round_up((size_t)ns * rows * 2 * sizeof(float), 256);
@@ -1748,6 +1764,15 @@ int mi_sdpa_f16_plan(const void *q, const int64_t q_strides[4], const void *k, c
     const bool vec = vec_addressable(a.q, a.qs, a.E) && vec_addressable(a.k, a.ks, a.E) && vec_addressable(a.v, a.vs, a.E);
     if (nsplit_out) *nsplit_out = (path == MI_SDPA_ROWS && Lq < 64) ? (one_pass_decode(a, vec) ? decode_splits(E, Lk, H, B) : rows_splits(Lq, Lk, H, B))
                                   : (path == MI_SDPA_FLASH && !has_bias && !flash_unsplit(E, Lq, Lk, H, B)) ? flash_splits(E, Lq, Lk, H, B) : 1;
+    return path;
+}
+
+int mi_sdpa_f16_plan_caps(const int64_t caps[6], const void *q, const int64_t q_strides[4], const void *k, const int64_t k_strides[4],
+                          const void *v, const int64_t v_strides[4], int has_bias, int has_kv_len,
+                          int64_t E, int64_t Lq, int64_t Lk, int64_t H, int64_t B, float scale, int *nsplit_out) {
+    mi_plan_caps_begin(caps);
+    const int path = mi_sdpa_f16_plan(q, q_strides, k, k_strides, v, v_strides, has_bias, has_kv_len, E, Lq, Lk, H, B, scale, nsplit_out);
+    mi_plan_caps_end();
     return path;
 }
 
@@ -1786,11 +1811,11 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
         } else if (pp) {
             dim3 grid((unsigned)ceil_div(Lq, 256), (unsigned)H, (unsigned)B);
             hipLaunchKernelGGL((flash_fwd_kernel<64, true>), grid, dim3(512), flash_lds_bytes(64), st, a);
-        } else if (flash_pair(E, Lq, Lk, H, B)) {
+        } else if (!flash_few_queries(E, Lq, Lk, H, B) && flash_pair(E, Lq, Lk, H, B)) {
             a.nsplit = 1;
             dim3 grid((unsigned)ceil_div(Lq, 64), (unsigned)H, (unsigned)B);
             hipLaunchKernelGGL(flash_pair_kernel, grid, dim3(512), flash_pair_lds_bytes(), st, a);
-        } else if (flash_short(E, Lq, Lk, H, B)) {
+        } else if (!flash_few_queries(E, Lq, Lk, H, B) && flash_short(E, Lq, Lk, H, B)) {
             a.nsplit = 1;
             dim3 grid((unsigned)ceil_div(Lq, 32), (unsigned)H, (unsigned)B);
             hipLaunchKernelGGL(flash_short_kernel<4>, grid, dim3(256), flash_short_lds_bytes(4), st, a);

@@ -67,6 +67,11 @@ class DeviceCaps(NamedTuple):
 MI355X = DeviceCaps(True, 16, 64, 160 * 1024, 1024, 256)
 
 
+def _caps_array(dev: DeviceCaps):
+    """The six values of mi_device_caps, for the planners that answer for a described device."""
+    return (C.c_int64 * 6)(int(dev.coopmat), dev.tile, dev.subgroup, dev.sharedbudget, dev.workgrouplimit, dev.cores)
+
+
 def caps() -> DeviceCaps:
     """Query the current device (context.jl:55)."""
     lib = L.init()
@@ -226,8 +231,8 @@ def mmplan(dev: DeviceCaps, out, A, B, bias=None):
         return Decline("nocoopmat")
     w_layout = L.W_KF if la[0] == 0 else L.W_FK
     lib = L.load()
-    path = lib.mi_gemm_f16_plan(out.data_ptr(), B.data_ptr(), A.data_ptr(), T, K, F, lo[1], lb[1], la[1],
-                                w_layout, _dtype_code(out), 1, 0, 0, 0)
+    path = lib.mi_gemm_f16_plan_caps(_caps_array(dev), out.data_ptr(), B.data_ptr(), A.data_ptr(), T, K, F, lo[1], lb[1], la[1],
+                                     w_layout, _dtype_code(out), 1, 0, 0, 0, None)
     return {1: MMMfmaPlan, 2: MMSkinnyPlan, 3: MMScalarPlan}.get(path, lambda _: Decline("extent"))(w_layout)
 
 
@@ -447,8 +452,9 @@ def sdpaplan(ctx: Ctx, q, k, v, bias=None, scale=None, kv_len=None):
         return Decline("nocoopmat")
     scale = (1.0 / math.sqrt(E)) if scale is None else float(scale)
     ns = C.c_int(1)
-    path = L.load().mi_sdpa_f16_plan(q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k), v.data_ptr(), _strides_elbh(v),
-                                     0, int(kv_len is not None), E, Lq, Lk, H, Bq, scale, C.byref(ns))
+    devcaps = _caps_array(ctx.dev)
+    path = L.load().mi_sdpa_f16_plan_caps(devcaps, q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k), v.data_ptr(), _strides_elbh(v),
+                                          0, int(kv_len is not None), E, Lq, Lk, H, Bq, scale, C.byref(ns))
     if bias is not None:
         # The fused kernel carries a mask whose keys are contiguous and whose fp16 rows start on 4-byte boundaries (any
         # other axis may broadcast); everything else is the rows kernel's.  The C planner sees only "a mask" and plans a
@@ -459,8 +465,8 @@ def sdpaplan(ctx: Ctx, q, k, v, bias=None, scale=None, kv_len=None):
         if fused:
             return FlashPlan(1)
         ns1 = C.c_int(1)
-        L.load().mi_sdpa_f16_plan(q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k), v.data_ptr(), _strides_elbh(v),
-                                  1, int(kv_len is not None), E, Lq, Lk, H, Bq, scale, C.byref(ns1))
+        L.load().mi_sdpa_f16_plan_caps(devcaps, q.data_ptr(), _strides_elbh(q), k.data_ptr(), _strides_elbh(k), v.data_ptr(), _strides_elbh(v),
+                                       1, int(kv_len is not None), E, Lq, Lk, H, Bq, scale, C.byref(ns1))
         return RowsSDPAPlan(ns1.value if Lq < 64 else 1) if path in (1, 2) else Decline("extent")
     if path == 1:
         return FlashPlan(ns.value)
@@ -700,6 +706,24 @@ def transposeLE_(ctx: Ctx, out, a):
     if rc != L.OK:
         raise DeclineError("mi_transpose_le_f16", rc)
     return out
+
+
+def relayout_weight(ctx: Ctx, w):
+    """A ``(K, F)`` weight held as ``[K][F]`` memory (the reference's hoisted layout, hoistcasts.jl:47-112) returned as
+    the same ``(K, F)`` tensor over ``[F][K]`` memory -- a transposed view of a new buffer -- through
+    ``mi_relayout_weight_f16``; a weight that already lies that way is returned as it is.  Once, at load."""
+    if w.dim() != 2 or not _is_f16_cuda(w):
+        raise DeclineError("relayout_weight: a 2-D fp16 device tensor", L.DECLINE_OPERANDS)
+    if w.stride(0) == 1 and w.shape[0] > 1:
+        return w
+    if w.stride(1) != 1:
+        raise DeclineError("relayout_weight: rows must be contiguous", L.DECLINE_OPERANDS)
+    K, F = w.shape
+    fk = torch.empty((F, K), dtype=w.dtype, device=w.device)
+    rc = L.init().mi_relayout_weight_f16(fk.data_ptr(), K, w.data_ptr(), w.stride(0), K, F, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_relayout_weight_f16", rc)
+    return fk.t()
 
 
 # ----------------------------------------------------------------------------- layer norm, add

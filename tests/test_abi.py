@@ -68,6 +68,43 @@ def test_gemm_planner():
     assert _gemm_plan(64, 64, 64, dt=7) == "decline"
 
 
+def test_planning_for_a_device_one_does_not_have():
+    """The reference's planners take a DeviceCaps value, so its tests ask about hardware they do not have
+    (test_flash.jl:328 `DeviceCaps(dev; cores=1)`, :363 `coopmat=false`, :373-377 a wave64 device).  The C planners
+    answer the same questions through the *_plan_caps entry points; the description does not outlive the call."""
+    lib = L.load()
+    caps = lambda mfma, cus: (C.c_int64 * 6)(mfma, 16, 64, 160 * 1024, 1024, cus)
+    ks, ns = C.c_int(0), C.c_int(0)
+
+    def gemm(c, T, K, F):
+        r = lib.mi_gemm_f16_plan_caps(c, 0x10000, 0x20000, 0x30000, T, K, F, F, K, F, L.W_KF, L.F16, 1, 0, 0, 0, C.byref(ks))
+        return L.GEMM_PATHS[r], ks.value
+
+    def sdpa(c, E, Lq, Lk, H, B):
+        d = lambda n: L.strides4(1, E, E * n, E * n * H)
+        r = lib.mi_sdpa_f16_plan_caps(c, 0x10000, d(Lq), 0x20000, d(Lk), 0x30000, d(Lk), 0, 0, E, Lq, Lk, H, B, 0.125, C.byref(ns))
+        return L.SDPA_PATHS[r], ns.value
+
+    # config 2's second MLP linear: 120 tiles of 128 x 128 leave half of 256 compute units idle, so K is cut in two;
+    # on 64 units the tiles alone fill the device twice over and nothing is cut; without a matrix unit there is no
+    # tiled path at all (mm_coopmat_plan's `dev.coopmat` gate, matmul.jl:172-179), the decode-sized kernel remains
+    assert gemm(None, 1500, 5120, 1280) == gemm(caps(1, 256), 1500, 5120, 1280) == ("mfma", 2)
+    assert gemm(caps(1, 64), 1500, 5120, 1280) == ("mfma", 1)
+    assert gemm(caps(1, 64), 300, 5120, 1280)[1] < gemm(caps(1, 1024), 300, 5120, 1280)[1]
+    assert gemm(caps(0, 256), 1500, 5120, 1280) == ("scalar", 1)
+    assert gemm(caps(0, 256), 4, 1280, 1280)[0] == "skinny"
+    # 23 queries over 4096 keys, the reference's flash-decoding case: the key splits follow the compute units
+    # (two workgroups per unit, splitcount, flash.jl:1288-1303); a one-unit device does not split, a device without a
+    # matrix unit gets the always-available path (Decline(:nocoopmat) -> three-pass, attention.jl:735-759)
+    assert sdpa(caps(1, 256), 16, 23, 4096, 8, 1) == ("flash", 16)
+    assert sdpa(caps(1, 48), 16, 23, 4096, 8, 1) == ("flash", 11)
+    assert sdpa(caps(1, 1), 16, 23, 4096, 8, 1) == ("rows", 1)
+    assert sdpa(caps(0, 256), 64, 4096, 4096, 16, 1)[0] == "rows"
+    assert sdpa(caps(1, 1), 64, 1, 1500, 20, 1) == ("rows", 1) and sdpa(caps(1, 256), 64, 1, 1500, 20, 1) == ("rows", 4)
+    # nothing leaks into the planners of the running device
+    assert _sdpa_plan(64, 4096, 4096, 16, 1) == ("flash", 1) and _gemm_plan(1500, 5120, 1280) == "mfma"
+
+
 def test_gemm_workspace():
     lib = L.load()
     assert lib.mi_gemm_f16_workspace(1500, 1280, 5120, L.W_KF, 1) == 0
@@ -113,6 +150,10 @@ def test_sdpa_planner():
     assert _sdpa_plan(64, 1, 700, 20, 1)[1] == 2                             # 11 passes: two rounds
     assert _sdpa_plan(64, 1, 1500, 20, 1, bias=1)[1] == 24                   # masked: the rows kernel, split 24 ways
     assert _sdpa_plan(64, 23, 17, 4, 1)[1] == 1
+    # 8 to 63 queries over a long key range on few (head, batch) tiles: the fused kernel with its keys cut over
+    # workgroups (the reference's flash-decoding case), not one workgroup per query row
+    assert _sdpa_plan(16, 23, 4096, 8, 1) == ("flash", 16) and _sdpa_plan(16, 23, 4096, 8, 1, bias=1)[0] == "rows"
+    assert _sdpa_plan(64, 23, 300, 8, 1)[0] == "rows" and _sdpa_plan(64, 23, 4096, 200, 1)[0] == "rows"
 
 
 def test_conv_planner_and_extents():

@@ -62,11 +62,28 @@ def test_decode_attention_keeps_the_two_workgroups_per_core_rule():
     assert nsplit(64, 1, 1500, 20, 1, bias=1) == P.splitcount(256, 1, 1500, 1, 64, 20) == 24
     assert nsplit(64, 1, 700, 20, 1, bias=1) == P.splitcount(256, 1, 700, 1, 64, 20) == 11
     for (Lq, Lk, H, B, bias) in [(1, 1500, 20, 4, 1), (1, 1500, 20, 8, 1), (1, 700, 20, 4, 1), (1, 1000, 20, 8, 1), (1, 4096, 8, 1, 1),
-                                 (3, 100, 2, 1, 0), (23, 4096, 8, 1, 0), (5, 100, 2, 1, 0), (2, 17, 4, 1, 0), (7, 64, 1, 1, 0), (1, 100000, 1, 1, 1)]:
+                                 (3, 100, 2, 1, 0), (23, 4096, 8, 1, 1), (5, 100, 2, 1, 0), (2, 17, 4, 1, 0), (7, 64, 1, 1, 0), (1, 100000, 1, 1, 1)]:
         rows = Lq * H * B
         mine = nsplit(64, Lq, Lk, H, B, bias)
         assert mine == max(1, min(P.cld(2 * 256, rows), P.cld(Lk, 64), 64)), (Lq, Lk, H, B)
         assert mine >= min(64, P.splitcount(256, Lq, Lk, 1, 64, H * B)), (Lq, Lk, H, B)
+    # 8 to 63 unmasked queries over 512 keys or more on few (head, batch) tiles take the fused kernel on one 128-query
+    # tile per (head, batch): the same two-workgroups-per-core aim, but a split is at least four 64-key blocks and there
+    # are at most 32 (the reference's rule would cut the 64 blocks of its 23 x 4096 case 64 ways on 256 cores; on its own
+    # 48 cores it gives 6, kernelplans.jl:300-312)
+    def few(E, Lq, Lk, H, B):
+        ns = C.c_int(0)
+        st = L.strides4(1, E, E * Lq, E * Lq * H)
+        sk = L.strides4(1, E, E * Lk, E * Lk * H)
+        assert L.SDPA_PATHS[lib.mi_sdpa_f16_plan(0x10000, st, 0x20000, sk, 0x30000, sk, 0, 0, E, Lq, Lk, H, B, 0.25, C.byref(ns))] == "flash"
+        return ns.value
+    for (Lq, Lk, H, B) in [(23, 4096, 8, 1), (8, 512, 1, 1), (63, 100000, 4, 2), (40, 1111, 4, 2), (23, 4096, 128, 1)]:
+        blocks = P.cld(Lk, 64)
+        rule = max(1, min(P.cld(2 * 256, H * B), blocks // 4, 32))
+        while rule > 1 and P.cld(blocks, rule) * (rule - 1) >= blocks:
+            rule -= 1
+        assert few(16, Lq, Lk, H, B) == rule, (Lq, Lk, H, B)
+    assert few(16, 23, 4096, 8, 1) == 16 and P.splitcount(48, 23, 4096, 16, 32, 8) == 6
     # the one-launch kernel's own count
     for (Lk, H, B, want) in [(448, 20, 1, 1), (448, 20, 8, 1), (512, 20, 1, 1), (700, 20, 1, 2), (1500, 20, 1, 4), (1500, 20, 4, 3),
                              (1500, 20, 8, 1), (4096, 8, 1, 11), (100000, 1, 1, 32)]:

@@ -112,10 +112,41 @@ def test_strided_heads_from_packed_qkv(ctx):
 
 
 def test_rows_path_small_lq_and_ragged(ctx):
-    # ragged shapes of test_flash.jl:189-190 as (E,Lq,Lk,H,B): (16,23,4096,8,1), (32,23,23,8,1), (16,23,17,4,1)
-    for (E, Lq, Lk, H, B) in [(16, 23, 4096, 8, 1), (32, 23, 23, 8, 1), (16, 23, 17, 4, 1), (64, 1, 448, 20, 4), (72, 5, 100, 2, 1), (20, 3, 50, 2, 2)]:
+    # ragged shapes of test_flash.jl:189-190 as (E,Lq,Lk,H,B): (32,23,23,8,1), (16,23,17,4,1)
+    for (E, Lq, Lk, H, B) in [(32, 23, 23, 8, 1), (16, 23, 17, 4, 1), (64, 1, 448, 20, 4), (72, 5, 100, 2, 1), (20, 3, 50, 2, 2)]:
         q, k, v = _qkv(B, H, Lq, Lk, E, 61)
         _check(ctx, q, k, v, expect="RowsSDPAPlan", what=f"rows {E},{Lq},{Lk},{H},{B}")
+
+
+def test_the_references_decoder_shapes_with_a_23_in_them(ctx):
+    """The other two ragged shapes of test_flash.jl:189-190, SAM 2.1's mask decoder attending the image and back:
+    (16,23,4096,8,1) -- 23 queries over 4096 keys, the reference's flash-decoding case (flash.jl:1288-1303), here the
+    fused kernel with the keys cut over workgroups and a merge -- and (16,4096,23,8,1), 4096 queries over 23 keys
+    (fewer keys than one block: a loop that counted whole blocks would run zero times)."""
+    import juliavision_amd as jv
+    q, k, v = _qkv(1, 8, 23, 4096, 16, 62)
+    plan = jv.sdpaplan(ctx, *(to_dev(t) for t in (q, k, v)))
+    assert type(plan).__name__ == "FlashPlan" and plan.nsplit > 1, plan
+    _check(ctx, q, k, v, expect="FlashPlan", what="23 queries over 4096 keys")
+    q, k, v = _qkv(1, 8, 4096, 23, 16, 63)
+    _check(ctx, q, k, v, expect="FlashPlan", what="4096 queries over 23 keys")
+    # the same few-query route with wider heads, a per-batch key count, and a key range that leaves a ragged last split
+    for (E, Lq, Lk, H, B, kv) in [(64, 23, 4096, 8, 1, None), (72, 40, 1111, 4, 2, [700, 1111]), (128, 8, 600, 2, 1, None), (64, 63, 2000, 20, 1, [1999])]:
+        q, k, v = _qkv(B, H, Lq, Lk, E, 64)
+        _check(ctx, q, k, v, kv_len=kv, expect="FlashPlan", what=f"few queries {E},{Lq},{Lk},{H},{B}")
+    # without the workspace for its partials the same call still runs (unsplit)
+    q, k, v = _qkv(1, 8, 23, 4096, 16, 65)
+    dq, dk, dv = (to_dev(t) for t in (q, k, v))
+    import torch
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    out = poison(torch.empty((1, 8, 23, 16), dtype=torch.float16, device="cuda"))
+    st = lambda t: L.strides4(1, t.stride(2), t.stride(1), t.stride(0))
+    rc = lib.mi_sdpa_f16(out.data_ptr(), L.F16, None, dq.data_ptr(), st(dq), dk.data_ptr(), st(dk), dv.data_ptr(), st(dv),
+                         None, 0, None, None, 16, 23, 4096, 8, 1, 0.25, None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == L.OK
+    torch.cuda.synchronize()
+    assert_parity(to_host(out), oracle.sdpa_ref_f32(q, k, v), what="few queries, no workspace")
 
 
 def test_additive_mask_and_kv_len_agree(ctx):
