@@ -76,3 +76,10 @@ extern "C" int mi_transpose_le_f16(void *out, const int64_t out_strides[4], cons
     }
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
+
+// A hoisted [K][F] weight re-laid as [F][K], once at model load: the 2-D case of the transpose above.
+extern "C" int mi_relayout_weight_f16(void *w_fk, int64_t ld_fk, const void *w_kf, int64_t ld_kf, int64_t K, int64_t F, void *stream) {
+    if (ld_kf < F || ld_fk < K) return MI_DECLINE_EXTENT;
+    const int64_t in_strides[4] = {1, ld_kf, 0, 0}, out_strides[4] = {1, ld_fk, 0, 0};
+    return mi_transpose_le_f16(w_fk, out_strides, w_kf, in_strides, F, K, 1, 1, stream);
+}

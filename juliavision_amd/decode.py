@@ -19,7 +19,7 @@ from typing import Callable, List, Optional
 import torch
 
 from . import _lib as L
-from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, matmul_heads_, sdpa, sdpa_append, transposeLE_
+from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, matmul_heads_, relayout_weight, sdpa, sdpa_append
 
 
 # Fold the cache write into the self-attention launch where the one-launch kernel covers the shape.
@@ -118,9 +118,7 @@ class DecoderLayerWeights:
             if w.stride(0) == 1:                           # already [F][K]
                 out[name] = w
                 continue
-            fk = torch.empty((w.shape[1], w.shape[0]), dtype=w.dtype, device=w.device)
-            transposeLE_(ctx, fk, w)
-            out[name] = fk.t()
+            out[name] = relayout_weight(ctx, w)
         return replace(self, **out)
 
 

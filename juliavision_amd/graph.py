@@ -91,17 +91,26 @@ class UnsupportedOp(NotImplementedError):
 
 # ----------------------------------------------------------------------------- schema
 
-def _const(x):
-    if isinstance(x, float) and not math.isfinite(x):
-        return "-inf" if x < 0 else ("inf" if x > 0 else "nan")
-    if isinstance(x, (int, float, bool, str)) or x is None:
-        return x
-    if isinstance(x, (list, tuple)):
-        return [_const(v) for v in x]
-    if isinstance(x, torch.dtype):
-        return str(x).replace("torch.", "")
-    if isinstance(x, torch.device):
-        return None
+def _json_dtype(dt) -> str:
+    return str(dt).replace("torch.", "")
+
+
+# How a literal argument of an exported node is written into the JSON: first matching row wins.  Non-finite floats
+# have no JSON form and travel as text; a device carries nothing the executor needs.
+_LITERAL_FORMS = (
+    (lambda x: isinstance(x, float) and math.isnan(x), lambda x: "nan"),
+    (lambda x: isinstance(x, float) and math.isinf(x), lambda x: "inf" if x > 0 else "-inf"),
+    (lambda x: x is None or isinstance(x, (bool, int, float, str)), lambda x: x),
+    (lambda x: isinstance(x, (list, tuple)), lambda x: [_literal(v) for v in x]),
+    (lambda x: isinstance(x, torch.dtype), _json_dtype),
+    (lambda x: isinstance(x, torch.device), lambda x: None),
+)
+
+
+def _literal(x):
+    for matches, encode in _LITERAL_FORMS:
+        if matches(x):
+            return encode(x)
     return str(x)
 
 
@@ -162,89 +171,142 @@ def evalexpr(expr, dims: Dict[str, int]) -> int:
     return int(math.floor(walk(ast.parse(str(expr), mode="eval").body)))
 
 
+class _SchemaWriter:
+    """Collects the records of one exported program in the reference's JSON schema (export_graphs.py:111-230:
+    ``buffers`` of kind weight / external / transient / view / host, ``ops`` with ``aten`` / ``in`` / ``out`` /
+    ``attrs``).  One method per kind of fx node; liveness is worked out afterwards from the finished records."""
+
+    SCALAR_RESULTS = (int, bool, float, torch.SymInt, torch.SymBool, torch.SymFloat)
+
+    def __init__(self, state_keys: Dict[str, str]):
+        self.state_keys = state_keys        # placeholder name -> state-dict key, for parameters, buffers and lifted constants
+        self.buffers: Dict[str, Dict[str, Any]] = {}
+        self.ops: List[Dict[str, Any]] = []
+        self.inputs: List[str] = []
+        self.outputs: List[str] = []
+        self.symbols: set = set()
+
+    # -- records
+    def _tensor_fields(self, val) -> Dict[str, Any]:
+        if isinstance(val, (tuple, list)):       # a tuple-returning op: one entry per element, None for non-tensors
+            return {"shapes": [list(v.shape) if hasattr(v, "shape") else None for v in val],
+                    "dtypes": [_json_dtype(v.dtype) if hasattr(v, "dtype") else None for v in val]}
+        if val is not None and hasattr(val, "shape"):
+            return {"shape": [_dim(d, self.symbols) for d in val.shape], "dtype": _json_dtype(val.dtype)}
+        return {}
+
+    def _buffer(self, nid: str, kind: str, val=None, **fields):
+        self.buffers[nid] = {"id": nid, "kind": kind, **self._tensor_fields(val), **fields}
+
+    # -- arguments of a call: tensor operands by name, everything else as attributes
+    def _operands_and_attrs(self, node):
+        import torch.fx as fx
+        operands: List[str] = []
+        attrs: Dict[str, Any] = {}
+
+        def tensor(a):
+            return isinstance(a, fx.Node)
+
+        for pos, a in enumerate(node.args):
+            key = f"arg{pos}"
+            if tensor(a):
+                operands.append(a.name)
+            elif isinstance(a, (list, tuple)) and any(tensor(v) for v in a):
+                # a list that mixes tensors and literals (cat's operands, index's indices): the tensors join the
+                # operands, the attribute keeps the list's shape with "$name" where a tensor stood
+                operands.extend(v.name for v in a if tensor(v))
+                attrs[key] = ["$" + v.name if tensor(v) else _literal(v) for v in a]
+            else:
+                attrs[key] = _literal(a)
+                _note_symbols(a, self.symbols)
+        for key, a in node.kwargs.items():
+            if tensor(a):
+                operands.append(a.name)
+            else:
+                attrs[key] = _literal(a)
+        return operands, attrs
+
+    # -- one method per fx node kind
+    def placeholder(self, node):
+        val = node.meta.get("val")
+        key = self.state_keys.get(node.name)
+        if key is None:
+            self._buffer(node.name, "external", val)
+            self.inputs.append(node.name)
+        else:
+            self._buffer(node.name, "weight", val, key=key)
+
+    def call_function(self, node):
+        target = str(node.target).replace("aten.", "")
+        if target in DROP_OPS:
+            return
+        operands, attrs = self._operands_and_attrs(node)
+        val = node.meta.get("val")
+        if isinstance(val, self.SCALAR_RESULTS):
+            # a size computed on the host (sym_size, h * w): a named scalar that views refer to as "$name"
+            self.buffers[node.name] = {"id": node.name, "kind": "host", "expr": _dim(val, self.symbols)}
+        elif target in VIEW_OPS or "getitem" in target:
+            self._buffer(node.name, "view", val, of=operands[0] if operands else None, op=target, attrs=attrs)
+        else:
+            self._buffer(node.name, "transient", val)
+            self.ops.append({"id": node.name, "aten": target, "in": operands, "out": node.name,
+                             "attrs": {k: v for k, v in attrs.items() if v is not None}})
+
+    def output(self, node):
+        import torch.fx as fx
+        results = node.args[0]
+        if not isinstance(results, (list, tuple)):
+            results = [results]
+        self.outputs.extend(r.name for r in results if isinstance(r, fx.Node))
+
+    def get_attr(self, node):
+        raise UnsupportedOp(f"get_attr node {node.name}: export the program with its constants lifted to inputs")
+
+    # -- after the walk
+    def _mark_liveness(self):
+        """A transient's ``live`` interval, in op indices: from the op that writes it to the last op that reads it,
+        directly or through any chain of views; a transient nobody reads lives to the end.  Results of the program
+        are the caller's memory (``external``) and carry no interval."""
+        def storage(bid):
+            seen = set()
+            while bid in self.buffers and self.buffers[bid]["kind"] == "view" and self.buffers[bid].get("of") and bid not in seen:
+                seen.add(bid)
+                bid = self.buffers[bid]["of"]
+            return bid
+
+        written = {op["out"]: i for i, op in enumerate(self.ops)}
+        last_read: Dict[str, int] = {}
+        for i, op in enumerate(self.ops):
+            for operand in op["in"]:
+                last_read[storage(operand)] = i
+        for bid, b in self.buffers.items():
+            if b["kind"] != "transient":
+                continue
+            if bid in self.outputs:
+                b["kind"] = "external"
+            else:
+                b["live"] = [written.get(bid, 0), last_read.get(bid, len(self.ops))]
+
+    def finish(self, name: str) -> Dict[str, Any]:
+        self._mark_liveness()
+        return {"name": name, "symbols": sorted(self.symbols), "inputs": self.inputs, "outputs": self.outputs,
+                "buffers": list(self.buffers.values()), "ops": self.ops, "fusion_groups": [], "barriers": []}
+
+
 def convert(ep, name: str = "graph") -> Dict[str, Any]:
     """``ExportedProgram`` -> the buffers/ops dictionary (the schema of export_graphs.py:111-230).  Parameters
     and buffers become ``weight`` buffers keyed by their state-dict name, user inputs and outputs ``external``,
     view ops ``view`` buffers that alias their parent, sizes computed on the host ``host`` scalars, everything
     else an op with a ``transient`` result and a ``live`` interval in op indices.  Symbolic extents stay
     expressions in torch's own symbol names (``s0`` ...), listed under ``symbols``."""
-    import torch.fx as fx
     sig = ep.graph_signature
-    key_of = dict(sig.inputs_to_parameters)
-    key_of.update(sig.inputs_to_buffers)
-    key_of.update(getattr(sig, "inputs_to_lifted_tensor_constants", {}))
-    buffers: Dict[str, Dict[str, Any]] = {}
-    ops: List[Dict[str, Any]] = []
-    inputs, outputs = [], []
-    born, last = {}, {}
-    symbols: set = set()
-
-    def describe(nid, val, kind, **extra):
-        b = {"id": nid, "kind": kind}
-        if isinstance(val, (tuple, list)):
-            b["shapes"] = [list(v.shape) if hasattr(v, "shape") else None for v in val]
-            b["dtypes"] = [str(v.dtype).replace("torch.", "") if hasattr(v, "dtype") else None for v in val]
-        elif val is not None and hasattr(val, "shape"):
-            b["shape"] = [_dim(d, symbols) for d in val.shape]
-            b["dtype"] = str(val.dtype).replace("torch.", "")
-        b.update(extra)
-        buffers[nid] = b
-
-    for n in ep.graph.nodes:
-        if n.op == "placeholder":
-            if n.name in key_of:
-                describe(n.name, n.meta.get("val"), "weight", key=key_of[n.name])
-            else:
-                describe(n.name, n.meta.get("val"), "external")
-                inputs.append(n.name)
-        elif n.op == "call_function":
-            target = str(n.target).replace("aten.", "")
-            if target in DROP_OPS:
-                continue
-            at = len(ops)
-            args, attrs = [], {}
-            for j, a in enumerate(n.args):
-                if isinstance(a, fx.Node):
-                    args.append(a.name)
-                    last[a.name] = at
-                elif isinstance(a, (list, tuple)) and any(isinstance(v, fx.Node) for v in a):
-                    for v in a:
-                        if isinstance(v, fx.Node):
-                            args.append(v.name)
-                            last[v.name] = at
-                    attrs[f"arg{j}"] = [f"${v.name}" if isinstance(v, fx.Node) else _const(v) for v in a]
-                else:
-                    attrs[f"arg{j}"] = _const(a)
-                    _note_symbols(a, symbols)
-            for k, v in n.kwargs.items():
-                if isinstance(v, fx.Node):
-                    args.append(v.name)
-                    last[v.name] = at
-                else:
-                    attrs[k] = _const(v)
-            val = n.meta.get("val")
-            born[n.name] = at
-            if isinstance(val, (int, bool, float, torch.SymInt, torch.SymBool, torch.SymFloat)):
-                # a size computed on the host (sym_size, h * w): a named scalar the views that use it refer to as "$name"
-                buffers[n.name] = {"id": n.name, "kind": "host", "expr": _dim(val, symbols)}
-                continue
-            if "getitem" in target or target in VIEW_OPS:
-                describe(n.name, val, "view", of=args[0] if args else None, op=target, attrs=attrs)
-                continue
-            describe(n.name, val, "transient")
-            ops.append({"id": n.name, "aten": target, "in": args, "out": n.name,
-                        "attrs": {k: v for k, v in attrs.items() if v is not None}})
-        elif n.op == "output":
-            flat = n.args[0] if isinstance(n.args[0], (list, tuple)) else [n.args[0]]
-            outputs += [a.name for a in flat if isinstance(a, fx.Node)]
-    for bid, b in buffers.items():
-        if b["kind"] == "transient":
-            if bid in outputs:
-                b["kind"] = "external"
-            else:
-                b["live"] = [born.get(bid, 0), last.get(bid, len(ops))]
-    return {"name": name, "symbols": sorted(symbols), "inputs": inputs, "outputs": outputs, "buffers": list(buffers.values()),
-            "ops": ops, "fusion_groups": [], "barriers": []}
+    state_keys: Dict[str, str] = {}
+    for table in ("inputs_to_parameters", "inputs_to_buffers", "inputs_to_lifted_tensor_constants"):
+        state_keys.update(getattr(sig, table, {}))
+    writer = _SchemaWriter(state_keys)
+    for node in ep.graph.nodes:
+        getattr(writer, node.op)(node)
+    return writer.finish(name)
 
 
 @dataclass

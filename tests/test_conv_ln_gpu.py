@@ -416,6 +416,16 @@ def test_standalone_activation_is_the_epilogue_function(ctx, kind):
     got, want = to_host(out).astype(np.float64), oracle.act_f16(a, kind).astype(np.float64)
     assert np.max(np.abs(got - want)) <= 2e-3 * max(1.0, np.max(np.abs(want)))        # device exp / rcp against libm: an ulp of fp16
     assert_parity(got, want, what=kind)
+    # the ends of the fp16 range: a linear whose sum overflowed hands the activation +-65504 or +inf, and the
+    # reference's expression returns them unchanged on the positive side and (signed) zero on the negative
+    edge = np.array([6.0, 14.0, 100.0, 1000.0, 65504.0, np.inf, -6.0, -14.0, -100.0, -1000.0, -65504.0], dtype=np.float16)
+    out = poison(torch.empty(edge.shape, dtype=torch.float16, device="cuda"))
+    jv.act_(ctx, out, to_dev(edge), kind)
+    torch.cuda.synchronize()
+    got, want = to_host(out), oracle.act_f16(edge, kind)
+    assert not np.isnan(got).any(), got
+    assert np.array_equal(got[3:6], want[3:6]) and np.array_equal(np.abs(got[7:]), np.abs(want[7:])), (got, want)
+    assert np.allclose(got.astype(np.float64)[:3], want.astype(np.float64)[:3], rtol=2e-3)
 
 
 def test_clamp_bit_exact(ctx):
