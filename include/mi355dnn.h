@@ -78,6 +78,19 @@ int mi_device_caps(int64_t out[6]);
  * launch ran at.  The caller keeps the buffer alive while it is registered.  Process-wide, not thread safe. */
 int mi_set_clock_probe(void *dev_u64x4);
 
+/* Ceiling probes (measurement aids, no counterpart in the reference).
+ * mi_probe_mfma: `workgroups` workgroups of eight waves run `steps` 64-deep steps of the 128 x 256 GEMM tile's
+ * arithmetic -- sixteen v_mfma_f32_32x32x16_f16 per wave and step, 2 x 8 x 16 x 32768 flop per workgroup and step --
+ * on operand fragments held in registers, with no memory operation in the loop; gelu != 0 adds the GEMM epilogue's
+ * arithmetic (bias, rounding, erf-GELU) on every accumulator value.  seed_f16: 65536 fp16 values the fragments are
+ * taken from (random values make the multipliers toggle as on real data); sink: 512 x workgroups floats that are never
+ * actually written.  240 workgroups x 20 steps with gelu is config 1's launch minus its memory traffic; a grid of many
+ * rounds is what the matrix units sustain at the clock the chip holds under that load.
+ * mi_probe_copy: out[0 .. bytes) = in[0 .. bytes), 16 bytes per lane and step; bytes % 16 == 0.  A kernel of known HBM
+ * traffic (bytes read + bytes written). */
+int mi_probe_mfma(void *sink, const void *seed_f16, int64_t workgroups, int64_t steps, int gelu, void *stream);
+int mi_probe_copy(void *out, const void *in, size_t bytes, void *stream);
+
 /* Device-side failures (no counterpart in the reference, whose kernels never wait for one another).  A few kernels
  * here exchange data between workgroups inside one launch and wait for each other a bounded time; a wait that gives
  * up cannot be reported by the call that enqueued the launch, so it is recorded in a sticky word in device memory.

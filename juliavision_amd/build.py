@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmi355dnn.so")
-SOURCES = ["gemm.hip", "sdpa.hip", "conv.hip", "convtranspose.hip", "layernorm.hip", "kvcache.hip", "layout.hip"]
+SOURCES = ["gemm.hip", "sdpa.hip", "conv.hip", "convtranspose.hip", "layernorm.hip", "kvcache.hip", "layout.hip", "probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 # -Xarch_device -fno-honor-nans: no kernel relies on NaN propagation (infinities stay honoured: they are the masks);

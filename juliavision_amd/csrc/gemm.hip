@@ -728,9 +728,23 @@ __device__ __noinline__ void sk_poison_region(void *Y, long ldY, int M, int N, i
     }
 }
 
+// With three 64-deep stages a ninth wave does nothing but request operand tiles (pp_loader).  A 1 KB
+// global_load_lds_dwordx4 takes the CU's vector-memory path sixteen clocks, so a wave that issues its share of a tile
+// stands at those instructions while its three partners' requests drain ahead of it -- 190 of the 750 clocks of a
+// memory phase, measured, against 530 clocks of the matrix phase, and moving the requests between a wave's own MFMAs
+// only moved the cost (716 clocks of matrix phase).  The loader wave issues all 48 requests of a tile, half in each
+// phase, waits for the tile the next phase will read, and joins every workgroup barrier; the eight matrix waves issue
+// no vector-memory instruction inside the loop.  Three waves then share one SIMD, which leaves 168 registers a wave:
+// the 256 x 256 tile (217) keeps the scheme in which every wave requests its own share.
+template <int BK, int STAGES, bool PINGPONG>
+constexpr bool pp_loader() { return PINGPONG && BK == 64 && STAGES == 3; }
+template <int BK, int STAGES, bool PINGPONG>
+constexpr int pp_threads() { return pp_loader<BK, STAGES, PINGPONG>() ? 576 : 512; }
+
 template <int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool B_KN, bool PINGPONG, bool SK = false>
-__global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
+__global__ __launch_bounds__((pp_threads<BK, STAGES, PINGPONG>())) void gemm_pp_kernel(GemmArgs p) {
     static_assert(WAVES_M * WAVES_N == 8, "two groups of four waves");
+    constexpr bool LOADER = pp_loader<BK, STAGES, PINGPONG>();
     static_assert(BK == 64 || BK == 32, "rows of 128 or 64 bytes");
     constexpr int NT = 512, KS = BK / 16, CPR = BK / 8, ROWB = BK * 2;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
@@ -771,42 +785,109 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
 
     // K-contiguous rows: LDS position pos of row r holds chunk pos ^ rowswz(r)
     auto rowswz = [](int r) { return BK == 64 ? (r & 7) ^ ((r >> 3) & 1) : (r >> 2) & 3; };
-    uint32_t aoffg[PA], boffg[PB];
-#pragma unroll
-    for (int i = 0; i < PA; i++) {
-        const int q = (i * 8 + wave) * 64 + lane, r = q / CPR, pos = q % CPR;
+    // per-lane byte offsets of the 1 KB slots that wave w of eight requests: slot i of the A part, slot i of the B part
+    auto a_offset = [&](int w, int i) {
+        const int q = (i * 8 + w) * 64 + lane, r = q / CPR, pos = q % CPR;
         const int c = pos ^ rowswz(r);
-        aoffg[i] = (uint32_t)(((long)(min(m0 + r, p.M - 1) - m0) * p.ldA + c * 8) * 2);
-    }
-#pragma unroll
-    for (int i = 0; i < PB; i++) {
-        const int q = (i * 8 + wave) * 64 + lane;
+        return (uint32_t)(((long)(min(m0 + r, p.M - 1) - m0) * p.ldA + c * 8) * 2);
+    };
+    auto b_offset = [&](int w, int i) {
+        const int q = (i * 8 + w) * 64 + lane;
         if (!B_KN) {
             const int r = q / CPR, pos = q % CPR;
             const int c = pos ^ rowswz(r);
-            boffg[i] = (uint32_t)(((long)(min(n0 + r, p.N - 1) - n0) * p.ldB + c * 8) * 2);
+            return (uint32_t)(((long)(min(n0 + r, p.N - 1) - n0) * p.ldB + c * 8) * 2);
         } else {
             constexpr int CPRB = BN / 8;
             const int k = q / CPRB, pos = q % CPRB;
             const int j = pos ^ ((k & 3) << 2);
-            boffg[i] = (uint32_t)(((long)k * p.ldB + (min(n0 + j * 8, p.NB - 8) - n0)) * 2);
+            return (uint32_t)(((long)k * p.ldB + (min(n0 + j * 8, p.NB - 8) - n0)) * 2);
+        }
+    };
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
+    auto barrier = [&]() {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    if constexpr (LOADER) {
+        if (wave == 8) {
+            // The loader wave.  Barrier b closes phase b - 1 (barrier 0 closes the prologue); tile t lives in stage
+            // t % 3, is read in phases 2t (leading group) and 2t + 1 (trailing group), and its stage is free from
+            // phase 2t + 2: tile kt + 2 is requested in phases 2kt and 2kt + 1, a half of its 48 slots in each, and
+            // has to have landed when phase 2kt + 3 ends.  Requests complete in order, so "tile t has landed" is
+            // "no more requests outstanding than were issued after it".
+            constexpr int PER_TILE = 8 * NL;
+            static_assert(PER_TILE <= 63, "vmcnt is a 6-bit counter");
+            uint32_t offa[8][PA], offb[8][PB];
+#pragma unroll
+            for (int w = 0; w < 8; w++) {
+#pragma unroll
+                for (int i = 0; i < PA; i++) offa[w][i] = a_offset(w, i);
+#pragma unroll
+                for (int i = 0; i < PB; i++) offb[w][i] = b_offset(w, i);
+            }
+            auto request = [&](int kt, int stage, int half) {      // half 0 / 1: the slots of waves 0-3 / 4-7; 2: all
+                const char *ab = reinterpret_cast<const char *>(Ag) + (long)kt * a_step;
+                const char *bb = reinterpret_cast<const char *>(Bg) + (long)kt * b_step;
+#pragma unroll
+                for (int w = 0; w < 8; w++) {
+                    if (half != 2 && (w >> 2) != half) continue;
+                    const uint32_t sa = lds0 + stage * STAGE_BYTES + w * 1024, sb = sa + A_BYTES;
+#pragma unroll
+                    for (int i = 0; i < PA; i++) {
+                        const uint32_t dst = __builtin_amdgcn_readfirstlane(sa + i * 8192);
+                        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offa[w][i]), "s"(ab), "s"(dst) : "memory");
+                    }
+#pragma unroll
+                    for (int i = 0; i < PB; i++) {
+                        const uint32_t dst = __builtin_amdgcn_readfirstlane(sb + i * 8192);
+                        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offb[w][i]), "s"(bb), "s"(dst) : "memory");
+                    }
+                }
+            };
+            request(0, 0, 2);
+            if (nk > 1) { request(1, 1, 2); asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory"); }
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            barrier();
+            for (int ph = 0; ph < 2 * nk; ph++) {
+                const int kt = ph >> 1, half = ph & 1, t = kt + 2;
+                if (t < nk) {
+                    const int stage = t % 3;
+                    if (half == 0) request(t, stage, 0); else request(t, stage, 1);
+                }
+                if (half == 1) {      // the next phase reads tile kt + 1
+                    if (t < nk) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory");
+                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                }
+                barrier();
+            }
+            return;
         }
     }
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
+    uint32_t aoffg[PA], boffg[PB];
+    if constexpr (!LOADER) {
+#pragma unroll
+        for (int i = 0; i < PA; i++) aoffg[i] = a_offset(wave, i);
+#pragma unroll
+        for (int i = 0; i < PB; i++) boffg[i] = b_offset(wave, i);
+    }
     // the wave's 1 KB slots inside a stage
     auto issue = [&](int kt, int stage) {
-        const char *ab = reinterpret_cast<const char *>(Ag) + (long)kt * a_step;
-        const char *bb = reinterpret_cast<const char *>(Bg) + (long)kt * b_step;
-        const uint32_t sa = lds0 + stage * STAGE_BYTES + wave * 1024, sb = sa + A_BYTES;
+        if constexpr (!LOADER) {
+            const char *ab = reinterpret_cast<const char *>(Ag) + (long)kt * a_step;
+            const char *bb = reinterpret_cast<const char *>(Bg) + (long)kt * b_step;
+            const uint32_t sa = lds0 + stage * STAGE_BYTES + wave * 1024, sb = sa + A_BYTES;
 #pragma unroll
-        for (int i = 0; i < PA; i++) {
-            const uint32_t dst = __builtin_amdgcn_readfirstlane(sa + i * 8192);
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(aoffg[i]), "s"(ab), "s"(dst) : "memory");
-        }
+            for (int i = 0; i < PA; i++) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(sa + i * 8192);
+                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(aoffg[i]), "s"(ab), "s"(dst) : "memory");
+            }
 #pragma unroll
-        for (int i = 0; i < PB; i++) {
-            const uint32_t dst = __builtin_amdgcn_readfirstlane(sb + i * 8192);
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(boffg[i]), "s"(bb), "s"(dst) : "memory");
+            for (int i = 0; i < PB; i++) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(sb + i * 8192);
+                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(boffg[i]), "s"(bb), "s"(dst) : "memory");
+            }
         }
     };
 
@@ -868,16 +949,15 @@ __global__ __launch_bounds__(512, 2) void gemm_pp_kernel(GemmArgs p) {
     const bool probe = p.clk && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0;
     if (probe) { p.clk[0] = clock64(); p.clk[1] = wall_clock64(); }
     // this wave's loads of tile kt + 1 have landed: only the tiles requested after it may still be in flight
+    // (with a loader wave the matrix waves have no requests of their own to wait for: the loader waits for the tile
+    // ahead of the barrier that everybody passes)
     auto wait_next = [&](int kt) {
-        const int newer = min(kt + STAGES - 1, nk - 1) - (kt + 1);
-        if (newer >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NL) : "memory");
-        else if (newer == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    };
-    auto barrier = [&]() {
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
+        if constexpr (!LOADER) {
+            const int newer = min(kt + STAGES - 1, nk - 1) - (kt + 1);
+            if (newer >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NL) : "memory");
+            else if (newer == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
     };
 
 #pragma unroll
@@ -1771,8 +1851,9 @@ int launch_pp(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     a.clk = g_clock_probe;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
     constexpr int lds = pp_lds_bytes<BM, BN, BK, STAGES>();
-    if (b_kn) hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, BK, STAGES, WM, WN, true, PP>), grid, dim3(512), lds, st, a);
-    else      hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, BK, STAGES, WM, WN, false, PP>), grid, dim3(512), lds, st, a);
+    constexpr int threads = pp_threads<BK, STAGES, PP>();
+    if (b_kn) hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, BK, STAGES, WM, WN, true, PP>), grid, dim3(threads), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, BK, STAGES, WM, WN, false, PP>), grid, dim3(threads), lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
@@ -1803,8 +1884,9 @@ int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
     a.clk = g_clock_probe;
     dim3 grid((unsigned)(8 * a.sk_tpx * split), 1);
     constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
-    if (b_kn) hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, 64, 3, 2, 4, true, true, true>), grid, dim3(512), lds, st, a);
-    else      hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, 64, 3, 2, 4, false, true, true>), grid, dim3(512), lds, st, a);
+    constexpr int threads = pp_threads<64, 3, true>();
+    if (b_kn) hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, 64, 3, 2, 4, true, true, true>), grid, dim3(threads), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, 64, 3, 2, 4, false, true, true>), grid, dim3(threads), lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 

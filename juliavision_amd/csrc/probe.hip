@@ -1,0 +1,89 @@
+// Measurement kernels (no counterpart in the reference): what the matrix units and the memory system of THIS box
+// deliver when nothing else is in the way, so that a benchmark can print the ceilings next to its results instead
+// of assuming the vendor's figures.
+//
+//   probe_mfma_kernel   the arithmetic of the 128 x 256 GEMM tile with every memory operation removed: eight waves
+//                       per workgroup, two per SIMD, each with a 2 x 2 block of 32 x 32 accumulators and, per 64-deep
+//                       step, sixteen v_mfma_f32_32x32x16_f16 on operand fragments that sit in registers (random
+//                       fp16 values, so the multipliers toggle as they do on real data); optionally the GEMM's
+//                       epilogue arithmetic (bias, rounding, erf-GELU on the rounded value) on all 64 values a lane
+//                       holds.  Nothing is stored unless the results are impossible, which the compiler cannot know.
+//   probe_copy_kernel   out[i] = in[i], sixteen bytes per lane and step: a kernel of known HBM traffic, for timing
+//                       the memory system and for scaling the FETCH_SIZE / WRITE_SIZE counters of rocprofv3.
+#include "common.hpp"
+
+namespace {
+
+__global__ __launch_bounds__(512, 2) void probe_mfma_kernel(float *sink, const half_t *seed, int steps, int gelu) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // operand fragments of the four k-steps of a 64-deep step: 2 of A and 2 of B each, distinct random values per lane
+    half8v fa[4][2], fb[4][2];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            fa[ks][j] = *reinterpret_cast<const half8v *>(seed + (((ks * 2 + j) * 8 + wave) * 64 + lane) * 8);
+            fb[ks][j] = *reinterpret_cast<const half8v *>(seed + (((8 + ks * 2 + j) * 8 + wave) * 64 + lane) * 8);
+        }
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    for (int s = 0; s < steps; s++) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks][i], fa[ks][j], acc[i][j], 0, 0, 0);
+        // keeps the loop a loop (no hoisting of the whole chain) without touching memory
+        asm volatile("" : "+v"(fa[0][0]));
+    }
+    float t = 0.0f;
+    const float bias = (float)fa[0][0][0];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float v = acc[i][j][r] * 1e-3f;
+                if (gelu) v = (float)(half_t)gelu_erf((float)(half_t)(v + bias));
+                t += v;
+            }
+    if (t == 12345.6789f) sink[blockIdx.x * 512 + threadIdx.x] = t;
+}
+
+__global__ __launch_bounds__(256) void probe_copy_kernel(u32x4 *out, const u32x4 *in, long n16) {
+    const long stride = (long)gridDim.x * 256;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) out[i] = in[i];
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_probe_mfma(void *sink, const void *seed_f16, int64_t workgroups, int64_t steps, int gelu, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!sink || !seed_f16 || !aligned_to(seed_f16, 16)) return MI_DECLINE_OPERANDS;
+    if (workgroups < 1 || workgroups > (1 << 20) || steps < 1 || steps > (1 << 24)) return MI_DECLINE_EXTENT;
+    hipLaunchKernelGGL(probe_mfma_kernel, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream,
+                       reinterpret_cast<float *>(sink), reinterpret_cast<const half_t *>(seed_f16), (int)steps, gelu);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_probe_copy(void *out, const void *in, size_t bytes, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!out || !in || !aligned_to(out, 16) || !aligned_to(in, 16) || bytes % 16) return MI_DECLINE_OPERANDS;
+    if (bytes == 0) return MI_OK;
+    const long n16 = (long)(bytes / 16);
+    const long want = ceil_div(n16, 256 * 8), cap = (long)mi_num_cus() * 16;
+    hipLaunchKernelGGL(probe_copy_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<u32x4 *>(out), reinterpret_cast<const u32x4 *>(in), n16);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+}  // extern "C"
