@@ -216,6 +216,42 @@ int mi_gemm_clamp_ln_f16(void *Y, void *H, const void *X, const void *W, const v
 
 size_t mi_gemm_f16_workspace(int64_t T, int64_t K, int64_t F, int w_layout, int64_t nbatch);
 
+/* ---- a layer norm with no pass of its own
+ * layernorm! followed by matmul! (layernorm.jl:125, matmul.jl:78-79) is, algebraically,
+ *     LN(x) . W + b  =  r (x . W') - r mu colsum(W') + b',      W'[k][n] = gamma[k] W[k][n],  b' = b + beta . W,
+ * with (mu, r) the row's mean and 1 / sqrt(var + eps): the GEMM can run on the RAW rows and apply a per-row scale and
+ * a rank-one correction in its store, if it knows (mu, r) -- and the GEMM that WROTE the rows can leave what is needed
+ * behind.  Three pieces:
+ *   mi_lnfold_prepare_f16   once per weight, at load: Wp = fp16(gamma W) in W's layout, colsum[F] (of the rounded Wp)
+ *                           and biasp[F] in fp32.  gamma, beta, bias may be NULL.
+ *   row statistics          stats[ceil(C / 32)][rows][2] fp32: for every 32-column segment of a row, the sum and the
+ *                           squares about the segment's own mean (segment-major, so that a wave reads the segments of
+ *                           64 consecutive rows as contiguous 512 bytes).  Written by mi_gemm_rowstats_f16 (mi_gemm_f16 with
+ *                           dense rows of Y, ldY = F, that also leaves the statistics of the final fp16 rows, after
+ *                           residual and clamp), by mi_lnfold_gemm_f16 (stats_out), or by mi_rowstats_f16 for rows that
+ *                           no GEMM of this library wrote (a block's first input).
+ *   mi_lnfold_gemm_f16      Y = epi(round(r (X . Wp) - r mu colsum + biasp)) (+ residual), (mu, r) combined per row
+ *                           from stats_in (segment sums -> mean; squares about that mean by the pairwise update, never
+ *                           as sum(x^2) - n mu^2).  nbatch planes share X and stats_in (sY, sW, sVec = plane strides of
+ *                           Y, Wp, colsum / biasp): q, k, v in one launch.  T > 8, K % 64 == 0, K >= 128, 16-byte rows;
+ *                           anything else returns a decline and the caller runs the two ops.
+ * What differs from the two ops: the reference rounds the normalised row to fp16 before the product; here the rounding
+ * sits on gamma W instead and the normalised row is never formed.  Same order of error (one fp16 rounding of one
+ * factor per product term), not the same bits: held to the 1e-2 / 0.9999 gate against layernorm -> GEMM, not to
+ * bit-identity (mi_ln_gemm_f16 is the bit-identical fold).  The reference's own plans name the fold of the norm into
+ * the GEMM as open work (plans/kernels-to-port.md item 3; plans/perf-plan.md:4074-4095). */
+int mi_lnfold_prepare_f16(void *Wp, float *colsum, float *biasp, const void *W, const void *gamma, const void *beta, const void *bias,
+                          int64_t K, int64_t F, int64_t ldW, int w_layout, void *stream);
+int mi_rowstats_f16(float *stats, const void *a, int64_t ld, int64_t C, int64_t rows, void *stream);
+int mi_gemm_rowstats_f16(void *Y, float *stats, const void *X, const void *W, const void *bias, const void *residual, float clamp,
+                         int64_t T, int64_t K, int64_t F, int64_t ldX, int64_t ldW,
+                         int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream);
+int mi_lnfold_gemm_f16(void *Y, float *stats_out, const void *X, const float *stats_in, float eps,
+                       const void *Wp, const float *colsum, const float *biasp, const void *residual, float clamp,
+                       int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                       int w_layout, int epi, int out_dtype,
+                       int64_t nbatch, int64_t sY, int64_t sW, int64_t sVec, void *ws, size_t ws_bytes, void *stream);
+
 /* mi_gemm_f16 without the workspace arguments, for callers that cannot allocate device memory and have no
  * workspace to hand over: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * It has no counterpart in the reference (whose kernels always draw scratch from the caller's bump workspace,

@@ -12,7 +12,7 @@ the weight-file reader.
 """
 from . import _lib  # noqa: F401
 from .kernels import (Ctx, Decline, DeclineError, DeviceCaps, MI355X, Workspace, act_, add_, batchedmatmul_, caps, clamp_, conv_plan,
-                      convolution_, convolution_nhwc_, convolution_tokens_, convolutiontranspose_, convsize, convtranspose_plan, convtransposesize, layernorm_, ln_matmul_, matmul_, matmul_heads_, matmul_ln_, mmplan, relayout_weight, scale_, sdpa, sdpa_append, sdpaplan, softmax_, transposeLE_)
+                      convolution_, convolution_nhwc_, convolution_tokens_, convolutiontranspose_, convsize, convtranspose_plan, convtransposesize, layernorm_, ln_matmul_, lnfold_matmul_, lnfold_prepare, matmul_rowstats_, rowstats_, rowstats_new, LnFoldedLinear, matmul_, matmul_heads_, matmul_ln_, mmplan, relayout_weight, scale_, sdpa, sdpa_append, sdpaplan, softmax_, transposeLE_)
 
 __all__ = ["Ctx", "Decline", "DeclineError", "DeviceCaps", "MI355X", "Workspace", "act_", "add_", "batchedmatmul_", "caps", "clamp_",
-           "conv_plan", "convolution_", "convolution_nhwc_", "convolution_tokens_", "convolutiontranspose_", "convsize", "convtranspose_plan", "convtransposesize", "layernorm_", "ln_matmul_", "matmul_", "matmul_heads_", "matmul_ln_", "mmplan", "relayout_weight", "scale_", "sdpa", "sdpa_append", "sdpaplan", "softmax_", "transposeLE_"]
+           "conv_plan", "convolution_", "convolution_nhwc_", "convolution_tokens_", "convolutiontranspose_", "convsize", "convtranspose_plan", "convtransposesize", "layernorm_", "ln_matmul_", "lnfold_matmul_", "lnfold_prepare", "matmul_rowstats_", "rowstats_", "rowstats_new", "LnFoldedLinear", "matmul_", "matmul_heads_", "matmul_ln_", "mmplan", "relayout_weight", "scale_", "sdpa", "sdpa_append", "sdpaplan", "softmax_", "transposeLE_"]

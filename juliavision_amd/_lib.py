@@ -47,6 +47,10 @@ SIGNATURES = {
     "mi_gemm_ln_f16": (_int, [_vp] * 8 + [_f32] + [_i64] * 5 + [_int] * 3 + [_vp, _sz, _vp]),
     "mi_gemm_clamp_ln_f16": (_int, [_vp] * 8 + [_f32, _f32] + [_i64] * 5 + [_int] * 3 + [_vp, _sz, _vp]),
     "mi_gemm_f16_workspace": (_sz, [_i64, _i64, _i64, _int, _i64]),
+    "mi_lnfold_prepare_f16": (_int, [_vp] * 7 + [_i64, _i64, _i64, _int, _vp]),
+    "mi_rowstats_f16": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
+    "mi_gemm_rowstats_f16": (_int, [_vp] * 6 + [_f32] + [_i64] * 5 + [_int] * 3 + [_vp, _sz, _vp]),
+    "mi_lnfold_gemm_f16": (_int, [_vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _f32] + [_i64] * 6 + [_int] * 3 + [_i64] * 4 + [_vp, _sz, _vp]),
     "mi_gemm_f16_noalloc": (_int, [_vp] * 5 + [_i64] * 6 + [_int] * 4 + [_vp]),
     "mi_gemm_f16_plan": (_int, [_vp] * 3 + [_i64] * 6 + [_int] * 2 + [_i64] * 4),
     "mi_gemm_f16_plan_caps": (_int, [_i64p] + [_vp] * 3 + [_i64] * 6 + [_int] * 2 + [_i64] * 4 + [C.POINTER(C.c_int)]),

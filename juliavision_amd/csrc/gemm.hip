@@ -63,6 +63,17 @@ struct GemmArgs {
     float *sk_part;
     unsigned *sk_flags;
     unsigned sk_epoch;
+    // Layer norm folded away (mi_lnfold_gemm_f16): A holds the raw rows, B carries gamma, and the store turns an
+    // accumulator into r (acc - mu colsum[n]) + biasp[n], with the row's (mu, r) combined from lnf_stats.
+    const float *lnf_stats;           // [lnf_nseg][M][2]: (sum, squares about its own mean) of each 32-column segment of a row
+    const float *lnf_colsum, *lnf_biasp;      // fp32[N], plane stride lnf_svec
+    long lnf_svec;
+    int lnf_nseg;
+    float lnf_eps;
+    // Row statistics of the result for a later folded norm: stats_out[n / 32][m] = (sum, squares about the mean) of the
+    // final fp16 values Y[m][32 (n / 32) .. + 32); stats_nseg segments per row.
+    float *stats_out;
+    int stats_nseg;
     int sk_spin;                      // polls before a wave gives up on its partners
     unsigned sk_pub_xor, sk_xcc_xor;  // zero in ordinary use: mi_test_exchange_faults makes the waits fail from the host side
     unsigned *status;                 // the device's sticky status word
@@ -173,6 +184,74 @@ __device__ __forceinline__ void tile_of(int pid, int nwg, int tiles_m, int tiles
     tn = in / gsz;
 }
 
+// What the store of a folded norm needs, fetched while the first operand tiles are on their way and parked in `slot`
+// (LDS past everything else the kernel keeps there: BM float2 (r, r mu), then BN column sums, then BN biases).
+//
+// A row's mean and reciprocal standard deviation over its K elements come from the per-segment statistics a producer
+// left (stats[seg][row] = (sum, squares about the segment's own mean)).  LPR lanes share a row, each with every LPR-th
+// segment, many loads in flight at a time (a lane that walked all segments one dependent load after the other held
+// the whole workgroup at its first barrier for 10 us).  One pass: the squares between the segments are taken about the
+// first segment's mean, which lies within a segment mean's spread of the row mean, so the final subtraction cancels
+// nothing that matters -- sum(x^2) - n mean^2 about zero would.  r = 1 / sqrt(var + eps), rmu = r * mean.
+// The caller synchronises the workgroup before anybody reads the slot.
+template <int BM, int BN, int NT, typename Args>
+__device__ __forceinline__ void lnf_stage(const Args &p, float2v *slot, int m0, int n0, long bz, int tid) {
+    if (!p.lnf_stats) return;
+    constexpr int LPR = NT >= 4 * BM ? 4 : NT >= 2 * BM ? 2 : 1;
+    static_assert(NT >= BM && (BM * LPR) % 64 == 0, "whole waves work on the rows");
+    if (tid < BM * LPR) {
+        const int row = tid / LPR, q = tid % LPR;
+        const float2v *seg = reinterpret_cast<const float2v *>(p.lnf_stats) + min(m0 + row, p.M - 1);
+        const float ref = seg[0][0] / (float)min(32, p.K);
+        float total = 0.0f, within = 0.0f, between = 0.0f;
+        // U loads in flight per lane: all of a row's segments in one trip to memory for K <= 1536 (2048 with four lanes a
+        // row) -- a trip costs 1 to 2 us here (the statistics were written by another kernel, on other XCDs), and the
+        // first operand tiles, requested before this, take about as long, so one trip is hidden and every further one
+        // is not (two and three batches of eight measured +3.3 and +4.3 us per launch)
+        constexpr int U = LPR == 4 ? 16 : 24;
+        for (int s0 = q; s0 < p.lnf_nseg; s0 += U * LPR) {
+            float2v v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int sg = s0 + u * LPR;
+                const float2v z = {0.0f, 0.0f};
+                v[u] = sg < p.lnf_nseg ? seg[(long)sg * p.M] : z;
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int sg = s0 + u * LPR;
+                if (sg < p.lnf_nseg) {
+                    const int left = p.K - 32 * sg;
+                    const float cnt = left >= 32 ? 32.0f : (float)left, inv = left >= 32 ? 1.0f / 32.0f : 1.0f / (float)left;
+                    const float d = fmaf(v[u][0], inv, -ref);
+                    total += v[u][0];
+                    within += v[u][1];
+                    between = fmaf(cnt * d, d, between);
+                }
+            }
+        }
+        if constexpr (LPR >= 2) { total += lane_xor<1>(total); within += lane_xor<1>(within); between += lane_xor<1>(between); }
+        if constexpr (LPR >= 4) { total += lane_xor<2>(total); within += lane_xor<2>(within); between += lane_xor<2>(between); }
+        if (q == 0) {
+            const float mu = total / (float)p.K, dm = mu - ref;
+            const float m2 = within + fmaxf(between - (float)p.K * dm * dm, 0.0f);
+            const float r = 1.0f / sqrtf(m2 / (float)p.K + p.lnf_eps);
+            const float2v o = {r, r * mu};
+            slot[row] = o;
+        }
+    }
+    // the tile's columns of colsum and biasp
+    for (int t = tid; t < BN / 2; t += NT) {
+        const int which = t / (BN / 4), c = (t % (BN / 4)) * 4, n = n0 + c;
+        const float *src = (which == 0 ? p.lnf_colsum : p.lnf_biasp) + bz * p.lnf_svec;
+        float4v v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (n + 3 < p.N) v = *reinterpret_cast<const float4v *>(src + n);
+        else for (int e = 0; e < 4; e++) if (n + e < p.N) v[e] = src[n + e];
+        *reinterpret_cast<float4v *>(reinterpret_cast<float *>(slot + BM) + which * BN + c) = v;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+
 // ------------------------------------------------------------------------------------------
 // Accumulator tile -> memory, shared by the tiled kernels.
 // acc[i][j][r]: n = n0 + wn*WTN + 32 i + 8 (r/4) + 4 (lane/32) + r%4,  m = m0 + wm*WTM + 32 j + lane%32.
@@ -203,9 +282,18 @@ __device__ __forceinline__ void load_col_bias(const GemmArgs &p, half4v (&cb)[TN
         }
 }
 
+// What the store of a folded layer norm carries (by value, so that it stays in registers): (r, r mu) of the lane's rows
+// m0 + wm WTM + 32 j + lane % 32, and the LDS copy of the tile's colsum (bn floats) followed by its biasp.
+template <int TM>
+struct LnFold {
+    bool on = false;
+    float r[TM] = {}, rmu[TM] = {};
+    const float *col = nullptr;
+    int bn = 0;
+};
 template <int EPI, int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
 __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], char *smem, int m0, int n0, int wm, int wn,
-                                               int wave, int lane, long bz) {
+                                               int wave, int lane, long bz, const LnFold<TM> ln = LnFold<TM>{}) {
     const int frow = lane & 31;
     const half_t *bias = p.bias ? p.bias + bz * p.sBias : nullptr;
     constexpr int SLD_H = WTN + 8;                 // halves per staged row (fp16 output)
@@ -220,13 +308,28 @@ __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc
         const float brow = (p.bias_mode == MI_BIAS_ROW && mrow + frow < p.M) ? (float)bias[mrow + frow] : 0.0f;
 #pragma unroll
         for (int i = 0; i < TN; i++) {
+            // folded layer norm: this lane's columns of colsum and biasp from their LDS copy, a 32-column group at a time
+            float4v lc4[4], lb4[4];
+            if (ln.on) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int nl = 32 * i + 8 * g + 4 * hl;
+                    lc4[g] = *reinterpret_cast<const float4v *>(ln.col + wn * WTN + nl);
+                    lb4[g] = *reinterpret_cast<const float4v *>(ln.col + ln.bn + wn * WTN + nl);
+                }
+            }
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int nl = 32 * i + 8 * g + 4 * hl;
                 const int n = n0 + wn * WTN + nl;
                 float v[4];
+                if (ln.on) {      // uniform: r (acc - mu colsum) + biasp
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + brow + (float)cb[i][g][e];
+                    for (int e = 0; e < 4; e++) v[e] = fmaf(acc[i][j][4 * g + e], ln.r[j], fmaf(-ln.rmu[j], lc4[g][e], lb4[g][e]));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + brow + (float)cb[i][g][e];
+                }
                 if (p.out_f32) {
                     float4v o = {v[0], v[1], v[2], v[3]};
                     *reinterpret_cast<float4v *>(reinterpret_cast<float *>(stage) + frow * SLD_F + nl) = o;
@@ -255,11 +358,13 @@ __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc
             }
         } else {
             constexpr int CPR = WTN / 8;
+            static_assert((32 * CPR) % 64 == 0 && CPR % 4 == 0, "whole waves walk the staged tile; four lanes hold a 32-column segment");
             for (int c = lane; c < 32 * CPR; c += 64) {
                 const int row = c / CPR, ch = c % CPR;
                 const int m = mrow + row, n = n0 + wn * WTN + ch * 8;
+                half8v x = {};
                 if (m < p.M && n < p.N) {
-                    half8v x = *reinterpret_cast<const half8v *>(reinterpret_cast<const half_t *>(stage) + row * SLD_H + ch * 8);
+                    x = *reinterpret_cast<const half8v *>(reinterpret_cast<const half_t *>(stage) + row * SLD_H + ch * 8);
                     const long off = bz * p.sY + (long)m * p.ldY + n;
                     half_t *yp = reinterpret_cast<half_t *>(p.Y) + off;
                     if constexpr (EPI != MI_EPI_NONE) {
@@ -288,6 +393,25 @@ __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc
                         }
                     }
                 }
+                if (p.stats_out) {      // uniform; the launcher admits it with 16-byte stores and N % 8 == 0 only
+                    // the four lanes of a quad hold the 32 columns of one segment of one row (chunks that lie past N
+                    // or below M count nothing): sum, then squares about the segment's own mean, both over the quad
+                    const bool have = m < p.M && n < p.N;
+                    float cnt = have ? 8.0f : 0.0f, sum = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) sum += have ? (float)x[e] : 0.0f;
+                    sum += lane_xor<1>(sum); sum += lane_xor<2>(sum);
+                    cnt += lane_xor<1>(cnt); cnt += lane_xor<2>(cnt);
+                    const float mean = sum / fmaxf(cnt, 1.0f);
+                    float sq = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) { const float d = (float)x[e] - mean; sq = have ? fmaf(d, d, sq) : sq; }
+                    sq += lane_xor<1>(sq); sq += lane_xor<2>(sq);
+                    if (have && (ch & 3) == 0) {
+                        const float2v o = {sum, sq};
+                        *reinterpret_cast<float2v *>(p.stats_out + ((long)(n / 32) * p.M + m) * 2) = o;
+                    }
+                }
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -298,12 +422,12 @@ __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc
 // instead of one per element.
 template <int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
 __device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], char *smem, int m0, int n0, int wm, int wn,
-                                           int wave, int lane, long bz) {
+                                           int wave, int lane, long bz, const LnFold<TM> ln = LnFold<TM>{}) {
     switch (p.epi) {
-    case MI_EPI_GELU_ERF: store_tile_epi<MI_EPI_GELU_ERF, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz); break;
-    case MI_EPI_GELU_TANH: store_tile_epi<MI_EPI_GELU_TANH, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz); break;
-    case MI_EPI_RELU: store_tile_epi<MI_EPI_RELU, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz); break;
-    default: store_tile_epi<MI_EPI_NONE, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz); break;
+    case MI_EPI_GELU_ERF: store_tile_epi<MI_EPI_GELU_ERF, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
+    case MI_EPI_GELU_TANH: store_tile_epi<MI_EPI_GELU_TANH, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
+    case MI_EPI_RELU: store_tile_epi<MI_EPI_RELU, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
+    default: store_tile_epi<MI_EPI_NONE, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
     }
 }
 
@@ -567,6 +691,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
     const int nk = p.K / BK;   // the launcher guarantees K % 64 == 0 and nk >= 2
     gload(0, 0);
     gload(1, 1);
+    // folded layer norm: (r, r mu) of the tile's rows, worked out while the first tiles are on their way and parked
+    // in LDS behind the operand buffers until the store (the barrier after the first LDS write covers it)
+    float2v *ln_slot = reinterpret_cast<float2v *>(smem + 2 * (BM * LD + BSZ) * 2);
+    if constexpr (!LNA) lnf_stage<BM, BN, NT>(p, ln_slot, m0, n0, bz, tid);
     if constexpr (LNA) {
         // One wave per row, all rows of a wave in flight at once (one trip to memory).  Rows past M repeat the last one.
         constexpr int NW = NT / 64, RB = BM / NW;
@@ -667,7 +795,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
         body(M2{}, kt + 1, 1, 0, 1);
     }
     __syncthreads();
-    store_tile<TM, TN, WTM, WTN, WAVES_M * WAVES_N, 2 * (BM * LD + BSZ) * 2>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz);
+    LnFold<TM> ln;
+    if (!LNA && p.lnf_stats) {
+        ln.on = true; ln.col = reinterpret_cast<const float *>(ln_slot + BM); ln.bn = BN;
+#pragma unroll
+        for (int j = 0; j < TM; j++) { const float2v v = ln_slot[wm * WTM + 32 * j + (lane & 31)]; ln.r[j] = v[0]; ln.rmu[j] = v[1]; }
+    }
+    store_tile<TM, TN, WTM, WTN, WAVES_M * WAVES_N, 2 * (BM * LD + BSZ) * 2>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -865,6 +999,12 @@ __global__ __launch_bounds__((pp_threads<BK, STAGES, PINGPONG>())) void gemm_pp_
             return;
         }
     }
+    // folded layer norm: (r, r mu) of the tile's rows, by the first BM / 64 matrix waves (they have nothing else to do
+    // until the first tile lands), parked in LDS behind the stages and the store's staging until the store; the barrier
+    // that closes the prologue covers it
+    constexpr int LN_SLOT_OFF = STAGES * STAGE_BYTES > 8 * 32 * (BN / 4 + 4) * 4 ? STAGES * STAGE_BYTES : 8 * 32 * (BN / 4 + 4) * 4;
+    float2v *ln_slot = reinterpret_cast<float2v *>(smem + LN_SLOT_OFF);
+    lnf_stage<BM, BN, 512>(p, ln_slot, m0, n0, bz, tid);
     uint32_t aoffg[PA], boffg[PB];
     if constexpr (!LOADER) {
 #pragma unroll
@@ -1092,7 +1232,13 @@ __global__ __launch_bounds__((pp_threads<BK, STAGES, PINGPONG>())) void gemm_pp_
         if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
         return;
     }
-    store_tile<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz);
+    LnFold<TM> ln;
+    if (p.lnf_stats) {
+        ln.on = true; ln.col = reinterpret_cast<const float *>(ln_slot + BM); ln.bn = BN;
+#pragma unroll
+        for (int j = 0; j < TM; j++) { const float2v v = ln_slot[wm * WTM + 32 * j + (lane & 31)]; ln.r[j] = v[0]; ln.rmu[j] = v[1]; }
+    }
+    store_tile<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln);
     if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
 }
 
@@ -1760,13 +1906,13 @@ int raise_lds(KernelT kern, int bytes) {
 template <int BM, int BN, int BK, int STAGES>
 constexpr int pp_lds_bytes() {
     constexpr int stages = STAGES * (BM + BN) * BK * 2, epi = 8 * 32 * (BN / 4 + 4) * 4;      // operand ring; epilogue staging of 8 waves
-    return stages > epi ? stages : epi;
+    return (stages > epi ? stages : epi) + BM * 8 + BN * 8;      // + a folded layer norm's (r, r mu) per row, colsum and biasp per column
 }
 
 template <int BM, int BN, int BK>
 constexpr int gemm_lds_bytes() {
     constexpr int kc = BN * (BK + 8), kn = BK * (BN + 32);       // B buffer in either layout
-    return 2 * (BM * (BK + 8) + (kc > kn ? kc : kn)) * 2;
+    return 2 * (BM * (BK + 8) + (kc > kn ? kc : kn)) * 2 + BM * 8 + BN * 8;      // + a folded layer norm's (r, r mu) per row, colsum and biasp per column
 }
 
 #define GEMM_BIG 128, 256, 64, 2, 2
@@ -2107,6 +2253,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.clk = nullptr;
     a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
     a.sk_spin = 0; a.sk_pub_xor = a.sk_xcc_xor = 0; a.status = nullptr;
+    a.lnf_stats = a.lnf_colsum = a.lnf_biasp = nullptr; a.lnf_svec = 0; a.lnf_nseg = 0; a.lnf_eps = 0.0f; a.stats_out = nullptr; a.stats_nseg = 0;
     return MI_OK;
 }
 
@@ -2133,15 +2280,26 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         const bool pipe = a.K % 64 == 0 && a.K >= 128;
         if ((a.cv.xp || a.ag.x) && !pipe) return MI_DECLINE_EXTENT;      // only the pipelined kernel gathers
         TilePlan tp = {4, 1, false};
+        // A folded norm on the way in or row statistics on the way out live in the tiled kernels' own store: those calls
+        // need the pipelined kernels, 16-byte rows, and K-slices only in the form that ends in that store (the in-launch
+        // exchange), never planes.
+        const bool in_store = a.lnf_stats || a.stats_out;
+        if (in_store) {
+            const bool rows16 = !a.out_f32 ? (a.N % 8 == 0 && a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)))
+                                           : (a.N % 4 == 0 && a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16));
+            if (!pipe || a.cv.xp || a.ag.x || !rows16 || (a.stats_out && a.out_f32)) return MI_DECLINE_EXTENT;
+        }
         if (pipe) {
-            tp = plan_tiles(a.M, a.N, a.K, nbatch, true);
+            tp = plan_tiles(a.M, a.N, a.K, nbatch, !a.lnf_stats);
             if (tp.split > 1 && !(ws && aligned_to(ws, 256) && ws_bytes >= plan_workspace_bytes(tp, a.M, a.N)))
                 tp = plan_tiles(a.M, a.N, a.K, nbatch, false);
+            if (in_store && tp.split > 1 && !(tp.peer && sk_usable())) tp = plan_tiles(a.M, a.N, a.K, nbatch, false);
         }
-        const int split = tp.split;
+        int split = tp.split;
         if (split > 1 && tp.peer && ws && aligned_to(ws, 256) && ws_bytes >= plan_workspace_bytes(tp, a.M, a.N)) {
             const int rc = tp.tile == 0 ? launch_pp_peer<128, 256>(a, b_kn, split, ws, st) : launch_pp_peer<128, 128>(a, b_kn, split, ws, st);
             if (rc != MI_DECLINE_EXTENT) return rc;     // declined (a gathered operand, a device that failed the probe): planes
+            if (in_store) { tp = plan_tiles(a.M, a.N, a.K, nbatch, false); split = 1; }
         }
         if (split > 1 && ws && aligned_to(ws, 256) && ws_bytes >= (size_t)split * a.M * a.N * sizeof(float)) {
             GemmArgs s1 = a;
@@ -2216,6 +2374,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     a.clk = nullptr;
     a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
     a.sk_spin = 0; a.sk_pub_xor = a.sk_xcc_xor = 0; a.status = nullptr;
+    a.lnf_stats = a.lnf_colsum = a.lnf_biasp = nullptr; a.lnf_svec = 0; a.lnf_nseg = 0; a.lnf_eps = 0.0f; a.stats_out = nullptr; a.stats_nseg = 0;
     a.Y = Y; a.A = (const half_t *)A; a.B = (const half_t *)B; a.bias = (const half_t *)bias; a.residual = out_f32 ? nullptr : (const half_t *)residual;
     a.M = M; a.N = N; a.NB = NB; a.K = K; a.ldY = ldY; a.ldA = ldA; a.ldB = ldB; a.sY = sY; a.sA = sA; a.sB = sB; a.sBias = 0;
     a.bias_mode = bias ? bias_mode : MI_BIAS_NONE; a.epi = epi; a.out_f32 = out_f32;
@@ -2435,6 +2594,42 @@ int mi_gemm_clamp_ln_f16(void *Y, void *H, const void *X, const void *W, const v
         if (rc != MI_OK) return rc;
     }
     return H ? mi_layernorm_f16(H, nullptr, nullptr, Y, gamma, beta, F, T, eps, stream) : MI_OK;
+}
+
+int mi_gemm_rowstats_f16(void *Y, float *stats, const void *X, const void *W, const void *bias, const void *residual, float clamp,
+                         int64_t T, int64_t K, int64_t F, int64_t ldX, int64_t ldW,
+                         int w_layout, int bias_mode, int epi, void *ws, size_t ws_bytes, void *stream) {
+    if (!stats || !aligned_to(stats, 8) || is_nan_arg(clamp)) return MI_DECLINE_OPERANDS;
+    GemmArgs a;
+    int rc = fill_args(a, Y, X, W, bias, residual, T, K, F, F, ldX, ldW, w_layout, bias_mode, epi, MI_F16, 0, 0, 0);
+    if (rc != MI_OK) return rc;
+    if (!g_ready) return MI_ERROR_DEVICE;
+    if (T == 0 || F == 0) return MI_OK;
+    if (gemm_path(a, w_layout == MI_W_KF, 1) != MI_GEMM_MFMA) return MI_DECLINE_EXTENT;
+    a.stats_out = stats; a.stats_nseg = (int)ceil_div(F, 32);
+    if (clamp > 0.0f) a.clamp = clamp;
+    return run_gemm(a, w_layout == MI_W_KF, 1, ws, ws_bytes, (hipStream_t)stream, 0);
+}
+
+int mi_lnfold_gemm_f16(void *Y, float *stats_out, const void *X, const float *stats_in, float eps,
+                       const void *Wp, const float *colsum, const float *biasp, const void *residual, float clamp,
+                       int64_t T, int64_t K, int64_t F, int64_t ldY, int64_t ldX, int64_t ldW,
+                       int w_layout, int epi, int out_dtype,
+                       int64_t nbatch, int64_t sY, int64_t sW, int64_t sVec, void *ws, size_t ws_bytes, void *stream) {
+    if (!stats_in || !colsum || !biasp || !aligned_to(stats_in, 8) || !aligned_to(colsum, 16) || !aligned_to(biasp, 16) || sVec % 4) return MI_DECLINE_OPERANDS;
+    if (is_nan_arg(eps) || is_nan_arg(clamp) || (stats_out && !aligned_to(stats_out, 8))) return MI_DECLINE_OPERANDS;
+    if (nbatch < 1 || nbatch > 65535 || (stats_out && (nbatch != 1 || ldY != F || out_dtype != MI_F16))) return MI_DECLINE_EXTENT;
+    GemmArgs a;
+    int rc = fill_args(a, Y, X, Wp, nullptr, residual, T, K, F, ldY, ldX, ldW, w_layout, MI_BIAS_NONE, epi, out_dtype, sY, 0, sW);
+    if (rc != MI_OK) return rc;
+    if (!g_ready) return MI_ERROR_DEVICE;
+    if (T == 0 || F == 0) return MI_OK;
+    if (T <= 8 || !mfma_addressable(a, w_layout == MI_W_KF)) return MI_DECLINE_EXTENT;      // decode-sized rows: mi_ln_gemv_f16
+    a.lnf_stats = stats_in; a.lnf_nseg = (int)ceil_div(K, 32); a.lnf_eps = eps;
+    a.lnf_colsum = colsum; a.lnf_biasp = biasp; a.lnf_svec = sVec;
+    if (stats_out) { a.stats_out = stats_out; a.stats_nseg = (int)ceil_div(F, 32); }
+    if (clamp > 0.0f) a.clamp = clamp;
+    return run_gemm(a, w_layout == MI_W_KF, nbatch, ws, ws_bytes, (hipStream_t)stream, MI_GEMM_MFMA);
 }
 
 // mi_gemm_f16 for callers that cannot allocate: the split-K / decode planes go to `scratch`, a file-scope

@@ -185,6 +185,59 @@ __global__ void add_any_kernel(half_t *o, const half_t *a, const half_t *b, long
     if (i < n) o[i] = (half_t)((float)a[i] + (float)b[i]);
 }
 
+
+// Row statistics for a layer norm that is folded into the GEMM reading the rows (mi_lnfold_gemm_f16): for every
+// 32-column segment of a row, (sum, squares about the segment's own mean) -- what the GEMM stores leave when they
+// produce the rows themselves -- stored segment-major.  A thread owns one segment of one row (64 bytes, four 16-byte
+// loads, no exchange between lanes); the lanes of a wave take consecutive rows, so its result is one contiguous store.
+__global__ __launch_bounds__(256) void rowstats_kernel(float *stats, const half_t *a, long ld, int C, long rows) {
+    const long g = (long)blockIdx.x * 256 + threadIdx.x;      // row
+    const int seg = blockIdx.y;
+    if (g >= rows) return;
+    const half_t *src = a + g * ld + 32 * seg;
+    const int chunks = min(4, (C - 32 * seg) / 8);             // C % 8 == 0
+    half8v t[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) if (i < chunks) t[i] = as_half8(ldg16(src + 8 * i));
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (i < chunks) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) sum += (float)t[i][j];
+        }
+    const float mean = sum / (float)(8 * chunks);
+    float sq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (i < chunks) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) { const float d = (float)t[i][j] - mean; sq = fmaf(d, d, sq); }
+        }
+    const float2v o = {sum, sq};
+    *reinterpret_cast<float2v *>(stats + ((long)seg * rows + g) * 2) = o;
+}
+
+// Load-time preparation of a folded norm: Wp = fp16(gamma[k] W[k][n]), colsum[n] = sum_k Wp[k][n] (of the ROUNDED
+// values: what the matrix units will multiply), biasp[n] = bias[n] + sum_k beta[k] W[k][n], both in fp32.  One thread per
+// output column walks K; run once per weight.
+__global__ __launch_bounds__(256) void lnfold_prepare_kernel(half_t *Wp, float *colsum, float *biasp, const half_t *W, const half_t *gamma,
+                                                             const half_t *beta, const half_t *bias, int K, int F, long ldW, int b_kn) {
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    if (n >= F) return;
+    float cs = 0.0f, bp = bias ? (float)bias[n] : 0.0f;
+    for (int k = 0; k < K; k++) {
+        const long at = b_kn ? (long)k * ldW + n : (long)n * ldW + k;
+        const float w = (float)W[at];
+        const half_t wp = (half_t)(gamma ? (float)gamma[k] * w : w);
+        Wp[at] = wp;
+        cs += (float)wp;
+        if (beta) bp = fmaf((float)beta[k], w, bp);
+    }
+    colsum[n] = cs;
+    biasp[n] = bp;
+}
+
 }  // namespace
 
 extern "C" {
@@ -269,6 +322,28 @@ int mi_add_f16(void *out, const void *a, const void *b, int64_t n, void *stream)
         hipLaunchKernelGGL(add_vec_kernel, dim3((unsigned)ceil_div(n / 8, 256)), dim3(256), 0, st, (half_t *)out, (const half_t *)a, (const half_t *)b, (long)(n / 8));
     else
         hipLaunchKernelGGL(add_any_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, (half_t *)out, (const half_t *)a, (const half_t *)b, (long)n);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_rowstats_f16(float *stats, const void *a, int64_t ld, int64_t C, int64_t rows, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!stats || !a || !aligned_to(stats, 8) || !aligned_to(a, 16)) return MI_DECLINE_OPERANDS;
+    if (C < 8 || C % 8 || ld < C || ld % 8 || rows < 0 || C > INT32_MAX) return MI_DECLINE_EXTENT;
+    if (rows == 0) return MI_OK;
+    if (ceil_div(C, 32) > 65535) return MI_DECLINE_EXTENT;
+    hipLaunchKernelGGL(rowstats_kernel, dim3((unsigned)ceil_div(rows, 256), (unsigned)ceil_div(C, 32)), dim3(256), 0, (hipStream_t)stream,
+                       stats, (const half_t *)a, (long)ld, (int)C, (long)rows);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_lnfold_prepare_f16(void *Wp, float *colsum, float *biasp, const void *W, const void *gamma, const void *beta, const void *bias,
+                          int64_t K, int64_t F, int64_t ldW, int w_layout, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!Wp || !colsum || !biasp || !W || (w_layout != MI_W_KF && w_layout != MI_W_FK)) return MI_DECLINE_OPERANDS;
+    if (K < 1 || F < 1 || K > INT32_MAX || F > INT32_MAX || ldW < (w_layout == MI_W_KF ? F : K)) return MI_DECLINE_EXTENT;
+    hipLaunchKernelGGL(lnfold_prepare_kernel, dim3((unsigned)ceil_div(F, 256)), dim3(256), 0, (hipStream_t)stream,
+                       (half_t *)Wp, colsum, biasp, (const half_t *)W, (const half_t *)gamma, (const half_t *)beta, (const half_t *)bias,
+                       (int)K, (int)F, (long)ldW, w_layout == MI_W_KF ? 1 : 0);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 

@@ -308,6 +308,119 @@ def matmul_ln_(ctx: Ctx, out, normed, A, B, gamma, beta, eps, bias=None, *, epi=
     return out
 
 
+# ----------------------------------------------------------------------------- a layer norm with no pass of its own
+
+@dataclass
+class LnFoldedLinear:
+    """A linear layer with the norm in front of it folded away (``mi_lnfold_prepare_f16``): ``wp`` = fp16(gamma W) as a
+    ``(K, F)`` tensor in W's memory layout, ``colsum`` / ``biasp`` fp32 ``(F,)``; ``planes`` > 1: ``F`` is that many
+    equal column bands run as planes of one launch (q, k, v)."""
+    wp: torch.Tensor
+    colsum: torch.Tensor
+    biasp: torch.Tensor
+    planes: int = 1
+
+
+def rowstats_segments(C: int) -> int:
+    return (C + 31) // 32
+
+
+def rowstats_new(rows: int, C: int, device="cuda") -> torch.Tensor:
+    """Storage for the row statistics of ``rows`` rows of ``C`` elements: (sum, squares about its mean) per 32-column
+    segment, segment-major ``(segments, rows, 2)``."""
+    return torch.empty((rowstats_segments(C), rows, 2), dtype=torch.float32, device=device)
+
+
+def lnfold_prepare(ctx: Ctx, W, gamma, beta, bias=None, planes: int = 1) -> LnFoldedLinear:
+    """Once per weight, at load: ``LN(x) . W + b = r (x . W') - r mu colsum(W') + b'`` with ``W' = gamma W`` and
+    ``b' = b + beta . W``.  ``W``: ``(K, F)`` fp16 in either memory layout; ``gamma`` / ``beta`` ``(K,)`` or None."""
+    lay = _mat2(W)
+    if W.dim() != 2 or not _is_f16_cuda(W) or lay is None:
+        raise DeclineError("lnfold_prepare: a 2-D fp16 device weight with one contiguous axis", L.DECLINE_OPERANDS)
+    K, F = W.shape
+    if F % planes:
+        raise DeclineError("lnfold_prepare: planes must divide F", L.DECLINE_EXTENT)
+    _check_vecs("lnfold_prepare", L.DECLINE_OPERANDS, ("gamma", gamma, K), ("beta", beta, K), ("bias", bias, F))
+    wp = torch.empty_like(W)                       # preserves W's strides (dense in its own layout)
+    if wp.stride() != W.stride():
+        raise DeclineError("lnfold_prepare: the weight must be dense in its layout", L.DECLINE_OPERANDS)
+    colsum = torch.empty((F,), dtype=torch.float32, device=W.device)
+    biasp = torch.empty((F,), dtype=torch.float32, device=W.device)
+    rc = L.init().mi_lnfold_prepare_f16(wp.data_ptr(), colsum.data_ptr(), biasp.data_ptr(), W.data_ptr(), _ptr(gamma), _ptr(beta), _ptr(bias),
+                                        K, F, lay[1], L.W_KF if lay[0] == 0 else L.W_FK, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_lnfold_prepare_f16", rc)
+    return LnFoldedLinear(wp, colsum, biasp, planes)
+
+
+def rowstats_(ctx: Ctx, stats, x):
+    """``stats`` (``rowstats_new``) of the rows of ``x`` ``(rows, C)`` fp16, rows contiguous: for rows no GEMM here wrote."""
+    if x.dim() != 2 or not _is_f16_cuda(x) or x.stride(1) != 1 or stats.dtype != torch.float32 or \
+            tuple(stats.shape) != (rowstats_segments(x.shape[1]), x.shape[0], 2) or not stats.is_contiguous():
+        raise DeclineError("rowstats_: operands", L.DECLINE_OPERANDS)
+    rc = L.init().mi_rowstats_f16(stats.data_ptr(), x.data_ptr(), x.stride(0), x.shape[1], x.shape[0], ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_rowstats_f16", rc)
+    return stats
+
+
+def matmul_rowstats_(ctx: Ctx, out, stats, A, B, bias=None, *, epi="none", residual=None, clamp=None):
+    """``matmul_`` into dense fp16 rows that also leaves ``stats`` (``rowstats_new(T, F)``) of the finished rows -- after
+    residual and clamp -- for a folded norm that reads them next (``lnfold_matmul_``)."""
+    plan = mmplan(ctx.dev, out, A, B, bias)
+    if not isinstance(plan, MMMfmaPlan):
+        raise DeclineError(f"matmul_rowstats_: the tiled kernels only (plan {plan})", L.DECLINE_EXTENT)
+    lib = L.init()
+    K, F = A.shape
+    T = B.shape[0]
+    la, lb = _mat2(A), _mat2(B)
+    if out.dtype != torch.float16 or not out.is_contiguous() or tuple(stats.shape) != (rowstats_segments(F), T, 2) or \
+            stats.dtype != torch.float32 or not stats.is_contiguous():
+        raise DeclineError("matmul_rowstats_: out dense fp16 (T,F), stats from rowstats_new(T, F)", L.DECLINE_OPERANDS)
+    if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
+        raise DeclineError("matmul_rowstats_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
+    bm = L.BIAS_NONE if bias is None else (L.BIAS_COL if bias.numel() == F else L.BIAS_ROW)
+    need = lib.mi_gemm_f16_workspace(T, K, F, plan.w_layout, 1)
+    ws = ctx.ws.scratch(need)
+    rc = lib.mi_gemm_rowstats_f16(out.data_ptr(), stats.data_ptr(), B.data_ptr(), A.data_ptr(), _ptr(bias), _ptr(residual),
+                                  0.0 if clamp is None else float(clamp), T, K, F, lb[1], la[1], plan.w_layout, bm, L.EPI[epi], ws, need, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_gemm_rowstats_f16", rc)
+    return out
+
+
+def lnfold_matmul_(ctx: Ctx, out, fw: LnFoldedLinear, B, stats, eps, *, epi="none", residual=None, stats_out=None, clamp=None):
+    """``out = epi(layernorm(B) . W + b) (+ residual)`` with no pass over ``B``: ``B`` ``(T, K)`` holds the RAW rows,
+    ``stats`` their row statistics (left by the GEMM that wrote them, or ``rowstats_``), ``fw`` the prepared weight.
+    ``fw.planes`` > 1: ``out`` is ``(T, F)`` whose ``planes`` column bands are written by the planes of one launch.
+    ``stats_out``: also leave the statistics of ``out``'s rows (single plane, dense ``out``).  Held to the parity gate
+    against ``layernorm_`` -> ``matmul_``, not to their bits."""
+    lib = L.init()
+    K, F = fw.wp.shape
+    T = B.shape[0]
+    la, lb, lo = _mat2(fw.wp), _mat2(B), _mat2(out)
+    if not _is_f16_cuda(B) or lb is None or lb[0] != 0 or B.shape[1] != K or lo is None or lo[0] != 0 or tuple(out.shape) != (T, F) or \
+            out.dtype not in (torch.float16, torch.float32):
+        raise DeclineError("lnfold_matmul_: operands", L.DECLINE_OPERANDS)
+    if tuple(stats.shape) != (rowstats_segments(K), T, 2) or stats.dtype != torch.float32 or not stats.is_contiguous():
+        raise DeclineError("lnfold_matmul_: stats must come from rowstats_new(T, K)", L.DECLINE_OPERANDS)
+    if residual is not None and (residual.shape != out.shape or residual.stride() != out.stride() or residual.dtype != torch.float16):
+        raise DeclineError("lnfold_matmul_: residual must match out's shape, strides and be fp16", L.DECLINE_OPERANDS)
+    P = fw.planes
+    Fp = F // P
+    w_layout = L.W_KF if la[0] == 0 else L.W_FK
+    sW = Fp if w_layout == L.W_KF else Fp * la[1]            # the next band of columns: F-contiguous, or Fp rows of K further
+    need = lib.mi_gemm_f16_workspace(T, K, Fp, w_layout, P)
+    ws = ctx.ws.scratch(need)
+    rc = lib.mi_lnfold_gemm_f16(out.data_ptr(), _ptr(stats_out), B.data_ptr(), stats.data_ptr(), float(eps),
+                                fw.wp.data_ptr(), fw.colsum.data_ptr(), fw.biasp.data_ptr(), _ptr(residual), 0.0 if clamp is None else float(clamp),
+                                T, K, Fp, lo[1], lb[1], la[1], w_layout, L.EPI[epi], _dtype_code(out),
+                                P, Fp, sW, Fp, ws, need, ctx.stream)
+    if rc != L.OK:
+        raise DeclineError("mi_lnfold_gemm_f16", rc)
+    return out
+
+
 LN_GEMM_KMAX = 512
 
 

@@ -40,14 +40,23 @@ def _oracle_layer(h, x, heads, eps):
     return oracle.gemm_f16(f, h["w2"], h["b2"], residual=x1)
 
 
-def test_config2_encoder_block_at_full_size(ctx):
+@pytest.mark.parametrize("folded", [False, True])
+def test_config2_encoder_block_at_full_size(ctx, folded):
+    """``folded``: the block in five launches, its norms folded into the linears that read them (no pass over the rows
+    for either), against the same oracle composition that runs them as ops of their own."""
     import torch
-    from juliavision_amd.encoder import EncoderBuffers, encoder_layer
+    from juliavision_amd import rowstats_
+    from juliavision_amd.encoder import EncoderBuffers, FoldedStats, encoder_layer, encoder_layer_folded, fold_layer_norms
     T, d, H, ffn = 1500, 1280, 20, 5120
     h, W = _layer(d, ffn, 1000)
     x = oracle.randn_f16((T, d), 999)
     out = poison(torch.empty((T, d), dtype=torch.float16, device="cuda"))
-    encoder_layer(ctx, W, to_dev(x), out, EncoderBuffers(T, d, ffn), H, 1e-5)
+    if folded:
+        dx, st = to_dev(x), FoldedStats(T, d)
+        rowstats_(ctx, st.x, dx)
+        encoder_layer_folded(ctx, fold_layer_norms(ctx, W), dx, out, EncoderBuffers(T, d, ffn), st, H, 1e-5)
+    else:
+        encoder_layer(ctx, W, to_dev(x), out, EncoderBuffers(T, d, ffn), H, 1e-5)
     torch.cuda.synchronize()
     want = _oracle_layer(h, x, H, 1e-5)
     assert_parity(to_host(out), want, what="config 2 encoder block")
@@ -56,7 +65,8 @@ def test_config2_encoder_block_at_full_size(ctx):
                   what="config 2 encoder block, update only")
 
 
-def test_config3_vit_s14_encoder_at_518(ctx):
+@pytest.mark.parametrize("folded", [False, True])
+def test_config3_vit_s14_encoder_at_518(ctx, folded):
     import torch
     from juliavision_amd.encoder import ViTEncoder, ViTWeights
     d, H, ffn, P, S, NL = 384, 6, 1536, 14, 518, 12
@@ -70,7 +80,7 @@ def test_config3_vit_s14_encoder_at_518(ctx):
     layers = [_layer(d, ffn, 100 + 50 * i) for i in range(NL)]
     norm_g, norm_b = oracle.randn_f16((d,), 5, 1.0, 0.02), oracle.randn_f16((d,), 6, 0.0, 0.02)
     W = ViTWeights(to_dev(patch_w), to_dev(patch_b), to_dev(cls), to_dev(pos), [l[1] for l in layers], to_dev(norm_g), to_dev(norm_b))
-    enc = ViTEncoder(W, (S, S), H, ffn)
+    enc = ViTEncoder(W, (S, S), H, ffn, fold_norms=ctx if folded else None)
     assert enc.T == T == 1370
     got = to_host(enc(ctx, to_dev(image)))
     torch.cuda.synchronize()
