@@ -97,7 +97,22 @@ def peak_probe(lib, stream):
         if rc != 0:
             raise RuntimeError(f"mi_probe_copy returned {rc}")
     t_cp, _ = timed(copy, 5)
-    return {"mfma_only_tflops": round(flop_fill / t_fill / 1e12, 1),
+    # one phase boundary of a would-be multi-phase persistent kernel: every compute unit's workgroup at a grid barrier
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    scratch = torch.zeros(16 + 8 * cus, dtype=torch.int32, device="cuda")
+    ROUNDS = 200
+
+    def barrier(payload):
+        rc = lib.mi_probe_grid_barrier(scratch.data_ptr(), cus, ROUNDS, payload, stream)
+        if rc != 0:
+            raise RuntimeError(f"mi_probe_grid_barrier returned {rc}")
+    t_bar, _ = timed(lambda: barrier(0), 5)
+    t_bar_x, _ = timed(lambda: barrier(1), 5)
+    gave_up = int(scratch[4].item())
+    return {"grid_barrier_us": round(t_bar * 1e6 / ROUNDS, 2), "grid_barrier_with_exchange_us": round(t_bar_x * 1e6 / ROUNDS, 2),
+            "grid_barrier": f"{cus} workgroups, agent-scope atomic add + poll per round; with exchange: 16 B published per workgroup "
+                            f"before and all {16 * cus} B read back after; {ROUNDS} rounds per launch" + ("; SOME WAITS GAVE UP" if gave_up else ""),
+            "mfma_only_tflops": round(flop_fill / t_fill / 1e12, 1),
             "mfma_only_frac_of_peak": round(flop_fill / t_fill / 1e12 / PEAK_F16_TFLOPS, 4),
             "mfma_only_grid": f"{WG} workgroups x 8 waves x {STEPS * 16} MFMAs (32x32x16 f16), no memory operations",
             "c1_no_memory_us": round(t_c1 * 1e6, 2), "c1_no_memory_us_min": round(t_c1_min * 1e6, 2),

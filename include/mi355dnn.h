@@ -87,8 +87,15 @@ int mi_set_clock_probe(void *dev_u64x4);
  * actually written.  240 workgroups x 20 steps with gelu is config 1's launch minus its memory traffic; a grid of many
  * rounds is what the matrix units sustain at the clock the chip holds under that load.
  * mi_probe_copy: out[0 .. bytes) = in[0 .. bytes), 16 bytes per lane and step; bytes % 16 == 0.  A kernel of known HBM
- * traffic (bytes read + bytes written). */
+ * traffic (bytes read + bytes written).
+ * mi_probe_grid_barrier: `workgroups` (<= compute units) workgroups meet `rounds` times at a barrier across the whole
+ * grid -- an agent-scope atomic add on a counter in device memory and a bounded poll -- and, with payload != 0, exchange
+ * 16 bytes each around it (write-through stores before, reads past the L2 after): what one phase boundary inside a
+ * multi-phase persistent kernel would cost.  scratch_u32: 64 + 32 x workgroups bytes of device memory, 16-byte aligned;
+ * word 4 is nonzero afterwards if some workgroup gave up waiting (it then ran on without waiting).  Not for use
+ * under graph capture (it clears its counter with a memset). */
 int mi_probe_mfma(void *sink, const void *seed_f16, int64_t workgroups, int64_t steps, int gelu, void *stream);
+int mi_probe_grid_barrier(void *scratch_u32, int64_t workgroups, int64_t rounds, int payload, void *stream);
 int mi_probe_copy(void *out, const void *in, size_t bytes, void *stream);
 
 /* Device-side failures (no counterpart in the reference, whose kernels never wait for one another).  A few kernels
@@ -102,7 +109,7 @@ int mi_probe_copy(void *out, const void *in, size_t bytes, void *stream);
 enum mi_device_status_bits {
     MI_DEVSTAT_EXCHANGE_TIMEOUT = 1,  /* split-K exchange of mi_gemm_f16: a partner workgroup did not arrive in time   */
     MI_DEVSTAT_EXCHANGE_XCD = 2,      /* split-K exchange: partner workgroups did not share an XCD (one L2)            */
-    MI_DEVSTAT_STEP_BARRIER = 4       /* mi_decoder_layer_step_f16: a workgroup gave up at a barrier between phases    */
+    MI_DEVSTAT_STEP_BARRIER = 4       /* a workgroup gave up at a barrier across the grid (mi_probe_grid_barrier's word) */
 };
 int mi_device_status(int reset);
 /* Process-wide switch for the in-launch split-K exchange of mi_gemm_f16 and its variants (on by default where the

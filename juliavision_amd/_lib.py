@@ -36,6 +36,7 @@ SIGNATURES = {
     "mi_set_clock_probe": (_int, [_vp]),
     "mi_probe_mfma": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "mi_probe_copy": (_int, [_vp, _vp, _sz, _vp]),
+    "mi_probe_grid_barrier": (_int, [_vp, _i64, _i64, _int, _vp]),
     "mi_device_status": (_int, [_int]),
     "mi_set_in_launch_exchange": (_int, [_int]),
     "mi_test_exchange_faults": (_int, [_int, C.c_uint, C.c_uint]),

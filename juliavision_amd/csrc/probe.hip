@@ -62,6 +62,38 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(u32x4 *out, const u32x4
     for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) out[i] = in[i];
 }
 
+// What a barrier across the whole grid costs on this device: `rounds` times, every workgroup adds itself to a counter
+// in device memory (an agent-scope atomic: the XCDs' L2s are not coherent with each other, so it is performed beyond
+// them) and polls it until all have arrived; with `payload`, every workgroup first publishes 16 bytes with write-through
+// stores and afterwards reads all of them back past its L2 -- the exchange a multi-phase kernel would need between phases
+// (a decode step's 2.5 KB activation row).  Every wait is bounded: a workgroup that gives up raises the sticky status word
+// and runs on without waiting, so the grid drains whatever happens.  The grid must be resident at once (<= one
+// workgroup per compute unit).
+__global__ __launch_bounds__(64) void probe_grid_barrier_kernel(unsigned *counter, unsigned *data, unsigned *status, int rounds, int payload, int spin_limit) {
+    const unsigned G = gridDim.x;
+    bool gave_up = false;
+    unsigned acc = 0;
+    for (int r = 0; r < rounds; r++) {
+        if (payload && threadIdx.x < 4)
+            __hip_atomic_store(data + ((r & 1) * G + blockIdx.x) * 4 + threadIdx.x, (unsigned)(r * 131 + blockIdx.x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (threadIdx.x == 0 && !gave_up) {
+            __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned want = (unsigned)(r + 1) * G;
+            int spins = 0;
+            while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
+                if (++spins > spin_limit) { gave_up = true; __hip_atomic_fetch_or(status, (unsigned)MI_DEVSTAT_STEP_BARRIER, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        __syncthreads();
+        if (payload) {
+            for (unsigned i = threadIdx.x; i < G * 4; i += 64) acc += __hip_atomic_load(data + (r & 1) * G * 4 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (acc == 0x12345u) data[0] = acc;
+}
+
 }  // namespace
 
 extern "C" {
@@ -72,6 +104,17 @@ int mi_probe_mfma(void *sink, const void *seed_f16, int64_t workgroups, int64_t 
     if (workgroups < 1 || workgroups > (1 << 20) || steps < 1 || steps > (1 << 24)) return MI_DECLINE_EXTENT;
     hipLaunchKernelGGL(probe_mfma_kernel, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream,
                        reinterpret_cast<float *>(sink), reinterpret_cast<const half_t *>(seed_f16), (int)steps, gelu);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
+int mi_probe_grid_barrier(void *scratch_u32, int64_t workgroups, int64_t rounds, int payload, void *stream) {
+    if (!mi_ready()) return MI_ERROR_DEVICE;
+    if (!scratch_u32 || !aligned_to(scratch_u32, 16)) return MI_DECLINE_OPERANDS;
+    if (workgroups < 1 || workgroups > mi_num_cus() || rounds < 1 || rounds > 100000) return MI_DECLINE_EXTENT;
+    unsigned *base = reinterpret_cast<unsigned *>(scratch_u32);      // [0]: counter, [4]: status, [16 ..): two rounds of payload
+    hipStream_t st = (hipStream_t)stream;
+    if (hipMemsetAsync(base, 0, 64, st) != hipSuccess) return MI_ERROR_LAUNCH;
+    hipLaunchKernelGGL(probe_grid_barrier_kernel, dim3((unsigned)workgroups), dim3(64), 0, st, base, base + 16, base + 4, (int)rounds, payload, 1 << 16);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
