@@ -302,10 +302,17 @@ __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc
     static_assert(STAGE_BYTES * NWAVES <= LDS_BYTES, "epilogue staging exceeds the operand LDS");
     char *stage = smem + wave * STAGE_BYTES;
     const int hl = lane >> 5;
+    // Row biases for all of the wave's rows before the first store (store_tile_simple says why).
+    float brow_j[TM];
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+        const int m = m0 + wm * WTM + 32 * j + frow;
+        brow_j[j] = (p.bias_mode == MI_BIAS_ROW && m < p.M) ? (float)bias[m] : 0.0f;
+    }
     static_for<TM>([&](auto J) {
         constexpr int j = decltype(J)::value;
         const int mrow = m0 + wm * WTM + 32 * j;
-        const float brow = (p.bias_mode == MI_BIAS_ROW && mrow + frow < p.M) ? (float)bias[mrow + frow] : 0.0f;
+        const float brow = brow_j[j];
 #pragma unroll
         for (int i = 0; i < TN; i++) {
             // folded layer norm: this lane's columns of colsum and biasp from their LDS copy, a 32-column group at a time
@@ -418,11 +425,133 @@ __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc
     });
 }
 
+// The common store: fp16 output in whole 16-byte chunks, column bias (or a folded layer norm), optional activation,
+// residual, clamp and row statistics; no row bias, no fp32 output, no ragged N.
+//
+// Loads and stores of a wave share one counter and complete in order, so a wait for a load -- wherever the compiler
+// places it -- is also a wait for every store issued before that load to be acknowledged: a trip of two microseconds
+// under the burst of all workgroups' stores.  The general store above pays it once per 32-row block of a wave's tile
+// and once per residual chunk (8 000 clocks of a 44 000-clock launch at 1500 x 1280 -> 5120).  Here nothing is fetched
+// behind a store that anybody then waits for: the caller's column bias is pinned in registers ahead of the first store,
+// and the residual chunks of block j + 1 are requested before block j's stores go out.
+// Same arithmetic as the general store (bias joined in fp32, one rounding, activation on the rounded value, residual,
+// clamp), so the two give the same bits.  Two staging areas a wave: block j + 1 is staged while block j's chunks are on
+// their way back from the LDS (a wave's LDS operations complete in order: no wait between staging a block and reading it).
+template <int EPI, int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
+__device__ __forceinline__ void store_tile_simple(const GemmArgs &p, float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], char *smem, int m0, int n0, int wm, int wn,
+                                                  int wave, int lane, long bz, const LnFold<TM> ln) {
+    constexpr int SLD_H = WTN + 8, BUF_BYTES = 32 * SLD_H * 2;      // halves per staged row; one staging area
+    constexpr int CPR = WTN / 8, RPI = 64 / CPR, NIT = 32 / RPI;     // 16-byte chunks per row; rows a wave covers at a time; chunks per lane and block
+    static_assert(2 * BUF_BYTES * NWAVES <= LDS_BYTES && 64 % CPR == 0 && CPR % 4 == 0, "two staging areas a wave; four lanes hold a 32-column segment");
+    char *const buf = smem + wave * 2 * BUF_BYTES;
+    const int frow = lane & 31, hl = lane >> 5;
+    const int ch = lane % CPR, r0 = lane / CPR;                      // this lane's chunks of a block: rows r0 + RPI t, columns 8 ch ..
+    const int mw = m0 + wm * WTM, n = n0 + wn * WTN + ch * 8;
+    const bool col_ok = n < p.N;                                     // N % 8 == 0: a chunk that starts below N ends below it
+    const long off0 = bz * p.sY + (long)(mw + r0) * p.ldY + n;
+    half_t *const ybase = reinterpret_cast<half_t *>(p.Y) + off0;
+    const half_t *const rbase = p.residual ? p.residual + off0 : nullptr;
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) asm volatile("" ::"v"(cb[i][g]));
+    auto stage = [&](auto J) {
+        constexpr int j = decltype(J)::value;
+        half_t *st = reinterpret_cast<half_t *>(buf + (j & 1) * BUF_BYTES) + frow * SLD_H + 4 * hl;
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int nl = 32 * i + 8 * g;
+                float v[4];
+                if (ln.on) {      // uniform: r (acc - mu colsum) + biasp, the tile's colsum and biasp from their LDS copy
+                    const float4v lc = *reinterpret_cast<const float4v *>(ln.col + wn * WTN + nl + 4 * hl);
+                    const float4v lb = *reinterpret_cast<const float4v *>(ln.col + ln.bn + wn * WTN + nl + 4 * hl);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = fmaf(acc[i][j][4 * g + e], ln.r[j], fmaf(-ln.rmu[j], lc[e], lb[e]));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + (float)cb[i][g][e];
+                }
+                const half4v o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                *reinterpret_cast<half4v *>(st + nl) = o;
+            }
+    };
+    half8v res[2][NIT];
+    auto fetch_residual = [&](auto J) {
+        constexpr int j = decltype(J)::value;
+#pragma unroll
+        for (int t = 0; t < NIT; t++) {
+            res[j & 1][t] = half8v{};
+            if (col_ok && mw + 32 * j + r0 + t * RPI < p.M) res[j & 1][t] = as_half8(ldg16(rbase + (long)(32 * j + t * RPI) * p.ldY));
+        }
+    };
+    if (rbase) fetch_residual(std::integral_constant<int, 0>{});
+    stage(std::integral_constant<int, 0>{});
+    static_for<TM>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+        const half_t *rd = reinterpret_cast<const half_t *>(buf + (j & 1) * BUF_BYTES) + r0 * SLD_H + ch * 8;
+        half8v x[NIT];
+#pragma unroll
+        for (int t = 0; t < NIT; t++) x[t] = *reinterpret_cast<const half8v *>(rd + t * RPI * SLD_H);
+        if constexpr (j + 1 < TM) {
+            stage(std::integral_constant<int, j + 1>{});
+            if (rbase) fetch_residual(std::integral_constant<int, j + 1>{});
+        }
+#pragma unroll
+        for (int t = 0; t < NIT; t++) {
+            const int m = mw + 32 * j + r0 + t * RPI;
+            const bool have = col_ok && m < p.M;
+            if constexpr (EPI != MI_EPI_NONE) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) x[t][e] = (half_t)apply_epi_c<EPI>((float)x[t][e]);
+            }
+            if (rbase) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) x[t][e] = (half_t)((float)x[t][e] + (float)res[j & 1][t][e]);
+            }
+            if (p.clamp > 0.0f) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) x[t][e] = (half_t)fminf(fmaxf((float)x[t][e], -p.clamp), p.clamp);
+            }
+            if (have) *reinterpret_cast<half8v *>(ybase + (long)(32 * j + t * RPI) * p.ldY) = x[t];
+            if (p.stats_out) {      // uniform
+                // the four lanes of a quad hold the 32 columns of one segment of one row (chunks that lie past N or
+                // below M count nothing): sum, then squares about the segment's own mean, both over the quad
+                float cnt = have ? 8.0f : 0.0f, sum = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) sum += have ? (float)x[t][e] : 0.0f;
+                sum += lane_xor<1>(sum); sum += lane_xor<2>(sum);
+                cnt += lane_xor<1>(cnt); cnt += lane_xor<2>(cnt);
+                const float mean = sum / fmaxf(cnt, 1.0f);
+                float sq = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) { const float d = (float)x[t][e] - mean; sq = have ? fmaf(d, d, sq) : sq; }
+                sq += lane_xor<1>(sq); sq += lane_xor<2>(sq);
+                if (have && (ch & 3) == 0) {
+                    const float2v o = {sum, sq};
+                    *reinterpret_cast<float2v *>(p.stats_out + ((long)(n / 32) * p.M + m) * 2) = o;
+                }
+            }
+        }
+    });
+}
+
 // The activation is a compile-time choice inside the store loops: one uniform branch per tile
 // instead of one per element.
 template <int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
 __device__ __forceinline__ void store_tile(const GemmArgs &p, float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], char *smem, int m0, int n0, int wm, int wn,
                                            int wave, int lane, long bz, const LnFold<TM> ln = LnFold<TM>{}) {
+    const bool simple = !p.out_f32 && p.vec_store && p.N % 8 == 0 && p.bias_mode != MI_BIAS_ROW;
+    if (simple) {
+        switch (p.epi) {
+        case MI_EPI_GELU_ERF: store_tile_simple<MI_EPI_GELU_ERF, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
+        case MI_EPI_GELU_TANH: store_tile_simple<MI_EPI_GELU_TANH, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
+        case MI_EPI_RELU: store_tile_simple<MI_EPI_RELU, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
+        default: store_tile_simple<MI_EPI_NONE, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
+        }
+        return;
+    }
     switch (p.epi) {
     case MI_EPI_GELU_ERF: store_tile_epi<MI_EPI_GELU_ERF, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
     case MI_EPI_GELU_TANH: store_tile_epi<MI_EPI_GELU_TANH, TM, TN, WTM, WTN, NWAVES, LDS_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln); break;
@@ -1243,6 +1372,236 @@ __global__ __launch_bounds__((pp_threads<BK, STAGES, PINGPONG>())) void gemm_pp_
 }
 
 // ------------------------------------------------------------------------------------------
+// Four matrix waves, one per SIMD, each with a BM x BN/4 strip of the tile, and a loader wave.
+//
+// The ping-pong kernel's 128 x 256 tile spends a third of its K loop in waits: per 64-deep tile its eight 64 x 64
+// waves read 8 x 16 KB of fragments for 1024 clocks of MFMAs per SIMD, a SIMD takes 32 B/clock from the LDS, and the
+// two phases of a tile came to 1590 clocks (measured with clock stamps; no different with every workgroup on one
+// L2-resident tile, so it is not memory).  A wave that owns 128 x 64 reads 24 KB for twice the MFMAs.  With one matrix
+// wave per SIMD there is no partner to alternate phases with; instead each wave overlaps its own work: three sets
+// of fragment registers (4 A + 2 B fragments of a 16-deep step), the reads of step s + 2 dealt one or two at a time
+// between the eight MFMAs of step s -- issued in one burst they held the wave at the LDS queue while its matrix pipe
+// ran dry -- and an MFMA in flight does not hold up the wave's LDS instructions.  128 accumulator registers + 72 of
+// fragments fit because at most two waves (a matrix wave and the loader) share a SIMD: 256 registers each.
+// Measured: 1290 to 1390 clocks a tile, and 1500 x 1280 -> 5120 in 23.1 us against 25.5 to 26.1 us.
+//
+// One workgroup barrier per tile, B_kt, taken by the matrix waves in the middle of tile kt's third step -- after the
+// last fragment read of the tile has returned, before the first read of tile kt + 1 -- and by the loader after it has
+// waited for tile kt + 1 to land.  Past B_kt stage kt % 3 is free, and the loader requests tile kt + 3 into it.
+template <int BM, int BN, int BK, bool B_KN>
+struct DirectTile {
+    static constexpr int CPR = BK / 8, ROWB = BK * 2, A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int SLOTS_A = A_BYTES / 1024, SLOTS_B = B_BYTES / 1024;      // 1 KB = one wave-wide request
+    __device__ __forceinline__ static int rowswz(int r) { return BK == 64 ? (r & 7) ^ ((r >> 3) & 1) : (r >> 2) & 3; }
+    // per-lane byte offset, from the tile's origin in memory, of what lands in 1 KB slot s of the A / B part of a stage
+    __device__ __forceinline__ static uint32_t a_offset(const GemmArgs &p, int m0, int s, int lane) {
+        const int q = s * 64 + lane, r = q / CPR, pos = q % CPR;
+        return (uint32_t)(((long)(min(m0 + r, p.M - 1) - m0) * p.ldA + (pos ^ rowswz(r)) * 8) * 2);
+    }
+    __device__ __forceinline__ static uint32_t b_offset(const GemmArgs &p, int n0, int s, int lane) {
+        const int q = s * 64 + lane;
+        if (!B_KN) {
+            const int r = q / CPR, pos = q % CPR;
+            return (uint32_t)(((long)(min(n0 + r, p.N - 1) - n0) * p.ldB + (pos ^ rowswz(r)) * 8) * 2);
+        } else {
+            constexpr int CPRB = BN / 8;
+            const int k = q / CPRB, pos = q % CPRB, j = pos ^ ((k & 3) << 2);
+            return (uint32_t)(((long)k * p.ldB + (min(n0 + j * 8, p.NB - 8) - n0)) * 2);
+        }
+    }
+    __device__ __forceinline__ static void request(const char *base, uint32_t off, uint32_t lds_dst) {
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_dst);
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(dst) : "memory");
+    }
+};
+
+template <int BM, int BN, bool B_KN>
+__global__ __launch_bounds__(320) void gemm_w4_kernel(GemmArgs p) {
+    constexpr int BK = 64, STAGES = 3, KS = 4;
+    using T = DirectTile<BM, BN, BK, B_KN>;
+    constexpr int ROWB = T::ROWB, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, PER_TILE = T::SLOTS_A + T::SLOTS_B;
+    constexpr int WTM = BM, WTN = BN / 4, TM = WTM / 32, TN = WTN / 32;
+    static_assert(TM * TN == 8 && PER_TILE <= 63, "128 accumulator registers a lane; vmcnt is a 6-bit counter");
+    static_assert(!B_KN || BN >= 128, "the [K][N] permutation moves a chunk by up to 12 places inside its row");
+    extern __shared__ __align__(16) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int tm_, tn_;
+    tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
+    // (the division inside tile_of runs on the vector unit: hand the results back to scalar registers, which the
+    // direct loads' base addresses have to be in)
+    const int m0 = __builtin_amdgcn_readfirstlane(tm_ * BM), n0 = __builtin_amdgcn_readfirstlane(tn_ * BN);
+    const long bz = blockIdx.y;
+    const int nk = p.K / BK;
+    const long a_step = BK * 2, b_step = B_KN ? (long)BK * p.ldB * 2 : BK * 2;
+    const char *Ag = reinterpret_cast<const char *>(p.A + bz * p.sA + (long)m0 * p.ldA);
+    const char *Bg = reinterpret_cast<const char *>(p.B + bz * p.sB + (B_KN ? (long)n0 : (long)n0 * p.ldB));
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
+    auto barrier = [&]() {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    if (wave == 4) {
+        uint32_t offa[T::SLOTS_A], offb[T::SLOTS_B];
+#pragma unroll
+        for (int s = 0; s < T::SLOTS_A; s++) offa[s] = T::a_offset(p, m0, s, lane);
+#pragma unroll
+        for (int s = 0; s < T::SLOTS_B; s++) offb[s] = T::b_offset(p, n0, s, lane);
+        auto request = [&](int kt, int stage) {
+            const char *ab = Ag + (long)kt * a_step, *bb = Bg + (long)kt * b_step;
+            const uint32_t sa = lds0 + stage * STAGE_BYTES, sb = sa + A_BYTES;
+#pragma unroll
+            for (int s = 0; s < T::SLOTS_A; s++) T::request(ab, offa[s], sa + s * 1024);
+#pragma unroll
+            for (int s = 0; s < T::SLOTS_B; s++) T::request(bb, offb[s], sb + s * 1024);
+        };
+        // requests complete in order: "tile t has landed" is "no more outstanding than were issued after it"
+        request(0, 0);
+        if (nk > 1) { request(1, 1); asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory"); }
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        barrier();                                                  // tile 0 has landed
+        if (nk > 2) request(2, 2);
+        for (int kt = 0; kt < nk; kt++) {
+            if (kt + 2 < nk) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory");      // tile kt + 1 has landed
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            barrier();                                              // B_kt
+            if (kt + 3 < nk) request(kt + 3, kt % 3);
+        }
+        return;
+    }
+    float2v *ln_slot = reinterpret_cast<float2v *>(smem + STAGES * STAGE_BYTES);
+    lnf_stage<BM, BN, 256>(p, ln_slot, m0, n0, bz, tid);
+
+    // fragment read offsets inside a stage (bytes): rows of A, and this wave's columns of B in either layout
+    const int frow = lane & 31, fhi = lane >> 5;
+    const int swz = T::rowswz(lane & 15);
+    int a_rd[KS], b_rd[KS], bt_rd[TN];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        const int cc = ((2 * ks + fhi) ^ swz) << 4;
+        a_rd[ks] = frow * ROWB + cc;
+        b_rd[ks] = A_BYTES + (wave * WTN + frow) * ROWB + cc;
+    }
+    {
+        const int kk = (lane >> 2) & 3;
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+            const int col = (wave * WTN + i * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4) ^ (kk << 5);
+            bt_rd[i] = A_BYTES + ((fhi * 8 + kk) * BN + col) * 2;
+        }
+    }
+    // fragment q of a 16-deep step: q < TM the A rows 32 q .., else the wave's B columns 32 (q - TM) ..
+    constexpr int NFRAG = TM + TN;
+    auto read_frag = [&](const char *st, int ks, int q, half8v (&a)[TM], half8v (&b)[TN]) {
+        if (q < TM) {
+            a[q] = *reinterpret_cast<const half8v *>(st + a_rd[ks] + q * 32 * ROWB);
+        } else if (!B_KN) {
+            b[q - TM] = *reinterpret_cast<const half8v *>(st + b_rd[ks] + (q - TM) * 32 * ROWB);
+        } else {
+            const char *bs = st + bt_rd[q - TM] + ks * 16 * BN * 2;
+            short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(bs));
+            short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(bs + 4 * BN * 2));
+            short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            b[q - TM] = __builtin_bit_cast(half8v, both);
+        }
+    };
+    auto read_step = [&](const char *st, int ks, half8v (&a)[TM], half8v (&b)[TN]) {
+#pragma unroll
+        for (int q = 0; q < NFRAG; q++) read_frag(st, ks, q, a, b);
+    };
+    float16v acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    // The MFMAs of rows [JLO, JHI) x all columns of one step, from fragment set (a, b), with the reads of step ks of
+    // the stage at st into set (da, db) dealt between them: a wave that issues its six or eight LDS instructions in
+    // one burst stands at them while the LDS queue drains, and its matrix pipe runs dry behind it.  The scheduling
+    // groups pin the order the source has: one MFMA, then the LDS reads that follow it.
+    auto step = [&](auto JLO, auto JHI, const half8v (&a)[TM], const half8v (&b)[TN], const char *st, int ks, half8v (&da)[TM], half8v (&db)[TN]) {
+        constexpr int jlo = decltype(JLO)::value, jhi = decltype(JHI)::value, NM = (jhi - jlo) * TN;
+        static_for<NM>([&](auto Mi) {
+            constexpr int m = decltype(Mi)::value, j = jlo + m / TN, i = m % TN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[i], a[j], acc[i][j], 0, 0, 0);
+            constexpr int q0 = (m * NFRAG) / NM, q1 = ((m + 1) * NFRAG) / NM;      // fragments [q0, q1) go behind MFMA m
+            static_for<q1 - q0>([&](auto Qi) { read_frag(st, ks, q0 + decltype(Qi)::value, da, db); });
+        });
+        static_for<NM>([&](auto Mi) {
+            constexpr int m = decltype(Mi)::value, q0 = (m * NFRAG) / NM, q1 = ((m + 1) * NFRAG) / NM;
+            constexpr int a_frags = (q1 < TM ? q1 : TM) - (q0 < TM ? q0 : TM), b_frags = (q1 - q0) - a_frags;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if constexpr (q1 > q0) __builtin_amdgcn_sched_group_barrier(0x100, a_frags + b_frags * (B_KN ? 2 : 1), 0);
+        });
+    };
+    auto mma = [&](auto JLO, auto JHI, const half8v (&a)[TM], const half8v (&b)[TN]) {
+        constexpr int jlo = decltype(JLO)::value, jhi = decltype(JHI)::value;
+#pragma unroll
+        for (int j = jlo; j < jhi; j++)
+#pragma unroll
+            for (int i = 0; i < TN; i++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[i], a[j], acc[i][j], 0, 0, 0);
+    };
+    const bool probe = p.clk && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0;
+    if (probe) { p.clk[0] = clock64(); p.clk[1] = wall_clock64(); }
+    // Three sets of fragment registers: step s of a tile whose rotation is R sits in set (R + s) % 3, and the reads run
+    // two steps ahead of the MFMAs (one step ahead, a wave's reads came back just too late: 6 KB per wave and step at the
+    // 32 B/clock a SIMD takes from the LDS is 190 of the 256 clocks its eight MFMAs last, before any queueing).  Four
+    // steps a tile, so the rotation advances by one per tile and the loop body is three tiles long.
+    half8v fa[3][TM], fb[3][TN];
+    half4v cb[TN][4];
+    load_col_bias<TN, WTN>(p, cb, n0, wave, lane, bz);              // sixteen registers held through the loop; no trip to memory after it
+    barrier();                                                      // tile 0 has landed
+    read_step(smem, 0, fa[0], fb[0]);
+    read_step(smem, 1, fa[1], fb[1]);
+    int stage = 0;
+    auto tile = [&](auto R, int kt) {
+        constexpr int r = decltype(R)::value, s0 = r % 3, s1 = (r + 1) % 3, s2 = (r + 2) % 3;
+        const char *st = smem + stage * STAGE_BYTES;
+        stage = stage == STAGES - 1 ? 0 : stage + 1;
+        const char *nx = smem + stage * STAGE_BYTES;
+        using std::integral_constant;
+        constexpr integral_constant<int, 0> J0{};
+        constexpr integral_constant<int, TM / 2> JH{};
+        constexpr integral_constant<int, TM> JE{};
+        // steps 0 and 1, with the reads of steps 2 and 3
+        step(J0, JE, fa[s0], fb[s0], st, 2, fa[s2], fb[s2]);
+        __builtin_amdgcn_sched_barrier(0);
+        step(J0, JE, fa[s1], fb[s1], st, 3, fa[s0], fb[s0]);
+        __builtin_amdgcn_sched_barrier(0);
+        // step 2: every fragment read of tile kt has returned before this wave lets the loader have the stage; the
+        // reads of the next tile's steps 0 and 1 follow the barrier (past the last tile they fetch nothing anybody uses)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        mma(J0, JH, fa[s2], fb[s2]);
+        __builtin_amdgcn_sched_barrier(0);
+        barrier();                                                  // B_kt
+        step(JH, JE, fa[s2], fb[s2], nx, 0, fa[s1], fb[s1]);
+        __builtin_amdgcn_sched_barrier(0);
+        // step 3
+        step(J0, JE, fa[s0], fb[s0], nx, 1, fa[s2], fb[s2]);
+        __builtin_amdgcn_sched_barrier(0);
+        (void)kt;
+    };
+    for (int kt = 0;;) {
+        tile(std::integral_constant<int, 0>{}, kt);
+        if (++kt == nk) break;
+        tile(std::integral_constant<int, 1>{}, kt);
+        if (++kt == nk) break;
+        tile(std::integral_constant<int, 2>{}, kt);
+        if (++kt == nk) break;
+    }
+    LnFold<TM> ln;
+    if (p.lnf_stats) {
+        ln.on = true; ln.col = reinterpret_cast<const float *>(ln_slot + BM); ln.bn = BN;
+#pragma unroll
+        for (int j = 0; j < TM; j++) { const float2v v = ln_slot[32 * j + (lane & 31)]; ln.r[j] = v[0]; ln.rmu[j] = v[1]; }
+    }
+    store_tile<TM, TN, WTM, WTN, 4, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, 0, wave, wave, lane, bz, ln);
+    if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
+}
+
+// ------------------------------------------------------------------------------------------
 // Scalar kernel: one thread per output, fp32 accumulation seeded with the bias,
 // any strides.  The arithmetic of the reference's mm2 (matmul.jl:17-27).
 __global__ void gemm_scalar_kernel(GemmArgs p, int b_kn) {
@@ -2003,6 +2362,24 @@ int launch_pp(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
+template <int BM, int BN>
+int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
+    if (a.K < 64 || a.K % 64 || a.cv.xp || a.ag.x) return MI_DECLINE_EXTENT;
+    a.tiles_m = (int)ceil_div(a.M, BM);
+    a.tiles_n = (int)ceil_div(a.N, BN);
+    a.group_m = a.tiles_m < 6 ? a.tiles_m : 6;
+    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
+                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
+    // per-lane load offsets are 32-bit byte offsets from the tile origin
+    if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? 64 : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;
+    a.clk = g_clock_probe;
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
+    constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
+    if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, true>), grid, dim3(320), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, false>), grid, dim3(320), lds, st, a);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
 bool sk_fits(int64_t M, int64_t N, int64_t K, int bm, int bn, int split);
 
 // The ping-pong kernel with `split` workgroups per tile exchanging their partial tiles (see the kernel).
@@ -2042,7 +2419,7 @@ int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
 int launch_tile(int tile, const GemmArgs &a, bool b_kn, int64_t nbatch, hipStream_t st) {
     const bool plain = !a.cv.xp && !a.ag.x;
     switch (tile) {
-        case 0: return plain ? launch_pp<128, 256, 64, 3, 2, 4, true>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
+        case 0: return plain ? launch_w4<128, 256>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
         case 1: return launch_pipe<192, 128, 2, 4>(a, b_kn, nbatch, st);
         case 2: return launch_pipe<128, 128, 2, 4>(a, b_kn, nbatch, st);
         case 3: return launch_pipe<64, 128, 2, 4>(a, b_kn, nbatch, st);
@@ -2423,8 +2800,8 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 0, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 1, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 2>, gemm_lds_bytes<128, 128, 64>());
-    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true>, pp_lds_bytes<128, 256, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, true>, pp_lds_bytes<128, 256, 64, 3>());
+    bad |= raise_lds(gemm_w4_kernel<128, 256, true>, pp_lds_bytes<128, 256, 64, 3>());
+    bad |= raise_lds(gemm_w4_kernel<128, 256, false>, pp_lds_bytes<128, 256, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, false, true, true>, pp_lds_bytes<128, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 256, 64, 3>());
