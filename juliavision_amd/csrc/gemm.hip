@@ -1415,17 +1415,18 @@ struct DirectTile {
     }
 };
 
-template <int BM, int BN, bool B_KN>
-__global__ __launch_bounds__(320) void gemm_w4_kernel(GemmArgs p) {
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool B_KN>
+__global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
     constexpr int BK = 64, STAGES = 3, KS = 4;
     using T = DirectTile<BM, BN, BK, B_KN>;
     constexpr int ROWB = T::ROWB, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, PER_TILE = T::SLOTS_A + T::SLOTS_B;
-    constexpr int WTM = BM, WTN = BN / 4, TM = WTM / 32, TN = WTN / 32;
-    static_assert(TM * TN == 8 && PER_TILE <= 63, "128 accumulator registers a lane; vmcnt is a 6-bit counter");
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
+    static_assert(WAVES_M * WAVES_N == 4 && TM * TN <= 8 && TM >= 2 && PER_TILE <= 63, "one matrix wave per SIMD; at most 128 accumulator registers a lane; vmcnt is a 6-bit counter");
     static_assert(!B_KN || BN >= 128, "the [K][N] permutation moves a chunk by up to 12 places inside its row");
     extern __shared__ __align__(16) char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     int tm_, tn_;
     tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
     // (the division inside tile_of runs on the vector unit: hand the results back to scalar registers, which the
@@ -1471,7 +1472,83 @@ __global__ __launch_bounds__(320) void gemm_w4_kernel(GemmArgs p) {
         return;
     }
     float2v *ln_slot = reinterpret_cast<float2v *>(smem + STAGES * STAGE_BYTES);
-    lnf_stage<BM, BN, 256>(p, ln_slot, m0, n0, bz, tid);
+    if (wave == 5) {
+        // The statistics wave of a folded layer norm (the launch has it only then).  The matrix waves need (r, r mu) of
+        // the tile's rows and the tile's columns of colsum and biasp at the store, not before: combining a row's
+        // K / 32 segment statistics in the prologue held every wave at the first barrier (5 000 clocks at 128 rows,
+        // 10 000 at 192: a trip to memory per batch of loads, then forty dependent steps a row).  This wave does it
+        // beside the K loop instead: tile kt covers segments 2 kt and 2 kt + 1 (K % 64 == 0), so between two barriers
+        // it takes in the two segments of each of its BM / 64 rows that it requested four tiles earlier, and the
+        // result is in the LDS slot when it arrives at the last barrier, which the matrix waves pass before they
+        // store.  Same arithmetic, in the same order per row, as lnf_stage with one lane a row.
+        constexpr int NR = BM / 64, AHEAD = 4;
+        static_assert(BM % 64 == 0 && NR * 2 * AHEAD <= 63, "whole rows per lane; vmcnt is a 6-bit counter");
+        for (int t = lane; t < BN / 2; t += 64) {
+            const int which = t / (BN / 4), c = (t % (BN / 4)) * 4, n = n0 + c;
+            const float *src = (which == 0 ? p.lnf_colsum : p.lnf_biasp) + bz * p.lnf_svec;
+            float4v v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (n + 3 < p.N) v = *reinterpret_cast<const float4v *>(src + n);
+            else for (int e = 0; e < 4; e++) if (n + e < p.N) v[e] = src[n + e];
+            *reinterpret_cast<float4v *>(reinterpret_cast<float *>(ln_slot + BM) + which * BN + c) = v;
+        }
+        const float2v *seg[NR];
+#pragma unroll
+        for (int i = 0; i < NR; i++) seg[i] = reinterpret_cast<const float2v *>(p.lnf_stats) + min(m0 + lane + 64 * i, p.M - 1);
+        float2v v[AHEAD][NR][2];
+        float ref[NR], total[NR], within[NR], between[NR];
+#pragma unroll
+        for (int i = 0; i < NR; i++) { ref[i] = 0.0f; total[i] = 0.0f; within[i] = 0.0f; between[i] = 0.0f; }
+        auto fetch = [&](auto SLOT, int kt) {
+            constexpr int sl = decltype(SLOT)::value;
+#pragma unroll
+            for (int i = 0; i < NR; i++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) v[sl][i][h] = seg[i][(long)(2 * kt + h) * p.M];
+        };
+        auto take = [&](auto SLOT, int kt) {
+            constexpr int sl = decltype(SLOT)::value;
+#pragma unroll
+            for (int i = 0; i < NR; i++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    if (kt == 0 && h == 0) ref[i] = v[sl][i][0][0] * (1.0f / 32.0f);
+                    const float d = fmaf(v[sl][i][h][0], 1.0f / 32.0f, -ref[i]);
+                    total[i] += v[sl][i][h][0];
+                    within[i] += v[sl][i][h][1];
+                    between[i] = fmaf(32.0f * d, d, between[i]);
+                }
+        };
+        // tiles 0 .. AHEAD - 1 are requested before the first barrier; tile kt + AHEAD right after tile kt is taken in
+        static_for<AHEAD>([&](auto S) { if (decltype(S)::value < nk) fetch(S, decltype(S)::value); });
+        barrier();
+        for (int kt0 = 0; kt0 < nk; kt0 += AHEAD) {
+            static_for<AHEAD>([&](auto S) {
+                const int kt = kt0 + decltype(S)::value;
+                if (kt < nk) {
+                    // requests complete in order: what was requested after tile kt may still be on its way
+                    if (kt + AHEAD - 1 < nk) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 1) * NR * 2) : "memory");
+                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    take(S, kt);
+                    if (kt + AHEAD < nk) fetch(S, kt + AHEAD);
+                    if (kt + 1 == nk) {
+#pragma unroll
+                        for (int i = 0; i < NR; i++) {
+                            const float mu = total[i] / (float)p.K, dm = mu - ref[i];
+                            const float m2 = within[i] + fmaxf(between[i] - (float)p.K * dm * dm, 0.0f);
+                            const float r = 1.0f / sqrtf(m2 / (float)p.K + p.lnf_eps);
+                            const float2v o = {r, r * mu};
+                            ln_slot[lane + 64 * i] = o;
+                        }
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    }
+                    barrier();                                      // B_kt
+                }
+            });
+        }
+        return;
+    }
+    // (a launch without the statistics wave and with a folded norm: combine in the prologue, as the other kernels do)
+    if (blockDim.x < 384) lnf_stage<BM, BN, 256>(p, ln_slot, m0, n0, bz, tid);
 
     // fragment read offsets inside a stage (bytes): rows of A, and this wave's columns of B in either layout
     const int frow = lane & 31, fhi = lane >> 5;
@@ -1480,14 +1557,14 @@ __global__ __launch_bounds__(320) void gemm_w4_kernel(GemmArgs p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
         const int cc = ((2 * ks + fhi) ^ swz) << 4;
-        a_rd[ks] = frow * ROWB + cc;
-        b_rd[ks] = A_BYTES + (wave * WTN + frow) * ROWB + cc;
+        a_rd[ks] = (wm * WTM + frow) * ROWB + cc;
+        b_rd[ks] = A_BYTES + (wn * WTN + frow) * ROWB + cc;
     }
     {
         const int kk = (lane >> 2) & 3;
 #pragma unroll
         for (int i = 0; i < TN; i++) {
-            const int col = (wave * WTN + i * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4) ^ (kk << 5);
+            const int col = (wn * WTN + i * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4) ^ (kk << 5);
             bt_rd[i] = A_BYTES + ((fhi * 8 + kk) * BN + col) * 2;
         }
     }
@@ -1551,7 +1628,7 @@ __global__ __launch_bounds__(320) void gemm_w4_kernel(GemmArgs p) {
     // steps a tile, so the rotation advances by one per tile and the loop body is three tiles long.
     half8v fa[3][TM], fb[3][TN];
     half4v cb[TN][4];
-    load_col_bias<TN, WTN>(p, cb, n0, wave, lane, bz);              // sixteen registers held through the loop; no trip to memory after it
+    load_col_bias<TN, WTN>(p, cb, n0, wn, lane, bz);              // sixteen registers held through the loop; no trip to memory after it
     barrier();                                                      // tile 0 has landed
     read_step(smem, 0, fa[0], fb[0]);
     read_step(smem, 1, fa[1], fb[1]);
@@ -1595,9 +1672,9 @@ __global__ __launch_bounds__(320) void gemm_w4_kernel(GemmArgs p) {
     if (p.lnf_stats) {
         ln.on = true; ln.col = reinterpret_cast<const float *>(ln_slot + BM); ln.bn = BN;
 #pragma unroll
-        for (int j = 0; j < TM; j++) { const float2v v = ln_slot[32 * j + (lane & 31)]; ln.r[j] = v[0]; ln.rmu[j] = v[1]; }
+        for (int j = 0; j < TM; j++) { const float2v v = ln_slot[wm * WTM + 32 * j + (lane & 31)]; ln.r[j] = v[0]; ln.rmu[j] = v[1]; }
     }
-    store_tile<TM, TN, WTM, WTN, 4, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, 0, wave, wave, lane, bz, ln);
+    store_tile<TM, TN, WTM, WTN, 4, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln);
     if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
 }
 
@@ -2362,7 +2439,7 @@ int launch_pp(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
-template <int BM, int BN>
+template <int BM, int BN, int WM, int WN>
 int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     if (a.K < 64 || a.K % 64 || a.cv.xp || a.ag.x) return MI_DECLINE_EXTENT;
     a.tiles_m = (int)ceil_div(a.M, BM);
@@ -2375,8 +2452,10 @@ int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     a.clk = g_clock_probe;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
     constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
-    if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, true>), grid, dim3(320), lds, st, a);
-    else      hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, false>), grid, dim3(320), lds, st, a);
+    // four matrix waves and the loader, plus the statistics wave of a folded layer norm
+    const dim3 block(a.lnf_stats ? 384 : 320);
+    if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, WM, WN, true>), grid, block, lds, st, a);
+    else      hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, WM, WN, false>), grid, block, lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
@@ -2419,8 +2498,8 @@ int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
 int launch_tile(int tile, const GemmArgs &a, bool b_kn, int64_t nbatch, hipStream_t st) {
     const bool plain = !a.cv.xp && !a.ag.x;
     switch (tile) {
-        case 0: return plain ? launch_w4<128, 256>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
-        case 1: return launch_pipe<192, 128, 2, 4>(a, b_kn, nbatch, st);
+        case 0: return plain ? launch_w4<128, 256, 1, 4>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
+        case 1: return plain ? launch_w4<192, 128, 2, 2>(a, b_kn, nbatch, st) : launch_pipe<192, 128, 2, 4>(a, b_kn, nbatch, st);
         case 2: return launch_pipe<128, 128, 2, 4>(a, b_kn, nbatch, st);
         case 3: return launch_pipe<64, 128, 2, 4>(a, b_kn, nbatch, st);
         case 5: return plain ? launch_pp<256, 256, 32, 4, 2, 4, true>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
@@ -2800,8 +2879,10 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 0, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 1, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 2>, gemm_lds_bytes<128, 128, 64>());
-    bad |= raise_lds(gemm_w4_kernel<128, 256, true>, pp_lds_bytes<128, 256, 64, 3>());
-    bad |= raise_lds(gemm_w4_kernel<128, 256, false>, pp_lds_bytes<128, 256, 64, 3>());
+    bad |= raise_lds(gemm_w4_kernel<128, 256, 1, 4, true>, pp_lds_bytes<128, 256, 64, 3>());
+    bad |= raise_lds(gemm_w4_kernel<128, 256, 1, 4, false>, pp_lds_bytes<128, 256, 64, 3>());
+    bad |= raise_lds(gemm_w4_kernel<192, 128, 2, 2, true>, pp_lds_bytes<192, 128, 64, 3>());
+    bad |= raise_lds(gemm_w4_kernel<192, 128, 2, 2, false>, pp_lds_bytes<192, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, false, true, true>, pp_lds_bytes<128, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 256, 64, 3>());
