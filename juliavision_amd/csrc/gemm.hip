@@ -991,6 +991,117 @@ __device__ __noinline__ void sk_poison_region(void *Y, long ldY, int M, int N, i
     }
 }
 
+// The end of a split-K launch whose K-slices exchange their partial tiles (the kernels above say how the workgroups
+// of a tile are placed): every wave sends the sub-tiles it does not keep to its partners, raises its flag, waits
+// (bounded) for the same wave of every partner, sums what arrived in slice order and stores its share.
+// sk_part[tile][owner][source][wave of NWAVES][slot][4][64 lanes][4]; flags [tile][slice][8].
+template <int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
+__device__ __forceinline__ void sk_finish(const GemmArgs &p, float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], char *smem, int sk_tile, int sk_s,
+                                          int m0, int n0, int wm, int wn, int wave, int lane, long bz) {
+    // A wave's accumulators are NQ = TM * TN sub-tiles of 32 x 32, q = i * TM + j; sub-tile q goes to slice q % S.
+    constexpr int NQ = TM * TN;
+    static_assert(TM == 2 && (TN == 1 || TN == 2), "two or four 32 x 32 sub-tiles per wave");
+    const int S = p.sk_S, NSL = NQ / S;                    // slices (2, or 4 when NQ = 4); sub-tiles a wave keeps
+    // sk_part[tile][owner][source][wave][slot][4][64 lanes][4]: four registers per lane and access, 1 KB per wave instruction
+    auto part_of = [&](int owner, int src) { return p.sk_part + ((((long)sk_tile * S + owner) * S + src) * NWAVES + wave) * (long)(NSL * 1024) + lane * 4; };
+    static_for<NQ>([&](auto Q) {
+        constexpr int q = decltype(Q)::value, i = q / TM, j = q % TM;
+        if (q % S != sk_s) {                               // uniform
+            float *dst = part_of(q % S, sk_s) + (q / S) * 1024;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const float4v v = {acc[i][j][4 * r4], acc[i][j][4 * r4 + 1], acc[i][j][4 * r4 + 2], acc[i][j][4 * r4 + 3]};
+                *reinterpret_cast<float4v *>(dst + r4 * 256) = v;
+            }
+        }
+    });
+    // the partials must have reached L2 before the flag can be seen
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned my_xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u;      // HW_REG_XCC_ID, bits 3:0
+    unsigned *myflag = p.sk_flags + ((long)sk_tile * S + sk_s) * 8 + wave;
+    if (lane == 0) SkExchange::publish(myflag, p.sk_epoch ^ p.sk_pub_xor, my_xcc);
+    // the sub-tiles this wave keeps (slot 0, and slot 1 when it keeps two)
+    float16v own[2];
+    static_for<NQ>([&](auto Q) {
+        constexpr int q = decltype(Q)::value, i = q / TM, j = q % TM;
+        if (q % S == sk_s) {                               // uniform
+            if (q / S == 0) own[0] = acc[i][j]; else own[1] = acc[i][j];
+        }
+    });
+    // Wait (bounded) for the same wave of every partner, then fetch everything they sent in one trip: at most three
+    // blocks of sixteen registers (three partners' one sub-tile, or one partner's one or two).  The three polls of a
+    // round are in flight together: a poll is a trip past the L1.  Co-residency of the partners is NOT guaranteed
+    // (another stream's kernel can hold an XCD's CUs): the bound is the guard, and a wave that runs into it says so.
+    unsigned *fl[3];
+#pragma unroll
+    for (int bi = 0; bi < 3; bi++) {
+        const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;      // S = 4: the bi-th partner in slice order
+        fl[bi] = p.sk_flags + ((long)sk_tile * S + src) * 8 + wave;
+    }
+    const unsigned *const cfl[3] = {fl[0], fl[1], fl[2]};
+    const sk::WaitResult wr = SkExchange::wait(cfl, S == 4 ? 3 : 1, p.sk_epoch, my_xcc ^ p.sk_xcc_xor, p.sk_spin);
+    asm volatile("" ::: "memory");
+    if (wr != sk::ARRIVED) {
+        // Loud failure: the sticky status word, NaN over this wave's share of Y, flags left as they are (the host
+        // zeroes the banks when it reads the status).  The wave still leaves the kernel normally.
+        if (lane == 0) __hip_atomic_fetch_or(p.status, wr == sk::TIMED_OUT ? (unsigned)MI_DEVSTAT_EXCHANGE_TIMEOUT : (unsigned)MI_DEVSTAT_EXCHANGE_XCD,
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // (the exchange runs unbatched launches only: bz = 0)
+        if (NSL == 1) sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * (sk_s % TM), n0 + wn * WTN + 32 * (sk_s / TM), 32, lane);
+        else sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * sk_s, n0 + wn * WTN, WTN, lane);
+        return;
+    }
+    // Ordinary loads: this CU has not touched these lines since the kernel began (its L1 was invalidated then), so
+    // they come from the L2 the partners' acknowledged stores are in (the wait has checked that it is this XCD's).
+    float4v blk[3][4];
+#pragma unroll
+    for (int bi = 0; bi < 3; bi++) {
+        const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;
+        if (S == 4 || bi < NSL) {
+            const float *from = part_of(sk_s, src) + (S == 4 ? 0 : bi * 1024);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) blk[bi][r4] = *reinterpret_cast<const float4v *>(from + r4 * 256);
+        }
+    }
+    float16v tot[2];                                       // summed in slice order, whoever does the summing
+    if (S == 4) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float x0 = blk[0][r >> 2][r & 3], x1 = blk[1][r >> 2][r & 3], x2 = blk[2][r >> 2][r & 3], o = own[0][r];
+            tot[0][r] = sk_s == 0 ? ((o + x0) + x1) + x2 : sk_s == 1 ? ((x0 + o) + x1) + x2 : sk_s == 2 ? ((x0 + x1) + o) + x2 : ((x0 + x1) + x2) + o;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            tot[0][r] = sk_s == 0 ? own[0][r] + blk[0][r >> 2][r & 3] : blk[0][r >> 2][r & 3] + own[0][r];
+            if (NQ == 4) tot[1][r] = sk_s == 0 ? own[1][r] + blk[1][r >> 2][r & 3] : blk[1][r >> 2][r & 3] + own[1][r];
+        }
+    }
+    // What the partners sent has arrived (the sums above used it).  The last wave to have consumed a partner's
+    // partials clears that partner's flag -- with two slices that is this wave, with four the third to count itself
+    // in -- so the next launch on this bank, which for a replayed graph carries this same epoch, starts from zero.
+    if (lane == 0) {
+#pragma unroll
+        for (int bi = 0; bi < 3; bi++)
+            if (S == 4 || bi == 0) SkExchange::release(fl[bi], fl[bi] + SK_WORDS, S == 4 ? 3 : 1);
+    }
+    // One kept sub-tile (S = NQ): q = s.  Two (S = 2 of four): q = s and s + 2, the 32-row half j = s at both
+    // 32-column halves.
+    if (NSL == 1) {
+        const int i = sk_s / TM, j = sk_s % TM;
+        float16v one[1][1] = {{tot[0]}};
+        half4v cb1[1][4];
+        // a 32-column store: the wave's column origin goes into n0 (the staging rows are as wide as the stored tile)
+        const int nw = n0 + wn * WTN + 32 * i;
+        load_col_bias<1, 32>(p, cb1, nw, 0, lane, bz);
+        store_tile<1, 1, WTM, 32, NWAVES, LDS_BYTES>(p, one, cb1, smem, m0 + 32 * j, nw, wm, 0, wave, lane, bz);
+    } else if constexpr (TN == 2) {
+        float16v two[2][1] = {{tot[0]}, {tot[1]}};
+        store_tile<1, 2, WTM, WTN, NWAVES, LDS_BYTES>(p, two, cb, smem, m0 + 32 * sk_s, n0, wm, wn, wave, lane, bz);
+    }
+    return;
+}
+
 // With three 64-deep stages a ninth wave does nothing but request operand tiles (pp_loader).  A 1 KB
 // global_load_lds_dwordx4 takes the CU's vector-memory path sixteen clocks, so a wave that issues its share of a tile
 // stands at those instructions while its three partners' requests drain ahead of it -- 190 of the 750 clocks of a
@@ -1256,108 +1367,7 @@ __global__ __launch_bounds__((pp_threads<BK, STAGES, PINGPONG>())) void gemm_pp_
         stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
     if constexpr (SK) {
-        // A wave's accumulators are NQ = TM * TN sub-tiles of 32 x 32, q = i * TM + j; sub-tile q goes to slice q % S.
-        constexpr int NQ = TM * TN;
-        static_assert(TM == 2 && (TN == 1 || TN == 2), "two or four 32 x 32 sub-tiles per wave");
-        const int S = p.sk_S, NSL = NQ / S;                    // slices (2, or 4 when NQ = 4); sub-tiles a wave keeps
-        // sk_part[tile][owner][source][wave][slot][4][64 lanes][4]: four registers per lane and access, 1 KB per wave instruction
-        auto part_of = [&](int owner, int src) { return p.sk_part + ((((long)sk_tile * S + owner) * S + src) * 8 + wave) * (long)(NSL * 1024) + lane * 4; };
-        static_for<NQ>([&](auto Q) {
-            constexpr int q = decltype(Q)::value, i = q / TM, j = q % TM;
-            if (q % S != sk_s) {                               // uniform
-                float *dst = part_of(q % S, sk_s) + (q / S) * 1024;
-#pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) {
-                    const float4v v = {acc[i][j][4 * r4], acc[i][j][4 * r4 + 1], acc[i][j][4 * r4 + 2], acc[i][j][4 * r4 + 3]};
-                    *reinterpret_cast<float4v *>(dst + r4 * 256) = v;
-                }
-            }
-        });
-        // the partials must have reached L2 before the flag can be seen
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const unsigned my_xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u;      // HW_REG_XCC_ID, bits 3:0
-        unsigned *myflag = p.sk_flags + ((long)sk_tile * S + sk_s) * 8 + wave;
-        if (lane == 0) SkExchange::publish(myflag, p.sk_epoch ^ p.sk_pub_xor, my_xcc);
-        // the sub-tiles this wave keeps (slot 0, and slot 1 when it keeps two)
-        float16v own[2];
-        static_for<NQ>([&](auto Q) {
-            constexpr int q = decltype(Q)::value, i = q / TM, j = q % TM;
-            if (q % S == sk_s) {                               // uniform
-                if (q / S == 0) own[0] = acc[i][j]; else own[1] = acc[i][j];
-            }
-        });
-        // Wait (bounded) for the same wave of every partner, then fetch everything they sent in one trip: at most three
-        // blocks of sixteen registers (three partners' one sub-tile, or one partner's one or two).  The three polls of a
-        // round are in flight together: a poll is a trip past the L1.  Co-residency of the partners is NOT guaranteed
-        // (another stream's kernel can hold an XCD's CUs): the bound is the guard, and a wave that runs into it says so.
-        unsigned *fl[3];
-#pragma unroll
-        for (int bi = 0; bi < 3; bi++) {
-            const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;      // S = 4: the bi-th partner in slice order
-            fl[bi] = p.sk_flags + ((long)sk_tile * S + src) * 8 + wave;
-        }
-        const unsigned *const cfl[3] = {fl[0], fl[1], fl[2]};
-        const sk::WaitResult wr = SkExchange::wait(cfl, S == 4 ? 3 : 1, p.sk_epoch, my_xcc ^ p.sk_xcc_xor, p.sk_spin);
-        asm volatile("" ::: "memory");
-        if (wr != sk::ARRIVED) {
-            // Loud failure: the sticky status word, NaN over this wave's share of Y, flags left as they are (the host
-            // zeroes the banks when it reads the status).  The wave still leaves the kernel normally.
-            if (lane == 0) __hip_atomic_fetch_or(p.status, wr == sk::TIMED_OUT ? (unsigned)MI_DEVSTAT_EXCHANGE_TIMEOUT : (unsigned)MI_DEVSTAT_EXCHANGE_XCD,
-                                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            // (the exchange runs unbatched launches only: bz = 0)
-            if (NSL == 1) sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * (sk_s % TM), n0 + wn * WTN + 32 * (sk_s / TM), 32, lane);
-            else sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * sk_s, n0 + wn * WTN, WTN, lane);
-            if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
-            return;
-        }
-        // Ordinary loads: this CU has not touched these lines since the kernel began (its L1 was invalidated then), so
-        // they come from the L2 the partners' acknowledged stores are in (the wait has checked that it is this XCD's).
-        float4v blk[3][4];
-#pragma unroll
-        for (int bi = 0; bi < 3; bi++) {
-            const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;
-            if (S == 4 || bi < NSL) {
-                const float *from = part_of(sk_s, src) + (S == 4 ? 0 : bi * 1024);
-#pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) blk[bi][r4] = *reinterpret_cast<const float4v *>(from + r4 * 256);
-            }
-        }
-        float16v tot[2];                                       // summed in slice order, whoever does the summing
-        if (S == 4) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float x0 = blk[0][r >> 2][r & 3], x1 = blk[1][r >> 2][r & 3], x2 = blk[2][r >> 2][r & 3], o = own[0][r];
-                tot[0][r] = sk_s == 0 ? ((o + x0) + x1) + x2 : sk_s == 1 ? ((x0 + o) + x1) + x2 : sk_s == 2 ? ((x0 + x1) + o) + x2 : ((x0 + x1) + x2) + o;
-            }
-        } else {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                tot[0][r] = sk_s == 0 ? own[0][r] + blk[0][r >> 2][r & 3] : blk[0][r >> 2][r & 3] + own[0][r];
-                if (NQ == 4) tot[1][r] = sk_s == 0 ? own[1][r] + blk[1][r >> 2][r & 3] : blk[1][r >> 2][r & 3] + own[1][r];
-            }
-        }
-        // What the partners sent has arrived (the sums above used it).  The last wave to have consumed a partner's
-        // partials clears that partner's flag -- with two slices that is this wave, with four the third to count itself
-        // in -- so the next launch on this bank, which for a replayed graph carries this same epoch, starts from zero.
-        if (lane == 0) {
-#pragma unroll
-            for (int bi = 0; bi < 3; bi++)
-                if (S == 4 || bi == 0) SkExchange::release(fl[bi], fl[bi] + SK_WORDS, S == 4 ? 3 : 1);
-        }
-        // One kept sub-tile (S = NQ): q = s.  Two (S = 2 of four): q = s and s + 2, the 32-row half j = s at both
-        // 32-column halves.
-        if (NSL == 1) {
-            const int i = sk_s / TM, j = sk_s % TM;
-            float16v one[1][1] = {{tot[0]}};
-            half4v cb1[1][4];
-            // a 32-column store: the wave's column origin goes into n0 (the staging rows are as wide as the stored tile)
-            const int nw = n0 + wn * WTN + 32 * i;
-            load_col_bias<1, 32>(p, cb1, nw, 0, lane, bz);
-            store_tile<1, 1, WTM, 32, 8, STAGES * STAGE_BYTES>(p, one, cb1, smem, m0 + 32 * j, nw, wm, 0, wave, lane, bz);
-        } else if constexpr (TN == 2) {
-            float16v two[2][1] = {{tot[0]}, {tot[1]}};
-            store_tile<1, 2, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, two, cb, smem, m0 + 32 * sk_s, n0, wm, wn, wave, lane, bz);
-        }
+        sk_finish<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, sk_tile, sk_s, m0, n0, wm, wn, wave, lane, bz);
         if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
         return;
     }
@@ -1415,7 +1425,7 @@ struct DirectTile {
     }
 };
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool B_KN>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool B_KN, bool SK = false>
 __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
     constexpr int BK = 64, STAGES = 3, KS = 4;
     using T = DirectTile<BM, BN, BK, B_KN>;
@@ -1427,16 +1437,30 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-    int tm_, tn_;
-    tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
-    // (the division inside tile_of runs on the vector unit: hand the results back to scalar registers, which the
-    // direct loads' base addresses have to be in)
+    int tm_, tn_, sk_s = 0, sk_tile = 0;
+    if constexpr (SK) {
+        // K-slice s of tile xcd * tpx + slot is workgroup (slot * S + s) * 8 + xcd: a tile's slices share an XCD (the
+        // ping-pong kernel's split-K instances say more); an XCD's run of the tile order is about square
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        sk_s = idx % p.sk_S;
+        sk_tile = xcd * p.sk_tpx + idx / p.sk_S;
+        if (sk_tile >= p.tiles_m * p.tiles_n) return;          // the whole workgroup: the last XCD's run may be short
+        const int width = p.group_m * p.tiles_n, g = sk_tile / width, in = sk_tile - g * width;
+        const int first = g * p.group_m, gsz = min(p.tiles_m - first, p.group_m);
+        tm_ = first + in % gsz;
+        tn_ = in / gsz;
+    } else {
+        tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
+    }
+    // (the divisions above run on the vector unit: hand the results back to scalar registers, which the direct loads'
+    // base addresses have to be in)
     const int m0 = __builtin_amdgcn_readfirstlane(tm_ * BM), n0 = __builtin_amdgcn_readfirstlane(tn_ * BN);
+    sk_s = __builtin_amdgcn_readfirstlane(sk_s);
     const long bz = blockIdx.y;
-    const int nk = p.K / BK;
+    const int nk = SK ? p.K / BK / p.sk_S : p.K / BK;      // the launcher guarantees whole BK-deep tiles per slice
     const long a_step = BK * 2, b_step = B_KN ? (long)BK * p.ldB * 2 : BK * 2;
-    const char *Ag = reinterpret_cast<const char *>(p.A + bz * p.sA + (long)m0 * p.ldA);
-    const char *Bg = reinterpret_cast<const char *>(p.B + bz * p.sB + (B_KN ? (long)n0 : (long)n0 * p.ldB));
+    const char *Ag = reinterpret_cast<const char *>(p.A + bz * p.sA + (long)m0 * p.ldA) + (SK ? (long)sk_s * nk * a_step : 0L);
+    const char *Bg = reinterpret_cast<const char *>(p.B + bz * p.sB + (B_KN ? (long)n0 : (long)n0 * p.ldB)) + (SK ? (long)sk_s * nk * b_step : 0L);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
     auto barrier = [&]() {
         asm volatile("" ::: "memory");
@@ -1667,6 +1691,11 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
         if (++kt == nk) break;
         tile(std::integral_constant<int, 2>{}, kt);
         if (++kt == nk) break;
+    }
+    if constexpr (SK) {
+        sk_finish<TM, TN, WTM, WTN, 4, STAGES * STAGE_BYTES>(p, acc, cb, smem, sk_tile, sk_s, m0, n0, wm, wn, wave, lane, bz);
+        if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
+        return;
     }
     LnFold<TM> ln;
     if (p.lnf_stats) {
@@ -2492,6 +2521,36 @@ int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
+// The four-wave kernel with two workgroups per 128 x 128 tile exchanging their partial tiles.
+int launch_w4_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
+    constexpr int BM = 128, BN = 128;
+    if (a.cv.xp || a.ag.x || split != 2 || !sk_usable() || !sk_fits(a.M, a.N, a.K, BM, BN, split)) return MI_DECLINE_EXTENT;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MI_ERROR_DEVICE;
+    a.tiles_m = (int)ceil_div(a.M, BM);
+    a.tiles_n = (int)ceil_div(a.N, BN);
+    a.group_m = 1;
+    while (a.group_m * a.group_m < (int)ceil_div((int64_t)a.tiles_m * a.tiles_n, 8) && a.group_m < a.tiles_m) a.group_m++;
+    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
+                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
+    if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? 64 : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;
+    const int tiles = a.tiles_m * a.tiles_n;
+    a.sk_S = split;
+    a.sk_tpx = (int)ceil_div(tiles, 8);
+    a.sk_part = reinterpret_cast<float *>(ws);
+    const unsigned launch = ++g_sk_epoch;
+    a.sk_epoch = sk::epoch_of(launch);
+    a.sk_flags = g_sk_flags_ptr[dev] + (size_t)(launch % SK_BANKS) * SK_FLAGS;
+    a.sk_spin = g_sk_spin; a.sk_pub_xor = g_sk_pub_xor; a.sk_xcc_xor = g_sk_xcc_xor;
+    a.status = g_status_ptr[dev];
+    a.clk = g_clock_probe;
+    dim3 grid((unsigned)(8 * a.sk_tpx * split), 1);
+    constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
+    if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, 2, 2, true, true>), grid, dim3(320), lds, st, a);
+    else      hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, 2, 2, false, true>), grid, dim3(320), lds, st, a);
+    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
+}
+
 // tile: index into TILE_MODELS.  The ping-pong kernels take ordinary operands only; a gathered operand (implicit-GEMM
 // convolution) planned onto one of their tiles runs the pipelined kernel's 128 x 256 tile instead: same K order per
 // output, same bits, and the plan (hence the workspace) stays a function of the extents alone.
@@ -2753,7 +2812,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         }
         int split = tp.split;
         if (split > 1 && tp.peer && ws && aligned_to(ws, 256) && ws_bytes >= plan_workspace_bytes(tp, a.M, a.N)) {
-            const int rc = tp.tile == 0 ? launch_pp_peer<128, 256>(a, b_kn, split, ws, st) : launch_pp_peer<128, 128>(a, b_kn, split, ws, st);
+            const int rc = tp.tile == 0 ? launch_pp_peer<128, 256>(a, b_kn, split, ws, st) : launch_w4_peer(a, b_kn, split, ws, st);
             if (rc != MI_DECLINE_EXTENT) return rc;     // declined (a gathered operand, a device that failed the probe): planes
             if (in_store) { tp = plan_tiles(a.M, a.N, a.K, nbatch, false); split = 1; }
         }
@@ -2883,8 +2942,8 @@ int mi_init(void) {
     bad |= raise_lds(gemm_w4_kernel<128, 256, 1, 4, false>, pp_lds_bytes<128, 256, 64, 3>());
     bad |= raise_lds(gemm_w4_kernel<192, 128, 2, 2, true>, pp_lds_bytes<192, 128, 64, 3>());
     bad |= raise_lds(gemm_w4_kernel<192, 128, 2, 2, false>, pp_lds_bytes<192, 128, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 128, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<128, 128, 64, 3, 2, 4, false, true, true>, pp_lds_bytes<128, 128, 64, 3>());
+    bad |= raise_lds(gemm_w4_kernel<128, 128, 2, 2, true, true>, pp_lds_bytes<128, 128, 64, 3>());
+    bad |= raise_lds(gemm_w4_kernel<128, 128, 2, 2, false, true>, pp_lds_bytes<128, 128, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 256, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, true, true>, pp_lds_bytes<128, 256, 64, 3>());
     bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, true, true>, pp_lds_bytes<256, 256, 32, 4>());
