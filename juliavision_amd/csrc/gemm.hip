@@ -2590,8 +2590,10 @@ int launch_mfma(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
 struct TileModel { int bm, bn; double step_lo, step_full, round, fixed; };
 constexpr int NTILES = 6;
 constexpr TileModel TILE_MODELS[NTILES] = {
-    {128, 256, 0.660, 0.970, 0.97, 5.6},
-    {192, 128, 0.545, 0.800, 0.93, 4.8},
+    // (the two tiles of the four-wave kernel, re-timed with it: 1500 x 5120 in 25.3 / 70.5 us at K = 1280 / 5120,
+    // 512 x 1280 in 16.3 / 47.2; 1500 x 3840 on 192 x 128 in 20.2 / 55.4, 512 x 1280 in 13.5 / 39.9)
+    {128, 256, 0.520, 0.760, 1.06, 7.0},
+    {192, 128, 0.420, 0.585, 1.00, 6.0},
     {128, 128, 0.428, 0.600, 1.00, 4.0},
     {64, 128, 0.318, 0.430, 0.90, 3.1},
     {64, 64, 0.235, 0.315, 0.73, 3.0},
@@ -2622,7 +2624,9 @@ double tile_cost_us(int64_t M, int64_t N, int64_t K, int64_t nbatch, int tile, i
 constexpr int SK_TILES[2] = {0, 2};      // indices into TILE_MODELS: 128 x 256, 128 x 128
 double sk_exchange_us(int64_t wg, int bm, int bn, int split) {
     const double mb = (double)wg * bm * bn * 4.0 * (split - 1) / split / 1e6;
-    return 3.0 + 0.45 * mb;      // fitted: 33.6 us measured on 1500 x 5120 -> 1280 (128 x 128, two slices), 37.8 (128 x 256, four)
+    // fitted: two slices, 29.8 us measured on 1500 x 5120 -> 1280 (128 x 128) and 39.7 on 1024 x 5120 -> 2560 (128 x 256);
+    // four slices (three partners to wait for), 40.8 on 1500 x 5120 -> 1280 and 31.0 on 512 x 5120 -> 1280 (128 x 256)
+    return split == 2 ? 2.0 + 0.3 * mb : 8.0 + 0.5 * mb;
 }
 size_t sk_workspace_bytes(int64_t M, int64_t N, int bm, int bn, int split) { return (size_t)(ceil_div(M, bm) * ceil_div(N, bn)) * split * bm * bn * 4; }
 bool sk_fits(int64_t M, int64_t N, int64_t K, int bm, int bn, int split) {
