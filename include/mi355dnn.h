@@ -72,8 +72,8 @@ int mi_init(void);
 int mi_device_caps(int64_t out[6]);
 
 /* Measurement aid (no counterpart in the reference).  While a device buffer of four uint64 is registered (NULL
- * clears it), workgroup 0 of every launch of the ping-pong GEMM kernels (the 128 x 256 and 256 x 256 tiles of
- * mi_gemm_f16 and its variants) stores {shader clock, constant 100 MHz clock} there when it starts and again after
+ * clears it), workgroup 0 of every launch of the four-wave GEMM kernel (the 128 x 256, 192 x 128 and split
+ * 128 x 128 tiles of mi_gemm_f16 and its variants) stores {shader clock, constant 100 MHz clock} there when it starts and again after
  * its last store: buf = {clk0, ref0, clk1, ref1}, and (clk1 - clk0) / (ref1 - ref0) x 100 MHz is the shader clock the
  * launch ran at.  The caller keeps the buffer alive while it is registered.  Process-wide, not thread safe. */
 int mi_set_clock_probe(void *dev_u64x4);

@@ -11,7 +11,7 @@
 #include <type_traits>
 #include <atomic>
 
-// Arrival flags of the split-K peer reduction (gemm_pp_kernel, SK): SK_BANKS banks of SK_FLAGS words, and as many
+// Arrival flags of the split-K peer reduction (gemm_w4_kernel, SK): SK_BANKS banks of SK_FLAGS words, and as many
 // counters behind them (word i's counter is word i + SK_WORDS).  A launch uses the bank its epoch selects, so launches
 // that overlap on one GPU (up to SK_BANKS of them) do not see each other's.  Every word is zero when the module loads
 // and zero again when a launch ends: the last consumer of a flag clears it (and its counter), so a captured launch --
@@ -53,11 +53,11 @@ struct GemmArgs {
     // Tiled kernels and the split-K plane sums: > 0 clamps the fp16 result to [-clamp, clamp] after the residual add,
     // as a separate aten::clamp on Y would (the overflow guard of exported fp16 encoder layers).
     float clamp;
-    // Measurement only (mi_set_clock_probe): workgroup 0 of a ping-pong launch stores {shader clock, 100 MHz clock}
+    // Measurement only (mi_set_clock_probe): workgroup 0 of a four-wave launch stores {shader clock, 100 MHz clock}
     // here when it starts and again after its last store.  Null in ordinary use.
     unsigned long long *clk;
     // Split-K with the partial tiles exchanged between the workgroups of a tile instead of written as planes
-    // (ping-pong kernel, SK instances): sk_S workgroups per tile, tiles dealt sk_tpx per XCD; partials in sk_part,
+    // (gemm_w4_kernel, SK instance): sk_S = 2 workgroups per tile, tiles dealt sk_tpx per XCD; partials in sk_part,
     // per-wave arrival flags in sk_flags (they carry sk_epoch; the last reader of a flag clears it).
     int sk_S, sk_tpx;
     float *sk_part;
@@ -934,41 +934,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, 2) void gemm_pipe_kernel(Gem
 }
 
 // ------------------------------------------------------------------------------------------
-// The ping-pong kernel: K % BK == 0, ordinary (ungathered) operands, eight waves.
+// Split-K without fp32 planes and without a second launch: the two workgroups of a tile (gemm_w4_kernel, SK) exchange
+// their partial tiles inside the launch.
 //
-// Operand tiles travel global -> LDS without passing through registers (global_load_lds_dwordx4: every lane
-// of a wave hands over 16 bytes, the wave's 1 KB lands contiguously at the LDS address in M0), STAGES BK-deep
-// stages deep, so a tile's loads are issued STAGES - 1 tiles ahead of its use and cost no VGPRs and no LDS-write
-// issue slots.  Unpadded rows would put every row of a fragment read on the same banks, and a direct load cannot pad
-// inside its 1 KB, so the 16-byte chunks are permuted instead: the chunk a lane fetches is chosen so that LDS
-// position `pos` of row r holds chunk pos ^ swz(r) (K-contiguous operands: swz = (r & 7) ^ ((r >> 3) & 1) for
-// 128-byte rows, (r >> 2) & 3 for 64-byte rows; the [K][N] operand: chunk ^ ((k & 3) << 2)), and the fragment
-// reads apply the same permutation.
-//
-// The two waves of a SIMD alternate between a memory phase (all fragment reads of a BK-deep tile plus the wave's
-// share of the loads of tile kt + STAGES - 1) and a matrix phase (the tile's 16 MFMAs): waves 0-3 (one per
-// SIMD) run one phase ahead of waves 4-7, a workgroup barrier closes every phase, and so one wave of each SIMD
-// always has a full phase of MFMAs queued while the other waits on LDS.  Every wave executes the same number of
-// barriers: the trailing group takes one extra at the start and none after its last matrix phase.
-//
-// Stage of tile t: t % STAGES.  A stage is free again once both groups have read it, i.e. after the barrier that
-// closes the trailing group's memory phase; tile t + STAGES is requested into it during the following memory phases
-// and has to have landed 2 (STAGES - 1) phases later: each wave waits for its own share (s_waitcnt vmcnt) ahead of the barrier that
-// precedes the leading group's first read of that tile.
-//
-// SK instances split K over the sk_S (2 or 4) workgroups of a tile without fp32 planes and without a second launch.
 // Workgroup pid runs on XCD pid % 8 (workgroups are dealt to the XCDs round robin; mi_init checks that this device
-// does so and the path stays off otherwise): pid = (slot * S + s) * 8 + xcd computes K-slice s of tile xcd * tpx + slot,
+// does so and the path stays off otherwise): pid = (slot * 2 + s) * 8 + xcd computes K-slice s of tile xcd * tpx + slot,
 // so the partners of a tile share an XCD, i.e. one L2, and are dispatched together.  After its K loop every wave owns
-// a quarter (S = 4) or half (S = 2) of its 64 x 64 accumulators -- the 32 x 32 sub-tiles q with q % S == s -- writes the
-// others into its partners' slots of sk_part (plain stores: they stay in the shared L2), waits for them to be
-// acknowledged, and raises its flag; it then waits (bounded) for the same wave of every partner, adds what they sent
-// in slice order (the result does not depend on which workgroup sums), and stores its share through the usual
-// epilogue.  Every workgroup publishes before it waits, so the waits are not circular among resident workgroups; the
-// launcher only checks that the grid fits an IDLE device in one round.  Under overlap (another stream's kernel holding
-// CUs) a partner may not be resident yet: the wait is bounded, and a wave that runs into the bound -- or finds its
-// partner on another XCD -- raises the device's sticky status word (mi_device_status), stores NaN over its share of Y
-// and releases nothing (sk_exchange.hpp has the protocol; tests/sk_exchange_host_test.cpp runs it on CPU threads).
+// half of its 64 x 64 accumulators -- the 32-row block s -- writes the other half into its partner's slot of sk_part
+// (plain stores: they stay in the shared L2), waits for them to be acknowledged, and raises its flag; it then waits
+// (bounded) for the same wave of its partner, adds what it sent in slice order (the result does not depend on which
+// workgroup sums), and stores its share through the usual epilogue.  Both workgroups publish before they wait, so the
+// waits are not circular among resident workgroups; the launcher only checks that the grid fits an IDLE device in
+// one round.  Under overlap (another stream's kernel holding CUs) a partner may not be resident yet: the wait is
+// bounded, and a wave that runs into the bound -- or finds its partner on another XCD -- raises the device's sticky
+// status word (mi_device_status), stores NaN over its share of Y and releases nothing (sk_exchange.hpp has the
+// protocol; tests/sk_exchange_host_test.cpp runs it on CPU threads, with one and with three partners).
+// (Four slices of a 128 x 256 tile were built and measured as well: three partners to wait for, 23 MB exchanged at
+// 1500 x 5120 -> 1280, 40.8 us against 29.8 us for two slices of 128 x 128.)
 struct SkDeviceMem {
     __device__ static unsigned load(const unsigned *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
     __device__ static void store(unsigned *p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -991,55 +973,42 @@ __device__ __noinline__ void sk_poison_region(void *Y, long ldY, int M, int N, i
     }
 }
 
-// The end of a split-K launch whose K-slices exchange their partial tiles (the kernels above say how the workgroups
-// of a tile are placed): every wave sends the sub-tiles it does not keep to its partners, raises its flag, waits
-// (bounded) for the same wave of every partner, sums what arrived in slice order and stores its share.
-// sk_part[tile][owner][source][wave of NWAVES][slot][4][64 lanes][4]; flags [tile][slice][8].
+// The end of a split-K launch whose two K-slices exchange their partial tiles: every wave sends the 32-row block it
+// does not keep to its partner, raises its flag, waits (bounded) for the same wave of the partner, sums what arrived
+// in slice order and stores its block.
+// sk_part[tile][owner][source][wave of NWAVES][column half][4][64 lanes][4]; flags [tile][slice][8].
 template <int TM, int TN, int WTM, int WTN, int NWAVES, int LDS_BYTES>
 __device__ __forceinline__ void sk_finish(const GemmArgs &p, float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], char *smem, int sk_tile, int sk_s,
                                           int m0, int n0, int wm, int wn, int wave, int lane, long bz) {
-    // A wave's accumulators are NQ = TM * TN sub-tiles of 32 x 32, q = i * TM + j; sub-tile q goes to slice q % S.
-    constexpr int NQ = TM * TN;
-    static_assert(TM == 2 && (TN == 1 || TN == 2), "two or four 32 x 32 sub-tiles per wave");
-    const int S = p.sk_S, NSL = NQ / S;                    // slices (2, or 4 when NQ = 4); sub-tiles a wave keeps
-    // sk_part[tile][owner][source][wave][slot][4][64 lanes][4]: four registers per lane and access, 1 KB per wave instruction
-    auto part_of = [&](int owner, int src) { return p.sk_part + ((((long)sk_tile * S + owner) * S + src) * NWAVES + wave) * (long)(NSL * 1024) + lane * 4; };
-    static_for<NQ>([&](auto Q) {
-        constexpr int q = decltype(Q)::value, i = q / TM, j = q % TM;
-        if (q % S != sk_s) {                               // uniform
-            float *dst = part_of(q % S, sk_s) + (q / S) * 1024;
+    static_assert(TM == 2 && TN == 2, "a wave's 64 x 64 accumulators: two 32-row blocks of two 32 x 32 sub-tiles");
+    // four registers per lane and access, 1 KB per wave instruction
+    auto part_of = [&](int owner, int src) { return p.sk_part + ((((long)sk_tile * 2 + owner) * 2 + src) * NWAVES + wave) * 2048L + lane * 4; };
+    float16v own[2];
+    static_for<2>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+        if (j == sk_s) {                                       // uniform: the block this wave keeps
+            own[0] = acc[0][j]; own[1] = acc[1][j];
+        } else {
+            float *dst = part_of(j, sk_s);
 #pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-                const float4v v = {acc[i][j][4 * r4], acc[i][j][4 * r4 + 1], acc[i][j][4 * r4 + 2], acc[i][j][4 * r4 + 3]};
-                *reinterpret_cast<float4v *>(dst + r4 * 256) = v;
-            }
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    const float4v v = {acc[i][j][4 * r4], acc[i][j][4 * r4 + 1], acc[i][j][4 * r4 + 2], acc[i][j][4 * r4 + 3]};
+                    *reinterpret_cast<float4v *>(dst + i * 1024 + r4 * 256) = v;
+                }
         }
     });
     // the partials must have reached L2 before the flag can be seen
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const unsigned my_xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u;      // HW_REG_XCC_ID, bits 3:0
-    unsigned *myflag = p.sk_flags + ((long)sk_tile * S + sk_s) * 8 + wave;
+    unsigned *myflag = p.sk_flags + ((long)sk_tile * 2 + sk_s) * 8 + wave;
+    unsigned *theirs = p.sk_flags + ((long)sk_tile * 2 + (1 - sk_s)) * 8 + wave;
     if (lane == 0) SkExchange::publish(myflag, p.sk_epoch ^ p.sk_pub_xor, my_xcc);
-    // the sub-tiles this wave keeps (slot 0, and slot 1 when it keeps two)
-    float16v own[2];
-    static_for<NQ>([&](auto Q) {
-        constexpr int q = decltype(Q)::value, i = q / TM, j = q % TM;
-        if (q % S == sk_s) {                               // uniform
-            if (q / S == 0) own[0] = acc[i][j]; else own[1] = acc[i][j];
-        }
-    });
-    // Wait (bounded) for the same wave of every partner, then fetch everything they sent in one trip: at most three
-    // blocks of sixteen registers (three partners' one sub-tile, or one partner's one or two).  The three polls of a
-    // round are in flight together: a poll is a trip past the L1.  Co-residency of the partners is NOT guaranteed
-    // (another stream's kernel can hold an XCD's CUs): the bound is the guard, and a wave that runs into it says so.
-    unsigned *fl[3];
-#pragma unroll
-    for (int bi = 0; bi < 3; bi++) {
-        const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;      // S = 4: the bi-th partner in slice order
-        fl[bi] = p.sk_flags + ((long)sk_tile * S + src) * 8 + wave;
-    }
-    const unsigned *const cfl[3] = {fl[0], fl[1], fl[2]};
-    const sk::WaitResult wr = SkExchange::wait(cfl, S == 4 ? 3 : 1, p.sk_epoch, my_xcc ^ p.sk_xcc_xor, p.sk_spin);
+    // Co-residency of the partner is NOT guaranteed (another stream's kernel can hold an XCD's CUs): the bound is the
+    // guard, and a wave that runs into it says so.
+    const unsigned *const cfl[3] = {theirs, theirs, theirs};
+    const sk::WaitResult wr = SkExchange::wait(cfl, 1, p.sk_epoch, my_xcc ^ p.sk_xcc_xor, p.sk_spin);
     asm volatile("" ::: "memory");
     if (wr != sk::ARRIVED) {
         // Loud failure: the sticky status word, NaN over this wave's share of Y, flags left as they are (the host
@@ -1047,338 +1016,26 @@ __device__ __forceinline__ void sk_finish(const GemmArgs &p, float16v (&acc)[TN]
         if (lane == 0) __hip_atomic_fetch_or(p.status, wr == sk::TIMED_OUT ? (unsigned)MI_DEVSTAT_EXCHANGE_TIMEOUT : (unsigned)MI_DEVSTAT_EXCHANGE_XCD,
                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         // (the exchange runs unbatched launches only: bz = 0)
-        if (NSL == 1) sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * (sk_s % TM), n0 + wn * WTN + 32 * (sk_s / TM), 32, lane);
-        else sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * sk_s, n0 + wn * WTN, WTN, lane);
+        sk_poison_region(p.Y, p.ldY, p.M, p.N, p.out_f32, m0 + wm * WTM + 32 * sk_s, n0 + wn * WTN, WTN, lane);
         return;
     }
     // Ordinary loads: this CU has not touched these lines since the kernel began (its L1 was invalidated then), so
-    // they come from the L2 the partners' acknowledged stores are in (the wait has checked that it is this XCD's).
-    float4v blk[3][4];
+    // they come from the L2 the partner's acknowledged stores are in (the wait has checked that it is this XCD's).
+    const float *from = part_of(sk_s, 1 - sk_s);
+    float4v blk[2][4];
 #pragma unroll
-    for (int bi = 0; bi < 3; bi++) {
-        const int src = S == 4 ? bi + (bi >= sk_s ? 1 : 0) : 1 - sk_s;
-        if (S == 4 || bi < NSL) {
-            const float *from = part_of(sk_s, src) + (S == 4 ? 0 : bi * 1024);
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) blk[bi][r4] = *reinterpret_cast<const float4v *>(from + r4 * 256);
-        }
-    }
-    float16v tot[2];                                       // summed in slice order, whoever does the summing
-    if (S == 4) {
+        for (int r4 = 0; r4 < 4; r4++) blk[i][r4] = *reinterpret_cast<const float4v *>(from + i * 1024 + r4 * 256);
+    float16v two[2][1];                                        // summed in slice order, whoever does the summing
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const float x0 = blk[0][r >> 2][r & 3], x1 = blk[1][r >> 2][r & 3], x2 = blk[2][r >> 2][r & 3], o = own[0][r];
-            tot[0][r] = sk_s == 0 ? ((o + x0) + x1) + x2 : sk_s == 1 ? ((x0 + o) + x1) + x2 : sk_s == 2 ? ((x0 + x1) + o) + x2 : ((x0 + x1) + x2) + o;
-        }
-    } else {
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            tot[0][r] = sk_s == 0 ? own[0][r] + blk[0][r >> 2][r & 3] : blk[0][r >> 2][r & 3] + own[0][r];
-            if (NQ == 4) tot[1][r] = sk_s == 0 ? own[1][r] + blk[1][r >> 2][r & 3] : blk[1][r >> 2][r & 3] + own[1][r];
-        }
-    }
-    // What the partners sent has arrived (the sums above used it).  The last wave to have consumed a partner's
-    // partials clears that partner's flag -- with two slices that is this wave, with four the third to count itself
-    // in -- so the next launch on this bank, which for a replayed graph carries this same epoch, starts from zero.
-    if (lane == 0) {
-#pragma unroll
-        for (int bi = 0; bi < 3; bi++)
-            if (S == 4 || bi == 0) SkExchange::release(fl[bi], fl[bi] + SK_WORDS, S == 4 ? 3 : 1);
-    }
-    // One kept sub-tile (S = NQ): q = s.  Two (S = 2 of four): q = s and s + 2, the 32-row half j = s at both
-    // 32-column halves.
-    if (NSL == 1) {
-        const int i = sk_s / TM, j = sk_s % TM;
-        float16v one[1][1] = {{tot[0]}};
-        half4v cb1[1][4];
-        // a 32-column store: the wave's column origin goes into n0 (the staging rows are as wide as the stored tile)
-        const int nw = n0 + wn * WTN + 32 * i;
-        load_col_bias<1, 32>(p, cb1, nw, 0, lane, bz);
-        store_tile<1, 1, WTM, 32, NWAVES, LDS_BYTES>(p, one, cb1, smem, m0 + 32 * j, nw, wm, 0, wave, lane, bz);
-    } else if constexpr (TN == 2) {
-        float16v two[2][1] = {{tot[0]}, {tot[1]}};
-        store_tile<1, 2, WTM, WTN, NWAVES, LDS_BYTES>(p, two, cb, smem, m0 + 32 * sk_s, n0, wm, wn, wave, lane, bz);
-    }
-    return;
-}
-
-// With three 64-deep stages a ninth wave does nothing but request operand tiles (pp_loader).  A 1 KB
-// global_load_lds_dwordx4 takes the CU's vector-memory path sixteen clocks, so a wave that issues its share of a tile
-// stands at those instructions while its three partners' requests drain ahead of it -- 190 of the 750 clocks of a
-// memory phase, measured, against 530 clocks of the matrix phase, and moving the requests between a wave's own MFMAs
-// only moved the cost (716 clocks of matrix phase).  The loader wave issues all 48 requests of a tile, half in each
-// phase, waits for the tile the next phase will read, and joins every workgroup barrier; the eight matrix waves issue
-// no vector-memory instruction inside the loop.  Three waves then share one SIMD, which leaves 168 registers a wave:
-// the 256 x 256 tile (217) keeps the scheme in which every wave requests its own share.
-template <int BK, int STAGES, bool PINGPONG>
-constexpr bool pp_loader() { return PINGPONG && BK == 64 && STAGES == 3; }
-template <int BK, int STAGES, bool PINGPONG>
-constexpr int pp_threads() { return pp_loader<BK, STAGES, PINGPONG>() ? 576 : 512; }
-
-template <int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool B_KN, bool PINGPONG, bool SK = false>
-__global__ __launch_bounds__((pp_threads<BK, STAGES, PINGPONG>())) void gemm_pp_kernel(GemmArgs p) {
-    static_assert(WAVES_M * WAVES_N == 8, "two groups of four waves");
-    constexpr bool LOADER = pp_loader<BK, STAGES, PINGPONG>();
-    static_assert(BK == 64 || BK == 32, "rows of 128 or 64 bytes");
-    constexpr int NT = 512, KS = BK / 16, CPR = BK / 8, ROWB = BK * 2;
-    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
-    constexpr int PA = BM * CPR / NT, PB = BN * CPR / NT;          // 1 KB load instructions per wave and tile
-    constexpr int NL = PA + PB;
-    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE_BYTES = A_BYTES + B_BYTES;
-    static_assert(BM % 64 == 0 && BN % 64 == 0 && PA >= 1 && PB >= 1 && STAGES >= 3 && STAGES <= 4, "tile shape");
-    static_assert(!B_KN || BN >= 128, "the [K][N] permutation moves a chunk by up to 12 places inside its row");
-    static_assert((STAGES - 2) * NL <= 63, "vmcnt is a 6-bit counter");
-    extern __shared__ __align__(16) char smem[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int grp = PINGPONG ? wave >> 2 : 0;
-    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-    int tm_, tn_, sk_s = 0, sk_tile = 0;
-    if constexpr (SK) {
-        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-        sk_s = idx % p.sk_S;
-        sk_tile = xcd * p.sk_tpx + idx / p.sk_S;
-        if (sk_tile >= p.tiles_m * p.tiles_n) return;          // the whole workgroup: the last XCD's run may be short
-        // an XCD's run of the tile order covers about as many row tiles as column tiles (group_m rows per column
-        // step), so its L2 pulls few panels of either operand: 1500 x 5120 -> 1280 fetched 156 MB with runs that
-        // walked whole columns of 12 row tiles
-        const int width = p.group_m * p.tiles_n, g = sk_tile / width, in = sk_tile - g * width;
-        const int first = g * p.group_m, gsz = min(p.tiles_m - first, p.group_m);
-        tm_ = first + in % gsz;
-        tn_ = in / gsz;
-    } else {
-        tile_of(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, p.group_m, tm_, tn_);
-    }
-    const int m0 = tm_ * BM, n0 = tn_ * BN;
-    const long bz = blockIdx.y;
-    const int nk = SK ? p.K / BK / p.sk_S : p.K / BK;      // the launcher guarantees whole BK-deep tiles per slice
-    // tile origins; the per-lane part of every load address is a 32-bit byte offset from these
-    const long a_step = BK * 2, b_step = B_KN ? (long)BK * p.ldB * 2 : BK * 2;       // bytes per BK-deep tile
-    const half_t *Ag = p.A + bz * p.sA + (long)m0 * p.ldA + (SK ? (long)sk_s * nk * (a_step / 2) : 0L);
-    const half_t *Bg = p.B + bz * p.sB + (B_KN ? (long)n0 : (long)n0 * p.ldB) + (SK ? (long)sk_s * nk * (b_step / 2) : 0L);
-
-    // K-contiguous rows: LDS position pos of row r holds chunk pos ^ rowswz(r)
-    auto rowswz = [](int r) { return BK == 64 ? (r & 7) ^ ((r >> 3) & 1) : (r >> 2) & 3; };
-    // per-lane byte offsets of the 1 KB slots that wave w of eight requests: slot i of the A part, slot i of the B part
-    auto a_offset = [&](int w, int i) {
-        const int q = (i * 8 + w) * 64 + lane, r = q / CPR, pos = q % CPR;
-        const int c = pos ^ rowswz(r);
-        return (uint32_t)(((long)(min(m0 + r, p.M - 1) - m0) * p.ldA + c * 8) * 2);
-    };
-    auto b_offset = [&](int w, int i) {
-        const int q = (i * 8 + w) * 64 + lane;
-        if (!B_KN) {
-            const int r = q / CPR, pos = q % CPR;
-            const int c = pos ^ rowswz(r);
-            return (uint32_t)(((long)(min(n0 + r, p.N - 1) - n0) * p.ldB + c * 8) * 2);
-        } else {
-            constexpr int CPRB = BN / 8;
-            const int k = q / CPRB, pos = q % CPRB;
-            const int j = pos ^ ((k & 3) << 2);
-            return (uint32_t)(((long)k * p.ldB + (min(n0 + j * 8, p.NB - 8) - n0)) * 2);
-        }
-    };
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)smem;
-    auto barrier = [&]() {
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-    };
-    if constexpr (LOADER) {
-        if (wave == 8) {
-            // The loader wave.  Barrier b closes phase b - 1 (barrier 0 closes the prologue); tile t lives in stage
-            // t % 3, is read in phases 2t (leading group) and 2t + 1 (trailing group), and its stage is free from
-            // phase 2t + 2: tile kt + 2 is requested in phases 2kt and 2kt + 1, a half of its 48 slots in each, and
-            // has to have landed when phase 2kt + 3 ends.  Requests complete in order, so "tile t has landed" is
-            // "no more requests outstanding than were issued after it".
-            constexpr int PER_TILE = 8 * NL;
-            static_assert(PER_TILE <= 63, "vmcnt is a 6-bit counter");
-            uint32_t offa[8][PA], offb[8][PB];
-#pragma unroll
-            for (int w = 0; w < 8; w++) {
-#pragma unroll
-                for (int i = 0; i < PA; i++) offa[w][i] = a_offset(w, i);
-#pragma unroll
-                for (int i = 0; i < PB; i++) offb[w][i] = b_offset(w, i);
-            }
-            auto request = [&](int kt, int stage, int half) {      // half 0 / 1: the slots of waves 0-3 / 4-7; 2: all
-                const char *ab = reinterpret_cast<const char *>(Ag) + (long)kt * a_step;
-                const char *bb = reinterpret_cast<const char *>(Bg) + (long)kt * b_step;
-#pragma unroll
-                for (int w = 0; w < 8; w++) {
-                    if (half != 2 && (w >> 2) != half) continue;
-                    const uint32_t sa = lds0 + stage * STAGE_BYTES + w * 1024, sb = sa + A_BYTES;
-#pragma unroll
-                    for (int i = 0; i < PA; i++) {
-                        const uint32_t dst = __builtin_amdgcn_readfirstlane(sa + i * 8192);
-                        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offa[w][i]), "s"(ab), "s"(dst) : "memory");
-                    }
-#pragma unroll
-                    for (int i = 0; i < PB; i++) {
-                        const uint32_t dst = __builtin_amdgcn_readfirstlane(sb + i * 8192);
-                        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offb[w][i]), "s"(bb), "s"(dst) : "memory");
-                    }
-                }
-            };
-            request(0, 0, 2);
-            if (nk > 1) { request(1, 1, 2); asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory"); }
-            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            barrier();
-            for (int ph = 0; ph < 2 * nk; ph++) {
-                const int kt = ph >> 1, half = ph & 1, t = kt + 2;
-                if (t < nk) {
-                    const int stage = t % 3;
-                    if (half == 0) request(t, stage, 0); else request(t, stage, 1);
-                }
-                if (half == 1) {      // the next phase reads tile kt + 1
-                    if (t < nk) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_TILE) : "memory");
-                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                }
-                barrier();
-            }
-            return;
-        }
-    }
-    // folded layer norm: (r, r mu) of the tile's rows, by the first BM / 64 matrix waves (they have nothing else to do
-    // until the first tile lands), parked in LDS behind the stages and the store's staging until the store; the barrier
-    // that closes the prologue covers it
-    constexpr int LN_SLOT_OFF = STAGES * STAGE_BYTES > 8 * 32 * (BN / 4 + 4) * 4 ? STAGES * STAGE_BYTES : 8 * 32 * (BN / 4 + 4) * 4;
-    float2v *ln_slot = reinterpret_cast<float2v *>(smem + LN_SLOT_OFF);
-    lnf_stage<BM, BN, 512>(p, ln_slot, m0, n0, bz, tid);
-    uint32_t aoffg[PA], boffg[PB];
-    if constexpr (!LOADER) {
-#pragma unroll
-        for (int i = 0; i < PA; i++) aoffg[i] = a_offset(wave, i);
-#pragma unroll
-        for (int i = 0; i < PB; i++) boffg[i] = b_offset(wave, i);
-    }
-    // the wave's 1 KB slots inside a stage
-    auto issue = [&](int kt, int stage) {
-        if constexpr (!LOADER) {
-            const char *ab = reinterpret_cast<const char *>(Ag) + (long)kt * a_step;
-            const char *bb = reinterpret_cast<const char *>(Bg) + (long)kt * b_step;
-            const uint32_t sa = lds0 + stage * STAGE_BYTES + wave * 1024, sb = sa + A_BYTES;
-#pragma unroll
-            for (int i = 0; i < PA; i++) {
-                const uint32_t dst = __builtin_amdgcn_readfirstlane(sa + i * 8192);
-                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(aoffg[i]), "s"(ab), "s"(dst) : "memory");
-            }
-#pragma unroll
-            for (int i = 0; i < PB; i++) {
-                const uint32_t dst = __builtin_amdgcn_readfirstlane(sb + i * 8192);
-                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(boffg[i]), "s"(bb), "s"(dst) : "memory");
-            }
-        }
-    };
-
-    // fragment read offsets inside a stage (bytes)
-    const int frow = lane & 31, fhi = lane >> 5;
-    const int swz = rowswz(lane & 15);
-    int a_rd[KS], b_rd[KS], bt_rd[TN];
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-        const int cc = ((2 * ks + fhi) ^ swz) << 4;
-        a_rd[ks] = (wm * WTM + frow) * ROWB + cc;
-        b_rd[ks] = A_BYTES + (wn * WTN + frow) * ROWB + cc;
-    }
-    {
-        const int kk = (lane >> 2) & 3;
-#pragma unroll
-        for (int i = 0; i < TN; i++) {
-            const int col = (wn * WTN + i * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4) ^ (kk << 5);
-            bt_rd[i] = A_BYTES + ((fhi * 8 + kk) * BN + col) * 2;
-        }
-    }
-    half8v fa[KS][TM], fb[KS][TN];
-    auto fread = [&](int stage) {
-        const char *st = smem + stage * STAGE_BYTES;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-#pragma unroll
-            for (int j = 0; j < TM; j++) fa[ks][j] = *reinterpret_cast<const half8v *>(st + a_rd[ks] + j * 32 * ROWB);
-            if (!B_KN) {
-#pragma unroll
-                for (int i = 0; i < TN; i++) fb[ks][i] = *reinterpret_cast<const half8v *>(st + b_rd[ks] + i * 32 * ROWB);
-            } else {
-#pragma unroll
-                for (int i = 0; i < TN; i++) {
-                    const char *bs = st + bt_rd[i] + ks * 16 * BN * 2;
-                    short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(bs));
-                    short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(bs + 4 * BN * 2));
-                    short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    fb[ks][i] = __builtin_bit_cast(half8v, both);
-                }
-            }
-        }
-    };
-    float16v acc[TN][TM];
-#pragma unroll
-    for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int j = 0; j < TM; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
-    auto mma = [&]() {
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++)
-#pragma unroll
-            for (int i = 0; i < TN; i++)
-#pragma unroll
-                for (int j = 0; j < TM; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks][i], fa[ks][j], acc[i][j], 0, 0, 0);
-    };
-    const bool probe = p.clk && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0;
-    if (probe) { p.clk[0] = clock64(); p.clk[1] = wall_clock64(); }
-    // this wave's loads of tile kt + 1 have landed: only the tiles requested after it may still be in flight
-    // (with a loader wave the matrix waves have no requests of their own to wait for: the loader waits for the tile
-    // ahead of the barrier that everybody passes)
-    auto wait_next = [&](int kt) {
-        if constexpr (!LOADER) {
-            const int newer = min(kt + STAGES - 1, nk - 1) - (kt + 1);
-            if (newer >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NL) : "memory");
-            else if (newer == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
-            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        }
-    };
-
-#pragma unroll
-    for (int t = 0; t < STAGES - 1; t++)
-        if (t < nk) issue(t, t);
-    wait_next(-1);                // tile 0
-    barrier();
-    if (grp == 1) barrier();
-    half4v cb[TN][4];
-    int stage = 0;
-    for (int kt = 0; kt < nk; kt++) {
-        // memory phase
-        fread(stage);
-        if (kt + STAGES - 1 < nk) issue(kt + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
-        if (kt + 1 == nk) load_col_bias<TN, WTN>(p, cb, n0, wn, lane, bz);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (grp == 1) wait_next(kt);
-        barrier();
-        // matrix phase
-        __builtin_amdgcn_s_setprio(1);
-        mma();
-        __builtin_amdgcn_s_setprio(0);
-        if (grp == 0) wait_next(kt);
-        // the trailing group's last matrix phase closes with no barrier (the leading group is already storing its
-        // tile): with the extra one it took at the start, both groups have then executed 2 nk + 1
-        if (!(PINGPONG && grp == 1 && kt + 1 == nk)) barrier();
-        stage = stage == STAGES - 1 ? 0 : stage + 1;
-    }
-    if constexpr (SK) {
-        sk_finish<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, sk_tile, sk_s, m0, n0, wm, wn, wave, lane, bz);
-        if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
-        return;
-    }
-    LnFold<TM> ln;
-    if (p.lnf_stats) {
-        ln.on = true; ln.col = reinterpret_cast<const float *>(ln_slot + BM); ln.bn = BN;
-#pragma unroll
-        for (int j = 0; j < TM; j++) { const float2v v = ln_slot[wm * WTM + 32 * j + (lane & 31)]; ln.r[j] = v[0]; ln.rmu[j] = v[1]; }
-    }
-    store_tile<TM, TN, WTM, WTN, 8, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln);
-    if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
+        for (int r = 0; r < 16; r++) two[i][0][r] = sk_s == 0 ? own[i][r] + blk[i][r >> 2][r & 3] : blk[i][r >> 2][r & 3] + own[i][r];
+    // What the partner sent has arrived (the sums above used it): this wave clears the partner's flag, so the next
+    // launch on this bank, which for a replayed graph carries this same epoch, starts from zero.
+    if (lane == 0) SkExchange::release(theirs, theirs + SK_WORDS, 1);
+    store_tile<1, 2, WTM, WTN, NWAVES, LDS_BYTES>(p, two, cb, smem, m0 + 32 * sk_s, n0, wm, wn, wave, lane, bz);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1439,8 +1096,10 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     int tm_, tn_, sk_s = 0, sk_tile = 0;
     if constexpr (SK) {
-        // K-slice s of tile xcd * tpx + slot is workgroup (slot * S + s) * 8 + xcd: a tile's slices share an XCD (the
-        // ping-pong kernel's split-K instances say more); an XCD's run of the tile order is about square
+        // K-slice s of tile xcd * tpx + slot is workgroup (slot * S + s) * 8 + xcd: a tile's slices share an XCD
+        // (sk_finish says more).  An XCD's run of the tile order covers about as many row tiles as column tiles, so
+        // its L2 pulls few panels of either operand: 1500 x 5120 -> 1280 fetched 156 MB with runs that walked whole
+        // columns of 12 row tiles
         const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
         sk_s = idx % p.sk_S;
         sk_tile = xcd * p.sk_tpx + idx / p.sk_S;
@@ -2368,11 +2027,10 @@ int raise_lds(KernelT kern, int bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? 0 : 1;
 }
 
-template <int BM, int BN, int BK, int STAGES>
-constexpr int pp_lds_bytes() {
-    constexpr int stages = STAGES * (BM + BN) * BK * 2, epi = 8 * 32 * (BN / 4 + 4) * 4;      // operand ring; epilogue staging of 8 waves
-    return (stages > epi ? stages : epi) + BM * 8 + BN * 8;      // + a folded layer norm's (r, r mu) per row, colsum and biasp per column
-}
+// LDS of the four-wave kernel: three 64-deep stages of both operands (the store's staging reuses them), then a folded
+// layer norm's (r, r mu) per row and colsum and biasp per column
+template <int BM, int BN>
+constexpr int w4_lds_bytes() { return 3 * (BM + BN) * 64 * 2 + BM * 8 + BN * 8; }
 
 template <int BM, int BN, int BK>
 constexpr int gemm_lds_bytes() {
@@ -2449,25 +2107,6 @@ int launch_pipe_ln(GemmArgs a, bool b_kn, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
-template <int BM, int BN, int BK, int STAGES, int WM, int WN, bool PP>
-int launch_pp(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
-    if (a.K < BK || a.K % BK || a.cv.xp || a.ag.x) return MI_DECLINE_EXTENT;
-    a.tiles_m = (int)ceil_div(a.M, BM);
-    a.tiles_n = (int)ceil_div(a.N, BN);
-    a.group_m = a.tiles_m < 6 ? a.tiles_m : 6;
-    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
-                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
-    // per-lane load offsets are 32-bit byte offsets from the tile origin
-    if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? BK : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;
-    a.clk = g_clock_probe;
-    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
-    constexpr int lds = pp_lds_bytes<BM, BN, BK, STAGES>();
-    constexpr int threads = pp_threads<BK, STAGES, PP>();
-    if (b_kn) hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, BK, STAGES, WM, WN, true, PP>), grid, dim3(threads), lds, st, a);
-    else      hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, BK, STAGES, WM, WN, false, PP>), grid, dim3(threads), lds, st, a);
-    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
-}
-
 template <int BM, int BN, int WM, int WN>
 int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     if (a.K < 64 || a.K % 64 || a.cv.xp || a.ag.x) return MI_DECLINE_EXTENT;
@@ -2480,7 +2119,7 @@ int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? 64 : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;
     a.clk = g_clock_probe;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
-    constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
+    constexpr int lds = w4_lds_bytes<BM, BN>();
     // four matrix waves and the loader, plus the statistics wave of a folded layer norm
     const dim3 block(a.lnf_stats ? 384 : 320);
     if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, WM, WN, true>), grid, block, lds, st, a);
@@ -2489,37 +2128,6 @@ int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
 }
 
 bool sk_fits(int64_t M, int64_t N, int64_t K, int bm, int bn, int split);
-
-// The ping-pong kernel with `split` workgroups per tile exchanging their partial tiles (see the kernel).
-template <int BM, int BN>
-int launch_pp_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
-    if (a.cv.xp || a.ag.x || !sk_usable() || !sk_fits(a.M, a.N, a.K, BM, BN, split)) return MI_DECLINE_EXTENT;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return MI_ERROR_DEVICE;
-    a.tiles_m = (int)ceil_div(a.M, BM);
-    a.tiles_n = (int)ceil_div(a.N, BN);
-    a.group_m = 1;
-    while (a.group_m * a.group_m < (int)ceil_div((int64_t)a.tiles_m * a.tiles_n, 8) && a.group_m < a.tiles_m) a.group_m++;
-    a.vec_store = a.out_f32 ? (a.ldY % 4 == 0 && a.sY % 4 == 0 && aligned_to(a.Y, 16))
-                            : (a.ldY % 8 == 0 && a.sY % 8 == 0 && aligned_to(a.Y, 16) && (!a.residual || aligned_to(a.residual, 16)));
-    if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? 64 : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;
-    const int tiles = a.tiles_m * a.tiles_n;
-    a.sk_S = split;
-    a.sk_tpx = (int)ceil_div(tiles, 8);
-    a.sk_part = reinterpret_cast<float *>(ws);
-    const unsigned launch = ++g_sk_epoch;
-    a.sk_epoch = sk::epoch_of(launch);
-    a.sk_flags = g_sk_flags_ptr[dev] + (size_t)(launch % SK_BANKS) * SK_FLAGS;
-    a.sk_spin = g_sk_spin; a.sk_pub_xor = g_sk_pub_xor; a.sk_xcc_xor = g_sk_xcc_xor;
-    a.status = g_status_ptr[dev];
-    a.clk = g_clock_probe;
-    dim3 grid((unsigned)(8 * a.sk_tpx * split), 1);
-    constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
-    constexpr int threads = pp_threads<64, 3, true>();
-    if (b_kn) hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, 64, 3, 2, 4, true, true, true>), grid, dim3(threads), lds, st, a);
-    else      hipLaunchKernelGGL((gemm_pp_kernel<BM, BN, 64, 3, 2, 4, false, true, true>), grid, dim3(threads), lds, st, a);
-    return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
-}
 
 // The four-wave kernel with two workgroups per 128 x 128 tile exchanging their partial tiles.
 int launch_w4_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
@@ -2545,14 +2153,14 @@ int launch_w4_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
     a.status = g_status_ptr[dev];
     a.clk = g_clock_probe;
     dim3 grid((unsigned)(8 * a.sk_tpx * split), 1);
-    constexpr int lds = pp_lds_bytes<BM, BN, 64, 3>();
+    constexpr int lds = w4_lds_bytes<BM, BN>();
     if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, 2, 2, true, true>), grid, dim3(320), lds, st, a);
     else      hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, 2, 2, false, true>), grid, dim3(320), lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
-// tile: index into TILE_MODELS.  The ping-pong kernels take ordinary operands only; a gathered operand (implicit-GEMM
-// convolution) planned onto one of their tiles runs the pipelined kernel's 128 x 256 tile instead: same K order per
+// tile: index into TILE_MODELS.  The four-wave kernel takes ordinary operands only; a gathered operand (implicit-GEMM
+// convolution) planned onto one of its tiles runs the pipelined kernel's same tile instead: same K order per
 // output, same bits, and the plan (hence the workspace) stays a function of the extents alone.
 int launch_tile(int tile, const GemmArgs &a, bool b_kn, int64_t nbatch, hipStream_t st) {
     const bool plain = !a.cv.xp && !a.ag.x;
@@ -2561,7 +2169,6 @@ int launch_tile(int tile, const GemmArgs &a, bool b_kn, int64_t nbatch, hipStrea
         case 1: return plain ? launch_w4<192, 128, 2, 2>(a, b_kn, nbatch, st) : launch_pipe<192, 128, 2, 4>(a, b_kn, nbatch, st);
         case 2: return launch_pipe<128, 128, 2, 4>(a, b_kn, nbatch, st);
         case 3: return launch_pipe<64, 128, 2, 4>(a, b_kn, nbatch, st);
-        case 5: return plain ? launch_pp<256, 256, 32, 4, 2, 4, true>(a, b_kn, nbatch, st) : launch_pipe<128, 256, 2, 4>(a, b_kn, nbatch, st);
         default: return launch_pipe<64, 64, 2, 2>(a, b_kn, nbatch, st);
     }
 }
@@ -2588,7 +2195,7 @@ int launch_mfma(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
 // the second launch (about 4 us) and the fp32 planes (0.25 us per MB).  Picking the cheapest estimate lands within
 // 1 % of the best measured choice on average over those shapes and within 6 % on 95 % of them.
 struct TileModel { int bm, bn; double step_lo, step_full, round, fixed; };
-constexpr int NTILES = 6;
+constexpr int NTILES = 5;
 constexpr TileModel TILE_MODELS[NTILES] = {
     // (the two tiles of the four-wave kernel, re-timed with it: 1500 x 5120 in 25.3 / 70.5 us at K = 1280 / 5120,
     // 512 x 1280 in 16.3 / 47.2; 1500 x 3840 on 192 x 128 in 20.2 / 55.4, 512 x 1280 in 13.5 / 39.9)
@@ -2597,9 +2204,6 @@ constexpr TileModel TILE_MODELS[NTILES] = {
     {128, 128, 0.428, 0.600, 1.00, 4.0},
     {64, 128, 0.318, 0.430, 0.90, 3.1},
     {64, 64, 0.235, 0.315, 0.73, 3.0},
-    // 256 x 256 (ping-pong kernel, 32-deep stages): 4096^3 in 120-123 us on one round of 256 workgroups, 8192^3 in
-    // 884-938 us on four; the lightly loaded step is scaled from the 128 x 256 tile's ratio
-    {256, 256, 1.200, 1.770, 1.00, 9.0},
 };
 struct TilePlan { int tile, split; bool peer; };      // peer: the K-slices exchange partial tiles in the kernel (no planes)
 
@@ -2615,24 +2219,19 @@ double tile_cost_us(int64_t M, int64_t N, int64_t K, int64_t nbatch, int tile, i
     return us;
 }
 
-// Split-K with the partials exchanged inside the launch (ping-pong kernel; 128 x 256 tiles in 2 or 4 K-slices, or
-// 128 x 128 tiles in 2; every workgroup resident at once): the tile's own estimate at that many workgroups, no planes
-// and no second launch, plus the exchange.  A workgroup writes and reads (S - 1) / S of its accumulators; what that
-// costs is set by how fast the burst drains -- 23 MB from 240 workgroups of 128 x 256 in four slices take 5 to 10 us
-// end to end (stores acknowledged after 1 to 10 us, every wave waiting for its slowest partner), 7.7 MB from 120 or 240
-// workgroups in two slices 2 to 3 us.
-constexpr int SK_TILES[2] = {0, 2};      // indices into TILE_MODELS: 128 x 256, 128 x 128
-double sk_exchange_us(int64_t wg, int bm, int bn, int split) {
-    const double mb = (double)wg * bm * bn * 4.0 * (split - 1) / split / 1e6;
-    // fitted: two slices, 29.8 us measured on 1500 x 5120 -> 1280 (128 x 128) and 39.7 on 1024 x 5120 -> 2560 (128 x 256);
-    // four slices (three partners to wait for), 40.8 on 1500 x 5120 -> 1280 and 31.0 on 512 x 5120 -> 1280 (128 x 256)
-    return split == 2 ? 2.0 + 0.3 * mb : 8.0 + 0.5 * mb;
+// Split-K with the partials exchanged inside the launch (four-wave kernel, 128 x 128 tiles in two K-slices, every
+// workgroup resident at once): the tile's own estimate at that many workgroups, no planes and no second launch, plus
+// the exchange.  A workgroup writes and reads half of its accumulators; what that costs is set by how fast the burst
+// drains -- 7.7 MB from 120 or 240 workgroups take 2 to 3 us end to end.
+constexpr int SK_TILE = 2;               // index into TILE_MODELS: 128 x 128
+double sk_exchange_us(int64_t wg, int bm, int bn) {
+    const double mb = (double)wg * bm * bn * 4.0 * 0.5 / 1e6;
+    return 2.0 + 0.3 * mb;               // fitted: 29.8 us measured on 1500 x 5120 -> 1280, 22.1 on 512 x 5120 -> 1280
 }
 size_t sk_workspace_bytes(int64_t M, int64_t N, int bm, int bn, int split) { return (size_t)(ceil_div(M, bm) * ceil_div(N, bn)) * split * bm * bn * 4; }
 bool sk_fits(int64_t M, int64_t N, int64_t K, int bm, int bn, int split) {
     const int64_t tiles = ceil_div(M, bm) * ceil_div(N, bn), tpx = ceil_div(tiles, 8);
-    return (split == 2 || (split == 4 && bn == 256)) && K % (64 * split) == 0 && K / split >= 128 && 8 * tpx * split <= mi_num_cus() &&
-           8 * tpx * split * 8 <= SK_FLAGS;
+    return split == 2 && bm == 128 && bn == 128 && K % 128 == 0 && K / 2 >= 128 && 8 * tpx * 2 <= mi_num_cus() && 8 * tpx * 2 * 8 <= SK_FLAGS;
 }
 // Before mi_init (planner queries without a device) the path is assumed: a workspace sized for it also holds the planes
 // the same split falls back to.
@@ -2648,7 +2247,7 @@ double sk_cost_us(int64_t M, int64_t N, int64_t K, int tile, int split) {
     const double load = (double)wg / (double)mi_num_cus();
     const double step = t.step_lo + (t.step_full - t.step_lo) * load;
     return 2.0 + (t.fixed - 2.0) * (0.4 + 0.6 / (double)split) + (t.fixed - 2.0) * 0.4 * load + (double)(K / (64 * split)) * step +
-           sk_exchange_us(wg, t.bm, t.bn, split);
+           sk_exchange_us(wg, t.bm, t.bn);
 }
 
 // The plan depends on the extents alone, so a GEMM gives the same bits whichever entry point issues it.
@@ -2663,10 +2262,9 @@ TilePlan plan_tiles(int64_t M, int64_t N, int64_t K, int64_t nbatch, bool may_sp
             if (us < best_us) { best_us = us; best = {tile, split, false}; }
         }
         if (max_split > 1 && sk_planned()) {
-            for (int tile : SK_TILES) {
-                if (!sk_fits(M, N, K, TILE_MODELS[tile].bm, TILE_MODELS[tile].bn, split)) continue;
-                const double us = sk_cost_us(M, N, K, tile, split);
-                if (us < best_us) { best_us = us; best = {tile, split, true}; }
+            if (sk_fits(M, N, K, TILE_MODELS[SK_TILE].bm, TILE_MODELS[SK_TILE].bn, split)) {
+                const double us = sk_cost_us(M, N, K, SK_TILE, split);
+                if (us < best_us) { best_us = us; best = {SK_TILE, split, true}; }
             }
         }
     }
@@ -2816,7 +2414,7 @@ int run_gemm(GemmArgs a, bool b_kn, int64_t nbatch, void *ws, size_t ws_bytes, h
         }
         int split = tp.split;
         if (split > 1 && tp.peer && ws && aligned_to(ws, 256) && ws_bytes >= plan_workspace_bytes(tp, a.M, a.N)) {
-            const int rc = tp.tile == 0 ? launch_pp_peer<128, 256>(a, b_kn, split, ws, st) : launch_w4_peer(a, b_kn, split, ws, st);
+            const int rc = launch_w4_peer(a, b_kn, split, ws, st);
             if (rc != MI_DECLINE_EXTENT) return rc;     // declined (a gathered operand, a device that failed the probe): planes
             if (in_store) { tp = plan_tiles(a.M, a.N, a.K, nbatch, false); split = 1; }
         }
@@ -2942,16 +2540,12 @@ int mi_init(void) {
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 0, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 1, 1>, gemm_lds_bytes<128, 128, 64>());
     bad |= raise_lds(gemm_pipe_kernel<128, 128, 2, 4, 2>, gemm_lds_bytes<128, 128, 64>());
-    bad |= raise_lds(gemm_w4_kernel<128, 256, 1, 4, true>, pp_lds_bytes<128, 256, 64, 3>());
-    bad |= raise_lds(gemm_w4_kernel<128, 256, 1, 4, false>, pp_lds_bytes<128, 256, 64, 3>());
-    bad |= raise_lds(gemm_w4_kernel<192, 128, 2, 2, true>, pp_lds_bytes<192, 128, 64, 3>());
-    bad |= raise_lds(gemm_w4_kernel<192, 128, 2, 2, false>, pp_lds_bytes<192, 128, 64, 3>());
-    bad |= raise_lds(gemm_w4_kernel<128, 128, 2, 2, true, true>, pp_lds_bytes<128, 128, 64, 3>());
-    bad |= raise_lds(gemm_w4_kernel<128, 128, 2, 2, false, true>, pp_lds_bytes<128, 128, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, true, true, true>, pp_lds_bytes<128, 256, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<128, 256, 64, 3, 2, 4, false, true, true>, pp_lds_bytes<128, 256, 64, 3>());
-    bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, true, true>, pp_lds_bytes<256, 256, 32, 4>());
-    bad |= raise_lds(gemm_pp_kernel<256, 256, 32, 4, 2, 4, false, true>, pp_lds_bytes<256, 256, 32, 4>());
+    bad |= raise_lds(gemm_w4_kernel<128, 256, 1, 4, true>, w4_lds_bytes<128, 256>());
+    bad |= raise_lds(gemm_w4_kernel<128, 256, 1, 4, false>, w4_lds_bytes<128, 256>());
+    bad |= raise_lds(gemm_w4_kernel<192, 128, 2, 2, true>, w4_lds_bytes<192, 128>());
+    bad |= raise_lds(gemm_w4_kernel<192, 128, 2, 2, false>, w4_lds_bytes<192, 128>());
+    bad |= raise_lds(gemm_w4_kernel<128, 128, 2, 2, true, true>, w4_lds_bytes<128, 128>());
+    bad |= raise_lds(gemm_w4_kernel<128, 128, 2, 2, false, true>, w4_lds_bytes<128, 128>());
     bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 1, 2>, lna_lds_bytes<128, 2, 4>(LNA_KMAX));
     bad |= raise_lds(gemm_pipe_kernel<64, 128, 2, 4, 0, 2>, lna_lds_bytes<128, 2, 4>(LNA_KMAX));
     bad |= raise_lds(gemm_pipe_kernel<64, 64, 2, 2, 1, 2>, lna_lds_bytes<64, 2, 2>(LNA_KMAX));

@@ -1,4 +1,4 @@
-// Arrival-flag protocol of the in-launch split-K exchange (gemm_pp_kernel, SK instances), written once for the
+// Arrival-flag protocol of the in-launch split-K exchange (gemm_w4_kernel, SK instance), written once for the
 // device and for a host model: the kernel instantiates it over agent-scope HIP atomics, the CPU test of the protocol
 // (tests/sk_exchange_host_test.cpp) over the compiler's __atomic builtins with one thread per wave.  No HIP header is
 // needed to read this file.

@@ -97,7 +97,7 @@ def test_folded_norm_with_everything_around_it(ctx):
 @pytest.mark.parametrize("T,K,F", [(1500, 5120, 1280), (1370, 384, 384), (1370, 1536, 384), (1500, 1280, 1280), (300, 256, 1024), (4096, 512, 256)])
 def test_a_gemm_leaves_the_statistics_of_its_rows(ctx, T, K, F):
     """The producer side, over the tiles and K-split forms the planner picks (the in-launch exchange at 1500 x 5120 ->
-    1280, 64 x 64 and 64 x 128 tiles, the ping-pong tile): Y carries mi_gemm_f16's bits, the statistics are those of the
+    1280, 64 x 64 and 64 x 128 tiles, the four-wave kernel's tiles): Y carries mi_gemm_f16's bits, the statistics are those of the
     final rows -- after the residual -- and a folded norm + linear that consumes them meets the two ops."""
     import torch
     import juliavision_amd as jv
