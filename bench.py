@@ -142,7 +142,52 @@ def parse_args():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (mi_probe_copy) three times, so that a rocprofv3 --pmc run "
                          "of this command holds a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
+    ap.add_argument("--phase-stamps", action="store_true",
+                    help="print where the waves of the four-wave GEMM kernel spend their clocks (mi_set_phase_probe) on config 1 "
+                         "in both weight layouts and on the encoder block's q/k/v, fc1 and fc2 launches, and exit")
     return ap.parse_args()
+
+
+def phase_stamps(lib, L, stream):
+    """Shader clocks per matrix wave, averaged over all waves of ten launches: before the K loop (launch, addresses, the
+    first operand tile's trip from memory), in the K loop (also per 64-deep tile, against the 1024 clocks -- 512 for the
+    split-K instance's 64 x 64 wave tiles -- its MFMAs occupy the SIMD), issuing the store, waiting for it to drain."""
+    import numpy as np
+    import torch
+    blk = EncoderBlock(lib, stream)
+    blk.step()
+    before, fc1, after = blk.calls_on(stream)
+    T, D, FF = blk.T, blk.D, blk.FF
+    p = lambda n: blk.d[n].data_ptr()
+    wfk = blk.d["w1"].t().contiguous()
+
+    def linear(layout, w, ldw):
+        return Call(lib.mi_gemm_f16, p("f"), p("o"), w, p("b1"), None, T, D, FF, FF, D, ldw, layout, L.BIAS_COL, L.EPI["none"], L.F16,
+                    blk._wsp, blk._ws_bytes, stream)
+    cases = [("c1 1500x1280->5120 W[K][F] + bias", linear(L.W_KF, p("w1"), FF), 240, D // 64, 1024),
+             ("c1 1500x1280->5120 W[F][K] + bias", linear(L.W_FK, wfk.data_ptr(), D), 240, D // 64, 1024),
+             ("block q/k/v: LN1 folded, 3 planes, 192x128 tiles", before[1], 80, D // 64, 768),
+             ("block fc1: LN2 folded + GELU, 128x256 tiles", fc1, 240, D // 64, 1024),
+             ("block fc2: + residual, 128x128 tiles in two K-slices", after[0], 240, FF // 128, 512)]
+    out = {}
+    for name, call, wgs, nk, mfma in cases:
+        for _ in range(30):
+            call()
+        buf = torch.zeros((wgs, 4, 4), dtype=torch.int64, device="cuda")
+        if lib.mi_set_phase_probe(buf.data_ptr(), wgs) != 0:
+            raise RuntimeError("mi_set_phase_probe")
+        acc = np.zeros(4)
+        for _ in range(10):
+            buf.zero_()
+            call()
+            torch.cuda.synchronize()
+            a = buf.cpu().numpy().astype(np.float64).reshape(-1, 4)
+            acc += a[a.sum(1) > 0].mean(0)
+        lib.mi_set_phase_probe(None, 0)
+        m = acc / 10
+        out[name] = {"before_loop": round(m[0]), "k_loop": round(m[1]), "k_loop_per_tile": round(m[1] / nk), "mfma_clocks_per_tile": mfma,
+                     "store_issue": round(m[2]), "store_drain": round(m[3]), "total": round(m.sum())}
+    return out
 
 
 # ----------------------------------------------------------------------------- helpers
@@ -1147,6 +1192,9 @@ def main():
             lib.mi_probe_copy(dst.data_ptr(), src.data_ptr(), src.numel(), stream)
         torch.cuda.synchronize()
         del src, dst
+    if args.phase_stamps:
+        print(json.dumps({"phase_stamps": phase_stamps(lib, L, stream)}, indent=1))
+        return
     if args.only is not None:
         print(json.dumps({"only": args.only, "detail": detail_benchmarks(lib, L, stream, args.only)}))
         return

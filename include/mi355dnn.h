@@ -77,6 +77,12 @@ int mi_device_caps(int64_t out[6]);
  * its last store: buf = {clk0, ref0, clk1, ref1}, and (clk1 - clk0) / (ref1 - ref0) x 100 MHz is the shader clock the
  * launch ran at.  The caller keeps the buffer alive while it is registered.  Process-wide, not thread safe. */
 int mi_set_clock_probe(void *dev_u64x4);
+/* A second measurement aid of the same kind.  While a device buffer of workgroups x 4 x 4 uint64 is registered (NULL
+ * clears it), matrix wave w of workgroup g < workgroups of every four-wave GEMM launch stores at buf[(g * 4 + w) * 4 ..]
+ * the shader clocks it spent {from its start to its K loop, in the K loop, issuing its store (for the split-K
+ * instance: exchange and store), waiting for the store to be acknowledged}.  Costs the launch five clock reads a wave
+ * while registered, a scalar branch otherwise.  Process-wide, not thread safe. */
+int mi_set_phase_probe(void *dev_u64, int64_t workgroups);
 
 /* Ceiling probes (measurement aids, no counterpart in the reference).
  * mi_probe_mfma: `workgroups` workgroups of eight waves run `steps` 64-deep steps of the 128 x 256 GEMM tile's

@@ -34,6 +34,7 @@ SIGNATURES = {
     "mi_init": (_int, []),
     "mi_device_caps": (_int, [_i64p]),
     "mi_set_clock_probe": (_int, [_vp]),
+    "mi_set_phase_probe": (_int, [_vp, _i64]),
     "mi_probe_mfma": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "mi_probe_copy": (_int, [_vp, _vp, _sz, _vp]),
     "mi_probe_grid_barrier": (_int, [_vp, _i64, _i64, _int, _vp]),

@@ -56,6 +56,10 @@ struct GemmArgs {
     // Measurement only (mi_set_clock_probe): workgroup 0 of a four-wave launch stores {shader clock, 100 MHz clock}
     // here when it starts and again after its last store.  Null in ordinary use.
     unsigned long long *clk;
+    // Measurement only (mi_set_phase_probe): every matrix wave of the first phase_wgs workgroups of a four-wave launch
+    // stores the shader clocks it spent {before its K loop, in it, issuing its store, waiting for the store to drain}.
+    unsigned long long *phase;
+    int phase_wgs;
     // Split-K with the partial tiles exchanged between the workgroups of a tile instead of written as planes
     // (gemm_w4_kernel, SK instance): sk_S = 2 workgroups per tile, tiles dealt sk_tpx per XCD; partials in sk_part,
     // per-wave arrival flags in sk_flags (they carry sk_epoch; the last reader of a flag clears it).
@@ -1094,6 +1098,7 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    const unsigned long long t_entry = p.phase ? clock64() : 0ull;
     int tm_, tn_, sk_s = 0, sk_tile = 0;
     if constexpr (SK) {
         // K-slice s of tile xcd * tpx + slot is workgroup (slot * S + s) * 8 + xcd: a tile's slices share an XCD
@@ -1305,6 +1310,9 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
     };
     const bool probe = p.clk && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0;
     if (probe) { p.clk[0] = clock64(); p.clk[1] = wall_clock64(); }
+    const bool phases = p.phase && (int)blockIdx.x < p.phase_wgs && blockIdx.y == 0;      // uniform
+    unsigned long long ph_t[4] = {0, 0, 0, t_entry};
+    auto phase_mark = [&](int i) { if (phases) ph_t[i] = clock64(); };
     // Three sets of fragment registers: step s of a tile whose rotation is R sits in set (R + s) % 3, and the reads run
     // two steps ahead of the MFMAs (one step ahead, a wave's reads came back just too late: 6 KB per wave and step at the
     // 32 B/clock a SIMD takes from the LDS is 190 of the 256 clocks its eight MFMAs last, before any queueing).  Four
@@ -1343,6 +1351,7 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
         __builtin_amdgcn_sched_barrier(0);
         (void)kt;
     };
+    phase_mark(0);
     for (int kt = 0;;) {
         tile(std::integral_constant<int, 0>{}, kt);
         if (++kt == nk) break;
@@ -1351,8 +1360,20 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
         tile(std::integral_constant<int, 2>{}, kt);
         if (++kt == nk) break;
     }
+    phase_mark(1);
+    auto phase_store = [&]() {
+        if (!phases) return;
+        const unsigned long long issued = clock64();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const unsigned long long done = clock64();
+        if (lane == 0) {
+            unsigned long long *t = p.phase + ((long)blockIdx.x * 4 + wave) * 4;
+            t[0] = ph_t[0] - ph_t[3]; t[1] = ph_t[1] - ph_t[0]; t[2] = issued - ph_t[1]; t[3] = done - issued;
+        }
+    };
     if constexpr (SK) {
         sk_finish<TM, TN, WTM, WTN, 4, STAGES * STAGE_BYTES>(p, acc, cb, smem, sk_tile, sk_s, m0, n0, wm, wn, wave, lane, bz);
+        phase_store();
         if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
         return;
     }
@@ -1363,6 +1384,7 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
         for (int j = 0; j < TM; j++) { const float2v v = ln_slot[wm * WTM + 32 * j + (lane & 31)]; ln.r[j] = v[0]; ln.rmu[j] = v[1]; }
     }
     store_tile<TM, TN, WTM, WTN, 4, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln);
+    phase_store();
     if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
 }
 
@@ -1963,6 +1985,8 @@ int g_cus = 256;
 thread_local int tl_plan_cus = 0;          // > 0: compute units to plan for
 thread_local bool tl_plan_mfma = true;     // false: the described device has no matrix unit
 unsigned long long *g_clock_probe = nullptr;      // mi_set_clock_probe
+unsigned long long *g_phase_probe = nullptr;      // mi_set_phase_probe
+int g_phase_wgs = 0;
 
 // Scratch of mi_gemm_f16_noalloc: every GPU the library runs on holds its own copy of this array, at its own
 // address, until the process ends.  Host code never uses the name as a pointer; g_scratch_ptr[device] is the
@@ -2118,6 +2142,7 @@ int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     // per-lane load offsets are 32-bit byte offsets from the tile origin
     if ((int64_t)BM * a.ldA * 2 >= (1ll << 31) || (int64_t)(b_kn ? 64 : BN) * a.ldB * 2 >= (1ll << 31)) return MI_DECLINE_EXTENT;
     a.clk = g_clock_probe;
+    a.phase = g_phase_probe; a.phase_wgs = g_phase_wgs;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
     constexpr int lds = w4_lds_bytes<BM, BN>();
     // four matrix waves and the loader, plus the statistics wave of a folded layer norm
@@ -2152,6 +2177,7 @@ int launch_w4_peer(GemmArgs a, bool b_kn, int split, void *ws, hipStream_t st) {
     a.sk_spin = g_sk_spin; a.sk_pub_xor = g_sk_pub_xor; a.sk_xcc_xor = g_sk_xcc_xor;
     a.status = g_status_ptr[dev];
     a.clk = g_clock_probe;
+    a.phase = g_phase_probe; a.phase_wgs = g_phase_wgs;
     dim3 grid((unsigned)(8 * a.sk_tpx * split), 1);
     constexpr int lds = w4_lds_bytes<BM, BN>();
     if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, 2, 2, true, true>), grid, dim3(320), lds, st, a);
@@ -2367,7 +2393,7 @@ int fill_args(GemmArgs &a, void *Y, const void *X, const void *W, const void *bi
     a.ag = NhwcGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
-    a.clk = nullptr;
+    a.clk = nullptr; a.phase = nullptr; a.phase_wgs = 0;
     a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
     a.sk_spin = 0; a.sk_pub_xor = a.sk_xcc_xor = 0; a.status = nullptr;
     a.lnf_stats = a.lnf_colsum = a.lnf_biasp = nullptr; a.lnf_svec = 0; a.lnf_nseg = 0; a.lnf_eps = 0.0f; a.stats_out = nullptr; a.stats_nseg = 0;
@@ -2488,7 +2514,7 @@ int mi_internal_gemm(void *Y, const void *A, const void *B, const void *bias, in
     a.ag = NhwcGather{};
     a.ln_gamma = a.ln_beta = nullptr; a.ln_eps = 0.0f; a.ln_on = 0;
     a.lnout = nullptr; a.lnout_gamma = a.lnout_beta = nullptr; a.lnout_eps = 0.0f; a.clamp = 0.0f;
-    a.clk = nullptr;
+    a.clk = nullptr; a.phase = nullptr; a.phase_wgs = 0;
     a.sk_S = 0; a.sk_tpx = 0; a.sk_part = nullptr; a.sk_flags = nullptr; a.sk_epoch = 0;
     a.sk_spin = 0; a.sk_pub_xor = a.sk_xcc_xor = 0; a.status = nullptr;
     a.lnf_stats = a.lnf_colsum = a.lnf_biasp = nullptr; a.lnf_svec = 0; a.lnf_nseg = 0; a.lnf_eps = 0.0f; a.stats_out = nullptr; a.stats_nseg = 0;
@@ -2563,6 +2589,13 @@ int mi_init(void) {
     sk_probe_current_device();      // a device that fails the probe only loses that path
     if (bad) return MI_ERROR_DEVICE;
     g_ready = true;
+    return MI_OK;
+}
+
+int mi_set_phase_probe(void *dev_u64, int64_t workgroups) {
+    if (workgroups < 0 || workgroups > (1 << 20) || (dev_u64 && !aligned_to(dev_u64, 8))) return MI_DECLINE_OPERANDS;
+    g_phase_probe = reinterpret_cast<unsigned long long *>(dev_u64);
+    g_phase_wgs = dev_u64 ? (int)workgroups : 0;
     return MI_OK;
 }
 
