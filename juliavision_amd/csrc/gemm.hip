@@ -429,6 +429,33 @@ __device__ __forceinline__ void store_tile_epi(const GemmArgs &p, float16v (&acc
     });
 }
 
+// Block j (32 rows) of a wave's accumulators -> its staging area `dst` (32 rows of WTN + 8 halves), rounded to fp16 once
+// with the column bias -- or the folded layer norm's r (acc - mu colsum) + biasp -- joined in fp32.
+template <int j, int TM, int TN, int WTN>
+__device__ __forceinline__ void stage_block(float16v (&acc)[TN][TM], const half4v (&cb)[TN][4], const LnFold<TM> &ln, int wn, char *dst, int lane) {
+    constexpr int SLD_H = WTN + 8;
+    const int frow = lane & 31, hl = lane >> 5;
+    half_t *st = reinterpret_cast<half_t *>(dst) + frow * SLD_H + 4 * hl;
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const int nl = 32 * i + 8 * g;
+            float v[4];
+            if (ln.on) {      // uniform; the tile's colsum and biasp from their LDS copy
+                const float4v lc = *reinterpret_cast<const float4v *>(ln.col + wn * WTN + nl + 4 * hl);
+                const float4v lb = *reinterpret_cast<const float4v *>(ln.col + ln.bn + wn * WTN + nl + 4 * hl);
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = fmaf(acc[i][j][4 * g + e], ln.r[j], fmaf(-ln.rmu[j], lc[e], lb[e]));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + (float)cb[i][g][e];
+            }
+            const half4v o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+            *reinterpret_cast<half4v *>(st + nl) = o;
+        }
+}
+
 // The common store: fp16 output in whole 16-byte chunks, column bias (or a folded layer norm), optional activation,
 // residual, clamp and row statistics; no row bias, no fp32 output, no ragged N.
 //
@@ -461,25 +488,7 @@ __device__ __forceinline__ void store_tile_simple(const GemmArgs &p, float16v (&
         for (int g = 0; g < 4; g++) asm volatile("" ::"v"(cb[i][g]));
     auto stage = [&](auto J) {
         constexpr int j = decltype(J)::value;
-        half_t *st = reinterpret_cast<half_t *>(buf + (j & 1) * BUF_BYTES) + frow * SLD_H + 4 * hl;
-#pragma unroll
-        for (int i = 0; i < TN; i++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int nl = 32 * i + 8 * g;
-                float v[4];
-                if (ln.on) {      // uniform: r (acc - mu colsum) + biasp, the tile's colsum and biasp from their LDS copy
-                    const float4v lc = *reinterpret_cast<const float4v *>(ln.col + wn * WTN + nl + 4 * hl);
-                    const float4v lb = *reinterpret_cast<const float4v *>(ln.col + ln.bn + wn * WTN + nl + 4 * hl);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) v[e] = fmaf(acc[i][j][4 * g + e], ln.r[j], fmaf(-ln.rmu[j], lc[e], lb[e]));
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * g + e] + (float)cb[i][g][e];
-                }
-                const half4v o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                *reinterpret_cast<half4v *>(st + nl) = o;
-            }
+        stage_block<j, TM, TN, WTN>(acc, cb, ln, wn, buf + (j & 1) * BUF_BYTES, lane);
     };
     half8v res[2][NIT];
     auto fetch_residual = [&](auto J) {
@@ -539,6 +548,52 @@ __device__ __forceinline__ void store_tile_simple(const GemmArgs &p, float16v (&
             }
         }
     });
+}
+
+// The store of a launch with an activation, shared between a matrix wave and the helper wave on its SIMD.  One wave
+// issues a vector instruction every eight clocks, a SIMD takes one every four: the erf-GELU of a 128 x 256 tile (a
+// reciprocal, an exponential and thirteen other vector instructions on each of 128 values a lane) cost a lone
+// matrix wave 14 600 clocks.  The matrix wave stages its 32-row blocks as in store_tile_simple and takes the first half
+// of each block's chunks, the helper the second half; a workgroup barrier per block says "block j is staged" (a
+// wave passes barrier j + 1 only when it has block j's chunks in registers, so staging block j + 2 over block j's area
+// after that barrier is safe).  Launches without residual, clamp or statistics only.
+__device__ __forceinline__ bool coop_store_applies(const GemmArgs &p) {
+    return p.epi != MI_EPI_NONE && !p.out_f32 && p.vec_store && p.N % 8 == 0 && p.bias_mode != MI_BIAS_ROW && !p.residual &&
+           !(p.clamp > 0.0f) && !p.stats_out;
+}
+template <int EPI, int TM, int WTN, bool HELPER, typename StageF, typename BarrierF>
+__device__ __forceinline__ void store_coop_epi(const GemmArgs &p, char *buf, int mw, int nw, int lane, long bz, StageF stage, BarrierF barrier) {
+    constexpr int SLD_H = WTN + 8, BUF_BYTES = 32 * SLD_H * 2;
+    constexpr int CPR = WTN / 8, RPI = 64 / CPR, NIT = 32 / RPI, T0 = HELPER ? NIT / 2 : 0, T1 = HELPER ? NIT : NIT / 2;
+    static_assert(NIT % 2 == 0, "the chunks of a block split in two");
+    const int ch = lane % CPR, r0 = lane / CPR;
+    const int n = nw + ch * 8;
+    const bool col_ok = n < p.N;
+    half_t *const ybase = reinterpret_cast<half_t *>(p.Y) + bz * p.sY + (long)(mw + r0) * p.ldY + n;
+    if constexpr (!HELPER) stage(std::integral_constant<int, 0>{});
+    static_for<TM>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+        barrier();                                             // block j is staged
+        const half_t *rd = reinterpret_cast<const half_t *>(buf + (j & 1) * BUF_BYTES) + r0 * SLD_H + ch * 8;
+        half8v x[T1 - T0];
+#pragma unroll
+        for (int t = T0; t < T1; t++) x[t - T0] = *reinterpret_cast<const half8v *>(rd + t * RPI * SLD_H);
+        if constexpr (!HELPER && j + 1 < TM) stage(std::integral_constant<int, j + 1>{});
+#pragma unroll
+        for (int t = T0; t < T1; t++) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[t - T0][e] = (half_t)apply_epi_c<EPI>((float)x[t - T0][e]);
+            if (col_ok && mw + 32 * j + r0 + t * RPI < p.M) *reinterpret_cast<half8v *>(ybase + (long)(32 * j + t * RPI) * p.ldY) = x[t - T0];
+        }
+    });
+}
+template <int TM, int WTN, bool HELPER, typename StageF, typename BarrierF>
+__device__ __forceinline__ void store_coop(const GemmArgs &p, char *buf, int mw, int nw, int lane, long bz, StageF stage, BarrierF barrier) {
+    switch (p.epi) {
+    case MI_EPI_GELU_ERF: store_coop_epi<MI_EPI_GELU_ERF, TM, WTN, HELPER>(p, buf, mw, nw, lane, bz, stage, barrier); break;
+    case MI_EPI_GELU_TANH: store_coop_epi<MI_EPI_GELU_TANH, TM, WTN, HELPER>(p, buf, mw, nw, lane, bz, stage, barrier); break;
+    default: store_coop_epi<MI_EPI_RELU, TM, WTN, HELPER>(p, buf, mw, nw, lane, bz, stage, barrier); break;
+    }
 }
 
 // The activation is a compile-time choice inside the store loops: one uniform branch per tile
@@ -1087,7 +1142,7 @@ struct DirectTile {
 };
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool B_KN, bool SK = false>
-__global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
+__global__ __launch_bounds__(512) void gemm_w4_kernel(GemmArgs p) {
     constexpr int BK = 64, STAGES = 3, KS = 4;
     using T = DirectTile<BM, BN, BK, B_KN>;
     constexpr int ROWB = T::ROWB, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, PER_TILE = T::SLOTS_A + T::SLOTS_B;
@@ -1131,6 +1186,15 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
+    // A launch with an activation has eight waves, and the four that do not multiply help with the store
+    // (store_coop_epi): wave 4 + w shares a SIMD with matrix wave w.
+    const bool coop = !SK && blockDim.x == 512 && coop_store_applies(p);      // uniform
+    constexpr int COOP_BUF = 2 * 32 * (WTN + 8) * 2;                         // a matrix wave's two staging areas
+    auto help_store = [&]() {
+        const int mwave = wave - 4;
+        store_coop<TM, WTN, true>(p, smem + mwave * COOP_BUF, m0 + (mwave % WAVES_M) * WTM, n0 + (mwave / WAVES_M) * WTN, lane, bz,
+                                  [](auto) {}, barrier);
+    };
     if (wave == 4) {
         uint32_t offa[T::SLOTS_A], offb[T::SLOTS_B];
 #pragma unroll
@@ -1157,11 +1221,19 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
             barrier();                                              // B_kt
             if (kt + 3 < nk) request(kt + 3, kt % 3);
         }
+        if (coop) help_store();
         return;
     }
     float2v *ln_slot = reinterpret_cast<float2v *>(smem + STAGES * STAGE_BYTES);
+    if (wave >= 5 && !(wave == 5 && p.lnf_stats)) {
+        // nothing to do beside the K loop: keep the barriers' count, then help with the store
+        barrier();
+        for (int kt = 0; kt < nk; kt++) barrier();
+        if (coop) help_store();
+        return;
+    }
     if (wave == 5) {
-        // The statistics wave of a folded layer norm (the launch has it only then).  The matrix waves need (r, r mu) of
+        // The statistics wave of a folded layer norm.  The matrix waves need (r, r mu) of
         // the tile's rows and the tile's columns of colsum and biasp at the store, not before: combining a row's
         // K / 32 segment statistics in the prologue held every wave at the first barrier (5 000 clocks at 128 rows,
         // 10 000 at 192: a trip to memory per batch of loads, then forty dependent steps a row).  This wave does it
@@ -1233,6 +1305,7 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
                 }
             });
         }
+        if (coop) help_store();
         return;
     }
     // (a launch without the statistics wave and with a folded norm: combine in the prologue, as the other kernels do)
@@ -1383,7 +1456,18 @@ __global__ __launch_bounds__(384) void gemm_w4_kernel(GemmArgs p) {
 #pragma unroll
         for (int j = 0; j < TM; j++) { const float2v v = ln_slot[wm * WTM + 32 * j + (lane & 31)]; ln.r[j] = v[0]; ln.rmu[j] = v[1]; }
     }
-    store_tile<TM, TN, WTM, WTN, 4, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln);
+    if (coop) {
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) asm volatile("" ::"v"(cb[i][g]));      // in registers ahead of the first store (store_tile_simple)
+        char *buf = smem + wave * COOP_BUF;
+        store_coop<TM, WTN, false>(p, buf, m0 + wm * WTM, n0 + wn * WTN, lane, bz,
+                                   [&](auto J) { constexpr int j = decltype(J)::value; stage_block<j, TM, TN, WTN>(acc, cb, ln, wn, buf + (j & 1) * (COOP_BUF / 2), lane); },
+                                   barrier);
+    } else {
+        store_tile<TM, TN, WTM, WTN, 4, STAGES * STAGE_BYTES>(p, acc, cb, smem, m0, n0, wm, wn, wave, lane, bz, ln);
+    }
     phase_store();
     if (probe) { p.clk[2] = clock64(); p.clk[3] = wall_clock64(); }
 }
@@ -2145,8 +2229,9 @@ int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     a.phase = g_phase_probe; a.phase_wgs = g_phase_wgs;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
     constexpr int lds = w4_lds_bytes<BM, BN>();
-    // four matrix waves and the loader, plus the statistics wave of a folded layer norm
-    const dim3 block(a.lnf_stats ? 384 : 320);
+    // four matrix waves and the loader, plus the statistics wave of a folded layer norm; eight waves when the store
+    // has an activation to compute (the four that do not multiply help with it)
+    const dim3 block(a.epi != MI_EPI_NONE ? 512 : a.lnf_stats ? 384 : 320);
     if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, WM, WN, true>), grid, block, lds, st, a);
     else      hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, WM, WN, false>), grid, block, lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
