@@ -550,15 +550,16 @@ __device__ __forceinline__ void store_tile_simple(const GemmArgs &p, float16v (&
     });
 }
 
-// The store of a launch with an activation, shared between a matrix wave and the helper wave on its SIMD.  One wave
-// issues a vector instruction every eight clocks, a SIMD takes one every four: the erf-GELU of a 128 x 256 tile (a
-// reciprocal, an exponential and thirteen other vector instructions on each of 128 values a lane) cost a lone
-// matrix wave 14 600 clocks.  The matrix wave stages its 32-row blocks as in store_tile_simple and takes the first half
-// of each block's chunks, the helper the second half; a workgroup barrier per block says "block j is staged" (a
-// wave passes barrier j + 1 only when it has block j's chunks in registers, so staging block j + 2 over block j's area
-// after that barrier is safe).  Launches without residual, clamp or statistics only.
-__device__ __forceinline__ bool coop_store_applies(const GemmArgs &p) {
-    return p.epi != MI_EPI_NONE && !p.out_f32 && p.vec_store && p.N % 8 == 0 && p.bias_mode != MI_BIAS_ROW && !p.residual &&
+// The four-wave kernel's store, shared between a matrix wave and the helper wave on its SIMD.  One wave issues a vector
+// instruction every eight clocks, a SIMD takes one every four: the erf-GELU of a 128 x 256 tile (a reciprocal, an
+// exponential and thirteen other vector instructions on each of 128 values a lane) cost a lone matrix wave 14 600
+// clocks, 8 100 with a helper, and the plain store gains too (1500 x 1280 -> 5120 + bias: 21.8 us against 22.8).  The
+// matrix wave stages its 32-row blocks as in store_tile_simple and takes the first half of each block's chunks, the
+// helper the second half; a workgroup barrier per block says "block j is staged" (a wave passes barrier j + 1 only
+// when it has block j's chunks in registers, so staging block j + 2 over block j's area after that barrier is safe).
+// Launches without residual, clamp or statistics only: the others keep store_tile_simple on the matrix waves alone.
+__host__ __device__ __forceinline__ bool coop_store_applies(const GemmArgs &p) {
+    return !p.out_f32 && p.vec_store && p.N % 8 == 0 && p.bias_mode != MI_BIAS_ROW && !p.residual &&
            !(p.clamp > 0.0f) && !p.stats_out;
 }
 template <int EPI, int TM, int WTN, bool HELPER, typename StageF, typename BarrierF>
@@ -592,7 +593,8 @@ __device__ __forceinline__ void store_coop(const GemmArgs &p, char *buf, int mw,
     switch (p.epi) {
     case MI_EPI_GELU_ERF: store_coop_epi<MI_EPI_GELU_ERF, TM, WTN, HELPER>(p, buf, mw, nw, lane, bz, stage, barrier); break;
     case MI_EPI_GELU_TANH: store_coop_epi<MI_EPI_GELU_TANH, TM, WTN, HELPER>(p, buf, mw, nw, lane, bz, stage, barrier); break;
-    default: store_coop_epi<MI_EPI_RELU, TM, WTN, HELPER>(p, buf, mw, nw, lane, bz, stage, barrier); break;
+    case MI_EPI_RELU: store_coop_epi<MI_EPI_RELU, TM, WTN, HELPER>(p, buf, mw, nw, lane, bz, stage, barrier); break;
+    default: store_coop_epi<MI_EPI_NONE, TM, WTN, HELPER>(p, buf, mw, nw, lane, bz, stage, barrier); break;
     }
 }
 
@@ -1186,8 +1188,8 @@ __global__ __launch_bounds__(512) void gemm_w4_kernel(GemmArgs p) {
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
-    // A launch with an activation has eight waves, and the four that do not multiply help with the store
-    // (store_coop_epi): wave 4 + w shares a SIMD with matrix wave w.
+    // A launch whose store the helpers can share (coop_store_applies) has eight waves, and the four that do not multiply
+    // take half of it (store_coop_epi): wave 4 + w shares a SIMD with matrix wave w.
     const bool coop = !SK && blockDim.x == 512 && coop_store_applies(p);      // uniform
     constexpr int COOP_BUF = 2 * 32 * (WTN + 8) * 2;                         // a matrix wave's two staging areas
     auto help_store = [&]() {
@@ -2229,9 +2231,9 @@ int launch_w4(GemmArgs a, bool b_kn, int64_t nbatch, hipStream_t st) {
     a.phase = g_phase_probe; a.phase_wgs = g_phase_wgs;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)nbatch);
     constexpr int lds = w4_lds_bytes<BM, BN>();
-    // four matrix waves and the loader, plus the statistics wave of a folded layer norm; eight waves when the store
-    // has an activation to compute (the four that do not multiply help with it)
-    const dim3 block(a.epi != MI_EPI_NONE ? 512 : a.lnf_stats ? 384 : 320);
+    // four matrix waves and the loader, plus the statistics wave of a folded layer norm; eight waves when the four that
+    // do not multiply can help with the store
+    const dim3 block(coop_store_applies(a) ? 512 : a.lnf_stats ? 384 : 320);
     if (b_kn) hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, WM, WN, true>), grid, block, lds, st, a);
     else      hipLaunchKernelGGL((gemm_w4_kernel<BM, BN, WM, WN, false>), grid, block, lds, st, a);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
