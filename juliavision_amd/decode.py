@@ -19,7 +19,7 @@ from typing import Callable, List, Optional
 import torch
 
 from . import _lib as L
-from .kernels import Ctx, DeclineError, _strides_elbh, layernorm_, ln_matmul_, matmul_, matmul_heads_, relayout_weight, sdpa, sdpa_append
+from .kernels import Ctx, DeclineError, Workspace, _strides_elbh, layernorm_, ln_matmul_, matmul_, matmul_heads_, relayout_weight, sdpa, sdpa_append
 
 
 # Fold the cache write into the self-attention launch where the one-launch kernel covers the shape.
@@ -188,6 +188,7 @@ class StepGraph:
         torch.cuda.synchronize()
         if restore is not None:
             restore()
+        Workspace.pin_all()                                # the capture holds addresses inside the workspaces from here on
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
             fn()

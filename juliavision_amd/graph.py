@@ -845,6 +845,8 @@ def _row_gather(g: Graph, o) -> Optional[tuple]:
     tb, ib = g.buffers[g.root(table)], g.buffers[ids]
     if tb["kind"] != "weight" or len(g.buffers[table].get("shape", [])) != 2 or ib.get("dtype") != "int64":
         return None
+    if tb.get("dtype") != "float16" or g.buffers[o["out"]].get("dtype") != "float16":      # mi_embedding_f16 gathers fp16 rows
+        return None
     return table, ids
 
 
@@ -924,6 +926,11 @@ def fold_patch_tokens(g: Graph) -> Graph:
         pb = g.buffers[pos]
         if pb["kind"] != "weight" or math.prod(pb["shape"]) != T * C or list(pb["shape"][-2:]) != [T, C] or \
                 list(g.buffers[other].get("shape", [])[-2:]) != [T, C]:
+            continue
+        # what the fused launch needs (mi_conv2d_tokens_f16): fp16 throughout, and token rows that start on 16 bytes --
+        # row 1 of every image, so C and T * C in whole 16-byte chunks.  Otherwise the ops stay as written.
+        f16 = lambda bid: g.buffers[bid].get("dtype") == "float16"
+        if C % 8 or (T * C) % 8 or not all(f16(b) for b in list(conv["in"]) + [cls, pos, conv["out"], add["out"]]):
             continue
         at = g.ops.index(add)
         g.ops[at] = {"id": add["id"], "aten": "patch_tokens", "in": list(conv["in"]) + [cls, pos], "out": add["out"],

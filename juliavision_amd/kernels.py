@@ -22,6 +22,8 @@ PyTorch is used only to own device memory and the stream.
 """
 from __future__ import annotations
 
+import weakref
+
 import ctypes as C
 import math
 from dataclasses import dataclass
@@ -88,22 +90,38 @@ class Workspace:
     next reset.  Grows by reallocation between ops, never inside one.
 
     A captured graph (``StepGraph``, ``Executor.replayable``) holds the addresses it was captured with -- split-K
-    planes, split-KV partials, convolution scratch -- for as long as it may be replayed.  So a buffer that was
-    ever handed out is never given back: growing retires the old buffer into ``_retired``, where it stays until
-    the workspace itself goes, and a replay after later growth still writes memory that nothing else owns.
-    Growing *during* a capture cannot work (the allocation would be captured too) and raises: run the step
-    eagerly once first, as both graph wrappers do, so that the workspace has reached its size."""
+    planes, split-KV partials, convolution scratch -- for as long as it may be replayed, and says so with ``pin()``.
+    From then on a buffer that is outgrown is retired into ``_retired`` instead of given back, where it stays until
+    the workspace itself goes, so a replay after later growth still writes memory that nothing else owns.  Before any
+    graph has pinned the workspace an outgrown buffer is simply dropped: the kernels already enqueued on it run on the
+    stream the allocator frees it on, so it is not reused under them.  (Buffers double, so even retired ones add up to
+    less than the current one.)  Growing *during* a capture cannot work (the allocation would be captured too) and
+    raises: run the step eagerly once first, as both graph wrappers do, so that the workspace has reached its size."""
 
     ALIGN = 256
+    _live = weakref.WeakSet()                             # every workspace alive: a capture pins them all (pin_all)
+
+    @classmethod
+    def pin_all(cls):
+        """Called by whoever captures a device graph of kernel launches: a capture does not know which workspaces the
+        launches inside it drew from, so all of them keep what they have handed out."""
+        for ws in list(cls._live):
+            ws.pin()
 
     def __init__(self, device="cuda", nbytes: int = 0):
         self.device = torch.device(device)
         self.buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=self.device)
         self.off = 0
         self._retired = []
+        self._pinned = False
+        Workspace._live.add(self)
 
     def reset(self):
         self.off = 0
+
+    def pin(self):
+        """A graph has captured addresses inside this workspace: nothing it handed out may be given back any more."""
+        self._pinned = True
 
     def scratch(self, nbytes: int) -> int:
         if nbytes <= 0:
@@ -113,7 +131,8 @@ class Workspace:
         if start + nbytes > self.buf.numel():
             if torch.cuda.is_current_stream_capturing():
                 raise RuntimeError(f"Workspace would have to grow to {nbytes} bytes inside a graph capture: run the step eagerly once before capturing it")
-            self._retired.append(self.buf)              # kernels already enqueued, and graphs already captured, keep using it
+            if self._pinned:
+                self._retired.append(self.buf)          # graphs already captured keep using it
             self.buf = torch.empty(max(2 * self.buf.numel(), nbytes + self.ALIGN), dtype=torch.uint8, device=self.device)
             self.off = 0
             base = self.buf.data_ptr()

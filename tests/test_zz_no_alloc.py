@@ -85,3 +85,45 @@ def test_noalloc_refuses_beyond_its_static_array():
     assert rc == L.DECLINE_SCRATCH_LIMIT
     torch.cuda.synchronize()
     assert bool(torch.isnan(y).all()), "a refused call wrote something"
+
+
+def test_noalloc_under_graph_capture():
+    """The callers this entry point exists for: the call is captured into a device graph (in the capture mode that turns
+    any allocation, free or synchronisation made by the thread into an error), replayed over changed inputs with eager
+    work in between, and every replay must give the bits of mi_gemm_f16 with a caller workspace; free device memory
+    does not shrink across the replays."""
+    import torch
+    from juliavision_amd import _lib as L
+    lib = L.init()
+    T, K, F = 200, 4096, 256
+    need = lib.mi_gemm_f16_workspace(T, K, F, L.W_FK, 1)
+    assert 0 < need <= L.NOALLOC_SCRATCH_BYTES
+    Wkf = oracle.randn_f16((K, F), 62, 0, 1.0)
+    dW, db = to_dev(np.ascontiguousarray(Wkf.T)), to_dev(oracle.randn_f16((F,), 63, 0, 0.02))
+    dX = to_dev(oracle.randn_f16((T, K), 61, 0, 1.0 / np.sqrt(K)))
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    got = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+    want = poison(torch.empty((T, F), dtype=torch.float16, device="cuda"))
+
+    def noalloc(stream):
+        return lib.mi_gemm_f16_noalloc(got.data_ptr(), dX.data_ptr(), dW.data_ptr(), db.data_ptr(), None, T, K, F, F, K, K,
+                                       L.W_FK, L.BIAS_COL, L.EPI["gelu"], L.F16, stream)
+    assert noalloc(torch.cuda.current_stream().cuda_stream) == L.OK      # a first call outside the capture, as a host would warm up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, capture_error_mode="global"):
+        assert noalloc(torch.cuda.current_stream().cuda_stream) == L.OK
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for seed in (71, 72, 73):
+        dX.copy_(to_dev(oracle.randn_f16((T, K), seed, 0, 1.0 / np.sqrt(K))))
+        poison(got)
+        graph.replay()
+        rc = lib.mi_gemm_f16(want.data_ptr(), dX.data_ptr(), dW.data_ptr(), db.data_ptr(), None, T, K, F, F, K, K,
+                             L.W_FK, L.BIAS_COL, L.EPI["gelu"], L.F16, ws.data_ptr(), need, torch.cuda.current_stream().cuda_stream)
+        assert rc == L.OK
+        torch.cuda.synchronize()
+        g, w = to_host(got), to_host(want)
+        assert np.all(np.isfinite(g)), "unwritten output"
+        assert np.array_equal(g.view(np.uint16), w.view(np.uint16)), f"replay with seed {seed} differs from mi_gemm_f16"
+    assert torch.cuda.mem_get_info()[0] >= free_before, "device memory shrank across replays of a call that allocates nothing"
