@@ -1198,11 +1198,26 @@ __global__ __launch_bounds__(512) void gemm_w4_kernel(GemmArgs p) {
                                   [](auto) {}, barrier);
     };
     if (wave == 4) {
+        // Per-lane offsets of the tile's 1 KB slots.  A tile that lies inside the operands needs no clamping, and its
+        // slots s and s + 2 differ by a constant (eight rows of a K-contiguous operand, 64 / (BN / 8) k-rows of the
+        // [K][N] one; the chunk permutation has period two in s): two offsets computed in full, the others one add
+        // each -- this wave alone stands between the launch and the first request, at a vector instruction every
+        // eight clocks.
         uint32_t offa[T::SLOTS_A], offb[T::SLOTS_B];
+        if (m0 + BM <= p.M && n0 + BN <= (B_KN ? p.NB : p.N)) {          // uniform
+            const uint32_t step_a = (uint32_t)(8 * p.ldA * 2), step_b = (uint32_t)((B_KN ? 64 / (BN / 8) : 8) * p.ldB * 2);
+            const uint32_t a0 = T::a_offset(p, m0, 0, lane), a1 = T::a_offset(p, m0, 1, lane);
+            const uint32_t b0 = T::b_offset(p, n0, 0, lane), b1 = T::b_offset(p, n0, 1, lane);
 #pragma unroll
-        for (int s = 0; s < T::SLOTS_A; s++) offa[s] = T::a_offset(p, m0, s, lane);
+            for (int s = 0; s < T::SLOTS_A; s++) offa[s] = ((s & 1) ? a1 : a0) + (uint32_t)(s & ~1) * step_a;
 #pragma unroll
-        for (int s = 0; s < T::SLOTS_B; s++) offb[s] = T::b_offset(p, n0, s, lane);
+            for (int s = 0; s < T::SLOTS_B; s++) offb[s] = ((s & 1) ? b1 : b0) + (uint32_t)(s & ~1) * step_b;
+        } else {
+#pragma unroll
+            for (int s = 0; s < T::SLOTS_A; s++) offa[s] = T::a_offset(p, m0, s, lane);
+#pragma unroll
+            for (int s = 0; s < T::SLOTS_B; s++) offb[s] = T::b_offset(p, n0, s, lane);
+        }
         auto request = [&](int kt, int stage) {
             const char *ab = Ag + (long)kt * a_step, *bb = Bg + (long)kt * b_step;
             const uint32_t sa = lds0 + stage * STAGE_BYTES, sb = sa + A_BYTES;
