@@ -462,14 +462,16 @@ def group_linears(g: Graph) -> Graph:
     as one launch of 180 tiles, 3 x 16 us apart).  The members keep their result buffers: planes of one allocation.
     Decode-sized members that all carry the same layer norm as their prologue (``fold_layernorm_prologues``) become one
     GEMV instead: the weights laid end to end along the output axis, the norm computed once, the results column bands
-    of one buffer -- the fused q/k/v projection of the hand-composed decoder layer."""
+    of one buffer -- the fused q/k/v projection of the hand-composed decoder layer.  Members whose norm was folded
+    away (``fold_norms_away``) run as the planes of one launch on the raw rows, their results column bands likewise."""
     def key(o):
         pos = {"linear.default": (0, 1, 2), "addmm.default": (1, 2, 0), "mm.default": (0, 1, None)}[o["aten"]]
         x, w = o["in"][pos[0]], o["in"][pos[1]]
         b = o["in"][pos[2]] if pos[2] is not None and len(o["in"]) > pos[2] else None
         return x, w, b
-    plain = lambda o: o["aten"] in LINEAR_OPS and not any(k in o["attrs"] for k in ("epilogue", "residual", "ln_out", "clamp"))
-    norm_of = lambda o: tuple(o["attrs"].get(k) for k in ("ln_in", "ln_in_gamma", "ln_in_beta", "ln_in_eps"))
+    plain = lambda o: o["aten"] in LINEAR_OPS and not any(k in o["attrs"] for k in ("epilogue", "residual", "ln_out", "clamp", "stats_out"))
+    norm_keys = ("ln_in", "ln_in_gamma", "ln_in_beta", "ln_in_eps", "lnf", "lnf_gamma", "lnf_beta", "lnf_eps")
+    norm_of = lambda o: tuple(o["attrs"].get(k) for k in norm_keys)
     done = set()
     for first in [o for o in g.ops if plain(o)]:
         if first["id"] in done or first not in g.ops:
@@ -511,9 +513,14 @@ def group_linears(g: Graph) -> Graph:
             # laid end to end along the output axis, the norm computed once, the results column bands of one buffer
             attrs.update({k: first["attrs"].get(k) for k in ("ln_in", "ln_in_gamma", "ln_in_beta", "ln_in_eps")})
             extra = [first["attrs"][k] for k in ("ln_in_gamma", "ln_in_beta") if first["attrs"].get(k)]
+        if first["attrs"].get("lnf"):
+            # members whose norm was folded away (fold_norms_away): planes of one launch over the raw rows, the prepared
+            # weights end to end along the output axis, the results column bands of one buffer
+            attrs.update({k: first["attrs"].get(k) for k in ("lnf", "lnf_gamma", "lnf_beta", "lnf_eps")})
+            extra = [first["attrs"][k] for k in ("lnf_gamma", "lnf_beta") if first["attrs"].get(k)]
         g.ops[at] = {"id": first["id"] + "_group", "aten": "linear_group", "in": [x0] + [m["w"] for m in spec] + [m["b"] for m in spec if m["b"]] + extra,
                      "out": first["out"], "attrs": attrs}
-        g.notes.append("one launch for " + ", ".join(m["out"] for m in spec) + (" (norm prologue shared)" if extra or attrs.get("ln_in") else ""))
+        g.notes.append("one launch for " + ", ".join(m["out"] for m in spec) + (" (norm prologue shared)" if attrs.get("ln_in") else " (on the raw rows)" if attrs.get("lnf") else ""))
     return g
 
 
@@ -636,6 +643,86 @@ def fold_layernorm_prologues(g: Graph) -> Graph:
     return g
 
 
+def fold_norms_away(g: Graph) -> Graph:
+    """A layer norm over the last axis that only linear ops read (through reshapes at most), over enough rows that the
+    tiled GEMMs run them (``kernels.lnfold_applies``), gets no pass of its own at all: ``LN(x) . W + b`` is
+    ``r (x . gamma W) - r mu colsum(gamma W) + (b + beta . W)``, so the linears run on the RAW rows with constants the
+    executor prepares once (``lnfold_prepare``) and need only each row's mean and reciprocal deviation, which come from
+    partial sums the GEMM that wrote those rows leaves behind (``stats_out`` on a linear op: ``matmul_rowstats_``) or,
+    for rows no linear op wrote (the graph's input, an embedding sum), from a small ``rowstats`` op where the norm
+    stood.  The normalised activations never exist in memory.  Held to the parity gate against the separate norm, not
+    to its bits.  Decode-sized norms are ``fold_layernorm_prologues``' (which runs first); what neither takes is left
+    for ``fold_layernorms``."""
+    for ln in [o for o in g.ops if o["aten"] in ("layer_norm.default", "native_layer_norm.default")]:
+        a = ln["attrs"]
+        x = ln["in"][0]
+        xb = g.buffers[x]
+        feat = (xb.get("shape") or [None])[-1]
+        if feat is None or list(a.get("arg1", [])) != [feat] or xb.get("dtype") != "float16":
+            continue
+        readers = _consumers(g, ln["out"])
+        if not readers or "<output>" in readers:
+            continue
+        if any(g.buffers[g.root(i)]["kind"] != "weight" for i in ln["in"][1:]):
+            continue                                    # gamma / beta must be constants: they go into the weights
+        T = math.prod(xb["shape"][:-1])
+        lins = []
+        for rid in sorted(readers, key=lambda r: g.ops.index(g.op(r))):
+            lin = g.op(rid)
+            if lin is None or lin["aten"] not in LINEAR_OPS or any(k in lin["attrs"] for k in ("ln_in", "ln_out", "lnf")):
+                break
+            xpos = {"linear.default": 0, "addmm.default": 1, "mm.default": 0}[lin["aten"]]
+            wpos = {"linear.default": 1, "addmm.default": 2, "mm.default": 1}[lin["aten"]]
+            at = lin["in"][xpos]
+            ok = True
+            while at != ln["out"]:
+                b = g.buffers[at]
+                if b["kind"] != "view" or not (b.get("op") in RESHAPES or "getitem" in b.get("op", "")) or \
+                        ("getitem" not in b.get("op", "") and (b.get("shape") or [None])[-1] != feat):
+                    ok = False
+                    break
+                at = b["of"]
+            if not ok or sum(1 for i in lin["in"] if i == lin["in"][xpos]) != 1:
+                break
+            wshape = g.buffers[lin["in"][wpos]].get("shape") or []
+            if len(wshape) != 2 or g.buffers[g.root(lin["in"][wpos])]["kind"] != "weight" or g.buffers[lin["out"]].get("dtype") != "float16":
+                break
+            if not K.lnfold_applies(T, feat, wshape[0] if lin["aten"] == "linear.default" else wshape[1]):
+                break
+            lins.append(lin)
+        if len(lins) != len(readers):
+            continue
+        # where the rows' statistics come from: the linear op that wrote them, if its GEMM can leave them ...
+        chain = [x]
+        while g.buffers[chain[-1]]["kind"] == "view":
+            chain.append(g.buffers[chain[-1]]["of"])
+        prod = g.op(chain[-1])
+        rides = prod is not None and prod["aten"] in LINEAR_OPS and not any(k in prod["attrs"] for k in ("ln_in", "ln_out")) and \
+            all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1]) and \
+            g.buffers[chain[-1]].get("dtype") == "float16" and (g.buffers[chain[-1]].get("shape") or [None])[-1] == feat
+        if rides:
+            wpos = {"linear.default": 1, "addmm.default": 2, "mm.default": 1}[prod["aten"]]
+            wshape = g.buffers[prod["in"][wpos]].get("shape") or []
+            rides = len(wshape) == 2 and K.rowstats_rides(T, wshape[1] if prod["aten"] == "linear.default" else wshape[0], feat)
+        if rides and prod["attrs"].get("stats_out"):
+            sid = prod["attrs"]["stats_out"]             # a second norm over the same rows
+        else:
+            sid = ln["id"] + "_rowstats"
+            g.buffers[sid] = {"id": sid, "kind": "transient", "shape": [K.rowstats_segments(feat), T, 2], "dtype": "float32"}
+            if rides:
+                prod["attrs"]["stats_out"] = sid
+            else:                                        # ... or one small pass over them where the norm stood
+                g.ops.insert(g.ops.index(ln), {"id": sid, "aten": "rowstats", "in": [x], "out": sid, "attrs": {}})
+        for lin in lins:
+            lin["attrs"].update(lnf=sid, lnf_gamma=ln["in"][1] if len(ln["in"]) > 1 else None,
+                                lnf_beta=ln["in"][2] if len(ln["in"]) > 2 else None, lnf_eps=a.get("arg4", a.get("eps", 1e-5)))
+        g.ops.remove(ln)
+        g.buffers[ln["out"]].update(kind="view", of=x, op="alias.default", attrs={})
+        g.notes.append(f"fold {ln['id']} away: " + ", ".join(l["id"] for l in lins) + " run on the raw rows, statistics from " +
+                       (prod["id"] if rides else "a rowstats op"))
+    return g
+
+
 def fold_layernorms(g: Graph) -> Graph:
     """A layer norm over the last axis whose input is (a reshaping view of) a linear op's output -- the residual
     stream after ``addmm`` + ``add``, normalised for the next block -- is written by that GEMM as a second result
@@ -647,7 +734,7 @@ def fold_layernorms(g: Graph) -> Graph:
         while g.buffers[chain[-1]]["kind"] == "view":
             chain.append(g.buffers[chain[-1]]["of"])
         prod = g.op(chain[-1])
-        if prod is None or prod["aten"] not in LINEAR_OPS or "ln_out" in prod["attrs"] or "ln_in" in prod["attrs"]:
+        if prod is None or prod["aten"] not in LINEAR_OPS or any(k in prod["attrs"] for k in ("ln_out", "ln_in", "lnf", "stats_out")):
             continue
         feat = (g.buffers[chain[-1]].get("shape") or [None])[-1]
         shapes_ok = all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1])
@@ -1142,8 +1229,8 @@ def prune(g: Graph) -> Graph:
 
 def optimize(g: Graph) -> Graph:
     g = fold_patch_tokens(fold_cache_step(fold_embedding_sum(g)))
-    return group_linears(fold_sdpa_transpose(fold_attention(fold_layernorms(fold_layernorm_prologues(
-        fold_clamps(fold_residuals(fold_layerscale(fold_activations(g)))))))))
+    return group_linears(fold_sdpa_transpose(fold_attention(fold_layernorms(fold_norms_away(fold_layernorm_prologues(
+        fold_clamps(fold_residuals(fold_layerscale(fold_activations(g))))))))))
 
 
 # ----------------------------------------------------------------------------- execution
@@ -1170,6 +1257,10 @@ class Executor:
         for o in graph.ops:                               # check every op has a handler before anything runs
             if o["aten"] not in self.HANDLERS:
                 raise UnsupportedOp(f"{graph.name}: no kernel on this path for aten.{o['aten']} (op {o['id']})")
+        for o in graph.ops:                               # row statistics a GEMM leaves for a folded norm
+            sid = o["attrs"].get("stats_out")
+            if sid is not None and sid not in self.t:
+                self.t[sid] = torch.empty(list(graph.buffers[sid]["shape"]), dtype=torch.float32, device=self.device)
         for o in graph.ops:                               # a norm folded into its producer: its result still needs a home
             nid = o["attrs"].get("ln_out")
             if nid is not None:
@@ -1180,7 +1271,7 @@ class Executor:
             if o["aten"] == "linear_group":               # the members' results are planes of one allocation
                 mem = o["attrs"]["members"]
                 b0 = graph.buffers[mem[0]["out"]]
-                if o["attrs"].get("ln_in"):               # ... or column bands of one (rows, n F) matrix
+                if o["attrs"].get("ln_in") or o["attrs"].get("lnf"):      # ... or column bands of one (rows, n F) matrix
                     F, rows = b0["shape"][-1], math.prod(b0["shape"][:-1])
                     bands = torch.empty((rows, len(mem) * F), dtype=_DTYPES[b0["dtype"]], device=self.device)
                     for i, m in enumerate(mem):
@@ -1290,6 +1381,18 @@ class Executor:
         out = self.t[o["out"]]
         res = self._rows(self.get(res_id)) if res_id else None
         self.ctx.ws.reset()
+        stats_out = self.t[attrs["stats_out"]] if attrs.get("stats_out") else None
+        if attrs.get("lnf"):                             # the norm in front folded away: prepared constants, raw rows
+            if ("lnf", o["id"]) not in self.scaled:
+                self.scaled[("lnf", o["id"])] = K.lnfold_prepare(self.ctx, w, self.get(attrs["lnf_gamma"]) if attrs.get("lnf_gamma") else None,
+                                                                 self.get(attrs["lnf_beta"]) if attrs.get("lnf_beta") else None, bias)
+            K.lnfold_matmul_(self.ctx, self._rows(out), self.scaled[("lnf", o["id"])], self._rows(x), self.t[attrs["lnf"]], attrs.get("lnf_eps", 1e-5),
+                             epi=attrs.get("epilogue", "none"), residual=res, stats_out=stats_out, clamp=attrs.get("clamp"))
+            return
+        if stats_out is not None:
+            K.matmul_rowstats_(self.ctx, self._rows(out), stats_out, w, self._rows(x), bias, epi=attrs.get("epilogue", "none"),
+                               residual=res, clamp=attrs.get("clamp"))
+            return
         if attrs.get("ln_out") is not None or attrs.get("clamp") is not None:
             has_ln = attrs.get("ln_out") is not None
             gamma = self.get(attrs["ln_gamma"]) if has_ln and attrs.get("ln_gamma") else None
@@ -1321,9 +1424,13 @@ class Executor:
                 bs.append(b)
             fk = all(w.stride(0) == 1 and w.stride(1) == w.shape[0] for w in ws)       # every member a transposed [F][K] matrix
             filled = [torch.zeros_like(next(x for x in bs if x is not None)) if b is None else b for b in bs] if any(b is not None for b in bs) else None
-            if o["attrs"].get("ln_in"):                   # end to end along the output axis, in the members' own memory layout
+            if o["attrs"].get("ln_in") or o["attrs"].get("lnf"):      # end to end along the output axis, in the members' own memory layout
                 W = torch.cat([w.t() for w in ws]).t() if fk else torch.cat([w.contiguous() for w in ws], dim=1)
                 B = None if filled is None else torch.cat(filled)
+                if o["attrs"].get("lnf"):
+                    a = o["attrs"]
+                    W = K.lnfold_prepare(self.ctx, W, self.get(a["lnf_gamma"]) if a.get("lnf_gamma") else None,
+                                         self.get(a["lnf_beta"]) if a.get("lnf_beta") else None, B, planes=len(mem))
             else:
                 W = torch.stack([w.t() for w in ws]).transpose(1, 2) if fk else torch.stack([w.contiguous() for w in ws])
                 B = None if filled is None else torch.stack(filled)
@@ -1331,6 +1438,10 @@ class Executor:
         W, B = self.scaled[o["id"]]
         x = self._rows(self.get(o["in"][0]))
         planes = self.t[o["id"]]
+        if o["attrs"].get("lnf"):
+            self.ctx.ws.reset()
+            K.lnfold_matmul_(self.ctx, planes, W, x, self.t[o["attrs"]["lnf"]], o["attrs"].get("lnf_eps", 1e-5))
+            return
         if o["attrs"].get("ln_in"):
             a = o["attrs"]
             self.ctx.ws.reset()
@@ -1401,6 +1512,10 @@ class Executor:
         """bmm(a (B,m,k), b (B,k,n)) -- batchedmatmul!, ops.jl:1393-1399."""
         a, b = self.get(o["in"][0]), self.get(o["in"][1])
         K.batchedmatmul_(self.ctx, self.t[o["out"]], b, a)
+
+    def _rowstats(self, o):
+        """The partial sums a folded norm's linears read, for rows no GEMM here wrote (``fold_norms_away``)."""
+        K.rowstats_(self.ctx, self.t[o["out"]], self._rows(self.get(o["in"][0])))
 
     def _layer_norm(self, o):
         ins, a = o["in"], o["attrs"]
@@ -1537,7 +1652,8 @@ class Executor:
                 "bmm.default": _bmm, "cat.default": _cat, **dict.fromkeys(SOFTMAX_OPS, _softmax),
                 "mul.Tensor": _scale, "div.Tensor": _scale, "clone.default": _clone, "clamp.default": _clamp,
                 "linear_group": _linear_group, "embedding.default": _embedding, "index.Tensor": _embedding,
-                "kv_len_from_position": _kv_len, "sdpa_append": _sdpa_append, "patch_tokens": _patch_tokens}
+                "kv_len_from_position": _kv_len, "sdpa_append": _sdpa_append, "patch_tokens": _patch_tokens,
+                "rowstats": _rowstats}
 
     def replayable(self, *inputs: torch.Tensor):
         """Run once eagerly (binds inputs, sizes the workspace, stacks folded constants), then capture the whole graph as

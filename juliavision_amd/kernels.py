@@ -344,6 +344,19 @@ def rowstats_segments(C: int) -> int:
     return (C + 31) // 32
 
 
+def lnfold_applies(T: int, K: int, F: int) -> bool:
+    """Whether ``lnfold_matmul_`` takes a ``(T, K) -> (T, F)`` linear (no GPU needed): the tiled kernels' pipelined form
+    (64-deep tiles, at least two of them) with 16-byte result rows, and enough rows that the tiled kernels are the ones
+    that would run it anyway."""
+    return T >= 64 and K >= 128 and K % 64 == 0 and F % 8 == 0
+
+
+def rowstats_rides(T: int, K: int, F: int) -> bool:
+    """Whether ``matmul_rowstats_`` takes a ``(T, K) -> (T, F)`` linear: the same conditions, seen from the GEMM that writes
+    the rows whose statistics are wanted."""
+    return lnfold_applies(T, K, F)
+
+
 def rowstats_new(rows: int, C: int, device="cuda") -> torch.Tensor:
     """Storage for the row statistics of ``rows`` rows of ``C`` elements: (sum, squares about its mean) per 32-column
     segment, segment-major ``(segments, rows, 2)``."""

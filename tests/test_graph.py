@@ -80,14 +80,26 @@ def test_rewrites_fold_activation_residuals_and_attention_layout():
     assert fc1["attrs"]["epilogue"] == "gelu" and g.buffers["gelu"]["kind"] == "view" and g.buffers["gelu"]["of"] == "linear_4"
     assert g.op("linear_3")["attrs"]["residual"] == "$x" and g.op("linear_5")["attrs"]["residual"] == "$add"
     assert g.op("scaled_dot_product_attention")["attrs"]["token_major"] is True
-    assert len(g.ops) == 6                                              # LN, q/k/v as one group, attention, 3 linears
+    assert len(g.ops) == 6                                              # row statistics of x, q/k/v as one group, attention, 3 linears
     grp = next(o for o in g.ops if o["aten"] == "linear_group")
     assert [m["out"] for m in grp["attrs"]["members"]] == ["linear", "linear_1", "linear_2"]
-    assert g.root("add_1") == "linear_5" and len(g.notes) == 6
-    # the second norm reads the residual stream that the out-projection writes: it became that GEMM's second result
+    assert g.root("add_1") == "linear_5" and len(g.notes) == 7
+    # 70 rows are enough for the tiled GEMMs: neither norm has a pass of its own.  The first reads the graph's input, whose
+    # row statistics one small op computes where the norm stood; q, k and v run on the raw rows as planes of one launch
+    assert g.op("layer_norm") is None and g.op("layer_norm_1") is None
+    assert [o["aten"] for o in g.ops][:2] == ["rowstats", "linear_group"] and g.ops[0]["in"] == ["x"]
+    assert grp["attrs"]["lnf"] == g.ops[0]["out"] and grp["attrs"]["lnf_gamma"] == "p_ln1_weight" and grp["attrs"]["lnf_beta"] == "p_ln1_bias"
+    assert g.buffers[g.ops[0]["out"]]["shape"] == [4, 70, 2] and g.buffers["layer_norm"]["of"] == "x"
+    # the second reads the residual stream the out-projection writes: that GEMM leaves the statistics, fc1 takes them
     proj = g.op("linear_3")
+    assert "ln_out" not in proj["attrs"] and fc1["attrs"]["lnf"] == proj["attrs"]["stats_out"] and fc1["attrs"]["lnf_eps"] == 1e-5
+    assert fc1["attrs"]["lnf_gamma"] == "p_ln2_weight" and g.buffers["layer_norm_1"]["of"] == "add"
+    # fewer rows than a tile is worth: the norms stay, the second as the out-projection's second result
+    ep40, _ = _export(_block(), T=40)
+    g40 = G.optimize(G.Graph.load(G.convert(ep40, "block")))
+    proj = g40.op("linear_3")
     assert proj["attrs"]["ln_out"] == "layer_norm_1" and proj["attrs"]["ln_gamma"] == "p_ln2_weight" and proj["attrs"]["ln_eps"] == 1e-5
-    assert g.op("layer_norm_1") is None and g.op("layer_norm") is not None           # the first norm reads the graph's input
+    assert g40.op("layer_norm_1") is None and g40.op("layer_norm") is not None and not any("lnf" in o["attrs"] for o in g40.ops)
     # an activation that something else also reads must stay where it is
     d = G.convert(ep, "block")
     d["outputs"].append("linear_4")
@@ -157,7 +169,7 @@ def test_decode_sized_norm_becomes_the_prologue_of_the_linear_that_reads_it():
     import torch
     from juliavision_amd import graph as G
     m = _mlp()
-    for rows, folded in ((4, True), (300, False)):
+    for rows, folded in ((4, True), (40, False), (300, None)):
         ep = torch.export.export(m, (torch.randn(1, rows, 256).half(),))
         g = G.optimize(G.Graph.load(G.convert(ep, "mlp")))
         fc1 = g.op("linear")
@@ -165,8 +177,11 @@ def test_decode_sized_norm_becomes_the_prologue_of_the_linear_that_reads_it():
             assert [o["aten"] for o in g.ops] == ["linear.default", "linear.default"], g.notes
             assert fc1["attrs"]["ln_in"] is True and fc1["attrs"]["ln_in_gamma"] == "p_ln_weight" and fc1["attrs"]["epilogue"] == "gelu"
             assert g.root(fc1["in"][0]) == "x"
-        else:           # a wide batch keeps the norm's own launch (the tiled kernel's prologue is the slower choice)
+        elif folded is False:   # between the two, the norm keeps its own launch (the tiled kernel's prologue is the slower choice)
             assert [o["aten"] for o in g.ops] == ["layer_norm.default", "linear.default", "linear.default"] and "ln_in" not in fc1["attrs"]
+        else:           # a wide batch: no pass for the norm at all -- statistics of the input rows, fc1 on the raw rows
+            assert [o["aten"] for o in g.ops] == ["rowstats", "linear.default", "linear.default"] and "ln_in" not in fc1["attrs"]
+            assert fc1["attrs"]["lnf"] == g.ops[0]["out"] and fc1["attrs"]["epilogue"] == "gelu" and g.root(fc1["in"][0]) == "x"
 
 
 @pytest.mark.gpu
@@ -279,7 +294,9 @@ def test_decomposed_export_folds_like_the_composite_one():
     assert aten.count("addmm.default") == 5 and aten.count("mm.default") == 1 and aten.count("native_layer_norm.default") == 2
     g = G.optimize(G.Graph.load(d))
     assert [o["aten"] for o in g.ops].count("gelu.default") == 0 and len(g.ops) == 6
-    assert [o["aten"] for o in g.ops].count("native_layer_norm.default") == 1         # the second one rides in the out-projection
+    # neither norm is left: the first became a pass over x for its row statistics, the second rides in the out-projection's store
+    assert [o["aten"] for o in g.ops].count("native_layer_norm.default") == 0 and g.ops[0]["aten"] == "rowstats"
+    assert sum("stats_out" in o["attrs"] for o in g.ops) == 1 and sum("lnf" in o["attrs"] for o in g.ops) == 2
     fc1 = next(o for o in g.ops if o["attrs"].get("epilogue") == "gelu")
     assert fc1["aten"] == "addmm.default" and g.root("gelu") == fc1["id"]       # gelu read the addmm through a view
     assert sum("residual" in o["attrs"] for o in g.ops) == 2
@@ -533,21 +550,25 @@ def test_patch_embedding_whose_feature_map_is_also_a_result_is_not_folded():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("B", [1, 2])
-def test_dinov2_like_encoder_runs_on_the_kernels(ctx, B):
+@pytest.mark.parametrize("B,image", [(1, 70), (2, 70), (1, 126), (2, 126)])
+def test_dinov2_like_encoder_runs_on_the_kernels(ctx, B, image):
+    """26 token rows per image at 70 x 70 (the norms keep a pass or ride as a GEMM's second result), 82 at 126 x 126 (the
+    norms between GEMMs are folded away: LayerScale, residual and row statistics in one store, the next GEMM on the raw rows)."""
     import torch
     from juliavision_amd import graph as G
-    m = _dinov2_like(seed=5)
-    x = torch.rand(B, 3, 70, 70).half()
+    m = _dinov2_like(seed=5, image=image)
+    x = torch.rand(B, 3, image, image).half()
     ep = torch.export.export(m, (x,)).run_decompositions()
     g = G.optimize(G.Graph.load(G.convert(ep, "vit")))
     assert g.ops[0]["aten"] == "patch_tokens"
+    tokens = (image // 14) ** 2 + 1
+    assert any("lnf" in o["attrs"] for o in g.ops) == (B * tokens >= 64)
     run = G.Executor(g, m.state_dict(), ctx)
     with torch.no_grad():
         want = m.float()(x.float()).numpy()
     got = run(x.cuda())
     torch.cuda.synchronize()
-    assert got.shape == (B, 26, 128)
+    assert got.shape == (B, tokens, 128)
     assert_parity(got.float().cpu().numpy(), want, what="DINOv2-like encoder from its exported graph")
 
 
@@ -660,18 +681,41 @@ def test_whisper_like_encoder_rewrites():
     assert sum(o["attrs"].get("epilogue") == "gelu" for o in g.ops) == 2 and sum("residual" in o["attrs"] for o in g.ops) == 4
 
 
-@pytest.mark.gpu
-def test_whisper_like_encoder_runs_on_the_kernels(ctx):
+def test_whisper_like_encoder_with_enough_rows_loses_its_norms():
+    """160 frames -> 80 token rows: every norm but the last (the graph's result) is folded away.  The first layer's reads the
+    stem's output (an add of the positions: no GEMM wrote it) and gets a rowstats op; every other one takes the statistics
+    the GEMM before it leaves next to its residual add and clamp."""
     import torch
     from juliavision_amd import graph as G
-    m = _whisper_like_encoder(seed=9)
-    x = torch.randn(1, 16, 60).half()
+    m = _whisper_like_encoder(frames=160)
+    g = G.optimize(G.Graph.load(G.convert(_export_keeping_sdpa(m, torch.randn(1, 16, 160).half()), "enc")))
+    left = [o["aten"] for o in g.ops]
+    assert left.count("rowstats") == 1 and left.count("native_layer_norm.default") == 0 and left.count("clamp.default") == 0, (left, g.notes)
+    grp = [o for o in g.ops if o["aten"] == "linear_group"]
+    assert len(grp) == 2 and all(o["attrs"].get("lnf") and len(o["attrs"]["members"]) == 3 for o in grp)
+    assert grp[0]["attrs"]["lnf"] == g.ops[left.index("rowstats")]["out"]
+    writers = [o for o in g.ops if "stats_out" in o["attrs"]]
+    assert len(writers) == 3 and all("residual" in o["attrs"] for o in writers)              # proj, fc2 of layer 0; proj of layer 1
+    assert writers[1]["attrs"]["clamp"] == 64504.0 and grp[1]["attrs"]["lnf"] == writers[1]["attrs"]["stats_out"]
+    fc1 = [o for o in g.ops if o["attrs"].get("epilogue") == "gelu" and o["aten"] != "convolution.default"]
+    assert [o["attrs"].get("lnf") for o in fc1] == [writers[0]["attrs"]["stats_out"], writers[2]["attrs"]["stats_out"]]
+    last = g.ops[-1]                                                                           # the final norm is returned: it stays a result
+    assert last["attrs"].get("ln_out") is not None and last["attrs"]["clamp"] == 64504.0 and "stats_out" not in last["attrs"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("frames", [60, 160])
+def test_whisper_like_encoder_runs_on_the_kernels(ctx, frames):
+    import torch
+    from juliavision_amd import graph as G
+    m = _whisper_like_encoder(seed=9, frames=frames)
+    x = torch.randn(1, 16, frames).half()
     run = G.Executor(G.optimize(G.Graph.load(G.convert(_export_keeping_sdpa(m, x), "enc"))), m.state_dict(), ctx)
     with torch.no_grad():
         want = m.float()(x.float()).numpy()
     got = run(x.cuda())
     torch.cuda.synchronize()
-    assert got.shape == (1, 30, 128)
+    assert got.shape == (1, frames // 2, 128)
     assert_parity(got.float().cpu().numpy(), want, what="Whisper-like encoder from its exported graph")
 
 
