@@ -28,7 +28,10 @@ after a linear rides in its GEMM store (``fold_residuals``; the reference's own
 next item, plans/perf-plan.md:4074-4095), and attention writes its output
 token-major when the graph transposes it straight back (``fold_sdpa_transpose``);
 attention exported as ``bmm`` + ``_softmax`` + ``bmm`` (DINOv2) is put back together
-(``fold_attention``).
+(``fold_attention``).  A layer norm that only linear ops read, over enough rows for
+the tiled GEMMs, gets no pass of its own (``fold_norms_away``): its readers run on
+the raw rows with prepared weights, the row statistics come out of the GEMM that
+wrote those rows.
 
 The decoder step (tools/export_whisper_decoder.py:90-240) is functional: it takes
 the self-attention cache, writes the new token's rows with ``index_copy`` /
