@@ -106,9 +106,15 @@ constexpr int flash_vld(int EP) { return EP == 96 ? EP : EP + 32; }
 // j + 1 are requested while block j is worked on (two register sets, like the scores) and join the scores, times
 // log2(e), ahead of the exponentials -- the reference's bias term of attention.jl:55-59, which its own fused kernel
 // declines (flash.jl:1327).
-template <int EP, bool PP, int KH = 1, int BIAS = 0>      // BIAS: 0 none, 1 fp16, 2 fp32
+// BIAS = 3: an fp16 mask that depends on the key only (the query axis broadcast: a padding mask (B, 1, 1, Lk), a per-head key
+// bias).  It costs no vector arithmetic at all: the extra k-step that subtracts the reference point also carries
+// mask[key] * log2(e) -- the key-side operand holds the key's mask value in two slots, the query-side operand log2(e)
+// split into an fp16 part just below it and the (positive) rest, so a -inf mask value gives -inf through both products
+// and never meets a zero or a negative factor.  The (b, h) row of the mask sits in LDS behind the stages, copied there
+// once, zero beyond the last key (FLASH_KEYMASK_MAX keys at most): a first product reads one value per lane and tile.
+template <int EP, bool PP, int KH = 1, int BIAS = 0>      // BIAS: 0 none, 1 fp16, 2 fp32, 3 fp16 by key only
 __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH == 1 && (BIAS == 0 || EP == 64)) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
-    static_assert(BIAS == 0 || (!PP && KH == 1) || (PP && KH == 2 && BIAS == 1 && EP == 64), "the mask rides in the four-wave form, and as fp16 in the key-halves form");
+    static_assert(BIAS == 0 || (!PP && KH == 1) || (PP && KH == 2 && (BIAS == 1 || BIAS == 3) && EP == 64), "the mask rides in the four-wave form, and as fp16 in the key-halves form");
     // PP with KH = 2: the two key-half groups of the eight-wave form (same 128 queries) take turns at the vector
     // and matrix units like the two query groups of the 256-query form do; every thread stages.
     constexpr int BC = 64, BR = (PP && KH == 1) ? 256 : 128, NT = (KH == 2 || PP) ? 512 : 256;     // NT: threads that stage K and V
@@ -122,6 +128,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     extern __shared__ __align__(16) char smem[];
     half_t (*Ks)[BCS * KLD] = reinterpret_cast<half_t (*)[BCS * KLD]>(smem);
     half_t (*Vs)[BCS * VLD] = reinterpret_cast<half_t (*)[BCS * VLD]>(smem + 3 * BCS * KLD * 2);
+    half_t *Ms = reinterpret_cast<half_t *>(smem + 3 * BCS * (KLD + VLD) * 2);       // BIAS 3: the mask row, then zeros
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int tid = threadIdx.x & (NT - 1);                  // index among the staging threads
@@ -251,6 +258,10 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
 #pragma unroll
     for (int j = 0; j < 8; j++) { kext[j] = (half_t)0.0f; qext[j] = (half_t)0.0f; }
     if (hl == 0) kext[0] = (half_t)1.0f;
+    if constexpr (BIAS == 3) {
+        // log2(e) = 1.4423828125 (the fp16 value below it) + 0.00031220...: both factors positive
+        if (hl == 0) { qext[1] = (half_t)1.4423828125f; qext[2] = (half_t)(1.44269504088896340736f - 1.4423828125f); }
+    }
     float m_ref = 0.0f, l_run = 0.0f;    // m_ref is always exactly representable in fp16
     bool first = true;
 
@@ -270,8 +281,19 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         }
         if (nblk > 0 && loader) store_kv(0);
         if (nblk > 1 && loader) store_from(kr1, vr1, 1);
+        if constexpr (BIAS == 3) {
+            // every block this workgroup walks, whole: keys past the last one read zero (the ragged block's own test
+            // excludes them), and so does the slot behind them, which the lanes that feed no mask value read
+            const unsigned short *mrow = reinterpret_cast<const unsigned short *>(p.bias) + (long)h * p.bs[2] + (long)b * p.bs[3];
+            for (int i = threadIdx.x; i <= nblk * BCS; i += (int)blockDim.x)
+                reinterpret_cast<unsigned short *>(Ms)[i] = i < p.Lk ? mrow[(long)i * p.bs[0]] : (unsigned short)0;
+        }
     }
     __syncthreads();
+    // BIAS 3: where a lane finds the mask value it feeds to the extra k-step (key l32 of a tile, from the lanes that hold
+    // k-slots 0..7; the others read the zero behind the row)
+    const int msel = hl == 0 ? 1 : 0;
+    const int moff = hl == 0 ? gk + l32 : nblk * BCS;
 
     // lane s of a 16-lane block addresses key (s/4), head-dim 4 (s%4) .. +3 of its 4 x 16 patch
     const int vtoff = (gk + 4 * hl + ((lane & 15) >> 2)) * VLD + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
@@ -279,7 +301,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // t = s*scale*log2(e) - M, straight out of the MFMA chain
-    auto qk = [&](float16v (&s)[2], int st) {
+    auto qk = [&](float16v (&s)[2], int st, int jblk) {
         const half_t *kbase = &Ks[st][ktoff];
 #pragma unroll
         for (int kt = 0; kt < 2; kt++) {
@@ -291,7 +313,13 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
 #pragma unroll
             for (int ks = 1; ks < KS; ks++)
                 s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8v *>(kp_ + 16 * ks), qf[ks], s[kt], 0, 0, 0);
-            if constexpr (!SEED) s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, s[kt], 0, 0, 0);
+            if constexpr (BIAS == 3) {
+                half8v kx = kext;
+                const half_t m = Ms[moff + (min(jblk, nblk - 1) * BCS + 32 * kt) * msel];      // (the product issued after the last block stays inside the row)
+                kx[1] = m;
+                kx[2] = m;
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kx, qext, s[kt], 0, 0, 0);
+            } else if constexpr (!SEED) s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kext, qext, s[kt], 0, 0, 0);
         }
     };
     // p = 2^t as fp16 MFMA operands; the row sum is kept in fp32 with plain adds (v_dot2_f32_f16 on the
@@ -313,12 +341,12 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
     // key0 + 32 kt + 8 g + 4 hl .. +3), raw as they lie in memory.  Runs past the last key read nothing.
     struct BiasRegs { u32x4 w[BIAS == 2 ? 8 : (BIAS == 1 ? 4 : 1)]; };
     const char *brow = nullptr;
-    if constexpr (BIAS != 0) {
+    if constexpr (BIAS == 1 || BIAS == 2) {
         const int qr = min(q0 + l32, p.Lq - 1);
         brow = reinterpret_cast<const char *>(p.bias) + ((long)qr * p.bs[1] + (long)h * p.bs[2] + (long)b * p.bs[3]) * (BIAS == 2 ? 4 : 2);
     }
     auto load_bias = [&](BiasRegs &br, int j) {
-        if constexpr (BIAS != 0) {
+        if constexpr (BIAS == 1 || BIAS == 2) {
             const int key0 = j * BCS + gk;
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
@@ -347,7 +375,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         }
     };
     auto add_bias = [&](float16v (&sc)[2], const BiasRegs &br) {
-        if constexpr (BIAS != 0) {
+        if constexpr (BIAS == 1 || BIAS == 2) {
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -367,10 +395,9 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         }
     };
     BiasRegs ba, bb;
-    if (nblk > 0) load_bias(ba, 0);
-
     float16v sa[2], sb[2];
-    if (nblk > 0) qk(sa, 0);
+    if constexpr (BIAS == 1 || BIAS == 2) { if (nblk > 0) load_bias(ba, 0); }
+    if (nblk > 0) qk(sa, 0, 0);
 
     // One key block: sc holds its scores (computed one iteration earlier), sn receives the next block's.
     auto iter = [&](auto MASK_, float16v (&sc)[2], float16v (&sn)[2], BiasRegs &bc, BiasRegs &bn, int j) {
@@ -379,7 +406,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         const int st = j % 3, st1 = (j + 1) % 3, st2 = (j + 2) % 3;
         const bool next2 = j + 2 < nblk && loader;
         if (next2) load_kv((j + 2) * BCS);
-        if constexpr (BIAS != 0) {
+        if constexpr (BIAS == 1 || BIAS == 2) {
             if (j + 1 < nblk) load_bias(bn, j + 1);
             add_bias(sc, bc);
         }
@@ -405,7 +432,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
         // assignment loses 4 %).  Between the ping-pong's halves priorities change nothing.
         if constexpr (!PP) {
             __builtin_amdgcn_s_setprio(1);
-            qk(sn, st1);
+            qk(sn, st1, j + 1);
         }
         half8v pf[2][2];
         float l_new = l_run;
@@ -489,7 +516,7 @@ __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH
                 }
         }
         if constexpr (PP) {
-            qk(sn, st1);         // the next block's scores, against the reference point as it stands now
+            qk(sn, st1, j + 1);  // the next block's scores, against the reference point as it stands now
             // the matrix half's fragment reads (V for the second product, K for the first) run ten ahead of the MFMAs
             // that consume them: config 3 18.9 -> 18.3 us, config 2 21.5 -> 21.0 us; six ahead or all 24 ahead lose
             constexpr int NRD = 4 * ET * 2 + 2 * KS, NMF = 4 * ET + 2 * KS + 2, AHEAD = 10;
@@ -1498,6 +1525,9 @@ __global__ void sdpa_merge_kernel(SdpaArgs p) {
 
 // ------------------------------------------------------------------------------------------
 constexpr int flash_lds_bytes(int EP) { return 3 * 64 * (EP + 8) * 2 + 3 * 64 * flash_vld(EP) * 2; }
+// A mask that depends on the key only rides in LDS behind the stages: whole key blocks (of `bcs` keys) and one zero
+constexpr int FLASH_KEYMASK_MAX = 4096;
+constexpr int flash_keymask_bytes(int64_t Lk, int bcs) { return (int)(((Lk + bcs - 1) / bcs * bcs + 1) * 2 + 15) / 16 * 16; }
 constexpr int flash_short_lds_bytes(int NW) { return NW * 64 * flash_vld(64) * 2; }
 constexpr int flash_pair_lds_bytes() { return 4 * (64 * (64 + 8) * 2 + 64 * flash_vld(64) * 2); }
 
@@ -1659,8 +1689,10 @@ int launch_decode(SdpaArgs &a, hipStream_t st) {
 }
 
 // A mask the fused kernel can carry: keys contiguous (a lane reads runs of four), the other axes any stride including
-// broadcast; fp16 runs are read as two dwords, so every row must start on a 4-byte boundary.
+// broadcast; fp16 runs are read as two dwords, so every row must start on a 4-byte boundary.  An fp16 mask with the
+// query axis broadcast has no such conditions.
 bool flash_bias_ok(const SdpaArgs &a) {
+    if (!a.bias_f32 && (a.bs[1] == 0 || a.Lq == 1) && a.Lk <= FLASH_KEYMASK_MAX) return aligned_to(a.bias, 2);      // the same for every query: copied to LDS a value at a time
     if (a.bs[0] != 1 && a.Lk != 1) return false;
     if (a.bias_f32) return aligned_to(a.bias, 4);
     return aligned_to(a.bias, 4) && a.bs[1] % 2 == 0 && a.bs[2] % 2 == 0 && a.bs[3] % 2 == 0;
@@ -1733,6 +1765,10 @@ int mi_sdpa_init() {
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false, 1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false, 1, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false, 1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 128)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 1, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false, 1, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false, 1, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 64)) != hipSuccess;
     return bad;
 }
 
@@ -1799,8 +1835,18 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
             a.nsplit = 1;
             dim3 grid((unsigned)ceil_div(Lq, 128), (unsigned)H, (unsigned)B);
             const bool f32 = a.bias_f32 != 0;
+            const bool halves = E <= 64 && ceil_div(Lq, 128) * H * B <= (int64_t)mi_num_cus() && Lk >= 256;
+            // an fp16 mask that is the same for every query (a padding mask, a per-head key bias) enters with the first
+            // product's extra k-step and costs no vector work
+            if (!f32 && (a.bs[1] == 0 || Lq == 1) && Lk <= FLASH_KEYMASK_MAX) {
+                const int m64 = flash_keymask_bytes(Lk, 64), m128 = flash_keymask_bytes(Lk, 128);
+                if (halves)       hipLaunchKernelGGL((flash_fwd_kernel<64, true, 2, 3>), grid, dim3(512), 2 * flash_lds_bytes(64) + m128, st, a);
+                else if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 3>), grid, dim3(256), flash_lds_bytes(64) + m64, st, a);
+                else if (E <= 96) hipLaunchKernelGGL((flash_fwd_kernel<96, false, 1, 3>), grid, dim3(256), flash_lds_bytes(96) + m64, st, a);
+                else              hipLaunchKernelGGL((flash_fwd_kernel<128, false, 1, 3>), grid, dim3(256), flash_lds_bytes(128) + m64, st, a);
+            }
             // an fp16 mask on a grid of at most one workgroup per CU: the key-halves form carries it too
-            if (E <= 64 && !f32 && ceil_div(Lq, 128) * H * B <= (int64_t)mi_num_cus() && Lk >= 256)
+            else if (halves && !f32)
                 hipLaunchKernelGGL((flash_fwd_kernel<64, true, 2, 1>), grid, dim3(512), 2 * flash_lds_bytes(64), st, a);
             else if (E <= 64) { if (f32) hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 2>), grid, dim3(256), flash_lds_bytes(64), st, a);
                                 else     hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 1>), grid, dim3(256), flash_lds_bytes(64), st, a); }

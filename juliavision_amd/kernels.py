@@ -605,8 +605,9 @@ def sdpaplan(ctx: Ctx, q, k, v, bias=None, scale=None, kv_len=None):
         # other axis may broadcast); everything else is the rows kernel's.  The C planner sees only "a mask" and plans a
         # dense fp16 one, so the mask's own layout is judged here, as mi_sdpa_f16 judges it at the call.
         bst = list(_bias_strides(bias, Lk, Lq, H, Bq))
-        fused = path == 1 and (bst[0] == 1 or Lk == 1) and bias.data_ptr() % 4 == 0 and \
-            (bias.dtype == torch.float32 or all(x % 2 == 0 for x in bst[1:]))
+        by_key = bias.dtype == torch.float16 and (bst[1] == 0 or Lq == 1) and Lk <= 4096    # the same for every query: no layout conditions
+        fused = path == 1 and (by_key or ((bst[0] == 1 or Lk == 1) and bias.data_ptr() % 4 == 0 and
+                                          (bias.dtype == torch.float32 or all(x % 2 == 0 for x in bst[1:]))))
         if fused:
             return FlashPlan(1)
         ns1 = C.c_int(1)

@@ -200,6 +200,41 @@ def test_additive_mask_rides_in_the_fused_kernel(ctx, B, H, Lq, Lk, E, kind):
         np.testing.assert_allclose(got.astype(np.float32), other.astype(np.float32), rtol=2e-3, atol=2e-3)
 
 
+@pytest.mark.parametrize("B,H,Lq,Lk,E,kind", [
+    (2, 3, 200, 136, 64, "values"),       # (B,1,1,Lk): random finite values, four-wave form, a ragged last block
+    (2, 3, 200, 333, 64, "holes"),        # 0 / -inf with masked keys anywhere, not only at the end; odd row length
+    (1, 20, 1500, 1500, 64, "holes"),     # config 2's grid: the eight-wave key-halves form
+    (2, 4, 300, 700, 64, "perhead"),      # (B,H,1,Lk): a different key bias per head, key-halves form
+    (3, 2, 150, 450, 64, "values"),       # key-halves form, second half of the last stage with two keys
+    (2, 2, 128, 130, 72, "holes"),        # the 96-wide instance
+    (1, 2, 192, 320, 128, "perhead"),     # the 128-wide instance
+    (1, 2, 128, 64, 64, "allmasked"),     # every key -inf: zeros, as kv_len = 0 gives
+    (1, 1, 128, 4096, 64, "holes"),       # the longest row that is kept in LDS
+    (1, 1, 128, 4160, 64, "holes"),       # longer ones are read like any other mask
+])
+def test_key_only_mask_enters_with_the_first_product(ctx, B, H, Lq, Lk, E, kind):
+    """An fp16 mask that is the same for every query -- a padding mask (B,1,1,Lk), a per-head key bias (B,H,1,Lk) -- is
+    added by the first product's extra k-step, not by vector instructions: held to the same oracle as the dense mask,
+    and to the dense-mask kernel's own result on the mask written out per query."""
+    q, k, v = _qkv(B, H, Lq, Lk, E, 187)
+    rng = np.random.default_rng(188)
+    Hm = H if kind == "perhead" else 1
+    if kind in ("values", "perhead"):
+        bias = (rng.standard_normal((B, Hm, 1, Lk)) * 3).astype(np.float16)
+    elif kind == "holes":
+        bias = np.where(rng.random((B, Hm, 1, Lk)) < 0.3, -np.inf, 0.0).astype(np.float16)
+        bias[..., 0] = 0.0                                             # at least one key stays
+    else:
+        bias = np.full((B, Hm, 1, Lk), -np.inf, dtype=np.float16)
+    got = _check(ctx, q, k, v, bias=bias, expect="FlashPlan", what=f"key-only mask {kind} {B},{H},{Lq},{Lk},{E}")
+    if kind == "allmasked":
+        assert np.all(got == 0)
+        return
+    dense = np.ascontiguousarray(np.broadcast_to(bias, (B, H, Lq, Lk)))
+    other = _check(ctx, q, k, v, bias=dense, what="the same mask written out per query")
+    np.testing.assert_allclose(got.astype(np.float32), other.astype(np.float32), rtol=2e-3, atol=2e-3)
+
+
 def test_mask_the_fused_kernel_cannot_read_takes_the_rows_kernel(ctx):
     q, k, v = _qkv(1, 2, 128, 129, 64, 90)
     bias = oracle.randn_f16((1, 2, 128, 129), 91)                     # fp16 rows of 129: every other row at a 2-byte offset
