@@ -114,7 +114,8 @@ constexpr int flash_vld(int EP) { return EP == 96 ? EP : EP + 32; }
 // once, zero beyond the last key (FLASH_KEYMASK_MAX keys at most): a first product reads one value per lane and tile.
 template <int EP, bool PP, int KH = 1, int BIAS = 0>      // BIAS: 0 none, 1 fp16, 2 fp32, 3 fp16 by key only
 __global__ __launch_bounds__((PP || KH == 2) ? 512 : 256, (EP <= 96 && !PP && KH == 1 && (BIAS == 0 || EP == 64)) ? 2 : 1) void flash_fwd_kernel(SdpaArgs p) {
-    static_assert(BIAS == 0 || (!PP && KH == 1) || (PP && KH == 2 && (BIAS == 1 || BIAS == 3) && EP == 64), "the mask rides in the four-wave form, and as fp16 in the key-halves form");
+    static_assert(BIAS == 0 || (!PP && KH == 1) || (PP && KH == 2 && (BIAS == 1 || BIAS == 3) && EP == 64) || (PP && BIAS == 3 && EP == 64),
+                  "the mask rides in the four-wave form, and as fp16 in the key-halves form; one that depends on the key only in every form");
     // PP with KH = 2: the two key-half groups of the eight-wave form (same 128 queries) take turns at the vector
     // and matrix units like the two query groups of the 256-query form do; every thread stages.
     constexpr int BC = 64, BR = (PP && KH == 1) ? 256 : 128, NT = (KH == 2 || PP) ? 512 : 256;     // NT: threads that stage K and V
@@ -1767,6 +1768,7 @@ int mi_sdpa_init() {
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false, 1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 2, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * flash_lds_bytes(64) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 128)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, false, 1, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 64)) != hipSuccess;
+    bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<64, true, 1, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(64) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<96, false, 1, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(96) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 64)) != hipSuccess;
     bad |= hipFuncSetAttribute(reinterpret_cast<const void *>(flash_fwd_kernel<128, false, 1, 3>), hipFuncAttributeMaxDynamicSharedMemorySize, flash_lds_bytes(128) + flash_keymask_bytes(FLASH_KEYMASK_MAX, 64)) != hipSuccess;
     return bad;
@@ -1840,7 +1842,13 @@ int mi_sdpa_f16(void *out, int out_dtype, const int64_t out_strides[4],
             // product's extra k-step and costs no vector work
             if (!f32 && (a.bs[1] == 0 || Lq == 1) && Lk <= FLASH_KEYMASK_MAX) {
                 const int m64 = flash_keymask_bytes(Lk, 64), m128 = flash_keymask_bytes(Lk, 128);
-                if (halves)       hipLaunchKernelGGL((flash_fwd_kernel<64, true, 2, 3>), grid, dim3(512), 2 * flash_lds_bytes(64) + m128, st, a);
+                // (the 256-query ping-pong form on the grids that run it unmasked: its first product, seeded with the
+                // reference point, gets the extra k-step for the mask alone)
+                if (E <= 64 && ceil_div(Lq, 256) * H * B * 4 >= (int64_t)mi_num_cus() * 3) {
+                    grid = dim3((unsigned)ceil_div(Lq, 256), (unsigned)H, (unsigned)B);
+                    hipLaunchKernelGGL((flash_fwd_kernel<64, true, 1, 3>), grid, dim3(512), flash_lds_bytes(64) + m64, st, a);
+                }
+                else if (halves)  hipLaunchKernelGGL((flash_fwd_kernel<64, true, 2, 3>), grid, dim3(512), 2 * flash_lds_bytes(64) + m128, st, a);
                 else if (E <= 64) hipLaunchKernelGGL((flash_fwd_kernel<64, false, 1, 3>), grid, dim3(256), flash_lds_bytes(64) + m64, st, a);
                 else if (E <= 96) hipLaunchKernelGGL((flash_fwd_kernel<96, false, 1, 3>), grid, dim3(256), flash_lds_bytes(96) + m64, st, a);
                 else              hipLaunchKernelGGL((flash_fwd_kernel<128, false, 1, 3>), grid, dim3(256), flash_lds_bytes(128) + m64, st, a);

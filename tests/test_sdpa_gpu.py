@@ -209,6 +209,8 @@ def test_additive_mask_rides_in_the_fused_kernel(ctx, B, H, Lq, Lk, E, kind):
     (2, 2, 128, 130, 72, "holes"),        # the 96-wide instance
     (1, 2, 192, 320, 128, "perhead"),     # the 128-wide instance
     (1, 2, 128, 64, 64, "allmasked"),     # every key -inf: zeros, as kv_len = 0 gives
+    (2, 48, 1024, 1024, 64, "holes"),     # a grid large enough for the 256-query ping-pong form
+    (3, 40, 700, 333, 64, "values"),      # ... ragged in queries and keys
     (1, 1, 128, 4096, 64, "holes"),       # the longest row that is kept in LDS
     (1, 1, 128, 4160, 64, "holes"),       # longer ones are read like any other mask
 ])
