@@ -700,9 +700,12 @@ def fold_norms_away(g: Graph) -> Graph:
         while g.buffers[chain[-1]]["kind"] == "view":
             chain.append(g.buffers[chain[-1]]["of"])
         prod = g.op(chain[-1])
+        dense_rows = all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1]) and \
+            (g.buffers[chain[-1]].get("shape") or [None])[-1] == feat
+        if not dense_rows:
+            continue                                    # a permuted or sliced view: its rows are not what the GEMMs and rowstats read
         rides = prod is not None and prod["aten"] in LINEAR_OPS and not any(k in prod["attrs"] for k in ("ln_in", "ln_out")) and \
-            all(g.buffers[c].get("op") in RESHAPES and (g.buffers[c].get("shape") or [None])[-1] == feat for c in chain[:-1]) and \
-            g.buffers[chain[-1]].get("dtype") == "float16" and (g.buffers[chain[-1]].get("shape") or [None])[-1] == feat
+            g.buffers[chain[-1]].get("dtype") == "float16"
         if rides:
             wpos = {"linear.default": 1, "addmm.default": 2, "mm.default": 1}[prod["aten"]]
             wshape = g.buffers[prod["in"][wpos]].get("shape") or []

@@ -184,6 +184,26 @@ def test_decode_sized_norm_becomes_the_prologue_of_the_linear_that_reads_it():
             assert fc1["attrs"]["lnf"] == g.ops[0]["out"] and fc1["attrs"]["epilogue"] == "gelu" and g.root(fc1["in"][0]) == "x"
 
 
+def test_norm_over_a_permuted_view_keeps_its_pass():
+    """The folded form reads the norm's input rows as the GEMM's operand: a channels-first tensor permuted in front of the
+    norm has no such rows, so the norm stays an op."""
+    import torch
+    import torch.nn as nn
+    from juliavision_amd import graph as G
+
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.ln, self.fc = nn.LayerNorm(256), nn.Linear(256, 512)
+
+        def forward(self, x):                       # (B, C, T)
+            return self.fc(self.ln(x.permute(0, 2, 1)))
+
+    ep = torch.export.export(M().eval().half(), (torch.randn(1, 256, 300).half(),))
+    g = G.optimize(G.Graph.load(G.convert(ep, "m")))
+    assert [o["aten"] for o in g.ops] == ["layer_norm.default", "linear.default"] and not any("lnf" in o["attrs"] for o in g.ops)
+
+
 @pytest.mark.gpu
 def test_decode_sized_norm_prologue_runs_on_the_kernels(ctx):
     import torch
