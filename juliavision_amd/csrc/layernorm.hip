@@ -219,10 +219,78 @@ __global__ __launch_bounds__(256) void rowstats_kernel(float *stats, const half_
 }
 
 // Load-time preparation of a folded norm: Wp = fp16(gamma[k] W[k][n]), colsum[n] = sum_k Wp[k][n] (of the ROUNDED
-// values: what the matrix units will multiply), biasp[n] = bias[n] + sum_k beta[k] W[k][n], both in fp32.  One thread per
-// output column walks K; run once per weight.
+// values: what the matrix units will multiply), biasp[n] = bias[n] + sum_k beta[k] W[k][n], both in fp32; run once per
+// weight.  A thread moves sixteen bytes of W at a time; the sums over k are partial sums of fixed k-subsets combined
+// in a fixed order (the same bits on every run).
+//   [K][F] weights: a workgroup owns 64 columns, its thread (chunk c of 8 columns, k-group g of 32) walks k = g, g + 32, ...
+//   [F][K] weights: a workgroup owns 8 columns, a group of 32 lanes walks one of them 256 k at a time
+template <bool B_KN>
 __global__ __launch_bounds__(256) void lnfold_prepare_kernel(half_t *Wp, float *colsum, float *biasp, const half_t *W, const half_t *gamma,
-                                                             const half_t *beta, const half_t *bias, int K, int F, long ldW, int b_kn) {
+                                                             const half_t *beta, const half_t *bias, int K, int F, long ldW) {
+    __shared__ float part[2][32][64];
+    const int tid = threadIdx.x;
+    if constexpr (B_KN) {
+        const int c = tid & 7, g = tid >> 3, n0 = blockIdx.x * 64 + c * 8;
+        float cs[8], bp[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) cs[e] = bp[e] = 0.0f;
+        if (n0 < F) {
+            for (int k = g; k < K; k += 32) {
+                const long at = (long)k * ldW + n0;
+                const half8v w = as_half8(ldg16(W + at));
+                const float gk = gamma ? (float)gamma[k] : 1.0f, bk = beta ? (float)beta[k] : 0.0f;
+                half8v o;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    o[e] = (half_t)(gamma ? gk * (float)w[e] : (float)w[e]);
+                    cs[e] += (float)o[e];
+                    bp[e] = fmaf(bk, (float)w[e], bp[e]);
+                }
+                *reinterpret_cast<half8v *>(Wp + at) = o;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) { part[0][g][c * 8 + e] = cs[e]; part[1][g][c * 8 + e] = bp[e]; }
+        __syncthreads();
+        if (tid < 64 && blockIdx.x * 64 + tid < F) {
+            const int n = blockIdx.x * 64 + tid;
+            float a = 0.0f, b = bias ? (float)bias[n] : 0.0f;
+            for (int q = 0; q < 32; q++) { a += part[0][q][tid]; b += part[1][q][tid]; }
+            colsum[n] = a;
+            biasp[n] = b;
+        }
+    } else {
+        const int l = tid & 31, n = blockIdx.x * 8 + (tid >> 5);
+        float cs = 0.0f, bp = 0.0f;
+        if (n < F) {
+            for (int k0 = l * 8; k0 < K; k0 += 256) {
+                const long at = (long)n * ldW + k0;
+                const half8v w = as_half8(ldg16(W + at));
+                half8v o;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    o[e] = (half_t)(gamma ? (float)gamma[k0 + e] * (float)w[e] : (float)w[e]);
+                    cs += (float)o[e];
+                    if (beta) bp = fmaf((float)beta[k0 + e], (float)w[e], bp);
+                }
+                *reinterpret_cast<half8v *>(Wp + at) = o;
+            }
+        }
+        part[0][tid >> 5][l] = cs;
+        part[1][tid >> 5][l] = bp;
+        __syncthreads();
+        if (l == 0 && n < F) {
+            float a = 0.0f, b = bias ? (float)bias[n] : 0.0f;
+            for (int q = 0; q < 32; q++) { a += part[0][tid >> 5][q]; b += part[1][tid >> 5][q]; }
+            colsum[n] = a;
+            biasp[n] = b;
+        }
+    }
+}
+
+// The same, an element at a time: weights whose rows do not start on sixteen bytes or whose extents are not multiples of 8.
+__global__ __launch_bounds__(256) void lnfold_prepare_any_kernel(half_t *Wp, float *colsum, float *biasp, const half_t *W, const half_t *gamma,
+                                                                 const half_t *beta, const half_t *bias, int K, int F, long ldW, int b_kn) {
     const int n = blockIdx.x * 256 + threadIdx.x;
     if (n >= F) return;
     float cs = 0.0f, bp = bias ? (float)bias[n] : 0.0f;
@@ -341,9 +409,14 @@ int mi_lnfold_prepare_f16(void *Wp, float *colsum, float *biasp, const void *W, 
     if (!mi_ready()) return MI_ERROR_DEVICE;
     if (!Wp || !colsum || !biasp || !W || (w_layout != MI_W_KF && w_layout != MI_W_FK)) return MI_DECLINE_OPERANDS;
     if (K < 1 || F < 1 || K > INT32_MAX || F > INT32_MAX || ldW < (w_layout == MI_W_KF ? F : K)) return MI_DECLINE_EXTENT;
-    hipLaunchKernelGGL(lnfold_prepare_kernel, dim3((unsigned)ceil_div(F, 256)), dim3(256), 0, (hipStream_t)stream,
-                       (half_t *)Wp, colsum, biasp, (const half_t *)W, (const half_t *)gamma, (const half_t *)beta, (const half_t *)bias,
-                       (int)K, (int)F, (long)ldW, w_layout == MI_W_KF ? 1 : 0);
+    hipStream_t st = (hipStream_t)stream;
+    half_t *o = (half_t *)Wp;
+    const half_t *w = (const half_t *)W, *g = (const half_t *)gamma, *be = (const half_t *)beta, *bi = (const half_t *)bias;
+    const bool kn = w_layout == MI_W_KF;
+    const bool vec = aligned_to(W, 16) && aligned_to(Wp, 16) && ldW % 8 == 0 && (kn ? F % 8 == 0 : K % 8 == 0);
+    if (!vec)    hipLaunchKernelGGL(lnfold_prepare_any_kernel, dim3((unsigned)ceil_div(F, 256)), dim3(256), 0, st, o, colsum, biasp, w, g, be, bi, (int)K, (int)F, (long)ldW, kn ? 1 : 0);
+    else if (kn) hipLaunchKernelGGL(lnfold_prepare_kernel<true>, dim3((unsigned)ceil_div(F, 64)), dim3(256), 0, st, o, colsum, biasp, w, g, be, bi, (int)K, (int)F, (long)ldW);
+    else         hipLaunchKernelGGL(lnfold_prepare_kernel<false>, dim3((unsigned)ceil_div(F, 8)), dim3(256), 0, st, o, colsum, biasp, w, g, be, bi, (int)K, (int)F, (long)ldW);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 

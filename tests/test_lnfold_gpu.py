@@ -52,6 +52,33 @@ def test_row_statistics(ctx, T, Cn, mean):
     assert np.allclose(mu, x64.mean(1), rtol=1e-5, atol=1e-5) and np.allclose(var, x64.var(1), rtol=1e-4)
 
 
+@pytest.mark.parametrize("K,F,layout,affine", [
+    (1280, 5120, "kf", True), (1280, 3840, "fk", True), (384, 1152, "kf", False), (512, 264, "fk", True),
+    (300, 1000, "kf", True),          # 16-byte rows, K not a multiple of the k-groups
+    (129, 70, "kf", True), (129, 70, "fk", True),     # no 16-byte rows: an element at a time
+])
+def test_prepared_constants(ctx, K, F, layout, affine):
+    """``lnfold_prepare``'s three results against numpy: ``Wp`` = fp16(gamma W) exactly (one rounding of the fp32 product),
+    ``colsum`` the column sums of the ROUNDED ``Wp`` and ``biasp`` = b + beta . W to fp32 summation error, in W's layout."""
+    import torch
+    import juliavision_amd as jv
+    W = oracle.randn_f16((K, F), 41, 0, 1.0 / np.sqrt(K))
+    g = oracle.randn_f16((K,), 42, 1.0, 0.2) if affine else None
+    be = oracle.randn_f16((K,), 43, 0, 0.3) if affine else None
+    b = oracle.randn_f16((F,), 44, 0, 0.1)
+    Wd = to_dev(W) if layout == "kf" else to_dev(np.ascontiguousarray(W.T)).t()
+    fw = jv.lnfold_prepare(ctx, Wd, None if g is None else to_dev(g), None if be is None else to_dev(be), to_dev(b))
+    torch.cuda.synchronize()
+    assert fw.wp.stride() == Wd.stride()
+    wp_want = (W.astype(np.float32) * (g.astype(np.float32)[:, None] if affine else np.float32(1))).astype(np.float16)
+    wp_got = fw.wp.cpu().numpy()
+    assert np.array_equal(wp_got, wp_want)
+    cs_want = wp_want.astype(np.float64).sum(0)
+    bp_want = b.astype(np.float64) + ((be.astype(np.float64)[:, None] * W.astype(np.float64)).sum(0) if affine else 0.0)
+    assert np.allclose(to_host(fw.colsum), cs_want, rtol=1e-5, atol=1e-5 * np.sqrt(K))
+    assert np.allclose(to_host(fw.biasp), bp_want, rtol=1e-5, atol=1e-5 * np.sqrt(K))
+
+
 def _folded(ctx, T, K, F, *, layout="kf", planes=1, epi="none", residual=False, mean=0.0, out_f32=False, gamma=True, beta=True, seed=21):
     import torch
     import juliavision_amd as jv
