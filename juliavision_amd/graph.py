@@ -1616,8 +1616,15 @@ class Executor:
         self.ctx.ws.reset()
         K.convolution_tokens_(self.ctx, out[:, 1:], x, w, bias, xy(a["arg3"]), xy(a["arg4"]), xy(a["arg5"]), residual=pos[1:],
                               act=a.get("epilogue", "none"))
-        for b in range(B):
-            K.add_(self.ctx, out[b, :1], cls, pos[:1])
+        if ("cls", o["id"]) not in self.scaled:          # cls + pos[0]: constants, added once
+            row = torch.empty((1, C), dtype=out.dtype, device=out.device)
+            K.add_(self.ctx, row, cls, pos[:1])
+            self.scaled[("cls", o["id"])] = row
+        row = self.scaled[("cls", o["id"])]
+        if B == 1:
+            K.add_(self.ctx, out[0, :1], cls, pos[:1])
+        else:                                           # one launch for every image: the row read with stride 0 along the batch
+            K.transposeLE_(self.ctx, out[:, :1].view(B, 1, C).unsqueeze(0), row.view(1, 1, C, 1).expand(1, B, C, 1))
 
     def _embedding(self, o):
         """embedding(table, ids) / index.Tensor(table, [ids]) along the first axis (ops.jl:1754-1783, 1524-1640); with
