@@ -305,7 +305,10 @@ int mi_gemm_f16_plan_caps(const int64_t caps[6], const void *Y, const void *X, c
  *   i.e. already in the layout the graph's following permute + reshape produces.
  *   bias: optional additive mask laid out (Lk,Lq,H,B) with element strides
  *   bias_strides[4]; a stride of 0 broadcasts that axis (attention.jl:55-59,
- *   launch.jl:72-75); bias_dtype MI_F16 / MI_F32.
+ *   launch.jl:72-75); bias_dtype MI_F16 / MI_F32.  An fp16 mask whose query
+ *   stride is 0 (a padding mask (B,1,1,Lk), a per-head key bias) over at most 4096
+ *   keys costs the fused kernel no time: give a padding mask in that form rather
+ *   than written out per query.
  *   kv_len: optional device int32[B]; keys >= kv_len[b] get weight exactly 0
  *   (what the decoder's 0 / finfo.min mask does, tools/export_whisper_decoder.py:158-165).
  *   A row with every key excluded yields zeros, not NaN (attention.jl:82-87).
