@@ -41,6 +41,37 @@ def test_attention_random_shapes(ctx, seed):
         assert_parity(to_host(out), oracle.sdpa_threepass_f16(q, k, v, bias, kv_len=lens), what=what)
 
 
+@pytest.mark.parametrize("seed", [5])
+def test_attention_random_key_masks(ctx, seed):
+    """Masks that are the same for every query -- (1,1,1,Lk), (B,1,1,Lk), (B,H,1,Lk), (1,H,1,Lk); values, or 0 / -inf holes --
+    over random extents on both sides of every form the fused kernel has and of the 4096-key limit of the LDS copy."""
+    import torch
+    import juliavision_amd as jv
+    rnd = random.Random(seed)
+    for it in range(60):
+        B, H = rnd.choice([1, 2, 3, 8]), rnd.choice([1, 2, 6, 16, 20, 40])
+        E = rnd.choice([64, 64, 64, 32, 72, 96, 128])
+        Lq, Lk = rnd.choice([64, rnd.randint(64, 400), rnd.randint(64, 1500)]), rnd.choice([rnd.randint(1, 2300), rnd.randint(3900, 4300)])
+        if B * H * Lq * Lk > 6.0e7:
+            H = max(1, int(6.0e7 / (B * Lq * Lk)))
+        shape = rnd.choice([(1, 1, 1, Lk), (B, 1, 1, Lk), (B, H, 1, Lk), (1, H, 1, Lk)])
+        holes = rnd.random() < 0.5
+        what = f"sdpa key mask seed{seed} #{it} B{B} H{H} Lq{Lq} Lk{Lk} E{E} mask{shape} holes={holes}"
+        print(what, flush=True)
+        q, k, v = oracle.randn_f16((B, H, Lq, E), it, 0, 1.5), oracle.randn_f16((B, H, Lk, E), it + 1000), oracle.randn_f16((B, H, Lk, E), it + 2000)
+        if holes:
+            gen = np.random.default_rng(seed * 1000 + it)
+            bias = np.where(gen.random(shape) < 0.4, -np.inf, 0.0).astype(np.float16)
+            bias[..., gen.integers(0, Lk)] = 0.0                     # a key stays in every row
+        else:
+            bias = oracle.randn_f16(shape, it + 3000, 0, 2.0)
+        out = poison(torch.empty((B, H, Lq, E), dtype=torch.float16, device="cuda"))
+        ctx.ws.reset()
+        jv.sdpa(ctx, to_dev(q), to_dev(k), to_dev(v), to_dev(bias), None, out=out)
+        torch.cuda.synchronize()
+        assert_parity(to_host(out), oracle.sdpa_threepass_f16(q, k, v, bias), what=what)
+
+
 @pytest.mark.parametrize("seed", [7, 23])
 def test_gemm_random_shapes(ctx, seed):
     import torch
