@@ -99,7 +99,7 @@ def peak_probe(lib, stream):
     t_cp, _ = timed(copy, 5)
     # one phase boundary of a would-be multi-phase persistent kernel: every compute unit's workgroup at a grid barrier
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    scratch = torch.zeros(16 + 8 * cus, dtype=torch.int32, device="cuda")
+    scratch = torch.zeros(576 + 8 * cus, dtype=torch.int32, device="cuda")
     ROUNDS = 200
 
     def barrier(payload):
@@ -109,8 +109,13 @@ def peak_probe(lib, stream):
     t_bar, _ = timed(lambda: barrier(0), 5)
     t_bar_x, _ = timed(lambda: barrier(1), 5)
     gave_up = int(scratch[4].item())
+    t_bar2, _ = timed(lambda: barrier(2), 5)
+    t_bar2_x, _ = timed(lambda: barrier(3), 5)
+    gave_up |= int(scratch[4].item())
     return {"grid_barrier_us": round(t_bar * 1e6 / ROUNDS, 2), "grid_barrier_with_exchange_us": round(t_bar_x * 1e6 / ROUNDS, 2),
-            "grid_barrier": f"{cus} workgroups, agent-scope atomic add + poll per round; with exchange: 16 B published per workgroup "
+            "grid_barrier_two_level_us": round(t_bar2 * 1e6 / ROUNDS, 2), "grid_barrier_two_level_with_exchange_us": round(t_bar2_x * 1e6 / ROUNDS, 2),
+            "grid_barrier": f"{cus} workgroups, agent-scope atomic add + poll per round (two-level: eight groups with a counter and a release "
+                            f"flag each); with exchange: 16 B published per workgroup "
                             f"before and all {16 * cus} B read back after; {ROUNDS} rounds per launch" + ("; SOME WAITS GAVE UP" if gave_up else ""),
             "mfma_only_tflops": round(flop_fill / t_fill / 1e12, 1),
             "mfma_only_frac_of_peak": round(flop_fill / t_fill / 1e12 / PEAK_F16_TFLOPS, 4),

@@ -95,11 +95,12 @@ int mi_set_phase_probe(void *dev_u64, int64_t workgroups);
  * mi_probe_copy: out[0 .. bytes) = in[0 .. bytes), 16 bytes per lane and step; bytes % 16 == 0.  A kernel of known HBM
  * traffic (bytes read + bytes written).
  * mi_probe_grid_barrier: `workgroups` (<= compute units) workgroups meet `rounds` times at a barrier across the whole
- * grid -- an agent-scope atomic add on a counter in device memory and a bounded poll -- and, with payload != 0, exchange
- * 16 bytes each around it (write-through stores before, reads past the L2 after): what one phase boundary inside a
- * multi-phase persistent kernel would cost.  scratch_u32: 64 + 32 x workgroups bytes of device memory, 16-byte aligned;
- * word 4 is nonzero afterwards if some workgroup gave up waiting (it then ran on without waiting).  Not for use
- * under graph capture (it clears its counter with a memset). */
+ * grid -- an agent-scope atomic add on a counter in device memory and a bounded poll -- and, with bit 0 of payload set,
+ * exchange 16 bytes each around it (write-through stores before, reads past the L2 after): what one phase boundary inside
+ * a multi-phase persistent kernel would cost.  Bit 1 of payload: the barrier in two levels (eight groups of workgroups
+ * with a counter and a release flag each, so that no address sees more than 32 arrivals or pollers).  scratch_u32:
+ * 2304 + 32 x workgroups bytes of device memory, 16-byte aligned; word 4 is nonzero afterwards if some workgroup gave up
+ * waiting (it then ran on without waiting).  Not for use under graph capture (it clears its counters with a memset). */
 int mi_probe_mfma(void *sink, const void *seed_f16, int64_t workgroups, int64_t steps, int gelu, void *stream);
 int mi_probe_grid_barrier(void *scratch_u32, int64_t workgroups, int64_t rounds, int payload, void *stream);
 int mi_probe_copy(void *out, const void *in, size_t bytes, void *stream);

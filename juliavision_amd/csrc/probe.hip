@@ -94,6 +94,44 @@ __global__ __launch_bounds__(64) void probe_grid_barrier_kernel(unsigned *counte
     if (acc == 0x12345u) data[0] = acc;
 }
 
+// The same barrier in two levels, so that no address sees more than 32 arrivals or 32 pollers: a workgroup adds itself to
+// the counter of its group (workgroup index mod 8: on a device that deals workgroups to its XCDs round robin, its XCD),
+// the last arrival of a group adds the group to the counter of groups, the last group releases everyone by writing the
+// round's number into each group's flag, and a workgroup polls its own group's flag.  Counters and flags sit 128 bytes
+// apart (`lines`: word 32 x (1 + g) the counter of group g, word 32 x 9 the counter of groups, word 32 x (10 + g) the
+// flag of group g); they only ever grow, so nothing is reset between rounds.  Waits are bounded like the flat form's.
+__global__ __launch_bounds__(64) void probe_grid_barrier2_kernel(unsigned *lines, unsigned *data, unsigned *status, int rounds, int payload, int spin_limit) {
+    const unsigned G = gridDim.x, grp = blockIdx.x & 7u;
+    const unsigned ngrp = G < 8u ? G : 8u, members = (G - grp + 7u) / 8u;
+    unsigned *mine = lines + 32 * (1 + grp), *groups = lines + 32 * 9, *flag = lines + 32 * (10 + grp);
+    bool gave_up = false;
+    unsigned acc = 0;
+    for (int r = 0; r < rounds; r++) {
+        if (payload && threadIdx.x < 4)
+            __hip_atomic_store(data + ((r & 1) * G + blockIdx.x) * 4 + threadIdx.x, (unsigned)(r * 131 + blockIdx.x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (threadIdx.x == 0 && !gave_up) {
+            const unsigned round1 = (unsigned)(r + 1);
+            if (__hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == round1 * members - 1u) {
+                if (__hip_atomic_fetch_add(groups, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == round1 * ngrp - 1u) {
+                    for (unsigned g = 0; g < ngrp; g++)
+                        __hip_atomic_store(lines + 32 * (10 + g), round1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            int spins = 0;
+            while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < round1) {
+                if (++spins > spin_limit) { gave_up = true; __hip_atomic_fetch_or(status, (unsigned)MI_DEVSTAT_STEP_BARRIER, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        __syncthreads();
+        if (payload) {
+            for (unsigned i = threadIdx.x; i < G * 4; i += 64) acc += __hip_atomic_load(data + (r & 1) * G * 4 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (acc == 0x12345u) data[0] = acc;
+}
+
 }  // namespace
 
 extern "C" {
@@ -110,11 +148,15 @@ int mi_probe_mfma(void *sink, const void *seed_f16, int64_t workgroups, int64_t 
 int mi_probe_grid_barrier(void *scratch_u32, int64_t workgroups, int64_t rounds, int payload, void *stream) {
     if (!mi_ready()) return MI_ERROR_DEVICE;
     if (!scratch_u32 || !aligned_to(scratch_u32, 16)) return MI_DECLINE_OPERANDS;
-    if (workgroups < 1 || workgroups > mi_num_cus() || rounds < 1 || rounds > 100000) return MI_DECLINE_EXTENT;
-    unsigned *base = reinterpret_cast<unsigned *>(scratch_u32);      // [0]: counter, [4]: status, [16 ..): two rounds of payload
+    if (workgroups < 1 || workgroups > mi_num_cus() || rounds < 1 || rounds > 100000 || payload < 0 || payload > 3) return MI_DECLINE_EXTENT;
+    // [0]: counter, [4]: status; flat form: two rounds of payload from word 16; two-level form: its counters and flags in
+    // words 32 .. 32 x 18, the payload behind them
+    unsigned *base = reinterpret_cast<unsigned *>(scratch_u32);
     hipStream_t st = (hipStream_t)stream;
-    if (hipMemsetAsync(base, 0, 64, st) != hipSuccess) return MI_ERROR_LAUNCH;
-    hipLaunchKernelGGL(probe_grid_barrier_kernel, dim3((unsigned)workgroups), dim3(64), 0, st, base, base + 16, base + 4, (int)rounds, payload, 1 << 16);
+    const bool two_level = (payload & 2) != 0;
+    if (hipMemsetAsync(base, 0, two_level ? 32 * 18 * 4 : 64, st) != hipSuccess) return MI_ERROR_LAUNCH;
+    if (two_level) hipLaunchKernelGGL(probe_grid_barrier2_kernel, dim3((unsigned)workgroups), dim3(64), 0, st, base, base + 32 * 18, base + 4, (int)rounds, payload & 1, 1 << 16);
+    else           hipLaunchKernelGGL(probe_grid_barrier_kernel, dim3((unsigned)workgroups), dim3(64), 0, st, base, base + 16, base + 4, (int)rounds, payload & 1, 1 << 16);
     return hipGetLastError() == hipSuccess ? MI_OK : MI_ERROR_LAUNCH;
 }
 
